@@ -1,0 +1,266 @@
+/*
+ * C ABI of the MI355X (gfx950) paged-KV decode path: the KV write through
+ * slot_mapping and paged-attention decode over block_tables / seq_lens.
+ *
+ * Every entry point takes plain device pointers, sizes and strides and returns
+ * an int status (0 = ok).  Nothing here allocates, frees or synchronises: work
+ * is enqueued on the hipStream_t the caller passes (NULL = the null stream), so
+ * every call is legal under HIP graph capture.  All pointers are device
+ * pointers unless a comment says "host".
+ *
+ * Reference interfaces these replace (paths relative to the xLLM tree):
+ *   xllm/core/kernels/ops_api.h:31-37          reshape_paged_cache / quant_to_paged_cache
+ *   xllm/core/kernels/param.h:122-157          ReshapePagedCacheParams (tensor contract)
+ *   xllm/core/kernels/cuda/cuda_ops_api.h:43-48,120-136   cuda::reshape_paged_cache, cuda::batch_decode (CSR form)
+ *   xllm/core/kernels/mlu/mlu_ops_api.h:66-77,126-145     quant_to_paged_cache, batch_decode (block_table form)
+ */
+#ifndef XLLM_HIP_PAGED_KV_H_
+#define XLLM_HIP_PAGED_KV_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define XLLM_HIP_ABI_VERSION 1
+
+/* A hipStream_t, passed as an opaque pointer so that C callers need no HIP headers. */
+typedef void* xllm_hip_stream_t;
+
+/* Element types.  Values are part of the ABI. */
+enum xllm_hip_dtype {
+  XLLM_HIP_BF16 = 0,
+  XLLM_HIP_FP16 = 1,
+  XLLM_HIP_FP32 = 2,
+  XLLM_HIP_FP8_E4M3 = 3, /* OCP e4m3fn, the encoding of torch.float8_e4m3fn */
+  XLLM_HIP_INT8 = 4
+};
+
+enum xllm_hip_status {
+  XLLM_HIP_OK = 0,
+  XLLM_HIP_INVALID_ARGUMENT = 1,    /* a size, stride, pointer or dtype violates the contract */
+  XLLM_HIP_UNSUPPORTED = 2,         /* valid request that no kernel here implements */
+  XLLM_HIP_WORKSPACE_TOO_SMALL = 3, /* see xllm_hip_paged_decode_workspace_bytes */
+  XLLM_HIP_RUNTIME_ERROR = 4        /* a HIP launch failed; see xllm_hip_last_error */
+};
+
+/*
+ * One layer's paged KV cache.  Logical coordinates are (block, slot, head, d);
+ * the element (block, slot, head, d) of K lives at
+ *   k_cache + block*stride_block + head*stride_head + slot*stride_slot + d      (elements)
+ * so both reference layouts are expressible without a copy:
+ *   NHD [n_blocks, block_size, Hkv, D] (xllm/core/distributed_runtime/llm_engine.cpp:574-577):
+ *        stride_block = bs*Hkv*D, stride_slot = Hkv*D, stride_head = D
+ *   HND [n_blocks, Hkv, block_size, D] (llm_engine.cpp:595-612, kernels/param.h:133-143):
+ *        stride_block = Hkv*bs*D, stride_head = bs*D, stride_slot = D
+ * HND is the native (fastest) layout of the decode kernel.  V uses the same
+ * strides as K.  head_dim is always contiguous.
+ *
+ * Quantised caches (dtype FP8_E4M3 or INT8) carry one fp32 scale per
+ * (block, slot, head) for K and for V (xllm/core/runtime/worker_impl.cpp:276-287:
+ * the cache shape minus its last dimension); element (block, slot, head) lives at
+ *   k_scale + block*scale_stride_block + head*scale_stride_head + slot*scale_stride_slot.
+ * A dequantised element is  (float)q * scale.
+ */
+typedef struct xllm_hip_kv_cache {
+  void* k_cache;
+  void* v_cache;  /* may be NULL for the write path when value is NULL */
+  float* k_scale; /* NULL unless dtype is FP8_E4M3 / INT8 */
+  float* v_scale;
+  int64_t num_blocks;
+  int32_t block_size;
+  int32_t num_kv_heads;
+  int32_t head_dim;
+  int32_t dtype; /* xllm_hip_dtype of the cache elements */
+  int64_t stride_block;
+  int64_t stride_head;
+  int64_t stride_slot;
+  int64_t scale_stride_block;
+  int64_t scale_stride_head;
+  int64_t scale_stride_slot;
+} xllm_hip_kv_cache;
+
+/*
+ * KV write through slot_mapping: for every token t with slot = slot_mapping[t],
+ *   block = slot / block_size, off = slot % block_size,
+ *   k_cache[block][off][h][d] = key[t*key_token_stride + h*head_dim + d]   (same for V)
+ * — the index math of reshape_paged_cache_kernel
+ * (xllm/core/kernels/cuda/reshape_paged_cache.cu:35-57), behind
+ * xllm::kernel::reshape_paged_cache (xllm/core/kernels/ops_api.cpp:150-180).
+ * Elements are copied verbatim (src_dtype must equal cache->dtype; BF16, FP16,
+ * FP32 or 1-byte types).  key/value are [num_tokens, Hkv, D] with the last two
+ * dimensions contiguous and a free token stride (they are slices of the fused
+ * qkv buffer).  value == NULL writes K only.  A negative slot or a slot beyond
+ * num_blocks*block_size is skipped (the reference would write out of bounds).
+ * Duplicate slots (padding rows all map to slot 0,
+ * xllm/core/framework/batch/batch_input_builder.cpp:517) are legal; which
+ * duplicate wins is unspecified, as in the reference.
+ */
+int xllm_hip_reshape_paged_cache(const xllm_hip_kv_cache* cache,
+                                 const void* key,
+                                 const void* value,
+                                 const int32_t* slot_mapping,
+                                 int64_t num_tokens,
+                                 int64_t key_token_stride,
+                                 int64_t value_token_stride,
+                                 int32_t src_dtype,
+                                 xllm_hip_stream_t stream);
+
+/*
+ * Quantising KV write: per token and per head, symmetric quantisation of the
+ * head_dim values followed by the same scatter as above, plus the scale store —
+ * xllm::kernel::quant_to_paged_cache (xllm/core/kernels/ops_api.cpp:196-210,
+ * xllm/core/kernels/mlu/mlu_ops_api.h:66-77).  src_dtype is BF16, FP16 or FP32;
+ * cache->dtype is INT8 (qmax 127) or FP8_E4M3 (qmax 448).
+ *   absmax = max_d |x_d|
+ *   scale  = max(absmax / qmax, min_scale)   min_scale = FLT_EPSILON (int8), 1/(448*512) (fp8)
+ *            (xllm/core/kernels/cuda/fp8_quant_utils.cuh:38-53)
+ *   q_d    = int8: clamp(rint(x_d / scale), -127, 127)   (round half to even)
+ *            fp8 : e4m3fn_rne(clamp(x_d / scale, -448, 448))  (fp8_quant_utils.cuh:112-131)
+ */
+int xllm_hip_quant_to_paged_cache(const xllm_hip_kv_cache* cache,
+                                  const void* key,
+                                  const void* value,
+                                  const int32_t* slot_mapping,
+                                  int64_t num_tokens,
+                                  int64_t key_token_stride,
+                                  int64_t value_token_stride,
+                                  int32_t src_dtype,
+                                  xllm_hip_stream_t stream);
+
+/*
+ * Paged-attention decode.
+ *
+ *   out[b*n + j, h, :] = sum_t softmax_t(sm_scale * q[b*n + j, h] . K[b, t, h/g]) * V[b, t, h/g]
+ *   t < seq_lens[b] - (n - 1 - j),   g = num_q_heads / num_kv_heads
+ *
+ * with K[b, t] found through the block table: block = table[b][t / block_size],
+ * slot = t % block_size.  n = q_per_seq query tokens per sequence; n = 1 is
+ * plain decode (xllm/core/kernels/mlu/mlu_ops_api.h:126-145 batch_decode,
+ * xllm/core/kernels/cuda/batch_decode.cpp:26-86).  n > 1 is speculative verify:
+ * the n draft tokens are the LAST n tokens of the sequence (already written to
+ * the cache) and token j sees seq_lens[b] - (n-1-j) keys, which is what the
+ * reference expresses by expanding every draft token into its own decode row
+ * with its own kv length (xllm/core/runtime/speculative_worker_impl.cpp:230-243).
+ *
+ * The block list of sequence b is given in one of two forms:
+ *   block_table form (mlu_ops_api.h:130-131): block_table != NULL, row b starts at
+ *       block_table + b*block_table_stride, padded with any valid block id;
+ *       seq_lens[b] is the kv length.
+ *   CSR form (cuda_ops_api.h:129-131): block_table == NULL; the list is
+ *       kv_indices[kv_indptr[b] .. kv_indptr[b+1]) and the kv length is
+ *       (kv_indptr[b+1]-kv_indptr[b]-1)*block_size + kv_last_page_len[b].
+ *
+ * q/out are [batch*n, num_q_heads, head_dim] of q_dtype (BF16, FP16 or FP32),
+ * head_dim contiguous, head stride = head_dim, token strides free.
+ * lse, if not NULL, receives the base-2 log-sum-exp of the scaled scores,
+ *   lse[row, h] = log2(sum_t 2^(log2(e) * sm_scale * q.k_t)),
+ * fp32 [batch*n, num_q_heads] — the quantity the reference's merge consumes
+ * (xllm/core/kernels/cuda/xattention/lse_combine.cu:61-73).
+ * A sequence with kv length 0 yields zeros (lse = -inf).
+ * window_left < 0 disables the sliding window; otherwise query at position p
+ * sees keys p - window_left .. p.
+ */
+typedef struct xllm_hip_decode_args {
+  const void* q;
+  void* out;
+  float* lse; /* may be NULL */
+  int64_t q_token_stride;
+  int64_t out_token_stride;
+  int32_t q_dtype;
+  int32_t batch;
+  int32_t q_per_seq;
+  int32_t num_q_heads;
+  float sm_scale;
+  int32_t window_left;
+  /* block_table form */
+  const int32_t* block_table;
+  int64_t block_table_stride;
+  int32_t max_blocks_per_seq; /* row length of block_table */
+  const int32_t* seq_lens;
+  /* CSR form (used when block_table == NULL) */
+  const int32_t* kv_indptr;
+  const int32_t* kv_indices;
+  const int32_t* kv_last_page_len;
+  /* Host-side hints, as the reference keeps them in AttentionMetadata
+   * (xllm/core/layers/common/attention_metadata.h:75-77).  max_seq_len must be
+   * >= every kv length; total_kv_len (0 = unknown) only tunes the split. */
+  int32_t max_seq_len;
+  int64_t total_kv_len;
+} xllm_hip_decode_args;
+
+/*
+ * Bytes of scratch xllm_hip_paged_decode needs for these sizes (split-KV
+ * partial results and the per-step schedule).  Depends on sizes only, never on
+ * the lengths, so one allocation serves every step.
+ */
+size_t xllm_hip_paged_decode_workspace_bytes(int32_t batch,
+                                             int32_t q_per_seq,
+                                             int32_t num_q_heads,
+                                             int32_t num_kv_heads,
+                                             int32_t head_dim);
+
+/*
+ * Build the per-step split-KV schedule from the kv lengths, on the device
+ * (no host read-back, unlike the reference's layer-0 plan,
+ * xllm/core/layers/cuda/flashinfer_planinfo.cpp:252-253,299-300).  The schedule
+ * is stored at the head of `workspace` and depends only on args' block
+ * list/length fields, batch, q_per_seq, num_q_heads and the cache's
+ * num_kv_heads/head_dim/block_size: it may be built once per step and reused
+ * by every layer's xllm_hip_paged_decode_run with the same workspace.
+ */
+int xllm_hip_paged_decode_plan(const xllm_hip_kv_cache* cache,
+                               const xllm_hip_decode_args* args,
+                               void* workspace,
+                               size_t workspace_bytes,
+                               xllm_hip_stream_t stream);
+
+/* Attention proper; requires a schedule built by xllm_hip_paged_decode_plan in `workspace`. */
+int xllm_hip_paged_decode_run(const xllm_hip_kv_cache* cache,
+                              const xllm_hip_decode_args* args,
+                              void* workspace,
+                              size_t workspace_bytes,
+                              xllm_hip_stream_t stream);
+
+/* plan + run in one call. */
+int xllm_hip_paged_decode(const xllm_hip_kv_cache* cache,
+                          const xllm_hip_decode_args* args,
+                          void* workspace,
+                          size_t workspace_bytes,
+                          xllm_hip_stream_t stream);
+
+/*
+ * Index-only conversion between the two block-list forms
+ * (xllm/core/framework/batch/batch_input_builder.cpp:438-494 builds both from
+ * the same sequences): fills block_table rows (padding with 0) and seq_lens
+ * from the CSR arrays.
+ */
+int xllm_hip_csr_to_block_table(const int32_t* kv_indptr,
+                                const int32_t* kv_indices,
+                                const int32_t* kv_last_page_len,
+                                int32_t batch,
+                                int32_t block_size,
+                                int32_t* block_table,
+                                int64_t block_table_stride,
+                                int32_t max_blocks_per_seq,
+                                int32_t* seq_lens,
+                                xllm_hip_stream_t stream);
+
+/* Message of the last non-OK status returned on this host thread ("" if none). */
+const char* xllm_hip_last_error(void);
+
+/* XLLM_HIP_ABI_VERSION the library was built with. */
+int xllm_hip_abi_version(void);
+
+/* Name of the kernel variant xllm_hip_paged_decode_run would pick for these
+ * arguments ("mfma_d128", "generic", ... or "" if unsupported); host-only, launches nothing. */
+const char* xllm_hip_paged_decode_variant(const xllm_hip_kv_cache* cache,
+                                          const xllm_hip_decode_args* args);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* XLLM_HIP_PAGED_KV_H_ */

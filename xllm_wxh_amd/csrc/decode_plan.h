@@ -1,0 +1,83 @@
+// Split-KV schedule of one decode step and the workspace layout that carries it.
+//
+// A sequence of kv length L is cut into chunks of `chunk_tokens` tokens (a
+// multiple of the 32-token tile): floor(L/C) full chunks and, if L % C != 0,
+// one tail chunk.  One work item = (sequence chunk, kv head, row group); the
+// kernel launched over the items writes one normalised partial output and its
+// base-2 log-sum-exp per item row, and the merge kernel combines a sequence's
+// partials with w_i = 2^(lse_i - lse_total) — the algebra of the reference's
+// two-partial merge (xllm/core/kernels/cuda/xattention/lse_combine.cu:61-73),
+// extended to any number of partials.
+//
+// Full chunks are numbered before tail chunks so that the hardware dispatcher,
+// which starts workgroups in index order, runs the equal-sized long items first
+// and fills the end of the launch with the short tails.
+#pragma once
+
+#include <stddef.h>
+#include <stdint.h>
+
+namespace xllm_hip {
+
+constexpr int kTileTokens = 32;       // tokens per MFMA tile; chunk sizes are multiples of it
+constexpr int kMinChunkTokens = 128;  // smallest split worth a partial round trip
+constexpr int kMaxTargetItems = 4096; // upper bound of the split target (sizes the workspace)
+constexpr int kMaxRowsPerItem = 32;   // query rows (g * n) one work item handles
+
+struct PlanHeader {
+  int32_t total_full;    // number of full sequence-chunks
+  int32_t total_tail;    // number of tail sequence-chunks
+  int32_t chunk_tokens;  // C
+  int32_t total_items;   // (total_full + total_tail) * num_kv_heads * row_groups
+  int32_t pad[12];
+};
+
+struct SeqChunk {
+  int32_t seq;    // sequence index b
+  int32_t chunk;  // chunk index within the sequence (token range [chunk*C, min(L, (chunk+1)*C)))
+};
+
+struct WorkspaceLayout {
+  size_t header;        // PlanHeader
+  size_t kv_len;        // int32 [B]
+  size_t full_prefix;   // int32 [B+1]  first full-chunk slot of sequence b
+  size_t tail_prefix;   // int32 [B+1]  tail-chunk slot (relative to total_full) of sequence b
+  size_t seq_chunks;    // SeqChunk [max_seq_chunks]
+  size_t partial_lse;   // float [max_seq_chunks][n][Hq]
+  size_t partial_out;   // float [max_seq_chunks][n][Hq][D]
+  size_t total_bytes;
+  int64_t max_seq_chunks;
+};
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+inline int row_groups(int q_per_seq, int num_q_heads, int num_kv_heads) {
+  const int rows = q_per_seq * (num_q_heads / num_kv_heads);
+  return (rows + kMaxRowsPerItem - 1) / kMaxRowsPerItem;
+}
+
+// Sum_b ceil(L_b / C) <= sum(L)/C + B and C >= sum(L)*Hkv*RG/target, hence the bound below
+// for every target <= kMaxTargetItems.
+inline WorkspaceLayout workspace_layout(int batch, int q_per_seq, int num_q_heads, int num_kv_heads, int head_dim) {
+  WorkspaceLayout w;
+  w.max_seq_chunks = (int64_t)kMaxTargetItems / num_kv_heads + batch + 1;
+  size_t off = 0;
+  w.header = off;
+  off += sizeof(PlanHeader);
+  w.kv_len = off;
+  off = align_up(off + sizeof(int32_t) * (size_t)batch, 64);
+  w.full_prefix = off;
+  off = align_up(off + sizeof(int32_t) * ((size_t)batch + 1), 64);
+  w.tail_prefix = off;
+  off = align_up(off + sizeof(int32_t) * ((size_t)batch + 1), 64);
+  w.seq_chunks = off;
+  off = align_up(off + sizeof(SeqChunk) * (size_t)w.max_seq_chunks, 256);
+  w.partial_lse = off;
+  off = align_up(off + sizeof(float) * (size_t)w.max_seq_chunks * q_per_seq * num_q_heads, 256);
+  w.partial_out = off;
+  off = align_up(off + sizeof(float) * (size_t)w.max_seq_chunks * q_per_seq * num_q_heads * head_dim, 256);
+  w.total_bytes = off;
+  return w;
+}
+
+}  // namespace xllm_hip

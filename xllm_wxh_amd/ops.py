@@ -1,0 +1,318 @@
+"""Operator mirror of xllm::kernel for the paged-KV decode path, over the C ABI.
+
+Names, argument meaning and error behaviour follow the reference operators:
+
+  reshape_paged_cache(params)   xllm/core/kernels/ops_api.cpp:150-180
+  quant_to_paged_cache(params)  xllm/core/kernels/ops_api.cpp:196-210
+  ReshapePagedCacheParams       xllm/core/kernels/param.h:122-157
+  batch_decode(...)             xllm/core/kernels/mlu/mlu_ops_api.h:126-145 (block_table form)
+  batch_decode_csr(...)         xllm/core/kernels/cuda/cuda_ops_api.h:120-136 (CSR form)
+
+Tensors are torch tensors on the GPU; this module only extracts pointers,
+sizes and strides and passes them, with torch's current stream, through ctypes.
+Outputs are pre-allocated by the caller and mutated in place, as in the
+reference.  The reference aborts on a contract violation (glog CHECK); here the
+library's non-zero status becomes an XllmHipError.
+
+Cache tensors are given in the HND logical shape [num_blocks, num_kv_heads,
+block_size, head_dim] with any strides whose last dimension is contiguous, so an
+NHD buffer [num_blocks, block_size, num_kv_heads, head_dim] (the CUDA backend's
+shape, xllm/core/distributed_runtime/llm_engine.cpp:574-577) is passed as
+`cache.permute(0, 2, 1, 3)` or with `kv_layout="NHD"`, without a copy.
+"""
+import ctypes
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+_DTYPES = {
+    torch.bfloat16: _lib.BF16,
+    torch.float16: _lib.FP16,
+    torch.float32: _lib.FP32,
+    torch.float8_e4m3fn: _lib.FP8_E4M3,
+    torch.int8: _lib.INT8,
+}
+
+
+def _dtype_code(t):
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise _lib.XllmHipError(_lib.INVALID_ARGUMENT, "unsupported dtype %s" % t.dtype)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _require(cond, msg):
+    if not cond:
+        raise _lib.XllmHipError(_lib.INVALID_ARGUMENT, msg)
+
+
+def _as_hnd(cache, kv_layout):
+    if cache is None:
+        return None
+    _require(cache.dim() == 4, "cache must be 4-D, got %d-D" % cache.dim())
+    if kv_layout == "NHD":
+        return cache.permute(0, 2, 1, 3)
+    _require(kv_layout == "HND", "kv_layout must be 'HND' or 'NHD'")
+    return cache
+
+
+def _cache_desc(k_cache, v_cache, k_scale, v_scale, kv_layout):
+    k = _as_hnd(k_cache, kv_layout)
+    v = _as_hnd(v_cache, kv_layout)
+    _require(k.is_cuda, "k_cache must live on the GPU")
+    _require(k.stride(3) == 1, "head_dim of k_cache must be contiguous")
+    if v is not None:
+        _require(v.shape == k.shape and v.dtype == k.dtype and v.stride() == k.stride(),
+                 "v_cache must match k_cache in shape, dtype and strides")
+    d = _lib.KvCacheDesc()
+    d.k_cache = k.data_ptr()
+    d.v_cache = v.data_ptr() if v is not None else None
+    d.num_blocks, d.num_kv_heads, d.block_size, d.head_dim = k.shape
+    d.dtype = _dtype_code(k)
+    d.stride_block, d.stride_head, d.stride_slot = k.stride(0), k.stride(1), k.stride(2)
+    if k_scale is not None:
+        ks = k_scale.permute(0, 2, 1) if kv_layout == "NHD" else k_scale
+        _require(ks.dtype == torch.float32 and tuple(ks.shape) == tuple(k.shape[:3]),
+                 "k_cache_scale must be float32 [num_blocks, num_kv_heads, block_size]")
+        d.k_scale = ks.data_ptr()
+        d.scale_stride_block, d.scale_stride_head, d.scale_stride_slot = ks.stride()
+        if v_scale is not None:
+            vs = v_scale.permute(0, 2, 1) if kv_layout == "NHD" else v_scale
+            _require(vs.dtype == torch.float32 and vs.shape == ks.shape and vs.stride() == ks.stride(),
+                     "v_cache_scale must match k_cache_scale")
+            d.v_scale = vs.data_ptr()
+    return d
+
+
+@dataclass
+class ReshapePagedCacheParams:
+    """Fields of xllm::kernel::ReshapePagedCacheParams (xllm/core/kernels/param.h:122-157)."""
+
+    key: torch.Tensor = None                       # [num_tokens, num_kv_heads, head_dim]
+    value: Optional[torch.Tensor] = None
+    k_cache: torch.Tensor = None                   # [num_blocks, num_kv_heads, block_size, head_dim]
+    v_cache: Optional[torch.Tensor] = None
+    slot_mapping: torch.Tensor = None              # [num_tokens] int32
+    direction: bool = False                        # false = CONTEXT2CACHE; true is not part of this path
+    k_cache_scale: Optional[torch.Tensor] = None   # [num_blocks, num_kv_heads, block_size] float32
+    v_cache_scale: Optional[torch.Tensor] = None
+    kv_layout: str = "HND"
+
+
+def _check_write_inputs(params):
+    key, value = params.key, params.value
+    _require(key is not None and params.k_cache is not None and params.slot_mapping is not None,
+             "key, k_cache and slot_mapping are required")
+    _require(not params.direction, "direction=true (cache to context) is not part of the decode path")
+    _require(key.dim() == 3, "key must be [num_tokens, num_kv_heads, head_dim]")
+    # keys and values should be continuous at n_kv_heads and head_dim dims
+    # (xllm/core/kernels/cuda/reshape_paged_cache.cu:68-69)
+    _require(key.stride(-1) == 1 and key.stride(-2) == key.size(-1),
+             "key must be contiguous in its last two dimensions")
+    if value is not None:
+        _require(value.shape == key.shape and value.dtype == key.dtype, "value must match key")
+        _require(value.stride(-1) == 1 and value.stride(-2) == value.size(-1),
+                 "value must be contiguous in its last two dimensions")
+        _require(params.v_cache is not None, "value given without v_cache")
+    else:
+        _require(params.v_cache is None, "v_cache given without value")
+    sm = params.slot_mapping
+    _require(sm.dtype == torch.int32 and sm.dim() == 1 and sm.is_contiguous(),
+             "slot_mapping must be a contiguous int32 vector")
+    _require(sm.numel() == key.size(0), "slot_mapping has %d entries for %d tokens" % (sm.numel(), key.size(0)))
+
+
+def reshape_paged_cache(params: ReshapePagedCacheParams) -> None:
+    """Verbatim KV write through slot_mapping."""
+    _check_write_inputs(params)
+    lib = _lib.load()
+    desc = _cache_desc(params.k_cache, params.v_cache, None, None, params.kv_layout)
+    _require(params.key.size(1) == desc.num_kv_heads and params.key.size(2) == desc.head_dim,
+             "key heads/head_dim do not match the cache")
+    key, value = params.key, params.value
+    _lib.check(lib.xllm_hip_reshape_paged_cache(
+        ctypes.byref(desc), _ptr(key), _ptr(value), _ptr(params.slot_mapping), key.size(0),
+        key.stride(0), value.stride(0) if value is not None else 0, _dtype_code(key), _stream()))
+
+
+def quant_to_paged_cache(params: ReshapePagedCacheParams) -> None:
+    """Per-token-per-head quantising KV write (int8 or fp8-e4m3 cache + fp32 scales)."""
+    _check_write_inputs(params)
+    # CHECK(params.k_cache_scale.has_value()) (xllm/core/kernels/ops_api.cpp:198-199)
+    _require(params.k_cache_scale is not None, "k_cache_scale is required for quant_to_paged_cache")
+    lib = _lib.load()
+    desc = _cache_desc(params.k_cache, params.v_cache, params.k_cache_scale, params.v_cache_scale,
+                       params.kv_layout)
+    _require(params.key.size(1) == desc.num_kv_heads and params.key.size(2) == desc.head_dim,
+             "key heads/head_dim do not match the cache")
+    key, value = params.key, params.value
+    _lib.check(lib.xllm_hip_quant_to_paged_cache(
+        ctypes.byref(desc), _ptr(key), _ptr(value), _ptr(params.slot_mapping), key.size(0),
+        key.stride(0), value.stride(0) if value is not None else 0, _dtype_code(key), _stream()))
+
+
+# ---------------------------------------------------------------------------------------
+# decode
+# ---------------------------------------------------------------------------------------
+
+_workspaces = {}
+
+
+def decode_workspace_bytes(batch, q_per_seq, num_q_heads, num_kv_heads, head_dim):
+    return _lib.load().xllm_hip_paged_decode_workspace_bytes(batch, q_per_seq, num_q_heads, num_kv_heads, head_dim)
+
+
+def get_workspace(device, nbytes):
+    """Process-wide scratch per device, grown on demand — the role of the reference's
+    FlashinferWorkspace singleton (xllm/core/layers/cuda/flashinfer_workspace.cpp:24-38).
+    Callers that must not allocate pass their own `workspace=` tensor instead."""
+    ws = _workspaces.get(device)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(int(nbytes), dtype=torch.uint8, device=device)
+        _workspaces[device] = ws
+    return ws
+
+
+def _decode_args(query, output, output_lse, block_table, seq_lens, csr, q_per_seq, scale, window_size_left,
+                 max_seq_len, desc):
+    _require(query.dim() in (3, 4), "query must be [tokens, heads, dim] or [batch, q_len, heads, dim]")
+    if query.dim() == 4:
+        # [batch, q_len, Hq, D] (xllm/core/layers/mlu/attention.cpp:263-264)
+        if q_per_seq is None:
+            q_per_seq = query.size(1)
+        _require(query.stride(0) == query.size(1) * query.stride(1), "4-D query must be dense over (batch, q_len)")
+        q3 = query.reshape(-1, query.size(2), query.size(3))
+        o3 = output.reshape(-1, output.size(-2), output.size(-1))
+        _require(o3.data_ptr() == output.data_ptr(), "output must be viewable as [tokens, heads, dim]")
+    else:
+        q3, o3 = query, output
+    q_per_seq = 1 if q_per_seq is None else int(q_per_seq)
+    _require(o3.dim() == 3 and o3.shape == q3.shape and o3.dtype == q3.dtype, "output must match query")
+    _require(q3.stride(2) == 1 and q3.stride(1) == q3.size(2), "query heads/head_dim must be contiguous")
+    _require(o3.stride(2) == 1 and o3.stride(1) == o3.size(2), "output heads/head_dim must be contiguous")
+    _require(q3.size(2) == desc.head_dim, "query head_dim %d != cache head_dim %d" % (q3.size(2), desc.head_dim))
+    _require(q3.size(0) % q_per_seq == 0, "query tokens not divisible by q_per_seq")
+
+    a = _lib.DecodeArgs()
+    a.q, a.out = q3.data_ptr(), o3.data_ptr()
+    a.q_token_stride, a.out_token_stride = q3.stride(0), o3.stride(0)
+    a.q_dtype = _dtype_code(q3)
+    a.batch = q3.size(0) // q_per_seq
+    a.q_per_seq = q_per_seq
+    a.num_q_heads = q3.size(1)
+    a.sm_scale = float(scale)
+    a.window_left = int(window_size_left) if window_size_left is not None else -1
+    if output_lse is not None:
+        _require(output_lse.dtype == torch.float32 and output_lse.is_contiguous()
+                 and output_lse.numel() == q3.size(0) * q3.size(1), "output_lse must be float32 [tokens, heads]")
+        a.lse = output_lse.data_ptr()
+    if csr is None:
+        _require(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.stride(1) == 1,
+                 "block_table must be int32 [batch, max_blocks]")
+        _require(seq_lens.dtype == torch.int32 and seq_lens.is_contiguous(), "seq_lens must be contiguous int32")
+        _require(block_table.size(0) == a.batch and seq_lens.numel() == a.batch,
+                 "block_table/seq_lens rows (%d/%d) != batch %d" % (block_table.size(0), seq_lens.numel(), a.batch))
+        a.block_table = block_table.data_ptr()
+        a.block_table_stride = block_table.stride(0)
+        a.max_blocks_per_seq = block_table.size(1)
+        a.seq_lens = seq_lens.data_ptr()
+    else:
+        indptr, indices, last_page_len = csr
+        for t in (indptr, indices, last_page_len):
+            _require(t.dtype == torch.int32 and t.is_contiguous(), "CSR arrays must be contiguous int32")
+        _require(indptr.numel() == a.batch + 1 and last_page_len.numel() == a.batch, "CSR arrays do not match batch")
+        a.kv_indptr, a.kv_indices, a.kv_last_page_len = indptr.data_ptr(), indices.data_ptr(), last_page_len.data_ptr()
+    a.max_seq_len = int(max_seq_len) if max_seq_len is not None else 0
+    a.total_kv_len = 0
+    return a, (q3, o3)
+
+
+def _run_decode(desc, args, workspace, device, plan=True, run=True):
+    lib = _lib.load()
+    need = lib.xllm_hip_paged_decode_workspace_bytes(args.batch, args.q_per_seq, args.num_q_heads,
+                                                     desc.num_kv_heads, desc.head_dim)
+    ws = workspace if workspace is not None else get_workspace(device, need)
+    wptr, wbytes = ctypes.c_void_p(ws.data_ptr()), ws.numel() * ws.element_size()
+    if plan and run:
+        _lib.check(lib.xllm_hip_paged_decode(ctypes.byref(desc), ctypes.byref(args), wptr, wbytes, _stream()))
+    elif plan:
+        _lib.check(lib.xllm_hip_paged_decode_plan(ctypes.byref(desc), ctypes.byref(args), wptr, wbytes, _stream()))
+    else:
+        _lib.check(lib.xllm_hip_paged_decode_run(ctypes.byref(desc), ctypes.byref(args), wptr, wbytes, _stream()))
+
+
+def batch_decode(query, k_cache, output, block_table, seq_lens, v_cache=None, output_lse=None,
+                 q_quant_scale=None, k_cache_quant_scale=None, v_cache_quant_scale=None, out_quant_scale=None,
+                 alibi_slope=None, mask=None, compute_dtype="float", max_seq_len=0, window_size_left=-1,
+                 window_size_right=-1, scale=1.0, return_lse=False, kv_cache_quant_bit_size=-1, *,
+                 q_per_seq=None, kv_layout="HND", workspace=None, plan=True, run=True):
+    """Paged decode in the block_table form; positional arguments as in
+    xllm::kernel::mlu::batch_decode (xllm/core/kernels/mlu/mlu_ops_api.h:126-145).
+
+    query/output: [batch, q_len, Hq, D] or [batch*q_len, Hq, D]; q_len > 1 is speculative verify
+    with a causal mask among the draft tokens.  Keyword-only extras: q_per_seq (for 3-D queries),
+    kv_layout, workspace (caller-owned scratch), plan/run (build the schedule once per step with
+    run=False, then reuse it for every layer with plan=False).
+    """
+    _require(v_cache is not None, "v_cache is required (MLA-style single-cache decode is outside this path)")
+    for name, t in (("q_quant_scale", q_quant_scale), ("out_quant_scale", out_quant_scale),
+                    ("alibi_slope", alibi_slope), ("mask", mask)):
+        if t is not None:
+            raise _lib.XllmHipError(_lib.UNSUPPORTED, "%s is not supported by the HIP decode path" % name)
+    _require(window_size_right is None or window_size_right < 0, "window_size_right must be -1 for decode")
+    quant = k_cache_quant_scale is not None
+    if kv_cache_quant_bit_size not in (-1, None):
+        _require(kv_cache_quant_bit_size == 8 and quant, "kv_cache_quant_bit_size=8 needs k/v_cache_quant_scale")
+    if quant:
+        _require(v_cache_quant_scale is not None, "v_cache_quant_scale is required with k_cache_quant_scale")
+    if return_lse:
+        _require(output_lse is not None, "return_lse=True needs a pre-allocated output_lse")
+    desc = _cache_desc(k_cache, v_cache, k_cache_quant_scale, v_cache_quant_scale, kv_layout)
+    args, _keep = _decode_args(query, output, output_lse if return_lse or output_lse is not None else None,
+                               block_table, seq_lens, None, q_per_seq, scale, window_size_left, max_seq_len, desc)
+    _run_decode(desc, args, workspace, query.device, plan, run)
+
+
+def batch_decode_csr(query, k_cache, v_cache, paged_kv_indptr, paged_kv_indices, paged_kv_last_page_len,
+                     window_left, sm_scale, output, output_lse=None, *, k_cache_scale=None, v_cache_scale=None,
+                     q_per_seq=None, kv_layout="NHD", workspace=None, plan=True, run=True):
+    """Paged decode in the CSR form of xllm::kernel::cuda::batch_decode
+    (xllm/core/kernels/cuda/cuda_ops_api.h:120-136; the FlashInfer plan/workspace/uri
+    arguments have no counterpart here).  The CUDA backend's cache layout is NHD."""
+    desc = _cache_desc(k_cache, v_cache, k_cache_scale, v_cache_scale, kv_layout)
+    args, _keep = _decode_args(query, output, output_lse, None, None,
+                               (paged_kv_indptr, paged_kv_indices, paged_kv_last_page_len), q_per_seq, sm_scale,
+                               window_left, 0, desc)
+    _run_decode(desc, args, workspace, query.device, plan, run)
+
+
+def decode_variant(query, k_cache, v_cache, block_table, seq_lens, k_cache_quant_scale=None,
+                   v_cache_quant_scale=None, q_per_seq=None, kv_layout="HND"):
+    """Name of the kernel variant batch_decode would run for these tensors."""
+    desc = _cache_desc(k_cache, v_cache, k_cache_quant_scale, v_cache_quant_scale, kv_layout)
+    out = torch.empty_like(query)
+    args, _keep = _decode_args(query, out, None, block_table, seq_lens, None, q_per_seq, 1.0, -1, 0, desc)
+    return _lib.load().xllm_hip_paged_decode_variant(ctypes.byref(desc), ctypes.byref(args)).decode()
+
+
+def csr_to_block_table(paged_kv_indptr, paged_kv_indices, paged_kv_last_page_len, block_size, max_blocks_per_seq):
+    """Index-only conversion CSR -> (block_table padded with 0, seq_lens)."""
+    batch = paged_kv_last_page_len.numel()
+    dev = paged_kv_indptr.device
+    table = torch.empty(batch, max_blocks_per_seq, dtype=torch.int32, device=dev)
+    seq_lens = torch.empty(batch, dtype=torch.int32, device=dev)
+    _lib.check(_lib.load().xllm_hip_csr_to_block_table(
+        _ptr(paged_kv_indptr), _ptr(paged_kv_indices), _ptr(paged_kv_last_page_len), batch, block_size,
+        _ptr(table), table.stride(0), max_blocks_per_seq, _ptr(seq_lens), _stream()))
+    return table, seq_lens
