@@ -1,0 +1,296 @@
+"""Paged-attention decode on the GPU against the fp32 oracle, through the C ABI.
+
+Tolerances (max-abs error of the output): 2e-2 for a bf16 KV cache, 5e-2 for fp8/int8 KV caches
+(compared with attention over the dequantised cache).  Tighter regression bounds are checked as well.
+The MFMA kernel rounds the probabilities to bf16 before the second MFMA (as tensor-core attention
+kernels do) and the output to bf16: each costs up to 2^-9 relative, i.e. about 1e-2 absolute on
+N(0,1) values when a sequence has only a handful of tokens (REG_TOL), and it averages out on long
+ones.  With a quantised cache the rounded weight is p * v_scale (REG_TOL_QUANT).
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import paged_kv_oracle as orc
+from tests.helpers import Case, TOL_BF16_KV, TOL_QUANT_KV, lse_err, max_abs_err
+from xllm_wxh_amd import _lib, ops
+
+pytestmark = pytest.mark.gpu
+
+REG_TOL = 1.2e-2
+REG_TOL_QUANT = 2.5e-2
+LSE_TOL = 1e-4
+
+
+def _check(case, window_left=-1, **kw):
+    ref, lse_ref = case.oracle(window_left)
+    out, lse = case.run(window_left, **kw)
+    assert not torch.isnan(out.float()).any()
+    e = max_abs_err(out, ref)
+    le = lse_err(lse, lse_ref)
+    print("   variant=%s err=%.3e lse_err=%.3e" % (case.variant(), e, le), flush=True)
+    assert e <= case.tol, e
+    assert e <= (REG_TOL_QUANT if case.kv in ("fp8", "int8") else REG_TOL), e
+    assert le <= LSE_TOL, le
+    return out, lse
+
+
+SHAPES = [
+    # B, Hq, Hkv, D, bs, lens, n
+    (2, 8, 2, 128, 16, [100, 33], 1),
+    (4, 32, 8, 128, 16, [1, 31, 32, 33], 1),
+    (3, 32, 8, 128, 16, [4096, 777, 128], 1),      # chunk boundaries of the split
+    (3, 32, 8, 128, 128, [4096, 129, 127], 1),
+    (2, 64, 8, 128, 32, [555, 64], 1),
+    (2, 8, 8, 128, 64, [300, 17], 1),              # MHA, g = 1
+    (2, 56, 8, 128, 16, [300, 517], 1),            # g = 7
+    (2, 64, 8, 128, 128, [3000, 517], 4),          # 32 query rows per kv head: two MFMA tiles
+    (2, 64, 4, 128, 16, [700, 90], 4),             # 64 rows: two row groups
+    (3, 32, 8, 128, 16, [5, 2, 3], 2),             # draft tokens at the very start of a sequence
+]
+
+
+@pytest.mark.parametrize("kv", ["bf16", "fp8", "int8"])
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "B%d_Hq%d_Hkv%d_D%d_bs%d_n%d_L%d" % (s[0], s[1], s[2], s[3], s[4], s[6], max(s[5])))
+def test_mfma_decode_matches_oracle(gpu, shape, kv):
+    B, Hq, Hkv, D, bs, lens, n = shape
+    print("case mfma", shape, kv, flush=True)
+    case = Case(B, Hq, Hkv, D, bs, lens, n=n, kv=kv, seed=11)
+    assert case.variant() == "mfma_d128"
+    _check(case)
+
+
+@pytest.mark.parametrize("kv,qdt", [("bf16", "bf16"), ("fp32", "fp32"), ("fp16", "fp16"), ("fp8", "bf16"), ("int8", "bf16")])
+@pytest.mark.parametrize("shape", [
+    (2, 14, 2, 64, 16, [300, 17], 1),
+    (2, 8, 2, 128, 16, [260, 33], 2),
+    (2, 6, 3, 80, 8, [70, 9], 1),
+    (1, 4, 1, 256, 16, [50], 1),
+], ids=lambda s: "Hq%d_Hkv%d_D%d_bs%d_n%d" % (s[1], s[2], s[3], s[4], s[6]))
+def test_generic_decode_matches_oracle(gpu, shape, kv, qdt, monkeypatch):
+    B, Hq, Hkv, D, bs, lens, n = shape
+    print("case generic", shape, kv, qdt, flush=True)
+    monkeypatch.setenv("XLLM_HIP_DECODE_FORCE_GENERIC", "1")
+    case = Case(B, Hq, Hkv, D, bs, lens, n=n, kv=kv, qdt=qdt, seed=5)
+    assert case.variant() == "generic"
+    ref, lse_ref = case.oracle()
+    out, lse = case.run()
+    e = max_abs_err(out, ref)
+    print("   err=%.3e" % e, flush=True)
+    assert e <= (1e-4 if qdt == "fp32" else 6e-3)  # the generic kernel keeps the probabilities in fp32
+    assert lse_err(lse, lse_ref) <= LSE_TOL
+
+
+@pytest.mark.parametrize("kv", ["bf16", "int8"])
+def test_nhd_layout_and_csr_form(gpu, kv):
+    print("case nhd/csr", kv, flush=True)
+    lens = [1000, 77, 16, 4000]
+    a = Case(4, 32, 8, 128, 16, lens, kv=kv, layout="HND", seed=3)
+    b = Case(4, 32, 8, 128, 16, lens, kv=kv, layout="NHD", seed=3)
+    out_a, lse_a = _check(a)
+    out_b, lse_b = _check(b)
+    assert torch.equal(out_a, out_b) and torch.equal(lse_a, lse_b)  # same values, only the strides differ
+    # CSR form of the same block lists (xllm/core/framework/batch/batch_input_builder.cpp:438-494)
+    lists = [a.table[i, : (L + 15) // 16] for i, L in enumerate(lens)]
+    indptr, indices, last = orc.build_paged_kv_csr(lists, lens, 16)
+    out_c = torch.empty_like(a.q)
+    dev = a.q.device
+    ops.batch_decode_csr(a.q, b.k_cache, b.v_cache, torch.from_numpy(indptr).to(dev), torch.from_numpy(indices).to(dev),
+                         torch.from_numpy(last).to(dev), -1, a.scale, out_c, k_cache_scale=b.k_scale,
+                         v_cache_scale=b.v_scale, kv_layout="NHD")
+    torch.cuda.synchronize()
+    assert torch.equal(out_c, out_a)
+    table, seq_lens = ops.csr_to_block_table(torch.from_numpy(indptr).to(dev), torch.from_numpy(indices).to(dev),
+                                             torch.from_numpy(last).to(dev), 16, a.table.shape[1])
+    torch.cuda.synchronize()
+    assert seq_lens.cpu().tolist() == lens
+    np.testing.assert_array_equal(table.cpu().numpy(), a.table)
+
+
+def test_kv_len_one_returns_value_row_exactly(gpu):
+    # xllm/core/runtime/cuda_graph_executor_test.cpp:150-151
+    print("case kv_len 1", flush=True)
+    case = Case(5, 32, 8, 128, 16, [1, 1, 1, 1, 1], seed=7)
+    out, _ = case.run()
+    v = case.v_cache.cpu()
+    for b in range(5):
+        blk = int(case.table[b, 0])
+        for h in range(32):
+            assert torch.equal(out[b, h].cpu(), v[blk, h // 4, 0])
+
+
+def test_fp8_bytes_decode_to_e4m3fn_values(gpu):
+    """Known-answer test of the in-register dequant: kv_len 1, scale 1 -> the output is the fp8 value."""
+    print("case fp8 KAT", flush=True)
+    bytes_ = torch.arange(256, dtype=torch.uint8)
+    bytes_ = bytes_[(bytes_ & 0x7F) != 0x7F]  # skip the two NaN encodings
+    vals = orc.e4m3fn_to_float(bytes_.numpy())
+    n = bytes_.numel()  # 254
+    B, Hkv, D, bs = 2, 1, 128, 16
+    kc = torch.zeros(B + 1, Hkv, bs, D, dtype=torch.uint8)
+    vc = torch.zeros(B + 1, Hkv, bs, D, dtype=torch.uint8)
+    vc[1, 0, 0, :] = bytes_[:128]
+    vc[2, 0, 0, :n - 128] = bytes_[128:]
+    dev = gpu
+    q = torch.randn(B, 4, D).to(torch.bfloat16).to(dev)
+    out = torch.empty_like(q)
+    ones = torch.ones(B + 1, Hkv, bs, device=dev)
+    ops.batch_decode(q, kc.view(torch.float8_e4m3fn).to(dev), out, torch.tensor([[1], [2]], dtype=torch.int32, device=dev),
+                     torch.tensor([1, 1], dtype=torch.int32, device=dev), vc.view(torch.float8_e4m3fn).to(dev), None, None,
+                     ones, ones, scale=1.0, kv_cache_quant_bit_size=8)
+    torch.cuda.synchronize()
+    got = out.float().cpu().numpy()
+    np.testing.assert_array_equal(got[0, 0], vals[:128])
+    np.testing.assert_array_equal(got[1, 2, : n - 128], vals[128:])
+    assert got[0, 0, 0x7E] == 448.0 and got[0, 0, 0x08] == 2.0 ** -6
+
+
+def test_block_table_permutation_invariance_is_bitwise(gpu):
+    print("case permutation", flush=True)
+    case = Case(3, 32, 8, 128, 16, [2000, 333, 48], seed=9)
+    out, lse = case.run()
+    perm = torch.randperm(case.nblocks, generator=torch.Generator().manual_seed(0))
+    k2, v2 = torch.empty_like(case.k_cache), torch.empty_like(case.v_cache)
+    k2[perm.to(gpu)] = case.k_cache
+    v2[perm.to(gpu)] = case.v_cache
+    table2 = perm[torch.from_numpy(case.table).long()].to(torch.int32).to(gpu)
+    out2 = torch.empty_like(out)
+    ops.batch_decode(case.q, k2, out2, table2, case.seq_lens, v2, scale=case.scale)
+    torch.cuda.synchronize()
+    assert torch.equal(out, out2)
+
+
+@pytest.mark.parametrize("kv", ["bf16", "fp8"])
+def test_garbage_outside_the_sequence_is_ignored(gpu, kv):
+    """Slots past seq_len, padded block-table entries and unused blocks may hold anything (NaN included)."""
+    print("case garbage", kv, flush=True)
+    lens = [37, 16, 1000, 5]
+    case = Case(4, 32, 8, 128, 16, lens, kv=kv, seed=13)
+    ref_out, _ = case.run()
+    used = np.zeros((case.nblocks, 16), bool)
+    for b, L in enumerate(lens):
+        for t in range(L):
+            used[case.table[b, t // 16], t % 16] = True
+    mask = torch.from_numpy(~used).to(gpu)  # [blocks, slots]
+    nan_bits = 0x7F if kv == "fp8" else None
+    for cache in (case.k_cache, case.v_cache):
+        c = cache.permute(0, 2, 1, 3)  # [blocks, slots, heads, dim] view
+        if kv == "fp8":
+            c.view(torch.uint8)[mask] = nan_bits
+        else:
+            c[mask] = float("nan")
+    if case.k_scale is not None:
+        case.k_scale.permute(0, 2, 1)[mask] = float("nan")
+        case.v_scale.permute(0, 2, 1)[mask] = float("inf")
+    # padded entries of the block table point at a block full of NaN (block 0 is never used by make_tables)
+    out, _ = case.run()
+    assert torch.equal(out, ref_out)
+
+
+def test_verify_rows_equal_expanded_decode_rows(gpu):
+    """n draft tokens with the causal mask == n expanded decode rows with kv lens L-n+1..L
+    (xllm/core/runtime/speculative_worker_impl.cpp:230-243)."""
+    print("case verify expansion", flush=True)
+    n = 4
+    lens = [900, 61, 4]
+    case = Case(3, 64, 8, 128, 16, lens, n=n, kv="int8", seed=17)
+    out, lse = _check(case)
+    table_x = case.block_table.repeat_interleave(n, dim=0).contiguous()
+    lens_x = torch.tensor([L - (n - 1 - j) for L in lens for j in range(n)], dtype=torch.int32, device=gpu)
+    out_x = torch.empty_like(out)
+    ops.batch_decode(case.q, case.k_cache, out_x, table_x, lens_x, case.v_cache, None, None, case.k_scale,
+                     case.v_scale, scale=case.scale, kv_cache_quant_bit_size=8)
+    torch.cuda.synchronize()
+    assert float((out.float() - out_x.float()).abs().max()) <= REG_TOL_QUANT
+
+
+def test_zero_length_and_empty_batch(gpu):
+    print("case zero length", flush=True)
+    case = Case(3, 32, 8, 128, 16, [0, 50, 0], seed=19)
+    out, lse = _check(case)
+    assert float(out[0].float().abs().max()) == 0.0 and float(out[2].float().abs().max()) == 0.0
+    assert torch.isneginf(lse[0]).all()
+    # empty batch: nothing to do, no error
+    q = torch.empty(0, 32, 128, dtype=torch.bfloat16, device=gpu)
+    ops.batch_decode(q, case.k_cache, torch.empty_like(q), torch.empty(0, 4, dtype=torch.int32, device=gpu),
+                     torch.empty(0, dtype=torch.int32, device=gpu), case.v_cache, scale=1.0)
+    torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("force_generic", [False, True])
+def test_sliding_window(gpu, force_generic, monkeypatch):
+    print("case window", force_generic, flush=True)
+    if force_generic:
+        monkeypatch.setenv("XLLM_HIP_DECODE_FORCE_GENERIC", "1")
+    case = Case(3, 32, 8, 128, 16, [3000, 517, 20], n=2, seed=21)
+    _check(case, window_left=100)
+    _check(case, window_left=0)
+
+
+@pytest.mark.parametrize("target", ["64", "4096"])
+def test_result_does_not_depend_on_the_split(gpu, target, monkeypatch):
+    print("case split target", target, flush=True)
+    monkeypatch.setenv("XLLM_HIP_DECODE_TARGET_ITEMS", target)
+    case = Case(4, 32, 8, 128, 16, [4096, 2500, 128, 129], seed=23)
+    _check(case)
+
+
+def test_plan_once_run_many(gpu):
+    """The schedule depends only on the lengths: build it once, reuse it for every layer's cache."""
+    print("case plan reuse", flush=True)
+    a = Case(3, 32, 8, 128, 16, [1500, 40, 700], seed=25)
+    b = Case(3, 32, 8, 128, 16, [1500, 40, 700], seed=25, value_seed=26)  # another layer: same tables, other values
+    assert np.array_equal(a.table, b.table)
+    ws = torch.empty(ops.decode_workspace_bytes(3, 1, 32, 8, 128), dtype=torch.uint8, device=gpu)
+    ref_a, _ = a.run(workspace=ws)
+    ref_b, _ = b.run(workspace=ws)
+    a.run(workspace=ws, run=False, lse=False)  # plan only
+    out_a, _ = a.run(workspace=ws, plan=False)
+    out_b, _ = b.run(workspace=ws, plan=False)
+    assert torch.equal(out_a, ref_a) and torch.equal(out_b, ref_b)
+
+
+def test_strided_query_rows(gpu):
+    """q is a slice of the fused qkv projection: its token stride is not Hq*D."""
+    print("case strided q", flush=True)
+    case = Case(2, 32, 8, 128, 16, [300, 40], seed=27)
+    ref, _ = case.run()
+    T, Hq, D = case.q.shape
+    fused = torch.zeros(T, (Hq + 16) * D, dtype=torch.bfloat16, device=gpu)
+    fused[:, : Hq * D] = case.q.view(T, -1)
+    q_view = fused[:, : Hq * D].view(T, Hq, D)
+    assert q_view.stride(0) == (Hq + 16) * D
+    out = torch.empty_like(case.q)
+    ops.batch_decode(q_view, case.k_cache, out, case.block_table, case.seq_lens, case.v_cache, scale=case.scale)
+    torch.cuda.synchronize()
+    assert torch.equal(out, ref)
+
+
+def test_4d_query_shape_of_the_mlu_caller(gpu):
+    # query.view({-1, 1, num_heads, head_size}) (xllm/core/layers/mlu/attention.cpp:263-264)
+    print("case 4-D query", flush=True)
+    case = Case(2, 32, 8, 128, 16, [300, 40], seed=29)
+    ref, _ = case.run()
+    q4 = case.q.view(2, 1, 32, 128)
+    out4 = torch.empty_like(q4)
+    ops.batch_decode(q4, case.k_cache, out4, case.block_table, case.seq_lens, case.v_cache, None, None, None, None,
+                     None, None, None, "float", 300, -1, -1, case.scale, False, -1)
+    torch.cuda.synchronize()
+    assert torch.equal(out4.view(2, 32, 128), ref)
+
+
+def test_errors(gpu):
+    case = Case(1, 32, 8, 128, 16, [20], seed=31)
+    out = torch.empty_like(case.q)
+    with pytest.raises(_lib.XllmHipError) as ei:
+        ops.batch_decode(case.q, case.k_cache, out, case.block_table, case.seq_lens, case.v_cache, scale=1.0,
+                         workspace=torch.empty(1024, dtype=torch.uint8, device=gpu))
+    assert ei.value.status == _lib.WORKSPACE_TOO_SMALL
+    with pytest.raises(_lib.XllmHipError):
+        ops.batch_decode(case.q, case.k_cache, out, case.block_table, case.seq_lens, case.v_cache, scale=1.0,
+                         alibi_slope=torch.zeros(32, device=gpu))
+    big = torch.zeros(2, 1, 16, 512, dtype=torch.bfloat16, device=gpu)
+    qb = torch.zeros(1, 1, 512, dtype=torch.bfloat16, device=gpu)
+    with pytest.raises(_lib.XllmHipError) as ei:
+        ops.batch_decode(qb, big, torch.empty_like(qb), case.block_table, case.seq_lens, big, scale=1.0)
+    assert ei.value.status == _lib.UNSUPPORTED

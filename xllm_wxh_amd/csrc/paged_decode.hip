@@ -782,17 +782,15 @@ __global__ void __launch_bounds__(256) csr_to_block_table_kernel(const int32_t* 
 
 enum Variant { kNone = 0, kMfmaD128 = 1, kGeneric = 2 };
 
+// Split target: about this many work items per launch.  One wave of the attention kernel occupies
+// one SIMD, and the chip has 256 CUs x 4 SIMDs.
 static int target_items() {
-  static int cached = 0;
-  if (cached == 0) {
-    int v = 2048;
-    if (const char* e = getenv("XLLM_HIP_DECODE_TARGET_ITEMS")) {
-      const int t = atoi(e);
-      if (t > 0) v = t;
-    }
-    cached = v > kMaxTargetItems ? kMaxTargetItems : v;
+  int v = 1024;
+  if (const char* e = getenv("XLLM_HIP_DECODE_TARGET_ITEMS")) {
+    const int t = atoi(e);
+    if (t > 0) v = t;
   }
-  return cached;
+  return v > kMaxTargetItems ? kMaxTargetItems : v;
 }
 
 static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
