@@ -1,0 +1,297 @@
+#!/usr/bin/env python3
+"""Benchmark of the paged-KV decode hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+A step is one decode-attention call (split schedule + attention + merge) over one batch of the
+workload, with q, the paged KV cache, the block table and the lengths already resident in HBM.
+Several disjoint KV pools are rotated from step to step so that the 256 MiB Infinity Cache cannot
+serve a repeat.  Prints ONE JSON line: the step time, the achieved HBM rate on the algorithmic
+bytes, the roofline of the dominant kernel and a CPU baseline (the torch-CPU restatement of the
+same path on the host cores).  The KV write of the step's new tokens is timed separately
+(`kv_write_us`).
+
+Two back-to-back regions of K steps each are run after the warm-up.  The first is bracketed by
+synchronisations only and gives `value`.  The second repeats the same K steps with a pair of HIP
+events recorded (by the library, on the launch stream) around the attention kernel of every step
+and gives the kernel's average duration for the roofline; the events cost a few microseconds per
+step, which is why they stay out of the region `value` is taken from.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+REPO = os.path.dirname(os.path.abspath(__file__))
+if REPO not in sys.path:
+    sys.path.insert(0, REPO)
+
+HBM_PEAK_GBPS = 8000.0
+DEFAULT_WORKLOAD = "cfg2_llama3_8b_b64_ctx4k"
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default=DEFAULT_WORKLOAD)
+    ap.add_argument("--pools", type=int, default=3, help="disjoint KV pools rotated between steps")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget of the CPU baseline leg")
+    return ap.parse_args()
+
+
+def build_pools(w, torch, ops, num_blocks, npools, device):
+    """KV pools in the native HND layout.  Quantised pools are produced by the path's own quantising
+    KV write from N(0,1) bf16 values, as the workload defines them."""
+    pools = []
+    gen = torch.Generator(device=device)
+    gen.manual_seed(1234)
+    shape = (num_blocks, w.num_kv_heads, w.block_size, w.head_dim)
+    for _ in range(npools):
+        if w.kv_dtype == "bf16":
+            k = torch.randn(shape, device=device, dtype=torch.bfloat16, generator=gen) * w.value_std
+            v = torch.randn(shape, device=device, dtype=torch.bfloat16, generator=gen) * w.value_std
+            pools.append((k, v, None, None))
+            continue
+        cdt = torch.int8 if w.kv_dtype == "int8" else torch.float8_e4m3fn
+        k = torch.empty(shape, device=device, dtype=cdt)
+        v = torch.empty(shape, device=device, dtype=cdt)
+        ks = torch.empty(shape[:3], device=device, dtype=torch.float32)
+        vs = torch.empty(shape[:3], device=device, dtype=torch.float32)
+        total_slots = num_blocks * w.block_size
+        chunk = 1 << 16
+        for s0 in range(0, total_slots, chunk):
+            t = min(chunk, total_slots - s0)
+            src_k = torch.randn(t, w.num_kv_heads, w.head_dim, device=device, dtype=torch.bfloat16, generator=gen)
+            src_v = torch.randn(t, w.num_kv_heads, w.head_dim, device=device, dtype=torch.bfloat16, generator=gen)
+            slots = torch.arange(s0, s0 + t, device=device, dtype=torch.int32)
+            ops.quant_to_paged_cache(ops.ReshapePagedCacheParams(
+                key=src_k, value=src_v, k_cache=k, v_cache=v, slot_mapping=slots, k_cache_scale=ks,
+                v_cache_scale=vs))
+        torch.cuda.synchronize()
+        pools.append((k, v, ks, vs))
+    return pools
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        sys.stderr.write("bench.py measures the decode path on ONE GPU; --gpus %d is not supported "
+                         "(the path has no cross-GPU step, each GPU would run this same kernel on its own "
+                         "KV-head or sequence shard).\n" % args.gpus)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    from xllm_wxh_amd import ops, workloads
+
+    if not torch.cuda.is_available():
+        sys.stderr.write("bench.py needs a GPU (torch.cuda.is_available() is False)\n")
+        sys.exit(2)
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    w = workloads.WORKLOADS[args.workload]
+    if w.kv_dtype == "fp32":
+        sys.stderr.write("workload %s is the CPU-reference case; pick a GPU workload\n" % w.name)
+        sys.exit(2)
+
+    seq_lens = workloads.make_seq_lens(w, seed=0)
+    table, num_blocks, lists = workloads.make_block_tables(w, seq_lens, seed=0)
+    pools = build_pools(w, torch, ops, num_blocks, args.pools, device)
+    T = w.batch * w.q_per_seq
+    gen = torch.Generator(device=device)
+    gen.manual_seed(99)
+    q = torch.randn(T, w.num_q_heads, w.head_dim, device=device, dtype=torch.bfloat16, generator=gen)
+    out = torch.empty_like(q)
+    block_table = torch.from_numpy(table).to(device)
+    seq_lens_d = torch.from_numpy(seq_lens).to(device)
+    ws = torch.empty(ops.decode_workspace_bytes(w.batch, w.q_per_seq, w.num_q_heads, w.num_kv_heads, w.head_dim),
+                     dtype=torch.uint8, device=device)
+    quant_bits = 8 if w.kv_dtype in ("fp8", "int8") else -1
+
+    def step(i, events=None):
+        k, v, ks, vs = pools[i % len(pools)]
+        ops.batch_decode(q, k, out, block_table, seq_lens_d, v, None, None, ks, vs, scale=w.sm_scale,
+                         q_per_seq=w.q_per_seq, workspace=ws, kv_cache_quant_bit_size=quant_bits,
+                         max_seq_len=int(seq_lens.max()), events=events)
+
+    variant = ops.decode_variant(q, pools[0][0], pools[0][1], block_table, seq_lens_d, pools[0][2], pools[0][3],
+                                 q_per_seq=w.q_per_seq)
+
+    # HIP events around the attention kernel of every timed step (recorded on the launch stream by
+    # the library itself).  torch creates the handles; the first record materialises them.
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    for a, b in ev:
+        a.record()
+        b.record()
+    handles = [(a.cuda_event, b.cuda_event) for a, b in ev]
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    us_per_step = (t1 - t0) * 1e6 / args.steps
+    for i in range(args.steps):
+        step(i, handles[i])
+    torch.cuda.synchronize()
+    us_per_step_with_events = (time.perf_counter() - t1) * 1e6 / args.steps
+    kern_us = sorted(a.elapsed_time(b) * 1e3 for a, b in ev)
+    kern_avg_us = sum(kern_us) / len(kern_us)
+
+    # the step's KV write, timed on its own
+    src_dt = torch.bfloat16
+    new_k = torch.randn(T, w.num_kv_heads, w.head_dim, device=device, dtype=src_dt, generator=gen)
+    new_v = torch.randn(T, w.num_kv_heads, w.head_dim, device=device, dtype=src_dt, generator=gen)
+    slots = torch.from_numpy(workloads.decode_slots(w, seq_lens, lists)).to(device)
+
+    def kv_write(i):
+        k, v, ks, vs = pools[i % len(pools)]
+        p = ops.ReshapePagedCacheParams(key=new_k, value=new_v, k_cache=k, v_cache=v, slot_mapping=slots,
+                                        k_cache_scale=ks, v_cache_scale=vs)
+        if ks is not None:
+            ops.quant_to_paged_cache(p)
+        else:
+            ops.reshape_paged_cache(p)
+
+    for i in range(5):
+        kv_write(i)
+    torch.cuda.synchronize()
+    t2 = time.perf_counter()
+    for i in range(args.steps):
+        kv_write(i)
+    torch.cuda.synchronize()
+    kv_write_us = (time.perf_counter() - t2) * 1e6 / args.steps
+
+    alg_bytes = workloads.algorithmic_bytes(w, seq_lens)
+    achieved_gbps = alg_bytes / us_per_step / 1e3
+    kern_gbps = alg_bytes / kern_avg_us / 1e3
+
+    traffic = None
+    tpath = os.path.join(REPO, "profiles", "hbm_traffic.json")
+    if os.path.exists(tpath):
+        traffic = json.load(open(tpath)).get(w.name, {}).get("traffic_bytes_per_launch")
+
+    result = {
+        "metric": "decode-attn us/step + achieved HBM GB/s (% of 8 TB/s), Llama-3-8B shape b64 ctx4k",
+        "value": round(us_per_step, 2),
+        "unit": "us/step",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(us_per_step / 1e3, 5),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if w.kv_dtype == "bf16" else "bf16 (KV %s)" % w.kv_dtype,
+        "data": "synthetic",
+        "config": {
+            "workload": w.name,
+            "description": w.description,
+            "batch": w.batch,
+            "q_per_seq": w.q_per_seq,
+            "num_q_heads": w.num_q_heads,
+            "num_kv_heads": w.num_kv_heads,
+            "head_dim": w.head_dim,
+            "block_size": w.block_size,
+            "kv_dtype": w.kv_dtype,
+            "sum_seq_len": int(seq_lens.sum()),
+            "max_seq_len": int(seq_lens.max()),
+            "kv_layout": "HND",
+            "kv_pools_rotated": len(pools),
+            "kernel_variant": variant,
+        },
+        "achieved_gbps": round(achieved_gbps, 1),
+        "pct_of_hbm_peak": round(100.0 * achieved_gbps / HBM_PEAK_GBPS, 2),
+        "algorithmic_bytes": int(alg_bytes),
+        "kv_write_us": round(kv_write_us, 2),
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "decode_mfma_d128_kernel" if variant == "mfma_d128" else "decode_generic_kernel",
+            "achieved": round(kern_gbps, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(kern_gbps / HBM_PEAK_GBPS, 4),
+            "traffic": traffic,
+            "kernel_avg_us": round(kern_avg_us, 2),
+            "kernel_min_us": round(kern_us[0], 2),
+            "kernel_max_us": round(kern_us[-1], 2),
+            "measured": "HIP events around the kernel in %d further steps (%.2f us/step with the events)"
+                        % (args.steps, us_per_step_with_events),
+        },
+    }
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(w, torch, pools[0], q, block_table, seq_lens, out, step, args)
+    print(json.dumps(result), flush=True)
+
+
+def cpu_baseline(w, torch, pool, q, block_table, seq_lens, out, step, args):
+    """The torch-CPU restatement of the same step on the host cores (baseline only).  Runs on a
+    bounded sample: the first `nseq` sequences of the batch, chosen so that the leg stays within
+    --cpu-seconds; the per-step figure is scaled to the whole batch by kv tokens."""
+    import numpy as np
+
+    from oracle import torch_cpu_path as tcp
+
+    cores = torch.get_num_threads()
+    k, v, ks, vs = pool
+    total_tokens = int(seq_lens.sum())
+    # sample: whole batch unless it is very large
+    nseq = w.batch
+    budget_tokens = 400_000
+    if total_tokens > budget_tokens:
+        csum = np.cumsum(seq_lens.astype(np.int64))
+        nseq = max(1, int(np.searchsorted(csum, budget_tokens)))
+    sample_tokens = int(seq_lens[:nseq].sum())
+    tbl = block_table[:nseq].cpu()
+    used = torch.unique(tbl.flatten())
+    remap = torch.zeros(int(k.size(0)), dtype=torch.long)
+    remap[used.long()] = torch.arange(used.numel())
+    tbl_c = remap[tbl.long()].to(torch.int32)
+    kc, vc = k[used.to(k.device).long()].cpu(), v[used.to(k.device).long()].cpu()
+    ksc = ks[used.to(k.device).long()].cpu() if ks is not None else None
+    vsc = vs[used.to(k.device).long()].cpu() if vs is not None else None
+    if ks is None:
+        kc, vc = kc.float(), vc.float()
+    qc = q[: nseq * w.q_per_seq].cpu().float()
+    lens_c = torch.from_numpy(seq_lens[:nseq].copy())
+
+    def run():
+        return tcp.paged_decode(qc, kc, vc, tbl_c, lens_c, w.sm_scale, q_per_seq=w.q_per_seq, k_scale=ksc,
+                                v_scale=vsc)
+
+    ref = run()  # warm-up, also the check below
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 3 and (time.perf_counter() - t_start) < args.cpu_seconds:
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    sample_us = sorted(times)[len(times) // 2] * 1e6
+    scaled_us = sample_us * total_tokens / max(sample_tokens, 1)
+    # sanity: the GPU result of the same pool agrees with the CPU one on the sample
+    step(0)
+    torch.cuda.synchronize()
+    err = float((out[: nseq * w.q_per_seq].float().cpu() - ref).abs().max())
+    return {
+        "value": round(scaled_us, 1),
+        "unit": "us/step",
+        "cores": cores,
+        "kind": "port",
+        "sample": "%d of %d sequences (%d of %d kv tokens), median of %d runs after 1 warm-up, %.0f us on the "
+                  "sample, scaled by kv tokens; torch-CPU fp32 gather+bmm+softmax+bmm"
+                  % (nseq, w.batch, sample_tokens, total_tokens, len(times), sample_us),
+        "gpu_vs_cpu_max_abs_err_on_sample": round(err, 5),
+    }
+
+
+if __name__ == "__main__":
+    main()

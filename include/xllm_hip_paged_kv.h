@@ -224,6 +224,20 @@ int xllm_hip_paged_decode_run(const xllm_hip_kv_cache* cache,
                               size_t workspace_bytes,
                               xllm_hip_stream_t stream);
 
+/*
+ * xllm_hip_paged_decode_run that also records two caller-created hipEvent_t on `stream`: ev_begin
+ * just before the attention kernel (the launch that streams the KV cache) and ev_end just after
+ * it, before the merge.  A measurement hook for benchmarks; it has no counterpart in the
+ * reference.  Either event may be NULL.
+ */
+int xllm_hip_paged_decode_run_timed(const xllm_hip_kv_cache* cache,
+                                    const xllm_hip_decode_args* args,
+                                    void* workspace,
+                                    size_t workspace_bytes,
+                                    xllm_hip_stream_t stream,
+                                    void* ev_begin,
+                                    void* ev_end);
+
 /* plan + run in one call. */
 int xllm_hip_paged_decode(const xllm_hip_kv_cache* cache,
                           const xllm_hip_decode_args* args,

@@ -289,3 +289,38 @@ def test_quant_to_paged_cache_scatter():
         np.testing.assert_array_equal(kc[s // bs, :, s % bs], qk[t])
         np.testing.assert_array_equal(ks[s // bs, :, s % bs], sk[t])
     assert np.count_nonzero(ks) == T * H
+
+
+# ---- torch-CPU restatement (the timed CPU baseline) -------------------------------------------
+
+
+@pytest.mark.parametrize("n", [1, 3])
+def test_torch_cpu_path_matches_numpy_oracle(n):
+    from oracle import torch_cpu_path as tcp
+
+    q, k, v, table, lens = _case(20, 3, 8, 2, 16, 4, [5, 9, 30], n=n)
+    ref, _ = orc.paged_decode(q, k, v, table, lens, 0.3, q_per_seq=n)
+    got = tcp.paged_decode(torch.from_numpy(q), torch.from_numpy(k), torch.from_numpy(v), torch.from_numpy(table),
+                           torch.from_numpy(lens), 0.3, q_per_seq=n)
+    np.testing.assert_allclose(got.numpy(), ref, atol=2e-5)
+
+
+def test_torch_cpu_path_quantised_and_write():
+    from oracle import torch_cpu_path as tcp
+
+    q, k, v, table, lens = _case(21, 2, 4, 2, 16, 4, [7, 12])
+    qk, sk = orc.quantize_per_token_head(k, "int8")
+    qv, sv = orc.quantize_per_token_head(v, "int8")
+    ref, _ = orc.paged_decode(q, qk, qv, table, lens, 0.3, k_scale=sk, v_scale=sv, kind="int8")
+    got = tcp.paged_decode(torch.from_numpy(q), torch.from_numpy(qk), torch.from_numpy(qv), torch.from_numpy(table),
+                           torch.from_numpy(lens), 0.3, k_scale=torch.from_numpy(sk), v_scale=torch.from_numpy(sv))
+    np.testing.assert_allclose(got.numpy(), ref, atol=2e-5)
+    # KV write by advanced indexing == the literal loops
+    slots = np.array([3, 17, 9], np.int32)
+    keys = np.random.default_rng(0).standard_normal((3, 2, 16)).astype(np.float32)
+    kc1, vc1 = k.copy(), v.copy()
+    orc.reshape_paged_cache_loops(slots, keys, keys * 2, kc1, vc1, "HND")
+    kc2, vc2 = torch.from_numpy(k.copy()), torch.from_numpy(v.copy())
+    tcp.reshape_paged_cache(torch.from_numpy(slots), torch.from_numpy(keys), torch.from_numpy(keys * 2), kc2, vc2)
+    np.testing.assert_array_equal(kc2.numpy(), kc1)
+    np.testing.assert_array_equal(vc2.numpy(), vc1)

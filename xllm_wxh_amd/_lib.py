@@ -31,6 +31,7 @@ EXPORTED_SYMBOLS = (
     "xllm_hip_paged_decode_workspace_bytes",
     "xllm_hip_paged_decode_plan",
     "xllm_hip_paged_decode_run",
+    "xllm_hip_paged_decode_run_timed",
     "xllm_hip_paged_decode",
     "xllm_hip_csr_to_block_table",
     "xllm_hip_last_error",
@@ -124,6 +125,8 @@ def load():
         fn = getattr(lib, name)
         fn.argtypes = [P(KvCacheDesc), P(DecodeArgs), vp, ctypes.c_size_t, vp]
         fn.restype = ctypes.c_int
+    lib.xllm_hip_paged_decode_run_timed.argtypes = [P(KvCacheDesc), P(DecodeArgs), vp, ctypes.c_size_t, vp, vp, vp]
+    lib.xllm_hip_paged_decode_run_timed.restype = ctypes.c_int
     lib.xllm_hip_csr_to_block_table.argtypes = [vp, vp, vp, i32, i32, vp, i64, i32, vp, vp]
     lib.xllm_hip_csr_to_block_table.restype = ctypes.c_int
     lib.xllm_hip_last_error.argtypes = []

@@ -992,6 +992,16 @@ extern "C" int xllm_hip_paged_decode_run(const xllm_hip_kv_cache* cache,
                                          void* workspace,
                                          size_t workspace_bytes,
                                          xllm_hip_stream_t stream) {
+  return xllm_hip_paged_decode_run_timed(cache, args, workspace, workspace_bytes, stream, nullptr, nullptr);
+}
+
+extern "C" int xllm_hip_paged_decode_run_timed(const xllm_hip_kv_cache* cache,
+                                               const xllm_hip_decode_args* args,
+                                               void* workspace,
+                                               size_t workspace_bytes,
+                                               xllm_hip_stream_t stream,
+                                               void* ev_begin,
+                                               void* ev_end) {
   DecodeParams p;
   if (int s = fill_params(cache, args, workspace, workspace_bytes, p)) return s;
   if (p.batch == 0) return XLLM_HIP_OK;
@@ -1004,6 +1014,9 @@ extern "C" int xllm_hip_paged_decode_run(const xllm_hip_kv_cache* cache,
   }
   hipStream_t st = (hipStream_t)stream;
   const unsigned grid = (unsigned)max_items(p);
+  if (ev_begin != nullptr && hipEventRecord((hipEvent_t)ev_begin, st) != hipSuccess) {
+    return fail(XLLM_HIP_RUNTIME_ERROR, "hipEventRecord(ev_begin) failed");
+  }
   if (v == kMfmaD128) {
     switch (cache->dtype) {
       case XLLM_HIP_BF16:
@@ -1032,6 +1045,9 @@ extern "C" int xllm_hip_paged_decode_run(const xllm_hip_kv_cache* cache,
     if (s) return s;
   }
   if (int s = check_launch("decode attention kernel")) return s;
+  if (ev_end != nullptr && hipEventRecord((hipEvent_t)ev_end, st) != hipSuccess) {
+    return fail(XLLM_HIP_RUNTIME_ERROR, "hipEventRecord(ev_end) failed");
+  }
 
   const int64_t rows = (int64_t)p.batch * p.n * p.num_q_heads;
   const unsigned mgrid = (unsigned)((rows + 7) / 8);

@@ -238,13 +238,20 @@ def _decode_args(query, output, output_lse, block_table, seq_lens, csr, q_per_se
     return a, (q3, o3)
 
 
-def _run_decode(desc, args, workspace, device, plan=True, run=True):
+def _run_decode(desc, args, workspace, device, plan=True, run=True, events=None):
     lib = _lib.load()
     need = lib.xllm_hip_paged_decode_workspace_bytes(args.batch, args.q_per_seq, args.num_q_heads,
                                                      desc.num_kv_heads, desc.head_dim)
     ws = workspace if workspace is not None else get_workspace(device, need)
     wptr, wbytes = ctypes.c_void_p(ws.data_ptr()), ws.numel() * ws.element_size()
-    if plan and run:
+    if events is not None:
+        # (ev_begin, ev_end): raw hipEvent_t handles recorded around the attention kernel
+        if plan:
+            _lib.check(lib.xllm_hip_paged_decode_plan(ctypes.byref(desc), ctypes.byref(args), wptr, wbytes, _stream()))
+        _lib.check(lib.xllm_hip_paged_decode_run_timed(ctypes.byref(desc), ctypes.byref(args), wptr, wbytes,
+                                                       _stream(), ctypes.c_void_p(events[0]),
+                                                       ctypes.c_void_p(events[1])))
+    elif plan and run:
         _lib.check(lib.xllm_hip_paged_decode(ctypes.byref(desc), ctypes.byref(args), wptr, wbytes, _stream()))
     elif plan:
         _lib.check(lib.xllm_hip_paged_decode_plan(ctypes.byref(desc), ctypes.byref(args), wptr, wbytes, _stream()))
@@ -256,14 +263,15 @@ def batch_decode(query, k_cache, output, block_table, seq_lens, v_cache=None, ou
                  q_quant_scale=None, k_cache_quant_scale=None, v_cache_quant_scale=None, out_quant_scale=None,
                  alibi_slope=None, mask=None, compute_dtype="float", max_seq_len=0, window_size_left=-1,
                  window_size_right=-1, scale=1.0, return_lse=False, kv_cache_quant_bit_size=-1, *,
-                 q_per_seq=None, kv_layout="HND", workspace=None, plan=True, run=True):
+                 q_per_seq=None, kv_layout="HND", workspace=None, plan=True, run=True, events=None):
     """Paged decode in the block_table form; positional arguments as in
     xllm::kernel::mlu::batch_decode (xllm/core/kernels/mlu/mlu_ops_api.h:126-145).
 
     query/output: [batch, q_len, Hq, D] or [batch*q_len, Hq, D]; q_len > 1 is speculative verify
     with a causal mask among the draft tokens.  Keyword-only extras: q_per_seq (for 3-D queries),
     kv_layout, workspace (caller-owned scratch), plan/run (build the schedule once per step with
-    run=False, then reuse it for every layer with plan=False).
+    run=False, then reuse it for every layer with plan=False), events (two raw hipEvent_t handles
+    recorded just before and just after the attention kernel, for benchmarks).
     """
     _require(v_cache is not None, "v_cache is required (MLA-style single-cache decode is outside this path)")
     for name, t in (("q_quant_scale", q_quant_scale), ("out_quant_scale", out_quant_scale),
@@ -281,7 +289,7 @@ def batch_decode(query, k_cache, output, block_table, seq_lens, v_cache=None, ou
     desc = _cache_desc(k_cache, v_cache, k_cache_quant_scale, v_cache_quant_scale, kv_layout)
     args, _keep = _decode_args(query, output, output_lse if return_lse or output_lse is not None else None,
                                block_table, seq_lens, None, q_per_seq, scale, window_size_left, max_seq_len, desc)
-    _run_decode(desc, args, workspace, query.device, plan, run)
+    _run_decode(desc, args, workspace, query.device, plan, run, events)
 
 
 def batch_decode_csr(query, k_cache, v_cache, paged_kv_indptr, paged_kv_indices, paged_kv_last_page_len,
