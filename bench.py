@@ -117,7 +117,7 @@ def main():
         k, v, ks, vs = pools[i % len(pools)]
         ops.batch_decode(q, k, out, block_table, seq_lens_d, v, None, None, ks, vs, scale=w.sm_scale,
                          q_per_seq=w.q_per_seq, workspace=ws, kv_cache_quant_bit_size=quant_bits,
-                         max_seq_len=int(seq_lens.max()), events=events)
+                         max_seq_len=int(seq_lens.max()), total_kv_len=int(seq_lens.sum()), events=events)
 
     variant = ops.decode_variant(q, pools[0][0], pools[0][1], block_table, seq_lens_d, pools[0][2], pools[0][3],
                                  q_per_seq=w.q_per_seq)

@@ -77,7 +77,10 @@ class Case:
         return orc.paged_decode(self.q_ref, self.k_ref, self.v_ref, self.table, self.lens, self.scale,
                                 q_per_seq=self.n, window_left=window_left)
 
-    def run(self, window_left=-1, lse=True, **kw):
+    def run(self, window_left=-1, lse=True, hints=False, **kw):
+        if hints:  # host-side lengths, as the reference's AttentionMetadata carries them
+            kw.setdefault("max_seq_len", int(self.lens.max()))
+            kw.setdefault("total_kv_len", int(self.lens.sum()))
         out = torch.full_like(self.q, float("nan"))
         lse_t = torch.full((self.q.size(0), self.Hq), float("nan"), dtype=torch.float32, device=self.q.device) \
             if lse else None

@@ -294,3 +294,19 @@ def test_errors(gpu):
     with pytest.raises(_lib.XllmHipError) as ei:
         ops.batch_decode(qb, big, torch.empty_like(qb), case.block_table, case.seq_lens, big, scale=1.0)
     assert ei.value.status == _lib.UNSUPPORTED
+
+
+@pytest.mark.parametrize("kv,n", [("bf16", 1), ("int8", 4)])
+def test_host_length_hints_select_the_unsplit_path(gpu, kv, n):
+    """With truthful max_seq_len / total_kv_len the library may skip the split and the merge launch;
+    with hints that are wrong the result must still be right."""
+    print("case hints", kv, n, flush=True)
+    lens = [700, 650, 702, 699, 640, 701, 688, 703] * 8  # 64 near-equal sequences: no split needed
+    case = Case(64, 64 if n == 4 else 32, 8, 128, 16, lens, n=n, kv=kv, seed=33)
+    ref, lse_ref = case.oracle()
+    for kw in ({}, {"hints": True}, {"max_seq_len": 16, "total_kv_len": 100}, {"max_seq_len": 1 << 20, "total_kv_len": 1 << 30}):
+        out, lse = case.run(**kw)
+        e = max_abs_err(out, ref)
+        print("   %s err=%.3e" % (kw, e), flush=True)
+        assert e <= (REG_TOL_QUANT if kv == "int8" else REG_TOL)
+        assert lse_err(lse, lse_ref) <= LSE_TOL

@@ -2,12 +2,14 @@
 //
 // A sequence of kv length L is cut into chunks of `chunk_tokens` tokens (a
 // multiple of the 32-token tile): floor(L/C) full chunks and, if L % C != 0,
-// one tail chunk.  One work item = (sequence chunk, kv head, row group); the
-// kernel launched over the items writes one normalised partial output and its
-// base-2 log-sum-exp per item row, and the merge kernel combines a sequence's
-// partials with w_i = 2^(lse_i - lse_total) — the algebra of the reference's
-// two-partial merge (xllm/core/kernels/cuda/xattention/lse_combine.cu:61-73),
-// extended to any number of partials.
+// one tail chunk (an empty sequence keeps one empty chunk).  One work item =
+// (sequence chunk, kv head, row group), run by one workgroup.  A sequence that
+// is a single chunk has its output rows written by that workgroup; a split
+// sequence gets one normalised partial output and its base-2 log-sum-exp per
+// chunk and row, and the merge kernel combines them with
+// w_i = 2^(lse_i - lse_total) — the algebra of the reference's two-partial merge
+// (xllm/core/kernels/cuda/xattention/lse_combine.cu:61-73), extended to any
+// number of partials.
 //
 // Full chunks are numbered before tail chunks so that the hardware dispatcher,
 // which starts workgroups in index order, runs the equal-sized long items first
@@ -20,7 +22,7 @@
 namespace xllm_hip {
 
 constexpr int kTileTokens = 32;       // tokens per MFMA tile; chunk sizes are multiples of it
-constexpr int kMinChunkTokens = 128;  // smallest split worth a partial round trip
+constexpr int kMinChunkTokens = 512;  // smallest split worth a partial round trip (128 tokens per wave)
 constexpr int kMaxTargetItems = 4096; // upper bound of the split target (sizes the workspace)
 constexpr int kMaxRowsPerItem = 32;   // query rows (g * n) one work item handles
 
@@ -42,6 +44,7 @@ struct WorkspaceLayout {
   size_t kv_len;        // int32 [B]
   size_t full_prefix;   // int32 [B+1]  first full-chunk slot of sequence b
   size_t tail_prefix;   // int32 [B+1]  tail-chunk slot (relative to total_full) of sequence b
+  size_t num_chunks;    // int32 [B]    chunks of sequence b (full + tail)
   size_t seq_chunks;    // SeqChunk [max_seq_chunks]
   size_t partial_lse;   // float [max_seq_chunks][n][Hq]
   size_t partial_out;   // float [max_seq_chunks][n][Hq][D]
@@ -70,6 +73,8 @@ inline WorkspaceLayout workspace_layout(int batch, int q_per_seq, int num_q_head
   off = align_up(off + sizeof(int32_t) * ((size_t)batch + 1), 64);
   w.tail_prefix = off;
   off = align_up(off + sizeof(int32_t) * ((size_t)batch + 1), 64);
+  w.num_chunks = off;
+  off = align_up(off + sizeof(int32_t) * (size_t)batch, 64);
   w.seq_chunks = off;
   off = align_up(off + sizeof(SeqChunk) * (size_t)w.max_seq_chunks, 256);
   w.partial_lse = off;

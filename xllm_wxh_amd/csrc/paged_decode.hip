@@ -1,11 +1,14 @@
 // Paged-attention decode for gfx950 (MI355X): split-KV ("flash decoding") over
 // block_tables / seq_lens with GQA, bf16 / fp8-e4m3 / int8 KV caches.
 //
-// Three launches per call, none of which reads anything back to the host:
-//   decode_plan_kernel   kv lengths -> chunk size, chunk table (once per step)
-//   decode_*_kernel      one wave per (sequence chunk, kv head, row group): streams the
-//                        chunk's K and V once and writes a normalised partial + log2-sum-exp
-//   decode_merge_kernel  combines a sequence's partials into the output rows
+// Launches per call, none of which reads anything back to the host:
+//   decode_plan_kernel   kv lengths -> chunk size, chunk table (one wave; once per step)
+//   decode_*_kernel      one workgroup per (sequence chunk, kv head, row group): its waves split
+//                        the chunk, stream its K and V once and combine their results through
+//                        LDS; a sequence that is a single chunk gets its output rows written
+//                        directly, otherwise a normalised partial + log2-sum-exp is written
+//   decode_merge_kernel  combines the partials of the sequences that were split; skipped when
+//                        the host-side length hints show that no sequence is split
 //
 // Semantics follow the reference's decode operators: head map kv = h / (Hq/Hkv)
 // and fp32 softmax as in xllm/core/layers/cuda/flashinfer_attention.cpp:61-88, the
@@ -39,6 +42,7 @@ struct DecodeParams {
   int32_t* kv_len;
   int32_t* full_prefix;
   int32_t* tail_prefix;
+  int32_t* num_chunks;
   SeqChunk* seq_chunks;
   float* partial_lse;
   float* partial_out;
@@ -64,6 +68,8 @@ struct DecodeParams {
   int32_t max_blocks_per_seq;
   int32_t window_left;
   int32_t target_items;
+  int32_t fixed_chunk;    // > 0: chunk size chosen on the host (1 << 30 = never split)
+  int32_t direct_single;  // the attention kernel writes the output rows of single-chunk sequences itself
   int32_t q_dtype;
   float scale_log2;  // sm_scale * log2(e)
 };
@@ -72,43 +78,24 @@ struct DecodeParams {
 // Plan: one workgroup.  kv lengths -> total -> chunk size -> prefix sums -> chunk table.
 // ---------------------------------------------------------------------------------
 
-constexpr int kPlanThreads = 1024;
-
-// Inclusive scan of (a, b) pairs over the workgroup; every thread gets its prefix and the totals.
-__device__ inline void block_scan2(int a, int b, int* s_a, int* s_b, int& incl_a, int& incl_b, int& tot_a,
-                                   int& tot_b) {
-  const int tid = threadIdx.x;
-  s_a[tid] = a;
-  s_b[tid] = b;
-  __syncthreads();
-  for (int off = 1; off < kPlanThreads; off <<= 1) {
-    int va = 0, vb = 0;
-    if (tid >= off) {
-      va = s_a[tid - off];
-      vb = s_b[tid - off];
+// Inclusive scan of (a, b) over the wave.
+__device__ inline void wave_scan2(int& a, int& b, int lane) {
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int ua = __shfl_up(a, o), ub = __shfl_up(b, o);
+    if (lane >= o) {
+      a += ua;
+      b += ub;
     }
-    __syncthreads();
-    s_a[tid] += va;
-    s_b[tid] += vb;
-    __syncthreads();
   }
-  incl_a = s_a[tid];
-  incl_b = s_b[tid];
-  tot_a = s_a[kPlanThreads - 1];
-  tot_b = s_b[kPlanThreads - 1];
-  __syncthreads();
 }
 
-__global__ void __launch_bounds__(kPlanThreads) decode_plan_kernel(DecodeParams p) {
-  __shared__ int s_a[kPlanThreads];
-  __shared__ int s_b[kPlanThreads];
-  __shared__ long long s_total[kPlanThreads / 64];
-  __shared__ int s_chunk;
-  const int tid = threadIdx.x;
+__global__ void __launch_bounds__(64) decode_plan_kernel(DecodeParams p) {
+  const int lane = threadIdx.x;
 
   // 1. kv lengths and their sum.
-  long long local = 0;
-  for (int b = tid; b < p.batch; b += kPlanThreads) {
+  long long total = 0;
+  for (int b = lane; b < p.batch; b += 64) {
     int len;
     if (p.kv_indptr != nullptr) {
       const int nb = p.kv_indptr[b + 1] - p.kv_indptr[b];
@@ -118,64 +105,80 @@ __global__ void __launch_bounds__(kPlanThreads) decode_plan_kernel(DecodeParams 
     }
     len = len > 0 ? len : 0;
     p.kv_len[b] = len;
-    local += len;
+    total += len;
   }
 #pragma unroll
-  for (int o = 32; o >= 1; o >>= 1) local += __shfl_xor(local, o);
-  if ((tid & 63) == 0) s_total[tid >> 6] = local;
-  __syncthreads();
-  if (tid == 0) {
-    long long total = 0;
-    for (int i = 0; i < kPlanThreads / 64; ++i) total += s_total[i];
-    // 2. Chunk size: split so that about target_items work items exist.
-    const long long work = total * p.num_kv_heads * p.row_groups;
-    long long c = (work + p.target_items - 1) / p.target_items;
-    c = (c + kTileTokens - 1) / kTileTokens * kTileTokens;
-    if (c < kMinChunkTokens) c = kMinChunkTokens;
-    if (c > (1 << 30)) c = 1 << 30;
-    s_chunk = (int)c;
-  }
-  __syncthreads();
-  const int chunk = s_chunk;
+  for (int o = 32; o >= 1; o >>= 1) total += __shfl_xor(total, o);
 
-  // 3. Prefix sums of the full-chunk and tail-chunk counts.
-  int run_full = 0, run_tail = 0;
-  for (int base = 0; base < p.batch; base += kPlanThreads) {
-    const int b = base + tid;
+  // 2. Chunk size: split so that about target_items work items exist.
+  const long long work = total * p.num_kv_heads * p.row_groups;
+  long long c = (work + p.target_items - 1) / p.target_items;
+  c = (c + kTileTokens - 1) / kTileTokens * kTileTokens;
+  if (c < kMinChunkTokens) c = kMinChunkTokens;
+  if (c > (1 << 30)) c = 1 << 30;
+  const int chunk = p.fixed_chunk > 0 ? p.fixed_chunk : (int)c;
+
+  // 3. Prefix sums of the full-chunk and tail-chunk counts (lengths are re-derived rather than
+  //    re-read so that no lane depends on another lane's global store).
+  auto length_of = [&](int b) {
+    int len;
+    if (p.kv_indptr != nullptr) {
+      const int nb = p.kv_indptr[b + 1] - p.kv_indptr[b];
+      len = nb > 0 ? (nb - 1) * p.block_size + p.kv_last_page_len[b] : 0;
+    } else {
+      len = p.seq_lens[b];
+    }
+    return len > 0 ? len : 0;
+  };
+  int total_full = 0, total_tail = 0;
+  for (int base = 0; base < p.batch; base += 64) {
+    const int b = base + lane;
     int nf = 0, nt = 0;
     if (b < p.batch) {
-      const int len = p.kv_len[b];
+      const int len = length_of(b);
       nf = len / chunk;
-      nt = (len - nf * chunk) > 0 ? 1 : 0;
+      nt = ((len - nf * chunk) > 0 || len == 0) ? 1 : 0;  // an empty sequence keeps one (empty) chunk: it writes zeros
     }
-    int incl_f, incl_t, tot_f, tot_t;
-    block_scan2(nf, nt, s_a, s_b, incl_f, incl_t, tot_f, tot_t);
+    int sf = nf, st = nt;
+    wave_scan2(sf, st, lane);
     if (b < p.batch) {
-      p.full_prefix[b] = run_full + incl_f - nf;
-      p.tail_prefix[b] = run_tail + incl_t - nt;
+      p.full_prefix[b] = total_full + sf - nf;
+      p.tail_prefix[b] = total_tail + st - nt;
+      p.num_chunks[b] = nf + nt;
     }
-    run_full += tot_f;
-    run_tail += tot_t;
+    total_full += __shfl(sf, 63);
+    total_tail += __shfl(st, 63);
   }
-  if (tid == 0) {
-    p.full_prefix[p.batch] = run_full;
-    p.tail_prefix[p.batch] = run_tail;
+  if (lane == 0) {
+    p.full_prefix[p.batch] = total_full;
+    p.tail_prefix[p.batch] = total_tail;
     PlanHeader h{};
-    h.total_full = run_full;
-    h.total_tail = run_tail;
+    h.total_full = total_full;
+    h.total_tail = total_tail;
     h.chunk_tokens = chunk;
-    h.total_items = (run_full + run_tail) * p.num_kv_heads * p.row_groups;
+    h.total_items = (total_full + total_tail) * p.num_kv_heads * p.row_groups;
     *p.hdr = h;
   }
-  __syncthreads();  // prefix arrays written by this workgroup are visible to it below
 
   // 4. Chunk table: full chunks first, then the tails.
-  for (int b = tid; b < p.batch; b += kPlanThreads) {
-    const int len = p.kv_len[b];
-    const int nf = len / chunk;
-    const int f0 = p.full_prefix[b];
-    for (int c = 0; c < nf; ++c) p.seq_chunks[f0 + c] = SeqChunk{b, c};
-    if (len - nf * chunk > 0) p.seq_chunks[run_full + p.tail_prefix[b]] = SeqChunk{b, nf};
+  int run_full = 0, run_tail = 0;
+  for (int base = 0; base < p.batch; base += 64) {
+    const int b = base + lane;
+    int nf = 0, nt = 0;
+    if (b < p.batch) {
+      const int len = length_of(b);
+      nf = len / chunk;
+      nt = ((len - nf * chunk) > 0 || len == 0) ? 1 : 0;  // an empty sequence keeps one (empty) chunk: it writes zeros
+    }
+    int sf = nf, st = nt;
+    wave_scan2(sf, st, lane);
+    if (b < p.batch) {
+      const int f0 = run_full + sf - nf;
+      for (int ci = 0; ci < nf; ++ci) p.seq_chunks[f0 + ci] = SeqChunk{b, ci};
+      if (nt) p.seq_chunks[total_full + run_tail + st - nt] = SeqChunk{b, nf};
+    }
+    run_full += __shfl(sf, 63);
+    run_tail += __shfl(st, 63);
   }
 }
 
@@ -219,9 +222,72 @@ __device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it)
 }
 
 // ---------------------------------------------------------------------------------
-// MFMA kernel, head_dim 128, bf16 queries.  One wave per work item.
+// Merge of the sequences that were split into several chunks:
+//   out = sum_i 2^(lse_i - lse) * partial_i,   lse = log2 sum_i 2^lse_i
+// in one pass over the partials with a running maximum.  32 threads per output row.
+// ---------------------------------------------------------------------------------
+
+template <int Q_DT>
+__global__ void __launch_bounds__(256) decode_merge_kernel(DecodeParams p) {
+  const int nhq = p.n * p.num_q_heads;
+  const int64_t row = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 5);
+  const int sub = threadIdx.x & 31;
+  if (row >= (int64_t)p.batch * nhq) return;
+  const int b = (int)(row / nhq);
+  const int cnt = p.num_chunks[b];
+  if (p.direct_single && cnt == 1) return;  // already written by the attention kernel
+  const int rem = (int)(row - (int64_t)b * nhq);  // j * Hq + head
+  const int j = rem / p.num_q_heads;
+  const int head = rem - j * p.num_q_heads;
+  const int D = p.head_dim;
+  const float neg_inf = -INFINITY;
+  const int f0 = p.full_prefix[b];
+  const int nf = p.full_prefix[b + 1] - f0;
+  const int tail_slot = p.hdr->total_full + p.tail_prefix[b];
+
+  float m = neg_inf, ssum = 0.0f;
+  float o[2][4] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};  // head_dim <= 256: two float4 per thread
+  for (int i = 0; i < cnt; ++i) {
+    const int sc = i < nf ? f0 + i : tail_slot;
+    const int64_t prow = (int64_t)sc * nhq + rem;
+    const float li = p.partial_lse[prow];
+    if (li == neg_inf) continue;
+    const float m_new = fmaxf(m, li);
+    const float a = __builtin_amdgcn_exp2f(m - m_new);
+    const float w = __builtin_amdgcn_exp2f(li - m_new);
+    ssum = ssum * a + w;
+    const float* po = p.partial_out + prow * D;
+#pragma unroll
+    for (int q4 = 0; q4 < 2; ++q4) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int d = (sub + 32 * q4) * 4 + e;
+        if (d < D) o[q4][e] = o[q4][e] * a + w * po[d];
+      }
+    }
+    m = m_new;
+  }
+  const float inv = ssum > 0.0f ? 1.0f / ssum : 0.0f;
+  const int64_t tok = (int64_t)b * p.n + j;
+  if (p.lse != nullptr && sub == 0) {
+    p.lse[tok * p.num_q_heads + head] = ssum > 0.0f ? m + __builtin_amdgcn_logf(ssum) : neg_inf;
+  }
+  const int64_t obase = tok * p.out_token_stride + (int64_t)head * D;
+#pragma unroll
+  for (int q4 = 0; q4 < 2; ++q4) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int d = (sub + 32 * q4) * 4 + e;
+      if (d < D) Elem<Q_DT>::store(p.out, obase + d, o[q4][e] * inv);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// MFMA kernel, head_dim 128, bf16 queries.  One workgroup of kWaves waves per work item; the waves
+// take equal, tile-aligned shares of the item's tokens and never synchronise until the end.
 //
-// Per 32-token tile the wave loads K and V rows with fully coalesced 16-byte
+// Per 32-token tile a wave loads K and V rows with fully coalesced 16-byte
 // loads, parks them in its private 16 KiB of LDS (row-major, 16-byte pieces
 // XOR-swizzled by row so that the fragment reads below are bank-conflict free),
 // and reads them back in MFMA operand order:
@@ -237,6 +303,8 @@ __device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it)
 constexpr int kLdsK = 0;
 constexpr int kLdsV = 8192;
 constexpr int kLdsWave = 16384;
+constexpr int kWaves = 4;       // waves per work item
+constexpr int kXchRow = 528;    // bytes per query row in the end-of-item exchange (128 floats + 16 pad)
 
 template <int KV_DT>
 struct KvStage;  // registers holding one tile in flight + how to park it in LDS
@@ -295,7 +363,7 @@ struct KvStage<XLLM_HIP_BF16> {
   __device__ inline void take_scales(f32x4 (&)[2], f32x4 (&)[2]) const {}
 };
 
-// Convert 16 quantised bytes to 16 bf16 (exact for both e4m3 and int8).
+// Convert 16 quantised bytes to 16 bf16: e4m3 values exactly, int8 values offset by +128 (exact).
 template <int KV_DT>
 __device__ inline void dequant16(const u32x4 raw, bf16x8& lo, bf16x8& hi) {
   union {
@@ -308,11 +376,13 @@ __device__ inline void dequant16(const u32x4 raw, bf16x8& lo, bf16x8& hi) {
       u.h[2 * w] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)raw[w], 1.0f, false);
       u.h[2 * w + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)raw[w], 1.0f, true);
     } else {
-      const uint32_t t = raw[w] ^ 0x80808080u;  // int8 + 128 as unsigned bytes
-      const float f0 = (float)(t & 0xffu) - 128.0f;
-      const float f1 = (float)((t >> 8) & 0xffu) - 128.0f;
-      const float f2 = (float)((t >> 16) & 0xffu) - 128.0f;
-      const float f3 = (float)(t >> 24) - 128.0f;
+      // int8 x -> bf16(x + 128): the unsigned byte converts in one instruction and 0..255 is exact
+      // in bf16; the kernel takes the 128 back out of the scores and of the output.
+      const uint32_t t = raw[w] ^ 0x80808080u;
+      const float f0 = (float)(t & 0xffu);
+      const float f1 = (float)((t >> 8) & 0xffu);
+      const float f2 = (float)((t >> 16) & 0xffu);
+      const float f3 = (float)(t >> 24);
       u.h[2 * w] = bf16x2{(__bf16)f0, (__bf16)f1};
       u.h[2 * w + 1] = bf16x2{(__bf16)f2, (__bf16)f3};
     }
@@ -406,14 +476,22 @@ template <>
 struct KvStage<XLLM_HIP_INT8> : KvStageQuant<XLLM_HIP_INT8> {};
 
 template <int KV_DT, int NT>
-__global__ void __launch_bounds__(64) decode_mfma_d128_kernel(DecodeParams p) {
+__global__ void __launch_bounds__(64 * kWaves, NT == 1 ? 2 : 1) decode_mfma_d128_kernel(DecodeParams p) {
   constexpr bool kQuant = KV_DT != XLLM_HIP_BF16;
-  __shared__ __attribute__((aligned(16))) uint8_t lds[kLdsWave];
+  // int8 rows sit in LDS as x + 128.  With K' = K + 128 and V' = V + 128:
+  //   q.K  = q.K' - 128 * sum_d q_d                    (qsum, once per query row)
+  //   sum_t w_t V_t = sum_t w_t V'_t - 128 * sum_t w_t  (wsum, tracked like the softmax denominator)
+  // Rows zeroed because they lie past the sequence end carry weight 0 in both sums.
+  constexpr bool kOffset = KV_DT == XLLM_HIP_INT8;
+  __shared__ __attribute__((aligned(16))) uint8_t lds_all[kWaves * kLdsWave];
+  __shared__ float lds_ml[kWaves * NT * 16 * 2];  // (running max, denominator) per wave and query row
 
   Item it;
   if (!decode_item(p, blockIdx.x, it)) return;
 
-  const int lane = threadIdx.x;
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  uint8_t* lds = lds_all + wave * kLdsWave;  // this wave's private K/V tile
   const int mi = lane & 15;  // MFMA row of A / column of B and D
   const int kg = lane >> 4;  // k-group of the operands; row block of D
   const float neg_inf = -INFINITY;
@@ -422,6 +500,7 @@ __global__ void __launch_bounds__(64) decode_mfma_d128_kernel(DecodeParams p) {
   int lim[NT];  // tokens >= lim are invisible to the row (causal among draft tokens)
   int lo[NT];   // tokens < lo are outside the sliding window
   bool valid[NT];
+  float qsum128[NT];  // 128 * sum_d q[r][d] (int8 offset correction of the scores)
   bf16x8 qf[NT][4];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
@@ -439,6 +518,18 @@ __global__ void __launch_bounds__(64) decode_mfma_d128_kernel(DecodeParams p) {
       if (valid[nt]) raw = *(const u32x4*)(qrow + c * 32 + kg * 8);
       qf[nt][c] = __builtin_bit_cast(bf16x8, raw);
     }
+    qsum128[nt] = 0.0f;
+    if (kOffset) {
+      float sq = 0.0f;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sq += (float)qf[nt][c][e];
+      }
+      sq += __shfl_xor(sq, 16);
+      sq += __shfl_xor(sq, 32);
+      qsum128[nt] = 128.0f * sq;
+    }
   }
 
   // Tile range.  With a sliding window, tiles wholly below every row's window are skipped.
@@ -449,15 +540,21 @@ __global__ void __launch_bounds__(64) decode_mfma_d128_kernel(DecodeParams p) {
     first &= ~(kTileTokens - 1);
     t0 = t0 > first ? t0 : first;
   }
+  // This wave's share of [t0, t_end).
+  const int span = it.t_end - t0;
+  const int share = span > 0 ? (((span + kWaves - 1) / kWaves + kTileTokens - 1) & ~(kTileTokens - 1)) : 0;
+  const int w_begin = t0 + wave * share;
+  const int w_end = min(it.t_end, w_begin + share);
   const int mask_hi_from = it.len - (p.n - 1);                                // tiles reaching past this need masks
   const int mask_lo_until = p.window_left >= 0 ? it.len - 1 - p.window_left : 0;  // tiles starting below this too
 
   f32x4 acc[NT][8];
-  float m_run[NT], l_run[NT];
+  float m_run[NT], l_run[NT], w_run[NT];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
     m_run[nt] = neg_inf;
     l_run[nt] = 0.0f;
+    w_run[nt] = 0.0f;
 #pragma unroll
     for (int dt = 0; dt < 8; ++dt) acc[nt][dt] = f32x4{0, 0, 0, 0};
   }
@@ -499,7 +596,9 @@ __global__ void __launch_bounds__(64) decode_mfma_d128_kernel(DecodeParams p) {
       for (int h = 0; h < 2; ++h) {
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) {
-          float v = s[h][nt][rr] * p.scale_log2;
+          float v = s[h][nt][rr];
+          if (kOffset) v -= qsum128[nt];
+          v *= p.scale_log2;
           if (kQuant) v *= ksc[h][rr];
           if (MASKED) {
             const int tok = tb + 16 * h + 4 * kg + rr;
@@ -544,6 +643,12 @@ __global__ void __launch_bounds__(64) decode_mfma_d128_kernel(DecodeParams p) {
       }
 #pragma unroll
       for (int i = 0; i < 8; ++i) pf[nt][i] = (__bf16)pv[i];
+      if (kOffset) {
+        float wt = 0.0f;  // sum of the weights as the MFMA will see them (after rounding to bf16)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) wt += (float)pf[nt][i];
+        w_run[nt] = w_run[nt] * alpha + wt;
+      }
     }
     // ---- O^T += V^T P^T ----
 #pragma unroll
@@ -560,9 +665,9 @@ __global__ void __launch_bounds__(64) decode_mfma_d128_kernel(DecodeParams p) {
     }
   };
 
-  if (t0 < it.t_end) {
-    stage.issue(p, it, t0, lane);
-    for (int tb = t0; tb < it.t_end; tb += kTileTokens) {
+  if (w_begin < w_end) {
+    stage.issue(p, it, w_begin, lane);
+    for (int tb = w_begin; tb < w_end; tb += kTileTokens) {
       const bool masked = (tb + kTileTokens > mask_hi_from) || (tb < mask_lo_until);
       if (masked) {
         stage.template park<true>(lds, tb, it.len, lane);
@@ -572,7 +677,7 @@ __global__ void __launch_bounds__(64) decode_mfma_d128_kernel(DecodeParams p) {
       // The scales of the tile being consumed must outlive the next issue.
       f32x4 ksc[2] = {}, vsc[2] = {};
       stage.take_scales(ksc, vsc);
-      if (tb + kTileTokens < it.t_end) stage.issue(p, it, tb + kTileTokens, lane);
+      if (tb + kTileTokens < w_end) stage.issue(p, it, tb + kTileTokens, lane);
       if (masked) {
         tile(tb, ksc, vsc, std::true_type{});
       } else {
@@ -581,24 +686,72 @@ __global__ void __launch_bounds__(64) decode_mfma_d128_kernel(DecodeParams p) {
     }
   }
 
-  // ---- normalised partial + base-2 log-sum-exp ----
+  // ---- combine the waves through LDS; each wave then finishes a 32-wide slice of head_dim ----
   const int nhq = p.n * p.num_q_heads;
+  const bool single = p.direct_single != 0 && p.num_chunks[it.b] == 1;
+  const int col = lane & 15;              // query row handled in the combine
+  const int d0 = 32 * wave + 8 * (lane >> 4);  // first of this lane's 8 output columns
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
     float l = l_run[nt];
     l += __shfl_xor(l, 16);
     l += __shfl_xor(l, 32);
-    if (!valid[nt]) continue;
-    const int r = it.rg * kMaxRowsPerItem + nt * 16 + mi;
-    const int j = r / p.group;
-    const int gq = r - j * p.group;
-    const int64_t prow = (int64_t)it.sc * nhq + (int64_t)j * p.num_q_heads + it.hk * p.group + gq;
-    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-    if (kg == 0) p.partial_lse[prow] = l > 0.0f ? m_run[nt] + __builtin_amdgcn_logf(l) : neg_inf;
-    float* po = p.partial_out + prow * 128 + 4 * kg;
+    float wsum = w_run[nt];
+    if (kOffset) {
+      wsum += __shfl_xor(wsum, 16);
+      wsum += __shfl_xor(wsum, 32);
+    }
+    if (nt > 0) __syncthreads();  // the previous round's reads are finished
 #pragma unroll
     for (int dt = 0; dt < 8; ++dt) {
-      *(f32x4*)(po + dt * 16) = acc[nt][dt] * inv;
+      f32x4 o = acc[nt][dt];
+      if (kOffset) o -= 128.0f * wsum;
+      *(f32x4*)(lds + mi * kXchRow + (dt * 16 + 4 * kg) * 4) = o;
+    }
+    if (kg == 0) {
+      lds_ml[((wave * NT + nt) * 16 + mi) * 2] = m_run[nt];
+      lds_ml[((wave * NT + nt) * 16 + mi) * 2 + 1] = l;
+    }
+    __syncthreads();
+
+    float m_all = neg_inf;
+#pragma unroll
+    for (int s = 0; s < kWaves; ++s) m_all = fmaxf(m_all, lds_ml[((s * NT + nt) * 16 + col) * 2]);
+    const float m_safe = m_all == neg_inf ? 0.0f : m_all;
+    float l_all = 0.0f;
+    f32x4 o_lo = {0, 0, 0, 0}, o_hi = {0, 0, 0, 0};
+#pragma unroll
+    for (int s = 0; s < kWaves; ++s) {
+      const float w = __builtin_amdgcn_exp2f(lds_ml[((s * NT + nt) * 16 + col) * 2] - m_safe);
+      l_all += w * lds_ml[((s * NT + nt) * 16 + col) * 2 + 1];
+      const uint8_t* src = lds_all + s * kLdsWave + col * kXchRow + d0 * 4;
+      o_lo += w * *(const f32x4*)(src);
+      o_hi += w * *(const f32x4*)(src + 16);
+    }
+    const int r = it.rg * kMaxRowsPerItem + nt * 16 + col;
+    if (r >= p.rows) continue;
+    const int j = r / p.group;
+    const int head = it.hk * p.group + (r - j * p.group);
+    const float inv = l_all > 0.0f ? 1.0f / l_all : 0.0f;
+    const float lse2 = l_all > 0.0f ? m_all + __builtin_amdgcn_logf(l_all) : neg_inf;
+    o_lo *= inv;
+    o_hi *= inv;
+    const int64_t tok = (int64_t)it.b * p.n + j;
+    if (single) {
+      bf16x8 ob;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        ob[e] = (__bf16)o_lo[e];
+        ob[4 + e] = (__bf16)o_hi[e];
+      }
+      *(bf16x8*)((uint16_t*)p.out + tok * p.out_token_stride + (int64_t)head * 128 + d0) = ob;
+      if (p.lse != nullptr && d0 == 0) p.lse[tok * p.num_q_heads + head] = lse2;
+    } else {
+      const int64_t prow = (int64_t)it.sc * nhq + (int64_t)j * p.num_q_heads + head;
+      float* po = p.partial_out + prow * 128 + d0;
+      *(f32x4*)(po) = o_lo;
+      *(f32x4*)(po + 4) = o_hi;
+      if (d0 == 0) p.partial_lse[prow] = lse2;
     }
   }
 }
@@ -693,67 +846,6 @@ __global__ void __launch_bounds__(64) decode_generic_kernel(DecodeParams p) {
 }
 
 // ---------------------------------------------------------------------------------
-// Merge: out = sum_i 2^(lse_i - lse) * partial_i,  lse = log2 sum_i 2^lse_i.
-// 32 threads per output row, 8 rows per workgroup.
-// ---------------------------------------------------------------------------------
-
-template <int Q_DT>
-__global__ void __launch_bounds__(256) decode_merge_kernel(DecodeParams p) {
-  const int nhq = p.n * p.num_q_heads;
-  const int64_t row = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 5);
-  const int sub = threadIdx.x & 31;
-  if (row >= (int64_t)p.batch * nhq) return;
-  const int b = (int)(row / nhq);
-  const int rem = (int)(row - (int64_t)b * nhq);  // j * Hq + head
-  const int j = rem / p.num_q_heads;
-  const int head = rem - j * p.num_q_heads;
-  const int D = p.head_dim;
-  const float neg_inf = -INFINITY;
-
-  const int f0 = p.full_prefix[b];
-  const int nf = p.full_prefix[b + 1] - f0;
-  const int has_tail = p.tail_prefix[b + 1] - p.tail_prefix[b];
-  const int tail_slot = p.hdr->total_full + p.tail_prefix[b];
-  const int cnt = nf + has_tail;
-
-  float mx = neg_inf;
-  for (int i = 0; i < cnt; ++i) {
-    const int sc = i < nf ? f0 + i : tail_slot;
-    mx = fmaxf(mx, p.partial_lse[(int64_t)sc * nhq + rem]);
-  }
-  float denom = 0.0f;
-  if (mx != neg_inf) {
-    for (int i = 0; i < cnt; ++i) {
-      const int sc = i < nf ? f0 + i : tail_slot;
-      denom += __builtin_amdgcn_exp2f(p.partial_lse[(int64_t)sc * nhq + rem] - mx);
-    }
-  }
-  const float lse = mx != neg_inf ? mx + __builtin_amdgcn_logf(denom) : neg_inf;
-  if (p.lse != nullptr && sub == 0) p.lse[(int64_t)(b * p.n + j) * p.num_q_heads + head] = lse;
-
-  const int64_t obase = (int64_t)(b * p.n + j) * p.out_token_stride + (int64_t)head * D;
-  for (int d4 = sub * 4; d4 < D; d4 += 128) {
-    float o[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    if (mx != neg_inf) {
-      for (int i = 0; i < cnt; ++i) {
-        const int sc = i < nf ? f0 + i : tail_slot;
-        const int64_t prow = (int64_t)sc * nhq + rem;
-        const float w = __builtin_amdgcn_exp2f(p.partial_lse[prow] - lse);
-        const float* po = p.partial_out + prow * D + d4;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          if (d4 + e < D) o[e] += w * po[e];
-        }
-      }
-    }
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      if (d4 + e < D) Elem<Q_DT>::store(p.out, obase + d4 + e, o[e]);
-    }
-  }
-}
-
-// ---------------------------------------------------------------------------------
 // CSR -> block_table / seq_lens.
 // ---------------------------------------------------------------------------------
 
@@ -782,15 +874,29 @@ __global__ void __launch_bounds__(256) csr_to_block_table_kernel(const int32_t* 
 
 enum Variant { kNone = 0, kMfmaD128 = 1, kGeneric = 2 };
 
-// Split target: about this many work items per launch.  One wave of the attention kernel occupies
-// one SIMD, and the chip has 256 CUs x 4 SIMDs.
-static int target_items() {
-  int v = 1024;
+// Split target: about this many work items (workgroups) per launch.  A workgroup of the MFMA kernel
+// is four waves, one per SIMD of a CU; two fit on a CU when the kernel needs at most 256 VGPRs
+// (up to 16 query rows per kv head), one otherwise.  The generic kernel runs one wave per item.
+constexpr int kNumCUs = 256;
+
+static int target_items(int variant_is_mfma, int rows_per_item) {
+  int v = variant_is_mfma ? (rows_per_item <= 16 ? 2 * kNumCUs : kNumCUs) : 8 * kNumCUs;
   if (const char* e = getenv("XLLM_HIP_DECODE_TARGET_ITEMS")) {
     const int t = atoi(e);
     if (t > 0) v = t;
   }
   return v > kMaxTargetItems ? kMaxTargetItems : v;
+}
+
+// Chunk size for a batch whose kv lengths sum to `total` — the formula decode_plan_kernel applies
+// on the device when the host has no length hints.
+static int64_t chunk_for(int64_t total, int num_kv_heads, int row_groups, int target) {
+  const int64_t work = total * num_kv_heads * row_groups;
+  int64_t c = (work + target - 1) / target;
+  c = (c + kTileTokens - 1) / kTileTokens * kTileTokens;
+  if (c < kMinChunkTokens) c = kMinChunkTokens;
+  if (c > (1 << 30)) c = 1 << 30;
+  return c;
 }
 
 static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
@@ -879,6 +985,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
   p.kv_len = (int32_t*)(ws + w.kv_len);
   p.full_prefix = (int32_t*)(ws + w.full_prefix);
   p.tail_prefix = (int32_t*)(ws + w.tail_prefix);
+  p.num_chunks = (int32_t*)(ws + w.num_chunks);
   p.seq_chunks = (SeqChunk*)(ws + w.seq_chunks);
   p.partial_lse = (float*)(ws + w.partial_lse);
   p.partial_out = (float*)(ws + w.partial_out);
@@ -903,7 +1010,19 @@ static int fill_params(const xllm_hip_kv_cache* c,
   p.log2_bs = is_pow2(c->block_size) ? ilog2(c->block_size) : 0;
   p.max_blocks_per_seq = a->max_blocks_per_seq;
   p.window_left = a->window_left;
-  p.target_items = target_items();
+  const Variant variant = pick_variant(c, a);
+  const int rows_per_item = p.rows < kMaxRowsPerItem ? p.rows : kMaxRowsPerItem;
+  p.target_items = target_items(variant == kMfmaD128, rows_per_item);
+  // Only the MFMA kernel finishes single-chunk sequences itself.  When the caller's host-side
+  // lengths (the reference keeps both in AttentionMetadata) show that the chunk the plan would
+  // pick covers the longest sequence, no sequence is split: the plan is told never to split
+  // (which stays correct even if the hints were wrong) and the merge launch is dropped.
+  p.direct_single = variant == kMfmaD128 ? 1 : 0;
+  p.fixed_chunk = 0;
+  if (p.direct_single && a->max_seq_len > 0 && a->total_kv_len > 0 &&
+      a->max_seq_len <= chunk_for(a->total_kv_len, p.num_kv_heads, p.row_groups, p.target_items)) {
+    p.fixed_chunk = 1 << 30;
+  }
   p.q_dtype = a->q_dtype;
   p.scale_log2 = a->sm_scale * 1.4426950408889634f;
   return XLLM_HIP_OK;
@@ -912,6 +1031,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
 // Upper bound of the work-item count for any lengths (see workspace_layout).
 static int64_t max_items(const DecodeParams& p) {
   const int64_t per = (int64_t)p.num_kv_heads * p.row_groups;
+  if (p.fixed_chunk == (1 << 30)) return (int64_t)p.batch * per;
   return ((int64_t)p.target_items / per + p.batch + 1) * per;
 }
 
@@ -919,9 +1039,9 @@ template <int KV_DT>
 static void launch_mfma(const DecodeParams& p, unsigned grid, hipStream_t st) {
   const int rows_per_item = p.rows < kMaxRowsPerItem ? p.rows : kMaxRowsPerItem;
   if (rows_per_item <= 16) {
-    decode_mfma_d128_kernel<KV_DT, 1><<<grid, 64, 0, st>>>(p);
+    decode_mfma_d128_kernel<KV_DT, 1><<<grid, 64 * kWaves, 0, st>>>(p);
   } else {
-    decode_mfma_d128_kernel<KV_DT, 2><<<grid, 64, 0, st>>>(p);
+    decode_mfma_d128_kernel<KV_DT, 2><<<grid, 64 * kWaves, 0, st>>>(p);
   }
 }
 
@@ -983,7 +1103,7 @@ extern "C" int xllm_hip_paged_decode_plan(const xllm_hip_kv_cache* cache,
   DecodeParams p;
   if (int s = fill_params(cache, args, workspace, workspace_bytes, p)) return s;
   if (p.batch == 0) return XLLM_HIP_OK;
-  decode_plan_kernel<<<1, kPlanThreads, 0, (hipStream_t)stream>>>(p);
+  decode_plan_kernel<<<1, 64, 0, (hipStream_t)stream>>>(p);
   return check_launch("decode_plan_kernel");
 }
 
@@ -1048,6 +1168,7 @@ extern "C" int xllm_hip_paged_decode_run_timed(const xllm_hip_kv_cache* cache,
   if (ev_end != nullptr && hipEventRecord((hipEvent_t)ev_end, st) != hipSuccess) {
     return fail(XLLM_HIP_RUNTIME_ERROR, "hipEventRecord(ev_end) failed");
   }
+  if (p.fixed_chunk == (1 << 30)) return XLLM_HIP_OK;  // nothing was split: the outputs are final
 
   const int64_t rows = (int64_t)p.batch * p.n * p.num_q_heads;
   const unsigned mgrid = (unsigned)((rows + 7) / 8);

@@ -185,7 +185,7 @@ def get_workspace(device, nbytes):
 
 
 def _decode_args(query, output, output_lse, block_table, seq_lens, csr, q_per_seq, scale, window_size_left,
-                 max_seq_len, desc):
+                 max_seq_len, desc, total_kv_len=0):
     _require(query.dim() in (3, 4), "query must be [tokens, heads, dim] or [batch, q_len, heads, dim]")
     if query.dim() == 4:
         # [batch, q_len, Hq, D] (xllm/core/layers/mlu/attention.cpp:263-264)
@@ -234,7 +234,7 @@ def _decode_args(query, output, output_lse, block_table, seq_lens, csr, q_per_se
         _require(indptr.numel() == a.batch + 1 and last_page_len.numel() == a.batch, "CSR arrays do not match batch")
         a.kv_indptr, a.kv_indices, a.kv_last_page_len = indptr.data_ptr(), indices.data_ptr(), last_page_len.data_ptr()
     a.max_seq_len = int(max_seq_len) if max_seq_len is not None else 0
-    a.total_kv_len = 0
+    a.total_kv_len = int(total_kv_len) if total_kv_len is not None else 0
     return a, (q3, o3)
 
 
@@ -263,7 +263,8 @@ def batch_decode(query, k_cache, output, block_table, seq_lens, v_cache=None, ou
                  q_quant_scale=None, k_cache_quant_scale=None, v_cache_quant_scale=None, out_quant_scale=None,
                  alibi_slope=None, mask=None, compute_dtype="float", max_seq_len=0, window_size_left=-1,
                  window_size_right=-1, scale=1.0, return_lse=False, kv_cache_quant_bit_size=-1, *,
-                 q_per_seq=None, kv_layout="HND", workspace=None, plan=True, run=True, events=None):
+                 q_per_seq=None, kv_layout="HND", workspace=None, plan=True, run=True, events=None,
+                 total_kv_len=0):
     """Paged decode in the block_table form; positional arguments as in
     xllm::kernel::mlu::batch_decode (xllm/core/kernels/mlu/mlu_ops_api.h:126-145).
 
@@ -271,7 +272,9 @@ def batch_decode(query, k_cache, output, block_table, seq_lens, v_cache=None, ou
     with a causal mask among the draft tokens.  Keyword-only extras: q_per_seq (for 3-D queries),
     kv_layout, workspace (caller-owned scratch), plan/run (build the schedule once per step with
     run=False, then reuse it for every layer with plan=False), events (two raw hipEvent_t handles
-    recorded just before and just after the attention kernel, for benchmarks).
+    recorded just before and just after the attention kernel, for benchmarks), total_kv_len (the
+    host-side sum of the kv lengths, AttentionMetadata.total_kv_len in the reference; together with
+    max_seq_len it lets the library drop the merge launch when no sequence needs splitting).
     """
     _require(v_cache is not None, "v_cache is required (MLA-style single-cache decode is outside this path)")
     for name, t in (("q_quant_scale", q_quant_scale), ("out_quant_scale", out_quant_scale),
@@ -288,20 +291,22 @@ def batch_decode(query, k_cache, output, block_table, seq_lens, v_cache=None, ou
         _require(output_lse is not None, "return_lse=True needs a pre-allocated output_lse")
     desc = _cache_desc(k_cache, v_cache, k_cache_quant_scale, v_cache_quant_scale, kv_layout)
     args, _keep = _decode_args(query, output, output_lse if return_lse or output_lse is not None else None,
-                               block_table, seq_lens, None, q_per_seq, scale, window_size_left, max_seq_len, desc)
+                               block_table, seq_lens, None, q_per_seq, scale, window_size_left, max_seq_len, desc,
+                               total_kv_len)
     _run_decode(desc, args, workspace, query.device, plan, run, events)
 
 
 def batch_decode_csr(query, k_cache, v_cache, paged_kv_indptr, paged_kv_indices, paged_kv_last_page_len,
                      window_left, sm_scale, output, output_lse=None, *, k_cache_scale=None, v_cache_scale=None,
-                     q_per_seq=None, kv_layout="NHD", workspace=None, plan=True, run=True):
+                     q_per_seq=None, kv_layout="NHD", workspace=None, plan=True, run=True, max_seq_len=0,
+                     total_kv_len=0):
     """Paged decode in the CSR form of xllm::kernel::cuda::batch_decode
     (xllm/core/kernels/cuda/cuda_ops_api.h:120-136; the FlashInfer plan/workspace/uri
     arguments have no counterpart here).  The CUDA backend's cache layout is NHD."""
     desc = _cache_desc(k_cache, v_cache, k_cache_scale, v_cache_scale, kv_layout)
     args, _keep = _decode_args(query, output, output_lse, None, None,
                                (paged_kv_indptr, paged_kv_indices, paged_kv_last_page_len), q_per_seq, sm_scale,
-                               window_left, 0, desc)
+                               window_left, max_seq_len, desc, total_kv_len)
     _run_decode(desc, args, workspace, query.device, plan, run)
 
 
