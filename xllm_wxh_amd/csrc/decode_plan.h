@@ -26,6 +26,29 @@ constexpr int kMinChunkTokens = 512;  // smallest split worth a partial round tr
 constexpr int kMaxTargetItems = 4096; // upper bound of the split target (sizes the workspace)
 constexpr int kMaxRowsPerItem = 32;   // query rows (g * n) one work item handles
 
+#if defined(__HIPCC__)
+#define XLLM_HIP_HD __host__ __device__
+#else
+#define XLLM_HIP_HD
+#endif
+
+// Chunk size for a batch whose kv lengths sum to `total` with maximum `max_len`: split so that
+// about `target` work items exist — four times as many when the batch is ragged (longest sequence
+// above 1.5x the mean), because then the items differ in size and the dispatcher needs slack to
+// balance them.  Shared by the device-side plan and by the host's check that nothing is split.
+XLLM_HIP_HD inline int choose_chunk(long long total, long long max_len, int batch, int num_kv_heads,
+                                    int row_groups, int target) {
+  long long t = target;
+  if (max_len * batch * 2 > total * 3) t *= 4;
+  if (t > kMaxTargetItems) t = kMaxTargetItems;
+  const long long work = total * num_kv_heads * row_groups;
+  long long c = (work + t - 1) / t;
+  c = (c + kTileTokens - 1) / kTileTokens * kTileTokens;
+  if (c < kMinChunkTokens) c = kMinChunkTokens;
+  if (c > (1 << 30)) c = 1 << 30;
+  return (int)c;
+}
+
 struct PlanHeader {
   int32_t total_full;    // number of full sequence-chunks
   int32_t total_tail;    // number of tail sequence-chunks

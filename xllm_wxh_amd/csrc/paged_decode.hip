@@ -93,8 +93,9 @@ __device__ inline void wave_scan2(int& a, int& b, int lane) {
 __global__ void __launch_bounds__(64) decode_plan_kernel(DecodeParams p) {
   const int lane = threadIdx.x;
 
-  // 1. kv lengths and their sum.
+  // 1. kv lengths, their sum and their maximum.
   long long total = 0;
+  int max_len = 0;
   for (int b = lane; b < p.batch; b += 64) {
     int len;
     if (p.kv_indptr != nullptr) {
@@ -106,17 +107,19 @@ __global__ void __launch_bounds__(64) decode_plan_kernel(DecodeParams p) {
     len = len > 0 ? len : 0;
     p.kv_len[b] = len;
     total += len;
+    max_len = len > max_len ? len : max_len;
   }
 #pragma unroll
-  for (int o = 32; o >= 1; o >>= 1) total += __shfl_xor(total, o);
+  for (int o = 32; o >= 1; o >>= 1) {
+    total += __shfl_xor(total, o);
+    const int other = __shfl_xor(max_len, o);
+    max_len = other > max_len ? other : max_len;
+  }
 
-  // 2. Chunk size: split so that about target_items work items exist.
-  const long long work = total * p.num_kv_heads * p.row_groups;
-  long long c = (work + p.target_items - 1) / p.target_items;
-  c = (c + kTileTokens - 1) / kTileTokens * kTileTokens;
-  if (c < kMinChunkTokens) c = kMinChunkTokens;
-  if (c > (1 << 30)) c = 1 << 30;
-  const int chunk = p.fixed_chunk > 0 ? p.fixed_chunk : (int)c;
+  // 2. Chunk size.
+  const int chunk = p.fixed_chunk > 0
+                        ? p.fixed_chunk
+                        : choose_chunk(total, max_len, p.batch, p.num_kv_heads, p.row_groups, p.target_items);
 
   // 3. Prefix sums of the full-chunk and tail-chunk counts (lengths are re-derived rather than
   //    re-read so that no lane depends on another lane's global store).
@@ -665,24 +668,38 @@ __global__ void __launch_bounds__(64 * kWaves, NT == 1 ? 2 : 1) decode_mfma_d128
     }
   };
 
+  // One tile's worth of global loads is always in flight while the previous tile is consumed.  A
+  // quantised tile is only half as many bytes, so two of them are kept in flight (two register
+  // stages, used alternately) to cover the same HBM latency.
+  auto consume = [&](KvStage<KV_DT>& st, int tb, int next_tb) {
+    const bool masked = (tb + kTileTokens > mask_hi_from) || (tb < mask_lo_until);
+    if (masked) {
+      st.template park<true>(lds, tb, it.len, lane);
+    } else {
+      st.template park<false>(lds, tb, it.len, lane);
+    }
+    // The scales of the tile being consumed must outlive the next issue into the same stage.
+    f32x4 ksc[2] = {}, vsc[2] = {};
+    st.take_scales(ksc, vsc);
+    if (next_tb < w_end) st.issue(p, it, next_tb, lane);
+    if (masked) {
+      tile(tb, ksc, vsc, std::true_type{});
+    } else {
+      tile(tb, ksc, vsc, std::false_type{});
+    }
+  };
   if (w_begin < w_end) {
-    stage.issue(p, it, w_begin, lane);
-    for (int tb = w_begin; tb < w_end; tb += kTileTokens) {
-      const bool masked = (tb + kTileTokens > mask_hi_from) || (tb < mask_lo_until);
-      if (masked) {
-        stage.template park<true>(lds, tb, it.len, lane);
-      } else {
-        stage.template park<false>(lds, tb, it.len, lane);
+    if (kQuant) {
+      KvStage<KV_DT> stage_b;
+      stage.issue(p, it, w_begin, lane);
+      if (w_begin + kTileTokens < w_end) stage_b.issue(p, it, w_begin + kTileTokens, lane);
+      for (int tb = w_begin; tb < w_end; tb += 2 * kTileTokens) {
+        consume(stage, tb, tb + 2 * kTileTokens);
+        if (tb + kTileTokens < w_end) consume(stage_b, tb + kTileTokens, tb + 3 * kTileTokens);
       }
-      // The scales of the tile being consumed must outlive the next issue.
-      f32x4 ksc[2] = {}, vsc[2] = {};
-      stage.take_scales(ksc, vsc);
-      if (tb + kTileTokens < w_end) stage.issue(p, it, tb + kTileTokens, lane);
-      if (masked) {
-        tile(tb, ksc, vsc, std::true_type{});
-      } else {
-        tile(tb, ksc, vsc, std::false_type{});
-      }
+    } else {
+      stage.issue(p, it, w_begin, lane);
+      for (int tb = w_begin; tb < w_end; tb += kTileTokens) consume(stage, tb, tb + kTileTokens);
     }
   }
 
@@ -888,17 +905,6 @@ static int target_items(int variant_is_mfma, int rows_per_item) {
   return v > kMaxTargetItems ? kMaxTargetItems : v;
 }
 
-// Chunk size for a batch whose kv lengths sum to `total` — the formula decode_plan_kernel applies
-// on the device when the host has no length hints.
-static int64_t chunk_for(int64_t total, int num_kv_heads, int row_groups, int target) {
-  const int64_t work = total * num_kv_heads * row_groups;
-  int64_t c = (work + target - 1) / target;
-  c = (c + kTileTokens - 1) / kTileTokens * kTileTokens;
-  if (c < kMinChunkTokens) c = kMinChunkTokens;
-  if (c > (1 << 30)) c = 1 << 30;
-  return c;
-}
-
 static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
 static Variant pick_variant(const xllm_hip_kv_cache* c, const xllm_hip_decode_args* a) {
@@ -1020,7 +1026,8 @@ static int fill_params(const xllm_hip_kv_cache* c,
   p.direct_single = variant == kMfmaD128 ? 1 : 0;
   p.fixed_chunk = 0;
   if (p.direct_single && a->max_seq_len > 0 && a->total_kv_len > 0 &&
-      a->max_seq_len <= chunk_for(a->total_kv_len, p.num_kv_heads, p.row_groups, p.target_items)) {
+      a->max_seq_len <= choose_chunk(a->total_kv_len, a->max_seq_len, p.batch, p.num_kv_heads, p.row_groups,
+                                     p.target_items)) {
     p.fixed_chunk = 1 << 30;
   }
   p.q_dtype = a->q_dtype;
@@ -1032,7 +1039,9 @@ static int fill_params(const xllm_hip_kv_cache* c,
 static int64_t max_items(const DecodeParams& p) {
   const int64_t per = (int64_t)p.num_kv_heads * p.row_groups;
   if (p.fixed_chunk == (1 << 30)) return (int64_t)p.batch * per;
-  return ((int64_t)p.target_items / per + p.batch + 1) * per;
+  int64_t t = 4 * (int64_t)p.target_items;  // choose_chunk may quadruple the target
+  if (t > kMaxTargetItems) t = kMaxTargetItems;
+  return (t / per + p.batch + 1) * per;
 }
 
 template <int KV_DT>
