@@ -40,6 +40,9 @@ def parse_args():
     ap.add_argument("--pools", type=int, default=3, help="disjoint KV pools rotated between steps")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget of the CPU baseline leg")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="run only a plain 1 GiB device-to-device copy a few times and exit: the known-size "
+                         "kernel against which the rocprofv3 FETCH_SIZE / WRITE_SIZE counters are scaled")
     return ap.parse_args()
 
 
@@ -94,6 +97,15 @@ def main():
         sys.exit(2)
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+    if args.copy_calibration:
+        src = torch.randn(1 << 29, device=device, dtype=torch.bfloat16)  # 1 GiB
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration": True, "bytes_read_per_launch": src.numel() * 2,
+                          "bytes_written_per_launch": src.numel() * 2, "launches": 10}))
+        return
     w = workloads.WORKLOADS[args.workload]
     if w.kv_dtype == "fp32":
         sys.stderr.write("workload %s is the CPU-reference case; pick a GPU workload\n" % w.name)

@@ -1,0 +1,157 @@
+"""The libtorch host side (C++ mirrors of xllm::kernel / xllm::layer for the decode path):
+host-only behaviour on the CPU, the whole write-then-attend dispatch on the GPU."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import paged_kv_oracle as orc
+from xllm_wxh_amd import build as xbuild
+
+
+@pytest.fixture(scope="module")
+def shim():
+    if not os.path.exists(xbuild.TORCH_SHIM_PATH):
+        xbuild.build_torch_shim(verbose=False)
+    from xllm_wxh_amd import _xllm_hip_torch
+
+    return _xllm_hip_torch
+
+
+def test_metadata_builder_matches_reference_known_answers(shim):
+    # cumulative layout of batch_test.cpp:176-189; kv_seq_lens = diff (attention_metadata_builder.cpp:105)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32)
+    md = shim.build_decode_metadata(i32([0, 9, 10, 11, 15]), i32([0, 9, 17, 33, 41]), i32([4, 23, 47, 56]),
+                                    i32([[1, 2, 3, 0, 0], [4, 5, 6, 7, 0], [8, 9, 10, 11, 12], [13, 14, 15, 0, 0]]),
+                                    9, 16, 41)
+    assert md.kv_seq_lens.tolist() == [9, 8, 16, 8]
+    assert md.q_seq_lens.tolist() == [9, 1, 1, 4]
+    assert md.max_seq_len == 16 and md.max_query_len == 9 and not md.is_dummy
+    dummy = shim.build_decode_metadata(i32([0, 0]), i32([0, 0]), i32([0]), i32([[0]]), 0, 0, 0)
+    assert dummy.is_dummy and dummy.slot_mapping.tolist() == [1]
+
+
+def test_kv_cache_scale_getters(shim):
+    k = torch.zeros(2, 1, 4, 8)
+    kv = shim.KVCache(k, k)
+    assert kv.get_k_cache_scale() is None and not kv.empty()
+    kv = shim.KVCache(k.to(torch.int8), k.to(torch.int8), torch.ones(2, 1, 4), torch.ones(2, 1, 4))
+    assert kv.get_k_cache_scale() is not None
+    kv = shim.KVCache(k.to(torch.int8), k.to(torch.int8), torch.empty(0), torch.empty(0))
+    assert kv.get_k_cache_scale() is None  # empty scale tensors mean "not quantised" (kv_cache.cpp:56-67)
+    assert shim.KVCache().empty()
+
+
+def test_contract_violations_throw_before_any_launch(shim):
+    p = shim.ReshapePagedCacheParams()
+    p.key = torch.zeros(3, 2, 8)
+    p.value = torch.zeros(3, 2, 8)
+    p.k_cache = torch.zeros(2, 2, 4, 8)
+    p.v_cache = torch.zeros(2, 2, 4, 8)
+    p.slot_mapping = torch.zeros(3, dtype=torch.int64)
+    with pytest.raises(RuntimeError, match="slot_mapping"):
+        shim.reshape_paged_cache(p)
+    p.slot_mapping = torch.zeros(3, dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="k_cache_scale is required"):
+        shim.quant_to_paged_cache(p)
+    with pytest.raises(RuntimeError, match="GPU"):
+        shim.reshape_paged_cache(p)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kv", ["bf16", "int8"])
+def test_attention_impl_write_then_attend(gpu, shim, kv):
+    """AttentionImpl::forward on a decode step: the new token's K/V land in the cache bit-exactly and
+    the output matches the oracle run on the updated cache."""
+    print("case shim AttentionImpl", kv, flush=True)
+    B, Hq, Hkv, D, bs = 5, 32, 8, 128, 16
+    lens = np.array([300, 17, 1, 4096, 64], np.int32)  # kv lengths including the new token
+    rng = np.random.default_rng(3)
+    need = (lens + bs - 1) // bs
+    nblocks = int(need.sum()) + 2
+    perm = rng.permutation(nblocks - 1) + 1
+    lists, o = [], 0
+    for b in range(B):
+        lists.append(perm[o:o + need[b]].astype(np.int32))
+        o += int(need[b])
+    table = orc.pad_block_tables(lists)
+    slots = np.array([orc.kv_cache_slots(lists[b], bs, int(lens[b]) - 1, int(lens[b]))[0] for b in range(B)], np.int32)
+    g = torch.Generator().manual_seed(5)
+    kf = torch.randn(nblocks, Hkv, bs, D, generator=g)
+    vf = torch.randn(nblocks, Hkv, bs, D, generator=g)
+    qkv = torch.randn(B, (Hq + 2 * Hkv) * D, generator=g).to(torch.bfloat16)  # fused projection output
+    q, k, v = qkv[:, : Hq * D], qkv[:, Hq * D:(Hq + Hkv) * D], qkv[:, (Hq + Hkv) * D:]
+    scale = 1.0 / float(np.sqrt(D))
+
+    k_new = k.float().numpy().reshape(B, Hkv, D)
+    v_new = v.float().numpy().reshape(B, Hkv, D)
+    if kv == "bf16":
+        kc, vc = kf.to(torch.bfloat16), vf.to(torch.bfloat16)
+        k_ref, v_ref = kc.float().numpy(), vc.float().numpy()
+        orc.reshape_paged_cache(slots, k_new, v_new, k_ref, v_ref, "HND")
+        cache = shim.KVCache(kc.to(gpu), vc.to(gpu))
+        k_deq, v_deq = k_ref, v_ref
+    else:
+        qk, sk = orc.quantize_per_token_head(kf.numpy(), "int8")
+        qv, sv = orc.quantize_per_token_head(vf.numpy(), "int8")
+        orc.quant_to_paged_cache(slots, k_new, v_new, qk, qv, sk, sv, "int8", "HND")
+        cache = shim.KVCache(torch.from_numpy(orc.quantize_per_token_head(kf.numpy(), "int8")[0]).to(gpu),
+                             torch.from_numpy(orc.quantize_per_token_head(vf.numpy(), "int8")[0]).to(gpu),
+                             torch.from_numpy(orc.quantize_per_token_head(kf.numpy(), "int8")[1]).to(gpu),
+                             torch.from_numpy(orc.quantize_per_token_head(vf.numpy(), "int8")[1]).to(gpu))
+        k_deq, v_deq = orc.dequantize(qk, sk, "int8"), orc.dequantize(qv, sv, "int8")
+    ref, _ = orc.paged_decode(q.float().numpy().reshape(B, Hq, D), k_deq, v_deq, table, lens, scale)
+
+    i32 = lambda a: torch.tensor(np.asarray(a), dtype=torch.int32, device=gpu)
+    cu_kv = np.concatenate([[0], np.cumsum(lens)])
+    md = shim.build_decode_metadata(i32(np.arange(B + 1)), i32(cu_kv), i32(slots), i32(table), 1, int(lens.max()),
+                                    int(lens.sum()))
+    attn = shim.AttentionImpl(Hq, D, scale, Hkv, -1)
+    qkv_d = qkv.to(gpu)
+    out, lse = attn.forward(md, qkv_d[:, : Hq * D], qkv_d[:, Hq * D:(Hq + Hkv) * D], qkv_d[:, (Hq + Hkv) * D:], cache)
+    torch.cuda.synchronize()
+    assert lse is None and tuple(out.shape) == (B, Hq * D)
+    # the write is bit-exact
+    if kv == "bf16":
+        assert np.array_equal(cache.get_k_cache().float().cpu().numpy(), k_ref)
+        assert np.array_equal(cache.get_v_cache().float().cpu().numpy(), v_ref)
+    else:
+        assert np.array_equal(cache.get_k_cache().cpu().numpy(), qk)
+        assert np.array_equal(cache.get_v_cache_scale().cpu().numpy(), sv)
+    err = float(np.abs(out.float().cpu().numpy().reshape(B, Hq, D) - ref).max())
+    print("   err %.3e" % err, flush=True)
+    assert err <= (5e-2 if kv == "int8" else 2e-2)
+
+    # dummy batch / empty step: untouched buffer of the right shape, nothing launched
+    md.is_dummy = True
+    out2, _ = attn.forward(md, qkv_d[:, : Hq * D], qkv_d[:, Hq * D:(Hq + Hkv) * D], qkv_d[:, (Hq + Hkv) * D:], cache)
+    assert tuple(out2.shape) == (B, Hq * D)
+    md.is_dummy = False
+    md.is_prefill = True
+    with pytest.raises(RuntimeError, match="decode path only"):
+        attn.forward(md, qkv_d[:, : Hq * D], qkv_d[:, Hq * D:(Hq + Hkv) * D], qkv_d[:, (Hq + Hkv) * D:], cache)
+
+
+@pytest.mark.gpu
+def test_cpp_ops_match_python_ops(gpu, shim):
+    print("case shim ops", flush=True)
+    from tests.helpers import Case
+
+    case = Case(3, 32, 8, 128, 16, [500, 33, 2000], seed=41)
+    ref, _ = case.run()
+    out = torch.empty_like(case.q).view(3, 1, 32, 128)
+    lse = torch.empty(3, 32, dtype=torch.float32, device=gpu)
+    shim.batch_decode(case.q.view(3, 1, 32, 128), case.k_cache, out, case.block_table, case.seq_lens, case.v_cache,
+                      lse, None, None, 2000, -1, case.scale, True, -1)
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(3, 32, 128), ref)
+    # CSR form with the CUDA backend's NHD cache shape
+    lists = [case.table[i, : (int(L) + 15) // 16] for i, L in enumerate(case.lens)]
+    indptr, indices, last = orc.build_paged_kv_csr(lists, case.lens, 16)
+    out_c = torch.empty_like(case.q)
+    shim.batch_decode_csr(case.q, case.k_cache.permute(0, 2, 1, 3).contiguous(),
+                          case.v_cache.permute(0, 2, 1, 3).contiguous(), torch.from_numpy(indptr).to(gpu),
+                          torch.from_numpy(indices).to(gpu), torch.from_numpy(last).to(gpu), -1, case.scale, out_c)
+    torch.cuda.synchronize()
+    assert torch.equal(out_c, ref)

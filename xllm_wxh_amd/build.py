@@ -58,6 +58,49 @@ def build_library(verbose=True, save_temps=False):
     return LIB_PATH
 
 
+TORCH_SHIM_NAME = "_xllm_hip_torch.so"
+TORCH_SHIM_PATH = os.path.join(PKG_DIR, TORCH_SHIM_NAME)
+TORCH_SHIM_SOURCES = ["ops_api.cpp", "attention.cpp", "pybind.cpp"]
+
+
+def build_torch_shim(verbose=True):
+    """Compile the libtorch host side (xllm::kernel / xllm::layer mirrors + pybind module) with g++.
+    Host code only: it reaches the GPU through the C ABI of LIB_PATH, which must exist."""
+    import sysconfig
+
+    import pybind11
+    import torch
+    from torch.utils import cpp_extension as ce
+
+    if not os.path.exists(LIB_PATH):
+        build_library(verbose=verbose)
+    build_dir = os.path.join(REPO_DIR, "build")
+    os.makedirs(build_dir, exist_ok=True)
+    shim_dir = os.path.join(CSRC_DIR, "torch_shim")
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    tmp_out = os.path.join(build_dir, TORCH_SHIM_NAME)
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           "-DTORCH_EXTENSION_NAME=_xllm_hip_torch",
+           "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI), "-Wno-deprecated-declarations"]
+    for inc in ce.include_paths() + [pybind11.get_include(), sysconfig.get_paths()["include"],
+                                      os.path.join(rocm, "include")]:
+        cmd += ["-isystem", inc]
+    cmd += [os.path.join(shim_dir, s) for s in TORCH_SHIM_SOURCES]
+    for lib_dir in ce.library_paths():
+        cmd += ["-L" + lib_dir, "-Wl,-rpath," + lib_dir]
+    cmd += ["-L" + PKG_DIR, "-Wl,-rpath,$ORIGIN", "-l:" + LIB_NAME, "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch",
+            "-ltorch_python", "-o", tmp_out]
+    if verbose:
+        print("[build]", " ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("g++ failed:\n" + proc.stdout)
+    os.replace(tmp_out, TORCH_SHIM_PATH)
+    return TORCH_SHIM_PATH
+
+
 if __name__ == "__main__":
     build_library(save_temps="--save-temps" in sys.argv)
     print(LIB_PATH)
+    if "--no-shim" not in sys.argv:
+        print(build_torch_shim())

@@ -1,0 +1,84 @@
+#include "attention.h"
+
+#include "ops_api.h"
+
+namespace xllm::layer {
+
+AttentionImpl::AttentionImpl(int64_t num_heads, int64_t head_size, float scale, int64_t num_kv_heads,
+                             int64_t sliding_window)
+    : num_heads_(num_heads), head_size_(head_size), scale_(scale), num_kv_heads_(num_kv_heads),
+      // window_left = sliding_window - 1; -1 disables it (xllm/core/layers/mlu/attention.cpp:60-63)
+      sliding_window_(sliding_window > -1 ? sliding_window - 1 : sliding_window) {}
+
+std::tuple<torch::Tensor, std::optional<torch::Tensor>> AttentionImpl::forward(
+    const AttentionMetadata& attn_metadata, torch::Tensor& query, torch::Tensor& key, torch::Tensor& value,
+    KVCache& kv_cache) {
+  std::optional<torch::Tensor> output_lse = std::nullopt;
+  torch::Tensor output = torch::empty_like(query);
+  // dummy batches and empty steps return the untouched buffer
+  // (xllm/core/layers/mlu/attention.cpp:80-82, xllm/core/layers/cuda/flashinfer_attention.cpp:120-123)
+  if (attn_metadata.is_dummy || attn_metadata.max_seq_len == 0) {
+    return {output.view({-1, num_heads_ * head_size_}), output_lse};
+  }
+  TORCH_CHECK(!attn_metadata.is_prefill && !attn_metadata.is_chunked_prefill,
+              "the HIP backend implements the decode path only (prefill is served elsewhere)");
+
+  torch::Tensor k_cache = kv_cache.get_k_cache();
+  torch::Tensor v_cache = kv_cache.get_v_cache();
+  std::optional<torch::Tensor> k_cache_scale = kv_cache.get_k_cache_scale();
+  std::optional<torch::Tensor> v_cache_scale = kv_cache.get_v_cache_scale();
+
+  // 1. KV write of the step's new tokens (write, then attend).
+  xllm::kernel::ReshapePagedCacheParams write;
+  write.key = key.view({-1, num_kv_heads_, head_size_});
+  write.value = value.view({-1, num_kv_heads_, head_size_});
+  write.k_cache = k_cache;
+  write.v_cache = v_cache;
+  write.slot_mapping = attn_metadata.slot_mapping;
+  if (k_cache_scale.has_value()) {
+    write.k_cache_scale = k_cache_scale;
+    write.v_cache_scale = v_cache_scale;
+    xllm::kernel::quant_to_paged_cache(write);
+  } else {
+    xllm::kernel::reshape_paged_cache(write);
+  }
+
+  // 2. Decode.
+  decoder_forward(attn_metadata, query, output, k_cache, v_cache, k_cache_scale, v_cache_scale);
+  return {output.view({-1, num_heads_ * head_size_}), output_lse};
+}
+
+void AttentionImpl::decoder_forward(const AttentionMetadata& attn_metadata, torch::Tensor& query,
+                                    torch::Tensor& output, const torch::Tensor& k_cache,
+                                    const torch::Tensor& v_cache, const std::optional<torch::Tensor>& k_cache_scale,
+                                    const std::optional<torch::Tensor>& v_cache_scale) {
+  std::optional<torch::Tensor> output_lse = std::nullopt;
+  // One decode row per query token by default (speculative verify arrives expanded into rows,
+  // xllm/core/runtime/speculative_worker_impl.cpp:230-243); a batch whose sequences all carry
+  // max_query_len > 1 tokens against one block-table row each is the multi-token form.
+  int64_t q_len = 1;
+  if (attn_metadata.max_query_len > 1 && attn_metadata.block_table.defined() &&
+      attn_metadata.block_table.size(0) * attn_metadata.max_query_len == query.size(0)) {
+    q_len = attn_metadata.max_query_len;
+  }
+  torch::Tensor q4 = query.view({-1, q_len, num_heads_, head_size_});
+  torch::Tensor o4 = output.view({-1, q_len, num_heads_, head_size_});
+  if (attn_metadata.block_table.defined() && attn_metadata.kv_seq_lens.defined()) {
+    xllm::kernel::hip::batch_decode(q4, k_cache, o4, attn_metadata.block_table, attn_metadata.kv_seq_lens, v_cache,
+                                    output_lse, std::nullopt, k_cache_scale, v_cache_scale, std::nullopt,
+                                    std::nullopt, std::nullopt, "float", attn_metadata.max_seq_len, sliding_window_,
+                                    -1, scale_, false, k_cache_scale.has_value() ? 8 : -1,
+                                    attn_metadata.total_kv_len);
+  } else {
+    TORCH_CHECK(attn_metadata.paged_kv_indptr.defined(), "neither block_table nor the CSR arrays are set");
+    TORCH_CHECK(!k_cache_scale.has_value(), "the CSR form serves unquantised caches");
+    torch::Tensor q3 = query.view({-1, num_heads_, head_size_});
+    torch::Tensor o3 = output.view({-1, num_heads_, head_size_});
+    // the CSR entry point takes the CUDA backend's NHD shape: hand it the NHD view of our HND cache
+    xllm::kernel::hip::batch_decode_csr(q3, k_cache.permute({0, 2, 1, 3}), v_cache.permute({0, 2, 1, 3}),
+                                        attn_metadata.paged_kv_indptr, attn_metadata.paged_kv_indices,
+                                        attn_metadata.paged_kv_last_page_len, sliding_window_, scale_, o3, output_lse);
+  }
+}
+
+}  // namespace xllm::layer

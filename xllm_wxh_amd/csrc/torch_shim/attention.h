@@ -1,0 +1,44 @@
+// Decode dispatch of the HIP backend: KV write, then paged decode — the role of
+// xllm::layer::AttentionImpl (xllm/core/layers/cuda/attention.h:41-46,
+// xllm/core/layers/mlu/attention.h:47-52; same constructor and forward signature on every backend).
+#pragma once
+
+#include <torch/torch.h>
+
+#include <optional>
+#include <tuple>
+
+#include "attention_metadata.h"
+#include "kv_cache.h"
+
+namespace xllm::layer {
+
+class AttentionImpl {
+ public:
+  AttentionImpl(int64_t num_heads, int64_t head_size, float scale, int64_t num_kv_heads, int64_t sliding_window);
+
+  // query [T, Hq*D], key/value [T, Hkv*D] (slices of the fused qkv buffer are fine).
+  // Returns (output [T, Hq*D], lse = nullopt).
+  std::tuple<torch::Tensor, std::optional<torch::Tensor>> forward(const AttentionMetadata& attn_metadata,
+                                                                   torch::Tensor& query,
+                                                                   torch::Tensor& key,
+                                                                   torch::Tensor& value,
+                                                                   KVCache& kv_cache);
+
+ private:
+  void decoder_forward(const AttentionMetadata& attn_metadata,
+                       torch::Tensor& query,
+                       torch::Tensor& output,
+                       const torch::Tensor& k_cache,
+                       const torch::Tensor& v_cache,
+                       const std::optional<torch::Tensor>& k_cache_scale,
+                       const std::optional<torch::Tensor>& v_cache_scale);
+
+  int64_t num_heads_;
+  int64_t head_size_;
+  float scale_;
+  int64_t num_kv_heads_;
+  int64_t sliding_window_;
+};
+
+}  // namespace xllm::layer

@@ -1,0 +1,56 @@
+// Batch-level attention inputs shared by every layer of a step: the fields of
+// xllm::layer::AttentionMetadata (xllm/core/layers/common/attention_metadata.h:68-153) that the
+// decode path reads, built from cumulative lengths the way
+// xllm/core/layers/common/attention_metadata_builder.cpp:29-124 does.
+#pragma once
+
+#include <torch/torch.h>
+
+namespace xllm::layer {
+
+struct AttentionMetadata {
+  torch::Tensor q_cu_seq_lens;
+  torch::Tensor kv_cu_seq_lens;
+  torch::Tensor kv_seq_lens;  // per sequence (diff of the cumulative lengths)
+  torch::Tensor q_seq_lens;
+  torch::Tensor block_table;   // [batch, max_blocks] int32, padded with 0
+  torch::Tensor slot_mapping;  // [num_tokens] int32
+  int64_t max_query_len = 0;
+  int64_t max_seq_len = 0;
+  int64_t total_kv_len = 0;
+  bool is_prefill = false;
+  bool is_chunked_prefill = false;
+  bool is_dummy = false;
+  bool is_causal = false;
+  // CSR form of the block lists (the CUDA backend's inputs).
+  torch::Tensor paged_kv_indptr;
+  torch::Tensor paged_kv_indices;
+  torch::Tensor paged_kv_last_page_len;
+};
+
+// Decode-step metadata from the batch builder's tensors: cumulative kv/q lengths [batch+1],
+// new_cache_slots, block_tables.  kv_seq_lens = diff(cumulative) (attention_metadata_builder.cpp:105);
+// a dummy batch (q_max_seq_len == 0) writes slot 1 only (:120-124).
+inline AttentionMetadata build_decode_metadata(const torch::Tensor& q_cu_seq_lens,
+                                               const torch::Tensor& kv_cu_seq_lens,
+                                               const torch::Tensor& new_cache_slots,
+                                               const torch::Tensor& block_tables,
+                                               int64_t q_max_seq_len,
+                                               int64_t kv_max_seq_len,
+                                               int64_t total_kv_len) {
+  AttentionMetadata m;
+  m.q_cu_seq_lens = q_cu_seq_lens;
+  m.kv_cu_seq_lens = kv_cu_seq_lens;
+  m.max_query_len = q_max_seq_len;
+  m.max_seq_len = kv_max_seq_len;
+  m.total_kv_len = total_kv_len;
+  m.slot_mapping = new_cache_slots;
+  m.block_table = block_tables;
+  m.kv_seq_lens = torch::diff(kv_cu_seq_lens).contiguous();
+  m.q_seq_lens = torch::diff(q_cu_seq_lens).contiguous();
+  m.is_dummy = q_max_seq_len == 0;
+  if (m.is_dummy) m.slot_mapping = torch::tensor({1}, new_cache_slots.options());
+  return m;
+}
+
+}  // namespace xllm::layer

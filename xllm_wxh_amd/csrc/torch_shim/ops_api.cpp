@@ -1,0 +1,260 @@
+#include "ops_api.h"
+
+#include <c10/hip/HIPStream.h>
+
+#include <mutex>
+#include <unordered_map>
+
+#include "../../../include/xllm_hip_paged_kv.h"
+
+namespace xllm::kernel {
+namespace {
+
+int32_t dtype_code(const torch::Tensor& t) {
+  switch (t.scalar_type()) {
+    case torch::kBFloat16:
+      return XLLM_HIP_BF16;
+    case torch::kHalf:
+      return XLLM_HIP_FP16;
+    case torch::kFloat:
+      return XLLM_HIP_FP32;
+    case torch::kFloat8_e4m3fn:
+      return XLLM_HIP_FP8_E4M3;
+    case torch::kChar:
+      return XLLM_HIP_INT8;
+    default:
+      TORCH_CHECK(false, "unsupported dtype ", t.scalar_type());
+  }
+}
+
+xllm_hip_stream_t current_stream(const torch::Tensor& t) {
+  return (xllm_hip_stream_t)c10::hip::getCurrentHIPStream(t.device().index()).stream();
+}
+
+void check_status(int status) {
+  TORCH_CHECK(status == XLLM_HIP_OK, "xllm_hip status ", status, ": ", xllm_hip_last_error());
+}
+
+// Cache descriptor from [blocks, heads, slots, dim]-shaped tensors of any strides.
+xllm_hip_kv_cache make_cache(const torch::Tensor& k,
+                             const std::optional<torch::Tensor>& v,
+                             const std::optional<torch::Tensor>& k_scale,
+                             const std::optional<torch::Tensor>& v_scale) {
+  TORCH_CHECK(k.defined() && k.dim() == 4, "k_cache must be [num_blocks, num_kv_heads, block_size, head_dim]");
+  TORCH_CHECK(k.is_cuda(), "k_cache must live on the GPU");
+  TORCH_CHECK(k.stride(3) == 1, "head_dim of k_cache must be contiguous");
+  xllm_hip_kv_cache c{};
+  c.k_cache = k.data_ptr();
+  if (v.has_value() && v->defined()) {
+    TORCH_CHECK(v->sizes() == k.sizes() && v->strides() == k.strides() && v->scalar_type() == k.scalar_type(),
+                "v_cache must match k_cache in shape, strides and dtype");
+    c.v_cache = v->data_ptr();
+  }
+  c.num_blocks = k.size(0);
+  c.num_kv_heads = (int32_t)k.size(1);
+  c.block_size = (int32_t)k.size(2);
+  c.head_dim = (int32_t)k.size(3);
+  c.dtype = dtype_code(k);
+  c.stride_block = k.stride(0);
+  c.stride_head = k.stride(1);
+  c.stride_slot = k.stride(2);
+  if (k_scale.has_value() && k_scale->defined()) {
+    TORCH_CHECK(k_scale->scalar_type() == torch::kFloat && k_scale->dim() == 3 && k_scale->size(0) == k.size(0) &&
+                    k_scale->size(1) == k.size(1) && k_scale->size(2) == k.size(2),
+                "k_cache_scale must be float32 [num_blocks, num_kv_heads, block_size]");
+    c.k_scale = k_scale->data_ptr<float>();
+    c.scale_stride_block = k_scale->stride(0);
+    c.scale_stride_head = k_scale->stride(1);
+    c.scale_stride_slot = k_scale->stride(2);
+    if (v_scale.has_value() && v_scale->defined()) {
+      TORCH_CHECK(v_scale->sizes() == k_scale->sizes() && v_scale->strides() == k_scale->strides() &&
+                      v_scale->scalar_type() == torch::kFloat,
+                  "v_cache_scale must match k_cache_scale");
+      c.v_scale = v_scale->data_ptr<float>();
+    }
+  }
+  return c;
+}
+
+void check_write_inputs(const ReshapePagedCacheParams& p) {
+  TORCH_CHECK(p.key.defined() && p.k_cache.defined() && p.slot_mapping.defined(),
+              "key, k_cache and slot_mapping are required");
+  TORCH_CHECK(!p.direction, "direction=true (cache to context) is not part of the decode path");
+  TORCH_CHECK(p.key.dim() == 3, "key must be [num_tokens, num_kv_heads, head_dim]");
+  // keys and values should be continuous at n_kv_heads and head_dim dims
+  TORCH_CHECK(p.key.stride(-1) == 1 && p.key.stride(-2) == p.key.size(-1),
+              "key must be contiguous in its last two dimensions");
+  if (p.value.has_value()) {
+    TORCH_CHECK(p.value->sizes() == p.key.sizes() && p.value->scalar_type() == p.key.scalar_type(),
+                "value must match key");
+    TORCH_CHECK(p.value->stride(-1) == 1 && p.value->stride(-2) == p.value->size(-1),
+                "value must be contiguous in its last two dimensions");
+    TORCH_CHECK(p.v_cache.has_value(), "value given without v_cache");
+  } else {
+    TORCH_CHECK(!p.v_cache.has_value(), "v_cache given without value");
+  }
+  TORCH_CHECK(p.slot_mapping.scalar_type() == torch::kInt && p.slot_mapping.dim() == 1 &&
+                  p.slot_mapping.is_contiguous() && p.slot_mapping.numel() == p.key.size(0),
+              "slot_mapping must be a contiguous int32 vector with one entry per token");
+  TORCH_CHECK(p.key.size(1) == p.k_cache.size(1) && p.key.size(2) == p.k_cache.size(3),
+              "key heads/head_dim do not match the cache");
+}
+
+}  // namespace
+
+void reshape_paged_cache(ReshapePagedCacheParams& params) {
+  check_write_inputs(params);
+  const xllm_hip_kv_cache cache = make_cache(params.k_cache, params.v_cache, std::nullopt, std::nullopt);
+  const bool has_v = params.value.has_value();
+  check_status(xllm_hip_reshape_paged_cache(&cache, params.key.data_ptr(), has_v ? params.value->data_ptr() : nullptr,
+                                            params.slot_mapping.data_ptr<int32_t>(), params.key.size(0),
+                                            params.key.stride(0), has_v ? params.value->stride(0) : 0,
+                                            dtype_code(params.key), current_stream(params.key)));
+}
+
+void quant_to_paged_cache(ReshapePagedCacheParams& params) {
+  check_write_inputs(params);
+  TORCH_CHECK(params.k_cache_scale.has_value(), "k_cache_scale is required for quant_to_paged_cache");
+  const xllm_hip_kv_cache cache =
+      make_cache(params.k_cache, params.v_cache, params.k_cache_scale, params.v_cache_scale);
+  const bool has_v = params.value.has_value();
+  check_status(xllm_hip_quant_to_paged_cache(&cache, params.key.data_ptr(), has_v ? params.value->data_ptr() : nullptr,
+                                             params.slot_mapping.data_ptr<int32_t>(), params.key.size(0),
+                                             params.key.stride(0), has_v ? params.value->stride(0) : 0,
+                                             dtype_code(params.key), current_stream(params.key)));
+}
+
+namespace hip {
+
+torch::Tensor decode_workspace(const torch::Device& device, size_t bytes) {
+  static std::mutex mu;
+  static std::unordered_map<int, torch::Tensor> per_device;
+  std::lock_guard<std::mutex> lock(mu);
+  torch::Tensor& ws = per_device[device.index()];
+  if (!ws.defined() || (size_t)ws.numel() < bytes) {
+    ws = torch::empty({(int64_t)bytes}, torch::TensorOptions().dtype(torch::kUInt8).device(device));
+  }
+  return ws;
+}
+
+namespace {
+
+void run_decode(const xllm_hip_kv_cache& cache, xllm_hip_decode_args& a, const torch::Tensor& q3) {
+  const size_t need =
+      xllm_hip_paged_decode_workspace_bytes(a.batch, a.q_per_seq, a.num_q_heads, cache.num_kv_heads, cache.head_dim);
+  torch::Tensor ws = decode_workspace(q3.device(), need);
+  check_status(xllm_hip_paged_decode(&cache, &a, ws.data_ptr(), (size_t)ws.numel(), current_stream(q3)));
+}
+
+void fill_q_out(xllm_hip_decode_args& a, const torch::Tensor& q3, torch::Tensor& o3, int64_t q_per_seq) {
+  TORCH_CHECK(q3.dim() == 3 && o3.dim() == 3 && o3.sizes() == q3.sizes() && o3.scalar_type() == q3.scalar_type(),
+              "output must match query [tokens, heads, head_dim]");
+  TORCH_CHECK(q3.stride(2) == 1 && q3.stride(1) == q3.size(2) && o3.stride(2) == 1 && o3.stride(1) == o3.size(2),
+              "query/output heads and head_dim must be contiguous");
+  TORCH_CHECK(q_per_seq >= 1 && q3.size(0) % q_per_seq == 0, "query tokens not divisible by q_len");
+  a.q = q3.data_ptr();
+  a.out = o3.data_ptr();
+  a.q_token_stride = q3.stride(0);
+  a.out_token_stride = o3.stride(0);
+  a.q_dtype = dtype_code(q3);
+  a.batch = (int32_t)(q3.size(0) / q_per_seq);
+  a.q_per_seq = (int32_t)q_per_seq;
+  a.num_q_heads = (int32_t)q3.size(1);
+}
+
+}  // namespace
+
+void batch_decode(const torch::Tensor& query,
+                  const torch::Tensor& k_cache,
+                  torch::Tensor& output,
+                  const torch::Tensor& block_table,
+                  const torch::Tensor& seq_lens,
+                  const std::optional<torch::Tensor>& v_cache,
+                  std::optional<torch::Tensor>& output_lse,
+                  const std::optional<torch::Tensor>& q_quant_scale,
+                  const std::optional<torch::Tensor>& k_cache_quant_scale,
+                  const std::optional<torch::Tensor>& v_cache_quant_scale,
+                  const std::optional<torch::Tensor>& out_quant_scale,
+                  const std::optional<torch::Tensor>& alibi_slope,
+                  const std::optional<torch::Tensor>& mask,
+                  const std::string& /*compute_dtype*/,
+                  int64_t max_seq_len,
+                  int64_t window_size_left,
+                  int64_t window_size_right,
+                  float scale,
+                  bool return_lse,
+                  int64_t kv_cache_quant_bit_size,
+                  int64_t total_kv_len) {
+  TORCH_CHECK(v_cache.has_value(), "v_cache is required (single-cache MLA decode is outside this path)");
+  TORCH_CHECK(!q_quant_scale.has_value() && !out_quant_scale.has_value() && !alibi_slope.has_value() &&
+                  !mask.has_value(),
+              "q/out quantisation, alibi and custom masks are not supported by the HIP decode path");
+  TORCH_CHECK(window_size_right < 0, "window_size_right must be -1 for decode");
+  const bool quant = k_cache_quant_scale.has_value();
+  TORCH_CHECK(kv_cache_quant_bit_size == -1 || (kv_cache_quant_bit_size == 8 && quant),
+              "kv_cache_quant_bit_size must be -1, or 8 together with k/v_cache_quant_scale");
+  TORCH_CHECK(!quant || v_cache_quant_scale.has_value(), "v_cache_quant_scale is required with k_cache_quant_scale");
+  TORCH_CHECK(query.dim() == 4 && output.dim() == 4, "query/output must be [batch, q_len, heads, head_dim]");
+  const xllm_hip_kv_cache cache = make_cache(k_cache, v_cache, k_cache_quant_scale, v_cache_quant_scale);
+
+  torch::Tensor q3 = query.view({-1, query.size(2), query.size(3)});
+  torch::Tensor o3 = output.view({-1, output.size(2), output.size(3)});
+  xllm_hip_decode_args a{};
+  fill_q_out(a, q3, o3, query.size(1));
+  TORCH_CHECK(q3.size(2) == cache.head_dim, "query head_dim does not match the cache");
+  a.sm_scale = scale;
+  a.window_left = (int32_t)window_size_left;
+  TORCH_CHECK(block_table.scalar_type() == torch::kInt && block_table.dim() == 2 && block_table.stride(1) == 1 &&
+                  block_table.size(0) == a.batch,
+              "block_table must be int32 [batch, max_blocks]");
+  TORCH_CHECK(seq_lens.scalar_type() == torch::kInt && seq_lens.is_contiguous() && seq_lens.numel() == a.batch,
+              "seq_lens must be contiguous int32 [batch]");
+  a.block_table = block_table.data_ptr<int32_t>();
+  a.block_table_stride = block_table.stride(0);
+  a.max_blocks_per_seq = (int32_t)block_table.size(1);
+  a.seq_lens = seq_lens.data_ptr<int32_t>();
+  a.max_seq_len = (int32_t)max_seq_len;
+  a.total_kv_len = total_kv_len;
+  if (return_lse) {
+    TORCH_CHECK(output_lse.has_value(), "return_lse needs a pre-allocated output_lse");
+  }
+  if (output_lse.has_value() && output_lse->defined()) {
+    TORCH_CHECK(output_lse->scalar_type() == torch::kFloat && output_lse->is_contiguous() &&
+                    output_lse->numel() == q3.size(0) * q3.size(1),
+                "output_lse must be contiguous float32 [tokens, heads]");
+    a.lse = output_lse->data_ptr<float>();
+  }
+  run_decode(cache, a, q3);
+}
+
+void batch_decode_csr(torch::Tensor query,
+                      torch::Tensor k_cache,
+                      torch::Tensor v_cache,
+                      torch::Tensor paged_kv_indptr,
+                      torch::Tensor paged_kv_indices,
+                      torch::Tensor paged_kv_last_page_len,
+                      int64_t window_left,
+                      double sm_scale,
+                      torch::Tensor output,
+                      std::optional<torch::Tensor>& output_lse) {
+  // NHD [blocks, block_size, Hkv, D] -> logical [blocks, Hkv, block_size, D] view
+  const xllm_hip_kv_cache cache =
+      make_cache(k_cache.permute({0, 2, 1, 3}), v_cache.permute({0, 2, 1, 3}), std::nullopt, std::nullopt);
+  xllm_hip_decode_args a{};
+  fill_q_out(a, query, output, 1);
+  a.sm_scale = (float)sm_scale;
+  a.window_left = (int32_t)window_left;
+  for (const torch::Tensor* t : {&paged_kv_indptr, &paged_kv_indices, &paged_kv_last_page_len}) {
+    TORCH_CHECK(t->scalar_type() == torch::kInt && t->is_contiguous(), "CSR arrays must be contiguous int32");
+  }
+  TORCH_CHECK(paged_kv_indptr.numel() == a.batch + 1 && paged_kv_last_page_len.numel() == a.batch,
+              "CSR arrays do not match the batch");
+  a.kv_indptr = paged_kv_indptr.data_ptr<int32_t>();
+  a.kv_indices = paged_kv_indices.data_ptr<int32_t>();
+  a.kv_last_page_len = paged_kv_last_page_len.data_ptr<int32_t>();
+  if (output_lse.has_value() && output_lse->defined()) a.lse = output_lse->data_ptr<float>();
+  run_decode(cache, a, query);
+}
+
+}  // namespace hip
+}  // namespace xllm::kernel

@@ -1,0 +1,70 @@
+// libtorch host side of the HIP backend: the operators of xllm/core/kernels/ops_api.h that lie on
+// the paged-KV decode path, plus the backend's batch_decode in both reference argument lists.
+// Every function only checks the tensor contract and forwards pointers, sizes and strides to the
+// C ABI (include/xllm_hip_paged_kv.h) on torch's current HIP stream; outputs are pre-allocated by
+// the caller and mutated in place.  A contract violation throws through TORCH_CHECK (the reference
+// aborts through glog CHECK: xllm/core/kernels/cuda/reshape_paged_cache.cu:68-69,
+// xllm/core/kernels/ops_api.cpp:198-199).
+#pragma once
+
+#include <torch/torch.h>
+
+#include <optional>
+#include <string>
+
+#include "param.h"
+
+namespace xllm::kernel {
+
+// xllm/core/kernels/ops_api.h:31 — verbatim KV write through slot_mapping.
+void reshape_paged_cache(ReshapePagedCacheParams& params);
+
+// xllm/core/kernels/ops_api.h:35-37 — per-token-per-head quantising KV write (int8 / fp8-e4m3).
+void quant_to_paged_cache(ReshapePagedCacheParams& params);
+
+namespace hip {
+
+// Argument list of xllm::kernel::mlu::batch_decode (xllm/core/kernels/mlu/mlu_ops_api.h:126-145).
+// query/output: [batch, q_len, Hq, D]; q_len > 1 = speculative verify, causal among the q_len tokens.
+void batch_decode(const torch::Tensor& query,
+                  const torch::Tensor& k_cache,
+                  torch::Tensor& output,
+                  const torch::Tensor& block_table,
+                  const torch::Tensor& seq_lens,
+                  const std::optional<torch::Tensor>& v_cache,
+                  std::optional<torch::Tensor>& output_lse,
+                  const std::optional<torch::Tensor>& q_quant_scale,
+                  const std::optional<torch::Tensor>& k_cache_quant_scale,
+                  const std::optional<torch::Tensor>& v_cache_quant_scale,
+                  const std::optional<torch::Tensor>& out_quant_scale,
+                  const std::optional<torch::Tensor>& alibi_slope,
+                  const std::optional<torch::Tensor>& mask,
+                  const std::string& compute_dtype,
+                  int64_t max_seq_len,
+                  int64_t window_size_left,
+                  int64_t window_size_right,
+                  float scale,
+                  bool return_lse,
+                  int64_t kv_cache_quant_bit_size,
+                  int64_t total_kv_len = 0);
+
+// Tensor arguments of xllm::kernel::cuda::batch_decode (xllm/core/kernels/cuda/cuda_ops_api.h:120-136)
+// without the FlashInfer uri / plan / workspaces, which have no counterpart here.
+// query/output: [tokens, Hq, D]; caches in the CUDA backend's NHD shape [blocks, block_size, Hkv, D].
+void batch_decode_csr(torch::Tensor query,
+                      torch::Tensor k_cache,
+                      torch::Tensor v_cache,
+                      torch::Tensor paged_kv_indptr,
+                      torch::Tensor paged_kv_indices,
+                      torch::Tensor paged_kv_last_page_len,
+                      int64_t window_left,
+                      double sm_scale,
+                      torch::Tensor output,
+                      std::optional<torch::Tensor>& output_lse);
+
+// Scratch of the decode kernels for this device, grown on demand — the role of the reference's
+// FlashinferWorkspace singleton (xllm/core/layers/cuda/flashinfer_workspace.cpp:24-38).
+torch::Tensor decode_workspace(const torch::Device& device, size_t bytes);
+
+}  // namespace hip
+}  // namespace xllm::kernel

@@ -1,0 +1,77 @@
+// Python binding of the libtorch host side, so that pytest can drive the C++ operators and the
+// AttentionImpl twin on the GPU box.
+#include <torch/extension.h>
+
+#include "attention.h"
+#include "ops_api.h"
+
+namespace py = pybind11;
+using xllm::KVCache;
+using xllm::kernel::ReshapePagedCacheParams;
+using xllm::layer::AttentionImpl;
+using xllm::layer::AttentionMetadata;
+
+PYBIND11_MODULE(_xllm_hip_torch, m) {
+  py::class_<ReshapePagedCacheParams>(m, "ReshapePagedCacheParams")
+      .def(py::init<>())
+      .def_readwrite("key", &ReshapePagedCacheParams::key)
+      .def_readwrite("value", &ReshapePagedCacheParams::value)
+      .def_readwrite("k_cache", &ReshapePagedCacheParams::k_cache)
+      .def_readwrite("v_cache", &ReshapePagedCacheParams::v_cache)
+      .def_readwrite("slot_mapping", &ReshapePagedCacheParams::slot_mapping)
+      .def_readwrite("direction", &ReshapePagedCacheParams::direction)
+      .def_readwrite("k_cache_scale", &ReshapePagedCacheParams::k_cache_scale)
+      .def_readwrite("v_cache_scale", &ReshapePagedCacheParams::v_cache_scale);
+  m.def("reshape_paged_cache", &xllm::kernel::reshape_paged_cache);
+  m.def("quant_to_paged_cache", &xllm::kernel::quant_to_paged_cache);
+  m.def("batch_decode",
+        [](const torch::Tensor& query, const torch::Tensor& k_cache, torch::Tensor output,
+           const torch::Tensor& block_table, const torch::Tensor& seq_lens, const std::optional<torch::Tensor>& v_cache,
+           std::optional<torch::Tensor> output_lse, const std::optional<torch::Tensor>& k_scale,
+           const std::optional<torch::Tensor>& v_scale, int64_t max_seq_len, int64_t window_size_left, float scale,
+           bool return_lse, int64_t kv_cache_quant_bit_size) {
+          xllm::kernel::hip::batch_decode(query, k_cache, output, block_table, seq_lens, v_cache, output_lse,
+                                          std::nullopt, k_scale, v_scale, std::nullopt, std::nullopt, std::nullopt,
+                                          "float", max_seq_len, window_size_left, -1, scale, return_lse,
+                                          kv_cache_quant_bit_size);
+        });
+  m.def("batch_decode_csr",
+        [](torch::Tensor query, torch::Tensor k_cache, torch::Tensor v_cache, torch::Tensor indptr, torch::Tensor indices,
+           torch::Tensor last_page_len, int64_t window_left, double sm_scale, torch::Tensor output) {
+          std::optional<torch::Tensor> lse = std::nullopt;
+          xllm::kernel::hip::batch_decode_csr(query, k_cache, v_cache, indptr, indices, last_page_len, window_left,
+                                              sm_scale, output, lse);
+        });
+
+  py::class_<KVCache>(m, "KVCache")
+      .def(py::init<>())
+      .def(py::init<torch::Tensor, torch::Tensor>())
+      .def(py::init<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor>())
+      .def("get_k_cache", &KVCache::get_k_cache)
+      .def("get_v_cache", &KVCache::get_v_cache)
+      .def("get_k_cache_scale", &KVCache::get_k_cache_scale)
+      .def("get_v_cache_scale", &KVCache::get_v_cache_scale)
+      .def("empty", &KVCache::empty);
+
+  py::class_<AttentionMetadata>(m, "AttentionMetadata")
+      .def(py::init<>())
+      .def_readwrite("kv_seq_lens", &AttentionMetadata::kv_seq_lens)
+      .def_readwrite("q_seq_lens", &AttentionMetadata::q_seq_lens)
+      .def_readwrite("block_table", &AttentionMetadata::block_table)
+      .def_readwrite("slot_mapping", &AttentionMetadata::slot_mapping)
+      .def_readwrite("max_query_len", &AttentionMetadata::max_query_len)
+      .def_readwrite("max_seq_len", &AttentionMetadata::max_seq_len)
+      .def_readwrite("total_kv_len", &AttentionMetadata::total_kv_len)
+      .def_readwrite("is_prefill", &AttentionMetadata::is_prefill)
+      .def_readwrite("is_chunked_prefill", &AttentionMetadata::is_chunked_prefill)
+      .def_readwrite("is_dummy", &AttentionMetadata::is_dummy)
+      .def_readwrite("paged_kv_indptr", &AttentionMetadata::paged_kv_indptr)
+      .def_readwrite("paged_kv_indices", &AttentionMetadata::paged_kv_indices)
+      .def_readwrite("paged_kv_last_page_len", &AttentionMetadata::paged_kv_last_page_len);
+  m.def("build_decode_metadata", &xllm::layer::build_decode_metadata);
+
+  py::class_<AttentionImpl>(m, "AttentionImpl")
+      .def(py::init<int64_t, int64_t, float, int64_t, int64_t>())
+      .def("forward", [](AttentionImpl& self, const AttentionMetadata& md, torch::Tensor query, torch::Tensor key,
+                         torch::Tensor value, KVCache& kv) { return self.forward(md, query, key, value, kv); });
+}
