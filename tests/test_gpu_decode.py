@@ -310,3 +310,74 @@ def test_host_length_hints_select_the_unsplit_path(gpu, kv, n):
         print("   %s err=%.3e" % (kw, e), flush=True)
         assert e <= (REG_TOL_QUANT if kv == "int8" else REG_TOL)
         assert lse_err(lse, lse_ref) <= LSE_TOL
+
+
+def test_decode_step_replays_under_hip_graph(gpu):
+    """KV write + plan + attention (+ merge) captured once in a HIP graph and replayed while the
+    lengths, slots and block tables change in the persistent input buffers (the way the reference's
+    graph executor feeds its attention, xllm/core/runtime/cuda_graph_executor_impl.cpp:129-180).
+    No host-side length hints are given under capture, so nothing in the graph depends on host
+    values.  Every replay is checked against the eager result, with eager work in between."""
+    print("case hip graph", flush=True)
+    B, Hq, Hkv, D, bs, max_blocks = 6, 32, 8, 128, 16, 300
+    nblocks = B * max_blocks + 1
+    g = torch.Generator().manual_seed(51)
+    k_cache = torch.randn(nblocks, Hkv, bs, D, generator=g).to(torch.bfloat16).to(gpu)
+    v_cache = torch.randn(nblocks, Hkv, bs, D, generator=g).to(torch.bfloat16).to(gpu)
+    perm = (torch.randperm(nblocks - 1, generator=g) + 1).to(torch.int32)
+    table_full = perm[: B * max_blocks].view(B, max_blocks)
+    # persistent buffers the graph reads
+    q = torch.zeros(B, Hq, D, dtype=torch.bfloat16, device=gpu)
+    new_k = torch.zeros(B, Hkv, D, dtype=torch.bfloat16, device=gpu)
+    new_v = torch.zeros(B, Hkv, D, dtype=torch.bfloat16, device=gpu)
+    slots = torch.zeros(B, dtype=torch.int32, device=gpu)
+    block_table = table_full.to(gpu).contiguous()
+    seq_lens = torch.ones(B, dtype=torch.int32, device=gpu)
+    out = torch.zeros(B, Hq, D, dtype=torch.bfloat16, device=gpu)
+    ws = torch.empty(ops.decode_workspace_bytes(B, 1, Hq, Hkv, D), dtype=torch.uint8, device=gpu)
+    scale = 1.0 / float(np.sqrt(D))
+
+    def step(o):
+        ops.reshape_paged_cache(ops.ReshapePagedCacheParams(key=new_k, value=new_v, k_cache=k_cache, v_cache=v_cache,
+                                                            slot_mapping=slots))
+        ops.batch_decode(q, k_cache, o, block_table, seq_lens, v_cache, scale=scale, workspace=ws)
+
+    def load_inputs(lens, seed):
+        gg = torch.Generator().manual_seed(seed)
+        q.copy_(torch.randn(B, Hq, D, generator=gg).to(torch.bfloat16))
+        new_k.copy_(torch.randn(B, Hkv, D, generator=gg).to(torch.bfloat16))
+        new_v.copy_(torch.randn(B, Hkv, D, generator=gg).to(torch.bfloat16))
+        lens_t = torch.tensor(lens, dtype=torch.int32)
+        pos = lens_t - 1
+        blk = table_full[torch.arange(B), (pos // bs).long()]
+        slots.copy_((blk * bs + pos % bs).to(torch.int32))
+        seq_lens.copy_(lens_t)
+
+    load_inputs([100, 20, 4000, 1, 777, 64], 0)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm-up on the capture stream
+        step(out)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step(out)
+    for it, lens in enumerate(([100, 20, 4000, 1, 777, 64], [4799, 3, 17, 2048, 1, 4800], [5, 5, 5, 5, 5, 5],
+                               [1000, 1001, 1002, 4003, 1004, 1005])):
+        load_inputs(lens, 10 + it)
+        k_before, v_before = k_cache.clone(), v_cache.clone()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        k_after = k_cache.clone()
+        # eager reference on the cache as it was before the replay
+        k_cache.copy_(k_before)
+        v_cache.copy_(v_before)
+        eager = torch.zeros_like(out)
+        step(eager)
+        torch.cuda.synchronize()
+        assert torch.equal(got, eager), "replay %d differs from eager" % it
+        assert torch.equal(k_after, k_cache)
+        # some unrelated eager work between replays
+        _ = (k_cache[:8].float() @ torch.ones(D, 4, device=gpu)).sum().item()

@@ -479,7 +479,7 @@ template <>
 struct KvStage<XLLM_HIP_INT8> : KvStageQuant<XLLM_HIP_INT8> {};
 
 template <int KV_DT, int NT>
-__global__ void __launch_bounds__(64 * kWaves, NT == 1 ? 2 : 1) decode_mfma_d128_kernel(DecodeParams p) {
+__global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_d128_kernel(DecodeParams p) {
   constexpr bool kQuant = KV_DT != XLLM_HIP_BF16;
   // int8 rows sit in LDS as x + 128.  With K' = K + 128 and V' = V + 128:
   //   q.K  = q.K' - 128 * sum_d q_d                    (qsum, once per query row)
@@ -488,6 +488,10 @@ __global__ void __launch_bounds__(64 * kWaves, NT == 1 ? 2 : 1) decode_mfma_d128
   constexpr bool kOffset = KV_DT == XLLM_HIP_INT8;
   __shared__ __attribute__((aligned(16))) uint8_t lds_all[kWaves * kLdsWave];
   __shared__ float lds_ml[kWaves * NT * 16 * 2];  // (running max, denominator) per wave and query row
+  // With two tiles of query rows the Q^T fragments live in LDS instead of 32 registers, which keeps
+  // the kernel within the 256 registers that let two workgroups share a CU.
+  constexpr bool kQInLds = NT > 1;
+  __shared__ __attribute__((aligned(16))) uint8_t lds_q[kQInLds ? NT * 4 * 64 * 16 : 16];
 
   Item it;
   if (!decode_item(p, blockIdx.x, it)) return;
@@ -533,7 +537,13 @@ __global__ void __launch_bounds__(64 * kWaves, NT == 1 ? 2 : 1) decode_mfma_d128
       sq += __shfl_xor(sq, 32);
       qsum128[nt] = 128.0f * sq;
     }
+    if (kQInLds) {
+      // every wave stores the same fragments and reads back only what it stored: no barrier needed
+#pragma unroll
+      for (int c = 0; c < 4; ++c) *(bf16x8*)(lds_q + ((nt * 4 + c) * 64 + lane) * 16) = qf[nt][c];
+    }
   }
+  uint32_t q_off = lane * 16;
 
   // Tile range.  With a sliding window, tiles wholly below every row's window are skipped.
   int t0 = it.t_begin;
@@ -577,17 +587,21 @@ __global__ void __launch_bounds__(64 * kWaves, NT == 1 ? 2 : 1) decode_mfma_d128
     constexpr bool MASKED = decltype(masked_tag)::value;
     // ---- S^T = K Q^T ----
     f32x4 s[2][NT];
+    if (kQInLds) asm volatile("" : "+v"(q_off));  // keeps the Q^T reads below inside the loop
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) s[h][nt] = f32x4{0, 0, 0, 0};
+    }
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        const bf16x8 kf = *(const bf16x8*)(lds + k_off[c] + h * 4096);
+    for (int c = 0; c < 4; ++c) {
+      const bf16x8 kf0 = *(const bf16x8*)(lds + k_off[c]);
+      const bf16x8 kf1 = *(const bf16x8*)(lds + k_off[c] + 4096);
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-          s[h][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[nt][c], s[h][nt], 0, 0, 0);
-        }
+      for (int nt = 0; nt < NT; ++nt) {
+        const bf16x8 qv = kQInLds ? *(const bf16x8*)(lds_q + q_off + (nt * 4 + c) * 1024) : qf[nt][c];
+        s[0][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf0, qv, s[0][nt], 0, 0, 0);
+        s[1][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf1, qv, s[1][nt], 0, 0, 0);
       }
     }
     // ---- online softmax, per query row (lane column) ----
@@ -689,7 +703,7 @@ __global__ void __launch_bounds__(64 * kWaves, NT == 1 ? 2 : 1) decode_mfma_d128
     }
   };
   if (w_begin < w_end) {
-    if (kQuant) {
+    if (kQuant && NT == 1) {
       KvStage<KV_DT> stage_b;
       stage.issue(p, it, w_begin, lane);
       if (w_begin + kTileTokens < w_end) stage_b.issue(p, it, w_begin + kTileTokens, lane);
@@ -892,12 +906,12 @@ __global__ void __launch_bounds__(256) csr_to_block_table_kernel(const int32_t* 
 enum Variant { kNone = 0, kMfmaD128 = 1, kGeneric = 2 };
 
 // Split target: about this many work items (workgroups) per launch.  A workgroup of the MFMA kernel
-// is four waves, one per SIMD of a CU; two fit on a CU when the kernel needs at most 256 VGPRs
-// (up to 16 query rows per kv head), one otherwise.  The generic kernel runs one wave per item.
+// is four waves, one per SIMD of a CU, and two workgroups fit on a CU (256 VGPRs, < 80 KiB of LDS).
+// The generic kernel runs one wave per item.
 constexpr int kNumCUs = 256;
 
-static int target_items(int variant_is_mfma, int rows_per_item) {
-  int v = variant_is_mfma ? (rows_per_item <= 16 ? 2 * kNumCUs : kNumCUs) : 8 * kNumCUs;
+static int target_items(int variant_is_mfma) {
+  int v = variant_is_mfma ? 2 * kNumCUs : 8 * kNumCUs;
   if (const char* e = getenv("XLLM_HIP_DECODE_TARGET_ITEMS")) {
     const int t = atoi(e);
     if (t > 0) v = t;
@@ -1017,8 +1031,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
   p.max_blocks_per_seq = a->max_blocks_per_seq;
   p.window_left = a->window_left;
   const Variant variant = pick_variant(c, a);
-  const int rows_per_item = p.rows < kMaxRowsPerItem ? p.rows : kMaxRowsPerItem;
-  p.target_items = target_items(variant == kMfmaD128, rows_per_item);
+  p.target_items = target_items(variant == kMfmaD128);
   // Only the MFMA kernel finishes single-chunk sequences itself.  When the caller's host-side
   // lengths (the reference keeps both in AttentionMetadata) show that the chunk the plan would
   // pick covers the longest sequence, no sequence is split: the plan is told never to split
