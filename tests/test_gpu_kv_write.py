@@ -87,8 +87,10 @@ def test_reshape_paged_cache_edge_cases(gpu):
     slots = torch.tensor([0, 0, -1, nb * bs, 17], dtype=torch.int32, device=gpu)
     ops.reshape_paged_cache(ops.ReshapePagedCacheParams(key=key, value=key, k_cache=kc, v_cache=vc, slot_mapping=slots))
     torch.cuda.synchronize()
+    # Two writers to one slot race (the reference's kernel has the same property); each 16-byte piece
+    # comes from one of them, so every element equals one of the two candidates.
     row0 = kc[0, :, 0, :]
-    assert torch.equal(row0, key[0]) or torch.equal(row0, key[1])
+    assert bool(((row0 == key[0]) | (row0 == key[1])).all())
     assert torch.equal(kc[1, :, 1, :], key[4])
     mask = torch.ones(nb, bs, dtype=torch.bool)
     mask[0, 0] = mask[1, 1] = False

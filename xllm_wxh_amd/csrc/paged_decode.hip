@@ -287,83 +287,128 @@ __global__ void __launch_bounds__(256) decode_merge_kernel(DecodeParams p) {
 }
 
 // ---------------------------------------------------------------------------------
-// MFMA kernel, head_dim 128, bf16 queries.  One workgroup of kWaves waves per work item; the waves
-// take equal, tile-aligned shares of the item's tokens and never synchronise until the end.
+// MFMA kernels, head_dim 128, bf16 queries.  One workgroup of four waves per work item.
 //
-// Per 32-token tile a wave loads K and V rows with fully coalesced 16-byte
-// loads, parks them in its private 16 KiB of LDS (row-major, 16-byte pieces
-// XOR-swizzled by row so that the fragment reads below are bank-conflict free),
-// and reads them back in MFMA operand order:
+// A tile is 32 tokens.  Its K and V rows are fetched with fully coalesced 16-byte loads, parked
+// in LDS (row-major, 16-byte pieces XOR-swizzled by row so that every access pattern below is
+// bank-conflict free) and read back in MFMA operand order:
 //   S^T[t][r]  = sum_d K[t][d] Q[r][d]      A = K tile (ds_read_b128), B = Q^T (registers)
 //   O^T[d][r] += sum_t V[t][d] P[r][t]      A = V^T tile (ds_read_b64_tr_b16), B = P^T (registers)
-// Computing the transposed products keeps a query row in one lane column for
-// both MFMAs, so the probabilities leave the first MFMA already laid out as the
-// second one's B operand and the softmax statistics are per-lane scalars.
-// Query rows r = j*g + gq (draft token j, head gq of the group) fill the 16
-// columns of an MFMA tile; NT tiles cover up to 16*NT rows.
+// Computing the transposed products keeps a query row in one lane column for both MFMAs, so the
+// probabilities leave the first MFMA already laid out as the second one's B operand and the
+// softmax statistics are per-lane scalars.  Query rows r = j*g + gq (draft token j, head gq of
+// the group) fill the 16 columns of an MFMA tile; a wave owns one such tile of rows.
+//
+// decode_mfma_d128_kernel        up to 16 rows per item: the four waves take a quarter of the
+//                                item's tokens each, stage their tiles privately and meet only
+//                                at the end.
+// decode_mfma_d128_rows32_kernel up to 32 rows per item: waves 0-1 own rows 0-15, waves 2-3 rows
+//                                16-31; a wave of each pair takes half of the tokens and the two
+//                                waves that share tokens also share the LDS tile — each fetches
+//                                and parks 16 of its 32 rows, then both read all of it — so K and
+//                                V still cross HBM once.
 // ---------------------------------------------------------------------------------
 
 constexpr int kLdsK = 0;
 constexpr int kLdsV = 8192;
-constexpr int kLdsWave = 16384;
-constexpr int kWaves = 4;       // waves per work item
-constexpr int kXchRow = 528;    // bytes per query row in the end-of-item exchange (128 floats + 16 pad)
-
-template <int KV_DT>
-struct KvStage;  // registers holding one tile in flight + how to park it in LDS
+constexpr int kLdsSc = 16384;    // fp32 scales of a quantised tile: K of tokens 0..31, then V
+constexpr int kLdsTile = 16640;  // one 32-token tile of K and V as bf16, plus the scales
+constexpr int kWaves = 4;        // waves per work item
+constexpr int kXchRow = 528;     // bytes per query row in the end-of-item exchange (128 floats + 16 pad)
 
 __device__ inline u32x4 ldg_stream(const void* p) {
   return __builtin_nontemporal_load((const u32x4*)p);
 }
 
-__device__ inline uint32_t swz(int row, int piece) { return (uint32_t)(row * 256 + ((piece ^ (row & 15)) << 4)); }
+// LDS placement of a tile: 32 rows of 256 bytes, the sixteen 16-byte pieces of a row permuted by an
+// XOR that depends on the row.  The LDS moves 128 bytes per clock, i.e. 8 lanes of a 16-byte access
+// or 16 lanes of an 8-byte access at a time, and pieces s and s+8 of a row share banks; each access
+// pattern of the kernel must therefore touch 8 different pieces (mod 8) per such group of lanes:
+//   K rows are read 16 rows at a time, same piece (MFMA A operand)  -> XOR with the row number;
+//   V rows are read 4 rows x 2 pieces at a time (transpose read)    -> XOR with twice the row number
+//     (bit 3 of the row goes to bit 0 so that rows r and r+8 differ in parity, see KvHalfQuant).
+__device__ inline uint32_t swz_k(int row, int piece) { return (uint32_t)(row * 256 + ((piece ^ (row & 15)) << 4)); }
+__device__ inline uint32_t swz_v(int row, int piece) {
+  return (uint32_t)(row * 256 + ((piece ^ (((row & 7) << 1) | ((row >> 3) & 1))) << 4));
+}
 
-// bf16 cache: 16 loads of 16 bytes per lane and tile (8 K + 8 V); lane = (row-in-load, piece).
+// Uniform (scalar-register) part of the addresses of 16 consecutive tokens starting at `tok`
+// (a multiple of 16, so they lie in one block): element offset of (block, kv head, slot) in the
+// cache and in the scale tensors.
+struct HalfBase {
+  int64_t elem;
+  int64_t scale;
+};
+
+__device__ inline HalfBase half_base(const DecodeParams& p, const Item& it, int tok) {
+  int bi = tok >> p.log2_bs;
+  bi = bi < it.nblk ? bi : it.nblk - 1;
+  const int64_t blk = __builtin_amdgcn_readfirstlane(it.ids[bi]);
+  const int64_t slot = tok & (p.block_size - 1);
+  HalfBase b;
+  b.elem = blk * p.stride_block + (int64_t)it.hk * p.stride_head + slot * p.stride_slot;
+  b.scale = blk * p.sc_stride_block + (int64_t)it.hk * p.sc_stride_head + slot * p.sc_stride_slot;
+  return b;
+}
+
+// KvHalf<KV>: the registers that hold 16 tokens (half a tile) of K and V in flight, the per-lane
+// geometry of their loads, and how they are parked in rows 16*h .. 16*h+15 of an LDS tile.
+template <int KV_DT>
+struct KvHalf;
+
+// bf16 cache: 8 loads of 16 bytes per lane (4 K + 4 V); a load instruction covers 4 rows:
+// lane = (row-in-load, piece).
 template <>
-struct KvStage<XLLM_HIP_BF16> {
-  u32x4 k[8];
-  u32x4 v[8];
+struct KvHalf<XLLM_HIP_BF16> {
+  // Row 4j + lrow differs from row lrow only in bits the lane does not own, so its swizzled LDS
+  // offset is the offset of row lrow with a j-dependent constant XORed in (plus j KiB): one register
+  // per array instead of one per row.
+  struct Geom {
+    uint32_t g_off;  // byte offset of (row lrow, piece) from the first of the 16 rows
+    uint32_t wk;     // LDS offset of K row lrow, piece
+    uint32_t wv;     // LDS offset of V row lrow, piece
+    int lrow;
+    __device__ inline void init(const DecodeParams& p, int lane) {
+      lrow = lane >> 4;
+      const int piece = lane & 15;
+      g_off = (uint32_t)((lrow * p.stride_slot + piece * 8) * 2);
+      wk = kLdsK + swz_k(lrow, piece);
+      wv = kLdsV + swz_v(lrow, piece);
+    }
+    // rows 4j + lrow (+16h): the K swizzle adds 4j; the V swizzle adds 8 for odd j, 1 for rows 8..15
+    __device__ inline uint32_t k_row(int j, int h) const {
+      return (wk ^ (uint32_t)((4 * j) << 4)) + j * 1024 + h * 4096;
+    }
+    __device__ inline uint32_t v_row(int j, int h) const {
+      return (wv ^ (uint32_t)((((j & 1) << 3) | (j >> 1)) << 4)) + j * 1024 + h * 4096;
+    }
+  };
+  u32x4 k[4];
+  u32x4 v[4];
 
-  __device__ inline void issue(const DecodeParams& p, const Item& it, int tb, int lane) {
-    const int lrow = lane >> 4, piece = lane & 15;
-    const int bs_mask = p.block_size - 1;
-    int bi0 = tb >> p.log2_bs, bi1 = (tb + 16) >> p.log2_bs;
-    bi0 = bi0 < it.nblk ? bi0 : it.nblk - 1;
-    bi1 = bi1 < it.nblk ? bi1 : it.nblk - 1;
-    const int64_t blk0 = it.ids[bi0], blk1 = it.ids[bi1];
-    const int64_t head_off = (int64_t)it.hk * p.stride_head + piece * 8;
-    const int64_t base0 = blk0 * p.stride_block + head_off + (int64_t)((tb & bs_mask) + lrow) * p.stride_slot;
-    const int64_t base1 = blk1 * p.stride_block + head_off + (int64_t)(((tb + 16) & bs_mask) + lrow) * p.stride_slot;
+  __device__ inline void issue(const DecodeParams& p, const Item& it, int tok, const Geom& g) {
+    const HalfBase b = half_base(p, it, tok);
+    const uint8_t* kb = p.k_cache + b.elem * 2;
+    const uint8_t* vb = p.v_cache + b.elem * 2;
+    const int64_t step = 4 * p.stride_slot * 2;  // four rows further, in bytes (uniform)
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int64_t o0 = (base0 + (int64_t)(4 * j) * p.stride_slot) * 2;
-      const int64_t o1 = (base1 + (int64_t)(4 * j) * p.stride_slot) * 2;
-      k[j] = ldg_stream(p.k_cache + o0);
-      k[j + 4] = ldg_stream(p.k_cache + o1);
-      v[j] = ldg_stream(p.v_cache + o0);
-      v[j + 4] = ldg_stream(p.v_cache + o1);
+      k[j] = ldg_stream(kb + j * step + g.g_off);
+      v[j] = ldg_stream(vb + j * step + g.g_off);
     }
   }
-
-  // Rows at or beyond `len` may hold anything (unwritten slots); zero them so that 0 * x stays 0.
+  // V rows at or beyond `len` may hold anything (unwritten slots); zero them so that 0 * x stays 0.
+  // (K rows need no such care: their scores are replaced by -inf.)
   template <bool MASKED>
-  __device__ inline void park(uint8_t* lds, int tb, int len, int lane) {
-    const int lrow = lane >> 4, piece = lane & 15;
+  __device__ inline void park(uint8_t* tile, int h, int tok, int len, const Geom& g) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int row = 4 * j + lrow;
-      u32x4 kk = k[j], vv = v[j];
-      if (MASKED && tb + row >= len) {
-        kk = u32x4{0, 0, 0, 0};
-        vv = u32x4{0, 0, 0, 0};
-      }
-      const uint32_t off = swz(row, piece);
-      *(u32x4*)(lds + kLdsK + off) = kk;
-      *(u32x4*)(lds + kLdsV + off) = vv;
+    for (int j = 0; j < 4; ++j) {
+      u32x4 vv = v[j];
+      if (MASKED && tok + 4 * j + g.lrow >= len) vv = u32x4{0, 0, 0, 0};
+      *(u32x4*)(tile + g.k_row(j, h)) = k[j];
+      *(u32x4*)(tile + g.v_row(j, h)) = vv;
     }
   }
-
-  __device__ inline void take_scales(f32x4 (&)[2], f32x4 (&)[2]) const {}
 };
 
 // Convert 16 quantised bytes to 16 bf16: e4m3 values exactly, int8 values offset by +128 (exact).
@@ -394,380 +439,314 @@ __device__ inline void dequant16(const u32x4 raw, bf16x8& lo, bf16x8& hi) {
   hi = u.v[1];
 }
 
-// 1-byte caches: 8 loads of 16 bytes per lane and tile (4 K + 4 V); lane = (row-in-load, 16-element piece),
-// plus the fp32 scales of the tile's tokens in the layout of the score registers.
+// 1-byte caches: 4 loads of 16 bytes per lane (2 K + 2 V).  A load instruction covers 8 rows of 128
+// bytes; a lane holds 16 consecutive elements, which become two 16-byte bf16 pieces (2c, 2c+1) of
+// one LDS row.  Lanes are assigned in quads so that the 8 lanes of an LDS write group hold pieces of
+// two rows whose swizzles differ in parity — rows r, r+1 for K and rows r, r+8 for V — which makes
+// the 8 pieces they write distinct mod 8.
+// The fp32 scales of the 16 tokens travel beside them: lanes 0-15 fetch the K scales, lanes 16-31
+// the V scales (one register), and park them after the tile, where every lane picks up the four it
+// needs for its score registers with one broadcast read per array and half.
 template <int KV_DT>
-struct KvStageQuant {
-  u32x4 k[4];
-  u32x4 v[4];
-  f32x4 ks[2];
-  f32x4 vs[2];
+struct KvHalfQuant {
+  // Load j (0, 1): K rows krow + 8j, V rows vrow + 4j.  As for the bf16 cache the LDS offsets of the
+  // further rows and of the second piece follow from one register by XOR.
+  struct Geom {
+    uint32_t gk_off;  // K: byte offset of (row krow, 16-byte chunk) from the first of the 16 rows
+    uint32_t gv_off;  // V: same under the V lane assignment
+    uint32_t wk;      // LDS offset of K row krow, piece 2 * chunk
+    uint32_t wv;      // LDS offset of V row vrow, piece 2 * chunk
+    uint32_t sc_g;    // byte offset of this lane's scale from the scale of the first of the 16 tokens
+    uint32_t sc_lds;  // where it is parked (before adding 64 bytes for the second half of the tile)
+    int vrow;
+    bool sc_on;       // lanes 0..31 carry a scale
+    bool sc_is_v;
+    __device__ inline void init(const DecodeParams& p, int lane) {
+      const int chunk = 4 * ((lane >> 3) & 1) + (lane & 3);
+      const int pair = (lane >> 2) & 1;
+      const int krow = 2 * (lane >> 4) + pair;  // rows r, r+1 alternate between quads (krow < 8)
+      vrow = (lane >> 4) + 8 * pair;            // rows r, r+8 alternate between quads (vrow & 7 < 4)
+      gk_off = (uint32_t)(krow * p.stride_slot + chunk * 16);
+      gv_off = (uint32_t)(vrow * p.stride_slot + chunk * 16);
+      wk = kLdsK + swz_k(krow, 2 * chunk);
+      wv = kLdsV + swz_v(vrow, 2 * chunk);
+      sc_g = (uint32_t)((lane & 15) * p.sc_stride_slot * 4);
+      sc_is_v = ((lane >> 4) & 1) != 0;
+      sc_lds = kLdsSc + (sc_is_v ? 128 : 0) + (lane & 15) * 4;
+      sc_on = lane < 32;
+    }
+    // K row krow + 8j: swizzle adds 8; V row vrow + 4j: swizzle adds 8; second piece: XOR 1.
+    __device__ inline uint32_t k_row(int j, int hi, int h) const {
+      return (wk ^ (uint32_t)(((j << 3) | hi) << 4)) + j * 2048 + h * 4096;
+    }
+    __device__ inline uint32_t v_row(int j, int hi, int h) const {
+      return (wv ^ (uint32_t)(((j << 3) | hi) << 4)) + j * 1024 + h * 4096;
+    }
+  };
+  u32x4 k[2];
+  u32x4 v[2];
+  float sc;
 
-  __device__ inline void issue(const DecodeParams& p, const Item& it, int tb, int lane) {
-    const int lrow = lane >> 3, piece = lane & 7;
-    const int kg = lane >> 4;
-    const int bs_mask = p.block_size - 1;
-    int bi0 = tb >> p.log2_bs, bi1 = (tb + 16) >> p.log2_bs;
-    bi0 = bi0 < it.nblk ? bi0 : it.nblk - 1;
-    bi1 = bi1 < it.nblk ? bi1 : it.nblk - 1;
-    const int64_t blk0 = it.ids[bi0], blk1 = it.ids[bi1];
-    const int slot0 = tb & bs_mask, slot1 = (tb + 16) & bs_mask;
-    const int64_t head_off = (int64_t)it.hk * p.stride_head + piece * 16;
-    const int64_t base0 = blk0 * p.stride_block + head_off + (int64_t)(slot0 + lrow) * p.stride_slot;
-    const int64_t base1 = blk1 * p.stride_block + head_off + (int64_t)(slot1 + lrow) * p.stride_slot;
+  __device__ inline void issue(const DecodeParams& p, const Item& it, int tok, const Geom& g) {
+    const HalfBase b = half_base(p, it, tok);
+    const uint8_t* kb = p.k_cache + b.elem;
+    const uint8_t* vb = p.v_cache + b.elem;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const int64_t o0 = base0 + (int64_t)(8 * j) * p.stride_slot;
-      const int64_t o1 = base1 + (int64_t)(8 * j) * p.stride_slot;
-      k[j] = ldg_stream(p.k_cache + o0);
-      k[j + 2] = ldg_stream(p.k_cache + o1);
-      v[j] = ldg_stream(p.v_cache + o0);
-      v[j + 2] = ldg_stream(p.v_cache + o1);
+      k[j] = ldg_stream(kb + j * 8 * p.stride_slot + g.gk_off);
+      v[j] = ldg_stream(vb + j * 4 * p.stride_slot + g.gv_off);
     }
-    // Scales of tokens tb + 16*s + 4*kg + rr, the tokens of this lane's score registers.
-    const int64_t s0 = blk0 * p.sc_stride_block + (int64_t)it.hk * p.sc_stride_head +
-                       (int64_t)(slot0 + 4 * kg) * p.sc_stride_slot;
-    const int64_t s1 = blk1 * p.sc_stride_block + (int64_t)it.hk * p.sc_stride_head +
-                       (int64_t)(slot1 + 4 * kg) * p.sc_stride_slot;
-    if (p.sc_stride_slot == 1) {
-      ks[0] = *(const f32x4*)(p.k_scale + s0);
-      ks[1] = *(const f32x4*)(p.k_scale + s1);
-      vs[0] = *(const f32x4*)(p.v_scale + s0);
-      vs[1] = *(const f32x4*)(p.v_scale + s1);
-    } else {
-#pragma unroll
-      for (int rr = 0; rr < 4; ++rr) {
-        ks[0][rr] = p.k_scale[s0 + rr * p.sc_stride_slot];
-        ks[1][rr] = p.k_scale[s1 + rr * p.sc_stride_slot];
-        vs[0][rr] = p.v_scale[s0 + rr * p.sc_stride_slot];
-        vs[1][rr] = p.v_scale[s1 + rr * p.sc_stride_slot];
-      }
-    }
+    const float* sb = (g.sc_is_v ? p.v_scale : p.k_scale) + b.scale;
+    if (g.sc_on) sc = *(const float*)((const uint8_t*)sb + g.sc_g);
   }
 
   template <bool MASKED>
-  __device__ inline void park(uint8_t* lds, int tb, int len, int lane) {
-    const int lrow = lane >> 3, piece = lane & 7;
+  __device__ inline void park(uint8_t* tile, int h, int tok, int len, const Geom& g) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int row = 8 * j + lrow;
+    for (int j = 0; j < 2; ++j) {
       bf16x8 klo, khi, vlo, vhi;
       dequant16<KV_DT>(k[j], klo, khi);
       dequant16<KV_DT>(v[j], vlo, vhi);
-      if (MASKED && tb + row >= len) {
+      if (MASKED && tok + g.vrow + 4 * j >= len) {
         const bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
-        klo = khi = vlo = vhi = z;
+        vlo = vhi = z;
       }
-      const uint32_t o_lo = swz(row, 2 * piece), o_hi = swz(row, 2 * piece + 1);
-      *(bf16x8*)(lds + kLdsK + o_lo) = klo;
-      *(bf16x8*)(lds + kLdsK + o_hi) = khi;
-      *(bf16x8*)(lds + kLdsV + o_lo) = vlo;
-      *(bf16x8*)(lds + kLdsV + o_hi) = vhi;
+      *(bf16x8*)(tile + g.k_row(j, 0, h)) = klo;
+      *(bf16x8*)(tile + g.k_row(j, 1, h)) = khi;
+      *(bf16x8*)(tile + g.v_row(j, 0, h)) = vlo;
+      *(bf16x8*)(tile + g.v_row(j, 1, h)) = vhi;
     }
-  }
-
-  __device__ inline void take_scales(f32x4 (&kss)[2], f32x4 (&vss)[2]) const {
-    kss[0] = ks[0];
-    kss[1] = ks[1];
-    vss[0] = vs[0];
-    vss[1] = vs[1];
+    if (g.sc_on) *(float*)(tile + g.sc_lds + h * 64) = sc;
   }
 };
 template <>
-struct KvStage<XLLM_HIP_FP8_E4M3> : KvStageQuant<XLLM_HIP_FP8_E4M3> {};
+struct KvHalf<XLLM_HIP_FP8_E4M3> : KvHalfQuant<XLLM_HIP_FP8_E4M3> {};
 template <>
-struct KvStage<XLLM_HIP_INT8> : KvStageQuant<XLLM_HIP_INT8> {};
+struct KvHalf<XLLM_HIP_INT8> : KvHalfQuant<XLLM_HIP_INT8> {};
 
-template <int KV_DT, int NT>
-__global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_d128_kernel(DecodeParams p) {
-  constexpr bool kQuant = KV_DT != XLLM_HIP_BF16;
+// State of one wave's tile of 16 query rows, and the attention over one parked tile.
+template <int KV_DT>
+struct RowTile {
+  static constexpr bool kQuant = KV_DT != XLLM_HIP_BF16;
   // int8 rows sit in LDS as x + 128.  With K' = K + 128 and V' = V + 128:
   //   q.K  = q.K' - 128 * sum_d q_d                    (qsum, once per query row)
   //   sum_t w_t V_t = sum_t w_t V'_t - 128 * sum_t w_t  (wsum, tracked like the softmax denominator)
   // Rows zeroed because they lie past the sequence end carry weight 0 in both sums.
-  constexpr bool kOffset = KV_DT == XLLM_HIP_INT8;
-  __shared__ __attribute__((aligned(16))) uint8_t lds_all[kWaves * kLdsWave];
-  __shared__ float lds_ml[kWaves * NT * 16 * 2];  // (running max, denominator) per wave and query row
-  // With two tiles of query rows the Q^T fragments live in LDS instead of 32 registers, which keeps
-  // the kernel within the 256 registers that let two workgroups share a CU.
-  constexpr bool kQInLds = NT > 1;
-  __shared__ __attribute__((aligned(16))) uint8_t lds_q[kQInLds ? NT * 4 * 64 * 16 : 16];
+  static constexpr bool kOffset = KV_DT == XLLM_HIP_INT8;
 
-  Item it;
-  if (!decode_item(p, blockIdx.x, it)) return;
+  bf16x8 qf[4];    // Q^T fragments (B operand) of the lane's query row
+  f32x4 acc[8];    // O^T accumulators: head-dim tile dt, rows 4*kg + rr
+  float m_run;     // running maximum of the log2-scaled scores
+  float l_run;     // this lane's share of the softmax denominator
+  float w_run;     // this lane's share of sum_t w_t (int8 only)
+  float qsum128;   // 128 * sum_d q[r][d] (int8 only)
+  int lim;         // tokens >= lim are invisible to the row (causal among draft tokens)
+  int lo;          // tokens < lo are outside the sliding window
+  int row;         // query row within (sequence, kv head); valid if < p.rows
+  uint32_t k_off0; // LDS offset of K row mi, piece kg        (piece 4c + kg: XOR c << 6)
+  uint32_t v_off0; // LDS offset of the transpose read, tile 0 (head-dim tile dt: XOR dt << 5)
+  int kg;
 
-  const int wave = threadIdx.x >> 6;
-  const int lane = threadIdx.x & 63;
-  uint8_t* lds = lds_all + wave * kLdsWave;  // this wave's private K/V tile
-  const int mi = lane & 15;  // MFMA row of A / column of B and D
-  const int kg = lane >> 4;  // k-group of the operands; row block of D
-  const float neg_inf = -INFINITY;
-
-  // Query rows of this lane's column, one per N tile.
-  int lim[NT];  // tokens >= lim are invisible to the row (causal among draft tokens)
-  int lo[NT];   // tokens < lo are outside the sliding window
-  bool valid[NT];
-  float qsum128[NT];  // 128 * sum_d q[r][d] (int8 offset correction of the scores)
-  bf16x8 qf[NT][4];
-#pragma unroll
-  for (int nt = 0; nt < NT; ++nt) {
-    const int r = it.rg * kMaxRowsPerItem + nt * 16 + mi;
-    valid[nt] = r < p.rows;
-    const int j = valid[nt] ? r / p.group : 0;
-    const int gq = valid[nt] ? r - j * p.group : 0;
-    lim[nt] = it.len - (p.n - 1 - j);
-    lo[nt] = p.window_left >= 0 ? lim[nt] - 1 - p.window_left : 0;
+  __device__ inline void init(const DecodeParams& p, const Item& it, int row_in_item, int lane) {
+    const int mi = lane & 15;  // MFMA row of A / column of B and D
+    kg = lane >> 4;            // k-group of the operands; row block of D
+    row = it.rg * kMaxRowsPerItem + row_in_item + mi;
+    const bool valid = row < p.rows;
+    const int j = valid ? row / p.group : 0;
+    const int gq = valid ? row - j * p.group : 0;
+    lim = it.len - (p.n - 1 - j);
+    lo = p.window_left >= 0 ? lim - 1 - p.window_left : 0;
     const uint16_t* qrow = (const uint16_t*)p.q + (int64_t)(it.b * p.n + j) * p.q_token_stride +
                            (int64_t)(it.hk * p.group + gq) * 128;
+    float sq = 0.0f;
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
       u32x4 raw = {0, 0, 0, 0};
-      if (valid[nt]) raw = *(const u32x4*)(qrow + c * 32 + kg * 8);
-      qf[nt][c] = __builtin_bit_cast(bf16x8, raw);
-    }
-    qsum128[nt] = 0.0f;
-    if (kOffset) {
-      float sq = 0.0f;
+      if (valid) raw = *(const u32x4*)(qrow + c * 32 + kg * 8);
+      qf[c] = __builtin_bit_cast(bf16x8, raw);
+      if (kOffset) {
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) sq += (float)qf[nt][c][e];
+        for (int e = 0; e < 8; ++e) sq += (float)qf[c][e];
       }
+    }
+    qsum128 = 0.0f;
+    if (kOffset) {
       sq += __shfl_xor(sq, 16);
       sq += __shfl_xor(sq, 32);
-      qsum128[nt] = 128.0f * sq;
+      qsum128 = 128.0f * sq;
     }
-    if (kQInLds) {
-      // every wave stores the same fragments and reads back only what it stored: no barrier needed
+    m_run = -INFINITY;
+    l_run = 0.0f;
+    w_run = 0.0f;
 #pragma unroll
-      for (int c = 0; c < 4; ++c) *(bf16x8*)(lds_q + ((nt * 4 + c) * 64 + lane) * 16) = qf[nt][c];
+    for (int dt = 0; dt < 8; ++dt) acc[dt] = f32x4{0, 0, 0, 0};
+    k_off0 = kLdsK + swz_k(mi, kg);
+    const int tau = 4 * kg + (mi >> 2);  // token row (within 16) this lane points the transpose read at
+    v_off0 = kLdsV + swz_v(tau, (mi & 3) >> 1) + (mi & 1) * 8;
+  }
+
+  // Attention of the 16 rows over the 32 tokens parked in `tile` (first token tb).
+  template <bool MASKED>
+  __device__ inline void attend(const uint8_t* tile, int tb, int len, float scale_log2) {
+    const float neg_inf = -INFINITY;
+    f32x4 ksc[2], vsc[2];  // scales of tokens tb + 16h + 4kg + rr
+    if (kQuant) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        ksc[h] = *(const f32x4*)(tile + kLdsSc + (16 * h + 4 * kg) * 4);
+        vsc[h] = *(const f32x4*)(tile + kLdsSc + 128 + (16 * h + 4 * kg) * 4);
+      }
     }
-  }
-  uint32_t q_off = lane * 16;
-
-  // Tile range.  With a sliding window, tiles wholly below every row's window are skipped.
-  int t0 = it.t_begin;
-  if (p.window_left >= 0) {
-    int first = it.len - p.n - p.window_left;  // window start of the earliest query row
-    first = first > 0 ? first : 0;
-    first &= ~(kTileTokens - 1);
-    t0 = t0 > first ? t0 : first;
-  }
-  // This wave's share of [t0, t_end).
-  const int span = it.t_end - t0;
-  const int share = span > 0 ? (((span + kWaves - 1) / kWaves + kTileTokens - 1) & ~(kTileTokens - 1)) : 0;
-  const int w_begin = t0 + wave * share;
-  const int w_end = min(it.t_end, w_begin + share);
-  const int mask_hi_from = it.len - (p.n - 1);                                // tiles reaching past this need masks
-  const int mask_lo_until = p.window_left >= 0 ? it.len - 1 - p.window_left : 0;  // tiles starting below this too
-
-  f32x4 acc[NT][8];
-  float m_run[NT], l_run[NT], w_run[NT];
-#pragma unroll
-  for (int nt = 0; nt < NT; ++nt) {
-    m_run[nt] = neg_inf;
-    l_run[nt] = 0.0f;
-    w_run[nt] = 0.0f;
-#pragma unroll
-    for (int dt = 0; dt < 8; ++dt) acc[nt][dt] = f32x4{0, 0, 0, 0};
-  }
-
-  // Per-lane LDS read offsets.
-  uint32_t k_off[4];
-#pragma unroll
-  for (int c = 0; c < 4; ++c) k_off[c] = kLdsK + swz(mi, c * 4 + kg);
-  const int tau = 4 * kg + (mi >> 2);  // token row (within a 16-token half) this lane points the transpose read at
-  uint32_t v_off[8];
-#pragma unroll
-  for (int dt = 0; dt < 8; ++dt) v_off[dt] = kLdsV + swz(tau, dt * 2 + ((mi & 3) >> 1)) + (mi & 1) * 8;
-
-  KvStage<KV_DT> stage;
-
-  auto tile = [&](int tb, const f32x4 (&ksc)[2], const f32x4 (&vsc)[2], auto masked_tag) {
-    constexpr bool MASKED = decltype(masked_tag)::value;
     // ---- S^T = K Q^T ----
-    f32x4 s[2][NT];
-    if (kQInLds) asm volatile("" : "+v"(q_off));  // keeps the Q^T reads below inside the loop
+    f32x4 s[2] = {f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}};
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const uint32_t ko = k_off0 ^ (uint32_t)(c << 6);
+      const bf16x8 kf0 = *(const bf16x8*)(tile + ko);
+      const bf16x8 kf1 = *(const bf16x8*)(tile + ko + 4096);
+      s[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf0, qf[c], s[0], 0, 0, 0);
+      s[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf1, qf[c], s[1], 0, 0, 0);
+    }
+    // ---- online softmax of the lane's query row ----
+    float x[8];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) s[h][nt] = f32x4{0, 0, 0, 0};
-    }
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const bf16x8 kf0 = *(const bf16x8*)(lds + k_off[c]);
-      const bf16x8 kf1 = *(const bf16x8*)(lds + k_off[c] + 4096);
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt) {
-        const bf16x8 qv = kQInLds ? *(const bf16x8*)(lds_q + q_off + (nt * 4 + c) * 1024) : qf[nt][c];
-        s[0][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf0, qv, s[0][nt], 0, 0, 0);
-        s[1][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf1, qv, s[1][nt], 0, 0, 0);
+      for (int rr = 0; rr < 4; ++rr) {
+        float v = s[h][rr];
+        if (kOffset) v -= qsum128;
+        v *= scale_log2;
+        if (kQuant) v *= ksc[h][rr];
+        if (MASKED) {
+          const int tok = tb + 16 * h + 4 * kg + rr;
+          v = (tok < lim && tok >= lo) ? v : neg_inf;
+        }
+        x[4 * h + rr] = v;
       }
     }
-    // ---- online softmax, per query row (lane column) ----
-    bf16x8 pf[NT];
+    float mt = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
+    mt = fmaxf(mt, __shfl_xor(mt, 16));
+    mt = fmaxf(mt, __shfl_xor(mt, 32));
+    const float m_new = fmaxf(m_run, mt);
+    const float m_safe = m_new == neg_inf ? 0.0f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_safe);
+    float psum = 0.0f;
+    float pv[8];
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      float x[8];
+    for (int i = 0; i < 8; ++i) {
+      const float e = __builtin_amdgcn_exp2f(x[i] - m_safe);
+      psum += e;
+      pv[i] = e;
+    }
+    if (kQuant) {
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) {
-          float v = s[h][nt][rr];
-          if (kOffset) v -= qsum128[nt];
-          v *= p.scale_log2;
-          if (kQuant) v *= ksc[h][rr];
+          float w = vsc[h][rr];
           if (MASKED) {
             const int tok = tb + 16 * h + 4 * kg + rr;
-            v = (tok < lim[nt] && tok >= lo[nt]) ? v : neg_inf;
+            w = tok < len ? w : 0.0f;
           }
-          x[4 * h + rr] = v;
+          pv[4 * h + rr] *= w;
         }
       }
-      float mt = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
-      mt = fmaxf(mt, __shfl_xor(mt, 16));
-      mt = fmaxf(mt, __shfl_xor(mt, 32));
-      const float m_new = fmaxf(m_run[nt], mt);
-      const float m_safe = m_new == neg_inf ? 0.0f : m_new;
-      const float alpha = __builtin_amdgcn_exp2f(m_run[nt] - m_safe);
-      float psum = 0.0f;
-      float pv[8];
+    }
+    l_run = l_run * alpha + psum;
+    m_run = m_new;
+    // Unconditional: a branch around the rescale splits the live ranges of the accumulator tuples
+    // and costs far more registers than the 32 multiplies cost issue slots.
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float e = __builtin_amdgcn_exp2f(x[i] - m_safe);
-        psum += e;
-        pv[i] = e;
-      }
-      if (kQuant) {
+    for (int dt = 0; dt < 8; ++dt) acc[dt] *= alpha;
+    bf16x8 pf;
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
+    for (int i = 0; i < 8; ++i) pf[i] = (__bf16)pv[i];
+    if (kOffset) {
+      float wt = 0.0f;  // sum of the weights as the MFMA will see them (after rounding to bf16)
 #pragma unroll
-          for (int rr = 0; rr < 4; ++rr) {
-            float w = vsc[h][rr];
-            if (MASKED) {
-              const int tok = tb + 16 * h + 4 * kg + rr;
-              w = tok < it.len ? w : 0.0f;
-            }
-            pv[4 * h + rr] *= w;
-          }
-        }
-      }
-      l_run[nt] = l_run[nt] * alpha + psum;
-      m_run[nt] = m_new;
-      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-#pragma unroll
-        for (int dt = 0; dt < 8; ++dt) acc[nt][dt] *= alpha;
-      }
-#pragma unroll
-      for (int i = 0; i < 8; ++i) pf[nt][i] = (__bf16)pv[i];
-      if (kOffset) {
-        float wt = 0.0f;  // sum of the weights as the MFMA will see them (after rounding to bf16)
-#pragma unroll
-        for (int i = 0; i < 8; ++i) wt += (float)pf[nt][i];
-        w_run[nt] = w_run[nt] * alpha + wt;
-      }
+      for (int i = 0; i < 8; ++i) wt += (float)pf[i];
+      w_run = w_run * alpha + wt;
     }
     // ---- O^T += V^T P^T ----
 #pragma unroll
     for (int dt = 0; dt < 8; ++dt) {
+      const uint32_t vo = v_off0 ^ (uint32_t)(dt << 5);
       const s16x4 a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (__attribute__((address_space(3))) s16x4*)(lds + v_off[dt]));
+          (__attribute__((address_space(3))) s16x4*)(tile + vo));
       const s16x4 a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (__attribute__((address_space(3))) s16x4*)(lds + v_off[dt] + 4096));
+          (__attribute__((address_space(3))) s16x4*)(tile + vo + 4096));
       const bf16x8 vf = __builtin_bit_cast(bf16x8, __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7));
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt) {
-        acc[nt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[nt], acc[nt][dt], 0, 0, 0);
-      }
-    }
-  };
-
-  // One tile's worth of global loads is always in flight while the previous tile is consumed.  A
-  // quantised tile is only half as many bytes, so two of them are kept in flight (two register
-  // stages, used alternately) to cover the same HBM latency.
-  auto consume = [&](KvStage<KV_DT>& st, int tb, int next_tb) {
-    const bool masked = (tb + kTileTokens > mask_hi_from) || (tb < mask_lo_until);
-    if (masked) {
-      st.template park<true>(lds, tb, it.len, lane);
-    } else {
-      st.template park<false>(lds, tb, it.len, lane);
-    }
-    // The scales of the tile being consumed must outlive the next issue into the same stage.
-    f32x4 ksc[2] = {}, vsc[2] = {};
-    st.take_scales(ksc, vsc);
-    if (next_tb < w_end) st.issue(p, it, next_tb, lane);
-    if (masked) {
-      tile(tb, ksc, vsc, std::true_type{});
-    } else {
-      tile(tb, ksc, vsc, std::false_type{});
-    }
-  };
-  if (w_begin < w_end) {
-    if (kQuant && NT == 1) {
-      KvStage<KV_DT> stage_b;
-      stage.issue(p, it, w_begin, lane);
-      if (w_begin + kTileTokens < w_end) stage_b.issue(p, it, w_begin + kTileTokens, lane);
-      for (int tb = w_begin; tb < w_end; tb += 2 * kTileTokens) {
-        consume(stage, tb, tb + 2 * kTileTokens);
-        if (tb + kTileTokens < w_end) consume(stage_b, tb + kTileTokens, tb + 3 * kTileTokens);
-      }
-    } else {
-      stage.issue(p, it, w_begin, lane);
-      for (int tb = w_begin; tb < w_end; tb += kTileTokens) consume(stage, tb, tb + kTileTokens);
+      acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, acc[dt], 0, 0, 0);
     }
   }
+};
 
-  // ---- combine the waves through LDS; each wave then finishes a 32-wide slice of head_dim ----
+// End of an item: the TW waves that share a set of 16 query rows exchange (m, l, acc) through LDS
+// (each wave's own 16 KiB region `xch_base + wave * xch_stride`), then each finishes 128/TW columns:
+// a sequence that is a single chunk gets its bf16 output rows (and LSE) written directly, a split
+// sequence a normalised fp32 partial and its log2-sum-exp.  All waves of the workgroup must call it.
+template <int KV_DT, int TW>
+__device__ inline void finish_item(const DecodeParams& p, const Item& it, RowTile<KV_DT>& rt, uint8_t* xch_base,
+                                   int xch_stride, float* lds_ml, int wave, int rs, int tw, int lane) {
+  constexpr bool kOffset = KV_DT == XLLM_HIP_INT8;
+  const float neg_inf = -INFINITY;
+  const int mi = lane & 15, kg = lane >> 4;
   const int nhq = p.n * p.num_q_heads;
   const bool single = p.direct_single != 0 && p.num_chunks[it.b] == 1;
-  const int col = lane & 15;              // query row handled in the combine
-  const int d0 = 32 * wave + 8 * (lane >> 4);  // first of this lane's 8 output columns
+  float l = rt.l_run;
+  l += __shfl_xor(l, 16);
+  l += __shfl_xor(l, 32);
+  float wsum = rt.w_run;
+  if (kOffset) {
+    wsum += __shfl_xor(wsum, 16);
+    wsum += __shfl_xor(wsum, 32);
+  }
+  uint8_t* mine = xch_base + wave * xch_stride;
 #pragma unroll
-  for (int nt = 0; nt < NT; ++nt) {
-    float l = l_run[nt];
-    l += __shfl_xor(l, 16);
-    l += __shfl_xor(l, 32);
-    float wsum = w_run[nt];
-    if (kOffset) {
-      wsum += __shfl_xor(wsum, 16);
-      wsum += __shfl_xor(wsum, 32);
-    }
-    if (nt > 0) __syncthreads();  // the previous round's reads are finished
-#pragma unroll
-    for (int dt = 0; dt < 8; ++dt) {
-      f32x4 o = acc[nt][dt];
-      if (kOffset) o -= 128.0f * wsum;
-      *(f32x4*)(lds + mi * kXchRow + (dt * 16 + 4 * kg) * 4) = o;
-    }
-    if (kg == 0) {
-      lds_ml[((wave * NT + nt) * 16 + mi) * 2] = m_run[nt];
-      lds_ml[((wave * NT + nt) * 16 + mi) * 2 + 1] = l;
-    }
-    __syncthreads();
+  for (int dt = 0; dt < 8; ++dt) {
+    f32x4 o = rt.acc[dt];
+    if (kOffset) o -= 128.0f * wsum;
+    *(f32x4*)(mine + mi * kXchRow + (dt * 16 + 4 * kg) * 4) = o;
+  }
+  if (kg == 0) {
+    lds_ml[(wave * 16 + mi) * 2] = rt.m_run;
+    lds_ml[(wave * 16 + mi) * 2 + 1] = l;
+  }
+  __syncthreads();
 
-    float m_all = neg_inf;
+  const int col = mi;  // query row handled in the combine
+  float m_all = neg_inf;
 #pragma unroll
-    for (int s = 0; s < kWaves; ++s) m_all = fmaxf(m_all, lds_ml[((s * NT + nt) * 16 + col) * 2]);
-    const float m_safe = m_all == neg_inf ? 0.0f : m_all;
-    float l_all = 0.0f;
+  for (int s = 0; s < TW; ++s) m_all = fmaxf(m_all, lds_ml[((rs * TW + s) * 16 + col) * 2]);
+  const float m_safe = m_all == neg_inf ? 0.0f : m_all;
+  float wgt[TW];
+  float l_all = 0.0f;
+#pragma unroll
+  for (int s = 0; s < TW; ++s) {
+    wgt[s] = __builtin_amdgcn_exp2f(lds_ml[((rs * TW + s) * 16 + col) * 2] - m_safe);
+    l_all += wgt[s] * lds_ml[((rs * TW + s) * 16 + col) * 2 + 1];
+  }
+  const int r = it.rg * kMaxRowsPerItem + rs * 16 + col;
+  if (r >= p.rows) return;
+  const int j = r / p.group;
+  const int head = it.hk * p.group + (r - j * p.group);
+  const float inv = l_all > 0.0f ? 1.0f / l_all : 0.0f;
+  const float lse2 = l_all > 0.0f ? m_all + __builtin_amdgcn_logf(l_all) : neg_inf;
+  const int64_t tok = (int64_t)it.b * p.n + j;
+  const int64_t prow = (int64_t)it.sc * nhq + (int64_t)j * p.num_q_heads + head;
+  constexpr int kCols = 128 / TW;  // columns this wave finishes: 8 per lane and pass
+#pragma unroll
+  for (int pass = 0; pass < kCols / 32; ++pass) {
+    const int d0 = kCols * tw + 32 * pass + 8 * kg;
     f32x4 o_lo = {0, 0, 0, 0}, o_hi = {0, 0, 0, 0};
 #pragma unroll
-    for (int s = 0; s < kWaves; ++s) {
-      const float w = __builtin_amdgcn_exp2f(lds_ml[((s * NT + nt) * 16 + col) * 2] - m_safe);
-      l_all += w * lds_ml[((s * NT + nt) * 16 + col) * 2 + 1];
-      const uint8_t* src = lds_all + s * kLdsWave + col * kXchRow + d0 * 4;
-      o_lo += w * *(const f32x4*)(src);
-      o_hi += w * *(const f32x4*)(src + 16);
+    for (int s = 0; s < TW; ++s) {
+      const uint8_t* src = xch_base + (rs * TW + s) * xch_stride + col * kXchRow + d0 * 4;
+      o_lo += wgt[s] * *(const f32x4*)(src);
+      o_hi += wgt[s] * *(const f32x4*)(src + 16);
     }
-    const int r = it.rg * kMaxRowsPerItem + nt * 16 + col;
-    if (r >= p.rows) continue;
-    const int j = r / p.group;
-    const int head = it.hk * p.group + (r - j * p.group);
-    const float inv = l_all > 0.0f ? 1.0f / l_all : 0.0f;
-    const float lse2 = l_all > 0.0f ? m_all + __builtin_amdgcn_logf(l_all) : neg_inf;
     o_lo *= inv;
     o_hi *= inv;
-    const int64_t tok = (int64_t)it.b * p.n + j;
     if (single) {
       bf16x8 ob;
 #pragma unroll
@@ -776,15 +755,159 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_d128_kernel(Decode
         ob[4 + e] = (__bf16)o_hi[e];
       }
       *(bf16x8*)((uint16_t*)p.out + tok * p.out_token_stride + (int64_t)head * 128 + d0) = ob;
-      if (p.lse != nullptr && d0 == 0) p.lse[tok * p.num_q_heads + head] = lse2;
     } else {
-      const int64_t prow = (int64_t)it.sc * nhq + (int64_t)j * p.num_q_heads + head;
       float* po = p.partial_out + prow * 128 + d0;
       *(f32x4*)(po) = o_lo;
       *(f32x4*)(po + 4) = o_hi;
-      if (d0 == 0) p.partial_lse[prow] = lse2;
     }
   }
+  if (tw == 0 && kg == 0) {
+    if (single) {
+      if (p.lse != nullptr) p.lse[tok * p.num_q_heads + head] = lse2;
+    } else {
+      p.partial_lse[prow] = lse2;
+    }
+  }
+}
+
+// Token range of an item after the sliding window has removed the tiles no row can see.
+__device__ inline int first_visible_tile(const DecodeParams& p, const Item& it) {
+  int t0 = it.t_begin;
+  if (p.window_left >= 0) {
+    int first = it.len - p.n - p.window_left;  // window start of the earliest query row
+    first = first > 0 ? first : 0;
+    first &= ~(kTileTokens - 1);
+    t0 = t0 > first ? t0 : first;
+  }
+  return t0;
+}
+
+template <int KV_DT>
+__global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_d128_kernel(DecodeParams p) {
+  __shared__ __attribute__((aligned(16))) uint8_t lds_all[kWaves * kLdsTile];
+  __shared__ float lds_ml[kWaves * 16 * 2];  // (running max, denominator) per wave and query row
+
+  Item it;
+  if (!decode_item(p, blockIdx.x, it)) return;
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: keeps the loop scalar
+  const int lane = threadIdx.x & 63;
+  uint8_t* tile = lds_all + wave * kLdsTile;  // this wave's private K/V tile
+
+  RowTile<KV_DT> rt;
+  rt.init(p, it, 0, lane);
+
+  // This wave's share of the item's tokens.
+  const int t0 = first_visible_tile(p, it);
+  const int span = it.t_end - t0;
+  const int share = span > 0 ? (((span + kWaves - 1) / kWaves + kTileTokens - 1) & ~(kTileTokens - 1)) : 0;
+  const int w_begin = t0 + wave * share;
+  const int w_end = min(it.t_end, w_begin + share);
+  const int mask_hi_from = it.len - (p.n - 1);                                    // tiles reaching past this need masks
+  const int mask_lo_until = p.window_left >= 0 ? it.len - 1 - p.window_left : 0;  // tiles starting below this too
+
+  typename KvHalf<KV_DT>::Geom geom;
+  geom.init(p, lane);
+  KvHalf<KV_DT> st[2];  // the two 16-token halves of the tile in flight
+
+  if (w_begin < w_end) {
+    st[0].issue(p, it, w_begin, geom);
+    st[1].issue(p, it, w_begin + 16, geom);
+    for (int tb = w_begin; tb < w_end; tb += kTileTokens) {
+      const bool masked = (tb + kTileTokens > mask_hi_from) || (tb < mask_lo_until);
+      // park the tile, then put the next tile's loads in flight while this one is consumed
+      if (masked) {
+        st[0].template park<true>(tile, 0, tb, it.len, geom);
+        st[1].template park<true>(tile, 1, tb + 16, it.len, geom);
+      } else {
+        st[0].template park<false>(tile, 0, tb, it.len, geom);
+        st[1].template park<false>(tile, 1, tb + 16, it.len, geom);
+      }
+      if (tb + kTileTokens < w_end) {
+        st[0].issue(p, it, tb + kTileTokens, geom);
+        st[1].issue(p, it, tb + kTileTokens + 16, geom);
+      }
+      if (masked) {
+        rt.template attend<true>(tile, tb, it.len, p.scale_log2);
+      } else {
+        rt.template attend<false>(tile, tb, it.len, p.scale_log2);
+      }
+    }
+  }
+  finish_item<KV_DT, kWaves>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, 0, wave, lane);
+}
+
+template <int KV_DT>
+__global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_d128_rows32_kernel(DecodeParams p) {
+  constexpr int TW = 2;  // waves per row set = token halves of the item
+  // [token half][buffer]: a tile is parked by the two waves that share the token half while both
+  // still read the previous tile from the other buffer, so one barrier per tile suffices.
+  __shared__ __attribute__((aligned(16))) uint8_t lds_all[TW * 2 * kLdsTile];
+  __shared__ float lds_ml[kWaves * 16 * 2];
+
+  Item it;
+  if (!decode_item(p, blockIdx.x, it)) return;
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int rs = wave >> 1;  // row set: query rows 16*rs .. 16*rs+15; also the tile half this wave fetches
+  const int tw = wave & 1;   // token half of the item
+  const int lane = threadIdx.x & 63;
+  uint8_t* tiles = lds_all + tw * 2 * kLdsTile;
+
+  RowTile<KV_DT> rt;
+  rt.init(p, it, 16 * rs, lane);
+
+  const int t0 = first_visible_tile(p, it);
+  const int span = it.t_end - t0;
+  const int share = span > 0 ? (((span + TW - 1) / TW + kTileTokens - 1) & ~(kTileTokens - 1)) : 0;
+  const int w_begin = t0 + tw * share;
+  const int w_end = min(it.t_end, w_begin + share);
+  // Every wave runs the same number of iterations (the barrier is workgroup wide); a wave whose
+  // token half is shorter idles through the tail.
+  const int iters = share / kTileTokens;
+  const int mask_hi_from = it.len - (p.n - 1);
+  const int mask_lo_until = p.window_left >= 0 ? it.len - 1 - p.window_left : 0;
+
+  typename KvHalf<KV_DT>::Geom geom;
+  geom.init(p, lane);
+  // Two register stages, used alternately: the loads of tiles i+1 and i+2 are in flight while tile
+  // i is consumed.  (A wave fetches only half a tile, so one stage would leave too few bytes in
+  // flight per CU to cover the HBM latency.)
+  KvHalf<KV_DT> mine[2];  // the 16 tokens this wave fetches: rows 16*rs .. of the tile
+
+  auto issue = [&](KvHalf<KV_DT>& m, int tb) {
+    if (tb < w_end) m.issue(p, it, tb + 16 * rs, geom);
+  };
+  auto step = [&](KvHalf<KV_DT>& m, int i) {
+    const int tb = w_begin + i * kTileTokens;
+    const bool live = tb < w_end;
+    uint8_t* tile = tiles + (i & 1) * kLdsTile;
+    const bool masked = (tb + kTileTokens > mask_hi_from) || (tb < mask_lo_until);
+    if (live) {
+      if (masked) {
+        m.template park<true>(tile, rs, tb + 16 * rs, it.len, geom);
+      } else {
+        m.template park<false>(tile, rs, tb + 16 * rs, it.len, geom);
+      }
+      issue(m, tb + 2 * kTileTokens);
+    }
+    __syncthreads();  // both halves of tile i are parked; everyone is done with tile i-1
+    if (live) {
+      if (masked) {
+        rt.template attend<true>(tile, tb, it.len, p.scale_log2);
+      } else {
+        rt.template attend<false>(tile, tb, it.len, p.scale_log2);
+      }
+    }
+  };
+  issue(mine[0], w_begin);
+  issue(mine[1], w_begin + kTileTokens);
+  for (int i = 0; i < iters; i += 2) {
+    step(mine[0], i);
+    if (i + 1 < iters) step(mine[1], i + 1);
+  }
+  __syncthreads();  // all tiles consumed before the buffers are reused for the exchange
+  finish_item<KV_DT, TW>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, rs, tw, lane);
 }
 
 // ---------------------------------------------------------------------------------
@@ -1061,9 +1184,9 @@ template <int KV_DT>
 static void launch_mfma(const DecodeParams& p, unsigned grid, hipStream_t st) {
   const int rows_per_item = p.rows < kMaxRowsPerItem ? p.rows : kMaxRowsPerItem;
   if (rows_per_item <= 16) {
-    decode_mfma_d128_kernel<KV_DT, 1><<<grid, 64 * kWaves, 0, st>>>(p);
+    decode_mfma_d128_kernel<KV_DT><<<grid, 64 * kWaves, 0, st>>>(p);
   } else {
-    decode_mfma_d128_kernel<KV_DT, 2><<<grid, 64 * kWaves, 0, st>>>(p);
+    decode_mfma_d128_rows32_kernel<KV_DT><<<grid, 64 * kWaves, 0, st>>>(p);
   }
 }
 
