@@ -311,8 +311,8 @@ __global__ void __launch_bounds__(256) decode_merge_kernel(DecodeParams p) {
 
 constexpr int kLdsK = 0;
 constexpr int kLdsV = 8192;
-constexpr int kLdsSc = 16384;    // fp32 scales of a quantised tile: K of tokens 0..31, then V
-constexpr int kLdsTile = 16640;  // one 32-token tile of K and V as bf16, plus the scales
+constexpr int kLdsSc = 16384;    // per-token factors of a quantised tile: three arrays of 32 floats
+constexpr int kLdsTile = 16768;  // one 32-token tile of K and V as 16-bit numbers, plus the factors
 constexpr int kWaves = 4;        // waves per work item
 constexpr int kXchRow = 528;     // bytes per query row in the end-of-item exchange (128 floats + 16 pad)
 
@@ -400,7 +400,7 @@ struct KvHalf<XLLM_HIP_BF16> {
   // V rows at or beyond `len` may hold anything (unwritten slots); zero them so that 0 * x stays 0.
   // (K rows need no such care: their scores are replaced by -inf.)
   template <bool MASKED>
-  __device__ inline void park(uint8_t* tile, int h, int tok, int len, const Geom& g) {
+  __device__ inline void park(uint8_t* tile, int h, int tok, int len, float, const Geom& g) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       u32x4 vv = v[j];
@@ -411,42 +411,64 @@ struct KvHalf<XLLM_HIP_BF16> {
   }
 };
 
-// Convert 16 quantised bytes to 16 bf16: e4m3 values exactly, int8 values offset by +128 (exact).
+// The 16-bit type the MFMAs compute in.  bf16 and e4m3 caches use bf16 (both convert exactly).  An
+// int8 cache uses fp16, because a byte u = x + 128 becomes the fp16 number 1024 + u by a byte
+// permute alone (0x6400 | u), 0.75 instructions per element instead of 1.75 through float; the
+// kernel takes the offset 1152 = 1024 + 128 back out of the scores and of the output.
 template <int KV_DT>
-__device__ inline void dequant16(const u32x4 raw, bf16x8& lo, bf16x8& hi) {
-  union {
-    bf16x2 h[8];
-    bf16x8 v[2];
-  } u;
+struct Mma {
+  typedef bf16x8 Op;
+  __device__ static inline f32x4 run(Op a, Op b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+  __device__ static inline uint32_t pack(float a, float b) {
+    return __builtin_bit_cast(uint32_t, bf16x2{(__bf16)a, (__bf16)b});
+  }
+};
+template <>
+struct Mma<XLLM_HIP_INT8> {
+  typedef f16x8 Op;
+  __device__ static inline f32x4 run(Op a, Op b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+  __device__ static inline uint32_t pack(float a, float b) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, f16x2));
+  }
+};
+constexpr float kInt8Offset = 1152.0f;
+
+// Convert 16 quantised bytes to 16 numbers of the MFMA operand type (two 16-byte pieces).
+template <int KV_DT>
+__device__ inline void dequant16(const u32x4 raw, u32x4& lo, u32x4& hi) {
+  uint32_t o[8];
 #pragma unroll
   for (int w = 0; w < 4; ++w) {
     if (KV_DT == XLLM_HIP_FP8_E4M3) {
-      u.h[2 * w] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)raw[w], 1.0f, false);
-      u.h[2 * w + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)raw[w], 1.0f, true);
+      o[2 * w] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)raw[w], 1.0f, false));
+      o[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)raw[w], 1.0f, true));
     } else {
-      // int8 x -> bf16(x + 128): the unsigned byte converts in one instruction and 0..255 is exact
-      // in bf16; the kernel takes the 128 back out of the scores and of the output.
-      const uint32_t t = raw[w] ^ 0x80808080u;
-      const float f0 = (float)(t & 0xffu);
-      const float f1 = (float)((t >> 8) & 0xffu);
-      const float f2 = (float)((t >> 16) & 0xffu);
-      const float f3 = (float)(t >> 24);
-      u.h[2 * w] = bf16x2{(__bf16)f0, (__bf16)f1};
-      u.h[2 * w + 1] = bf16x2{(__bf16)f2, (__bf16)f3};
+      const uint32_t t = raw[w] ^ 0x80808080u;                         // bytes x + 128
+      o[2 * w] = __builtin_amdgcn_perm(0x64646464u, t, 0x04010400u);      // (0x64, u1, 0x64, u0)
+      o[2 * w + 1] = __builtin_amdgcn_perm(0x64646464u, t, 0x04030402u);  // (0x64, u3, 0x64, u2)
     }
   }
-  lo = u.v[0];
-  hi = u.v[1];
+  lo = u32x4{o[0], o[1], o[2], o[3]};
+  hi = u32x4{o[4], o[5], o[6], o[7]};
 }
 
 // 1-byte caches: 4 loads of 16 bytes per lane (2 K + 2 V).  A load instruction covers 8 rows of 128
-// bytes; a lane holds 16 consecutive elements, which become two 16-byte bf16 pieces (2c, 2c+1) of
-// one LDS row.  Lanes are assigned in quads so that the 8 lanes of an LDS write group hold pieces of
+// bytes; a lane holds 16 consecutive elements, which become two 16-byte pieces (2c, 2c+1) of one
+// LDS row.  Lanes are assigned in quads so that the 8 lanes of an LDS write group hold pieces of
 // two rows whose swizzles differ in parity — rows r, r+1 for K and rows r, r+8 for V — which makes
 // the 8 pieces they write distinct mod 8.
 // The fp32 scales of the 16 tokens travel beside them: lanes 0-15 fetch the K scales, lanes 16-31
-// the V scales (one register), and park them after the tile, where every lane picks up the four it
-// needs for its score registers with one broadcast read per array and half.
+// the V scales (one register).  What is parked after the tile is what the softmax wants per token,
+// worked out once by the lane that holds the scale:
+//   kscl = k_scale * sm_scale * log2(e)    score x = s * kscl + lv
+//   lv   = log2(v_scale)                   weight w = 2^(x - max x) = p * v_scale / 2^max, never above 1
+//   rvs  = 1 / v_scale                     denominator share p = w * rvs
+// so the V scale rides inside the exponent: the weights given to the MFMA use the full range of a
+// 16-bit float whatever the scales are, and no separate multiply by v_scale is needed.
 template <int KV_DT>
 struct KvHalfQuant {
   // Load j (0, 1): K rows krow + 8j, V rows vrow + 4j.  As for the bf16 cache the LDS offsets of the
@@ -457,8 +479,9 @@ struct KvHalfQuant {
     uint32_t wk;      // LDS offset of K row krow, piece 2 * chunk
     uint32_t wv;      // LDS offset of V row vrow, piece 2 * chunk
     uint32_t sc_g;    // byte offset of this lane's scale from the scale of the first of the 16 tokens
-    uint32_t sc_lds;  // where it is parked (before adding 64 bytes for the second half of the tile)
+    uint32_t sc_lds;  // where kscl / lv is parked (before adding 64 bytes for the second half of the tile)
     int vrow;
+    int sc_tok;       // token (of the 16) whose scale this lane carries
     bool sc_on;       // lanes 0..31 carry a scale
     bool sc_is_v;
     __device__ inline void init(const DecodeParams& p, int lane) {
@@ -470,9 +493,10 @@ struct KvHalfQuant {
       gv_off = (uint32_t)(vrow * p.stride_slot + chunk * 16);
       wk = kLdsK + swz_k(krow, 2 * chunk);
       wv = kLdsV + swz_v(vrow, 2 * chunk);
-      sc_g = (uint32_t)((lane & 15) * p.sc_stride_slot * 4);
+      sc_tok = lane & 15;
+      sc_g = (uint32_t)(sc_tok * p.sc_stride_slot * 4);
       sc_is_v = ((lane >> 4) & 1) != 0;
-      sc_lds = kLdsSc + (sc_is_v ? 128 : 0) + (lane & 15) * 4;
+      sc_lds = kLdsSc + (sc_is_v ? 128 : 0) + sc_tok * 4;
       sc_on = lane < 32;
     }
     // K row krow + 8j: swizzle adds 8; V row vrow + 4j: swizzle adds 8; second piece: XOR 1.
@@ -501,22 +525,28 @@ struct KvHalfQuant {
   }
 
   template <bool MASKED>
-  __device__ inline void park(uint8_t* tile, int h, int tok, int len, const Geom& g) {
+  __device__ inline void park(uint8_t* tile, int h, int tok, int len, float scale_log2, const Geom& g) {
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      bf16x8 klo, khi, vlo, vhi;
+      u32x4 klo, khi, vlo, vhi;
       dequant16<KV_DT>(k[j], klo, khi);
       dequant16<KV_DT>(v[j], vlo, vhi);
-      if (MASKED && tok + g.vrow + 4 * j >= len) {
-        const bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
-        vlo = vhi = z;
-      }
-      *(bf16x8*)(tile + g.k_row(j, 0, h)) = klo;
-      *(bf16x8*)(tile + g.k_row(j, 1, h)) = khi;
-      *(bf16x8*)(tile + g.v_row(j, 0, h)) = vlo;
-      *(bf16x8*)(tile + g.v_row(j, 1, h)) = vhi;
+      if (MASKED && tok + g.vrow + 4 * j >= len) vlo = vhi = u32x4{0, 0, 0, 0};
+      *(u32x4*)(tile + g.k_row(j, 0, h)) = klo;
+      *(u32x4*)(tile + g.k_row(j, 1, h)) = khi;
+      *(u32x4*)(tile + g.v_row(j, 0, h)) = vlo;
+      *(u32x4*)(tile + g.v_row(j, 1, h)) = vhi;
     }
-    if (g.sc_on) *(float*)(tile + g.sc_lds + h * 64) = sc;
+    if (g.sc_on) {
+      // A V scale of zero (an all-zero row) would put -inf into the exponent and lose the token's
+      // share of the denominator; 2^-100 keeps it and still makes the row's contribution vanish.
+      const float vs = fmaxf(sc, 0x1p-100f);
+      float a = g.sc_is_v ? __builtin_amdgcn_logf(vs) : sc * scale_log2;
+      float r = __builtin_amdgcn_rcpf(vs);
+      if (MASKED && tok + g.sc_tok >= len) a = r = 0.0f;  // slots past the end may hold anything
+      *(float*)(tile + g.sc_lds + h * 64) = a;
+      if (g.sc_is_v) *(float*)(tile + g.sc_lds + 128 + h * 64) = r;
+    }
   }
 };
 template <>
@@ -524,25 +554,53 @@ struct KvHalf<XLLM_HIP_FP8_E4M3> : KvHalfQuant<XLLM_HIP_FP8_E4M3> {};
 template <>
 struct KvHalf<XLLM_HIP_INT8> : KvHalfQuant<XLLM_HIP_INT8> {};
 
+// max / sum over the four lanes (kg = 0..3) that share a query row: lanes l, l^16, l^32, l^48.
+// v_permlane16_swap exchanges the odd 16-lane rows of its first operand with the even rows of its
+// second, v_permlane32_swap the upper half of the first with the lower half of the second; fed the
+// same value twice they leave (rows 0,0,2,2 | rows 1,1,3,3) and (lower, lower | upper, upper).
+// Written as asm because the compiler's builtin hands back the first result twice; the leading
+// s_nop is the wait a VALU result needs before a lane permute may read it.
+__device__ inline void lane_swap16(float& a, float& b) {
+  asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+__device__ inline void lane_swap32(float& a, float& b) {
+  asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+__device__ inline float kg_max(float v) {
+  float a = v, b = v;
+  lane_swap16(a, b);
+  a = b = fmaxf(a, b);
+  lane_swap32(a, b);
+  return fmaxf(a, b);
+}
+__device__ inline float kg_sum(float v) {
+  float a = v, b = v;
+  lane_swap16(a, b);
+  a = b = a + b;
+  lane_swap32(a, b);
+  return a + b;
+}
+
 // State of one wave's tile of 16 query rows, and the attention over one parked tile.
 template <int KV_DT>
 struct RowTile {
   static constexpr bool kQuant = KV_DT != XLLM_HIP_BF16;
-  // int8 rows sit in LDS as x + 128.  With K' = K + 128 and V' = V + 128:
-  //   q.K  = q.K' - 128 * sum_d q_d                    (qsum, once per query row)
-  //   sum_t w_t V_t = sum_t w_t V'_t - 128 * sum_t w_t  (wsum, tracked like the softmax denominator)
+  // int8 rows sit in LDS as x + 1152.  With K' = K + 1152 and V' = V + 1152:
+  //   q.K  = q.K' - 1152 * sum_d q_d                     the constant is the MFMA's initial C operand
+  //   sum_t w_t V_t = sum_t w_t V'_t - 1152 * sum_t w_t   sum_t w_t comes from one more MFMA whose A
+  //                                                       operand is all ones (wacc)
   // Rows zeroed because they lie past the sequence end carry weight 0 in both sums.
   static constexpr bool kOffset = KV_DT == XLLM_HIP_INT8;
+  typedef typename Mma<KV_DT>::Op Op;
 
-  bf16x8 qf[4];    // Q^T fragments (B operand) of the lane's query row
+  Op qf[4];        // Q^T fragments (B operand) of the lane's query row
   f32x4 acc[8];    // O^T accumulators: head-dim tile dt, rows 4*kg + rr
-  float m_run;     // running maximum of the log2-scaled scores
+  f32x4 wacc;      // sum of the weights as the MFMA saw them (int8 only)
+  float m_run;     // running maximum of the log2-scaled scores (of score + log2 v_scale if quantised)
   float l_run;     // this lane's share of the softmax denominator
-  float w_run;     // this lane's share of sum_t w_t (int8 only)
-  float qsum128;   // 128 * sum_d q[r][d] (int8 only)
+  float s_init;    // initial value of the score accumulators: -1152 * sum_d q[r][d] (int8), else 0
   int lim;         // tokens >= lim are invisible to the row (causal among draft tokens)
   int lo;          // tokens < lo are outside the sliding window
-  int row;         // query row within (sequence, kv head); valid if < p.rows
   uint32_t k_off0; // LDS offset of K row mi, piece kg        (piece 4c + kg: XOR c << 6)
   uint32_t v_off0; // LDS offset of the transpose read, tile 0 (head-dim tile dt: XOR dt << 5)
   int kg;
@@ -550,7 +608,7 @@ struct RowTile {
   __device__ inline void init(const DecodeParams& p, const Item& it, int row_in_item, int lane) {
     const int mi = lane & 15;  // MFMA row of A / column of B and D
     kg = lane >> 4;            // k-group of the operands; row block of D
-    row = it.rg * kMaxRowsPerItem + row_in_item + mi;
+    const int row = it.rg * kMaxRowsPerItem + row_in_item + mi;
     const bool valid = row < p.rows;
     const int j = valid ? row / p.group : 0;
     const int gq = valid ? row - j * p.group : 0;
@@ -563,21 +621,23 @@ struct RowTile {
     for (int c = 0; c < 4; ++c) {
       u32x4 raw = {0, 0, 0, 0};
       if (valid) raw = *(const u32x4*)(qrow + c * 32 + kg * 8);
-      qf[c] = __builtin_bit_cast(bf16x8, raw);
-      if (kOffset) {
+      const bf16x8 qb = __builtin_bit_cast(bf16x8, raw);
+      if constexpr (kOffset) {
+        // bf16 -> fp16 is exact for magnitudes in [2^-14, 65504]; smaller ones lose low bits only
 #pragma unroll
-        for (int e = 0; e < 8; ++e) sq += (float)qf[c][e];
+        for (int e = 0; e < 8; ++e) {
+          const _Float16 hq = (_Float16)(float)qb[e];
+          qf[c][e] = hq;
+          sq += (float)hq;
+        }
+      } else {
+        qf[c] = __builtin_bit_cast(Op, qb);
       }
     }
-    qsum128 = 0.0f;
-    if (kOffset) {
-      sq += __shfl_xor(sq, 16);
-      sq += __shfl_xor(sq, 32);
-      qsum128 = 128.0f * sq;
-    }
+    s_init = kOffset ? -kInt8Offset * kg_sum(sq) : 0.0f;
     m_run = -INFINITY;
     l_run = 0.0f;
-    w_run = 0.0f;
+    wacc = f32x4{0, 0, 0, 0};
 #pragma unroll
     for (int dt = 0; dt < 8; ++dt) acc[dt] = f32x4{0, 0, 0, 0};
     k_off0 = kLdsK + swz_k(mi, kg);
@@ -587,25 +647,27 @@ struct RowTile {
 
   // Attention of the 16 rows over the 32 tokens parked in `tile` (first token tb).
   template <bool MASKED>
-  __device__ inline void attend(const uint8_t* tile, int tb, int len, float scale_log2) {
+  __device__ inline void attend(const uint8_t* tile, int tb, float scale_log2) {
     const float neg_inf = -INFINITY;
-    f32x4 ksc[2], vsc[2];  // scales of tokens tb + 16h + 4kg + rr
+    f32x4 kscl[2], lv[2], rvs[2];  // per-token factors of tokens tb + 16h + 4kg + rr
     if (kQuant) {
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
-        ksc[h] = *(const f32x4*)(tile + kLdsSc + (16 * h + 4 * kg) * 4);
-        vsc[h] = *(const f32x4*)(tile + kLdsSc + 128 + (16 * h + 4 * kg) * 4);
+        kscl[h] = *(const f32x4*)(tile + kLdsSc + (16 * h + 4 * kg) * 4);
+        lv[h] = *(const f32x4*)(tile + kLdsSc + 128 + (16 * h + 4 * kg) * 4);
+        rvs[h] = *(const f32x4*)(tile + kLdsSc + 256 + (16 * h + 4 * kg) * 4);
       }
     }
     // ---- S^T = K Q^T ----
-    f32x4 s[2] = {f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}};
+    f32x4 s[2];
+    s[0] = s[1] = f32x4{s_init, s_init, s_init, s_init};
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
       const uint32_t ko = k_off0 ^ (uint32_t)(c << 6);
-      const bf16x8 kf0 = *(const bf16x8*)(tile + ko);
-      const bf16x8 kf1 = *(const bf16x8*)(tile + ko + 4096);
-      s[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf0, qf[c], s[0], 0, 0, 0);
-      s[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf1, qf[c], s[1], 0, 0, 0);
+      const Op kf0 = *(const Op*)(tile + ko);
+      const Op kf1 = *(const Op*)(tile + ko + 4096);
+      s[0] = Mma<KV_DT>::run(kf0, qf[c], s[0]);
+      s[1] = Mma<KV_DT>::run(kf1, qf[c], s[1]);
     }
     // ---- online softmax of the lane's query row ----
     float x[8];
@@ -613,10 +675,7 @@ struct RowTile {
     for (int h = 0; h < 2; ++h) {
 #pragma unroll
       for (int rr = 0; rr < 4; ++rr) {
-        float v = s[h][rr];
-        if (kOffset) v -= qsum128;
-        v *= scale_log2;
-        if (kQuant) v *= ksc[h][rr];
+        float v = kQuant ? __builtin_fmaf(s[h][rr], kscl[h][rr], lv[h][rr]) : s[h][rr] * scale_log2;
         if (MASKED) {
           const int tok = tb + 16 * h + 4 * kg + rr;
           v = (tok < lim && tok >= lo) ? v : neg_inf;
@@ -624,50 +683,41 @@ struct RowTile {
         x[4 * h + rr] = v;
       }
     }
-    float mt = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
-    mt = fmaxf(mt, __shfl_xor(mt, 16));
-    mt = fmaxf(mt, __shfl_xor(mt, 32));
+    const float mt =
+        kg_max(fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7]))));
     const float m_new = fmaxf(m_run, mt);
     const float m_safe = m_new == neg_inf ? 0.0f : m_new;
+    const bool moved = __builtin_amdgcn_ballot_w64(m_new != m_run) != 0;
     const float alpha = __builtin_amdgcn_exp2f(m_run - m_safe);
-    float psum = 0.0f;
-    float pv[8];
+    l_run *= alpha;
+    m_run = m_new;
+    float w[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const float e = __builtin_amdgcn_exp2f(x[i] - m_safe);
-      psum += e;
-      pv[i] = e;
-    }
-    if (kQuant) {
+    for (int h = 0; h < 2; ++h) {
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {
-#pragma unroll
-        for (int rr = 0; rr < 4; ++rr) {
-          float w = vsc[h][rr];
-          if (MASKED) {
-            const int tok = tb + 16 * h + 4 * kg + rr;
-            w = tok < len ? w : 0.0f;
-          }
-          pv[4 * h + rr] *= w;
-        }
+      for (int rr = 0; rr < 4; ++rr) {
+        const float e = __builtin_amdgcn_exp2f(x[4 * h + rr] - m_safe);
+        w[4 * h + rr] = e;
+        l_run = kQuant ? __builtin_fmaf(e, rvs[h][rr], l_run) : l_run + e;
       }
     }
-    l_run = l_run * alpha + psum;
-    m_run = m_new;
-    // Unconditional: a branch around the rescale splits the live ranges of the accumulator tuples
-    // and costs far more registers than the 32 multiplies cost issue slots.
-#pragma unroll
-    for (int dt = 0; dt < 8; ++dt) acc[dt] *= alpha;
-    bf16x8 pf;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) pf[i] = (__bf16)pv[i];
-    if (kOffset) {
-      float wt = 0.0f;  // sum of the weights as the MFMA will see them (after rounding to bf16)
-#pragma unroll
-      for (int i = 0; i < 8; ++i) wt += (float)pf[i];
-      w_run = w_run * alpha + wt;
+    const u32x4 pw = {Mma<KV_DT>::pack(w[0], w[1]), Mma<KV_DT>::pack(w[2], w[3]), Mma<KV_DT>::pack(w[4], w[5]),
+                      Mma<KV_DT>::pack(w[6], w[7])};
+    const Op pf = __builtin_bit_cast(Op, pw);
+    // ---- O^T = O^T * alpha + V^T P^T ----
+    // The accumulators need rescaling only when some row's maximum moved, which becomes rare a few
+    // tiles into a sequence.  Both variants of the product are written out, so that each path ends
+    // in the MFMAs that define the accumulators (a branch around the multiplies alone makes the
+    // compiler shuffle the accumulator registers on every tile).
+    if (moved) {
+      accumulate<true>(tile, pf, alpha);
+    } else {
+      accumulate<false>(tile, pf, alpha);
     }
-    // ---- O^T += V^T P^T ----
+  }
+
+  template <bool RESCALE>
+  __device__ inline void accumulate(const uint8_t* tile, const Op pf, float alpha) {
 #pragma unroll
     for (int dt = 0; dt < 8; ++dt) {
       const uint32_t vo = v_off0 ^ (uint32_t)(dt << 5);
@@ -675,8 +725,16 @@ struct RowTile {
           (__attribute__((address_space(3))) s16x4*)(tile + vo));
       const s16x4 a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
           (__attribute__((address_space(3))) s16x4*)(tile + vo + 4096));
-      const bf16x8 vf = __builtin_bit_cast(bf16x8, __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7));
-      acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, acc[dt], 0, 0, 0);
+      const Op vf = __builtin_bit_cast(Op, __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7));
+      f32x4 c = acc[dt];
+      if (RESCALE) c *= alpha;
+      acc[dt] = Mma<KV_DT>::run(vf, pf, c);
+    }
+    if (kOffset) {
+      const u32x4 ones = {0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u};  // fp16 1.0
+      f32x4 c = wacc;
+      if (RESCALE) c *= alpha;
+      wacc = Mma<KV_DT>::run(__builtin_bit_cast(Op, ones), pf, c);
     }
   }
 };
@@ -693,19 +751,12 @@ __device__ inline void finish_item(const DecodeParams& p, const Item& it, RowTil
   const int mi = lane & 15, kg = lane >> 4;
   const int nhq = p.n * p.num_q_heads;
   const bool single = p.direct_single != 0 && p.num_chunks[it.b] == 1;
-  float l = rt.l_run;
-  l += __shfl_xor(l, 16);
-  l += __shfl_xor(l, 32);
-  float wsum = rt.w_run;
-  if (kOffset) {
-    wsum += __shfl_xor(wsum, 16);
-    wsum += __shfl_xor(wsum, 32);
-  }
+  const float l = kg_sum(rt.l_run);
   uint8_t* mine = xch_base + wave * xch_stride;
 #pragma unroll
   for (int dt = 0; dt < 8; ++dt) {
     f32x4 o = rt.acc[dt];
-    if (kOffset) o -= 128.0f * wsum;
+    if (kOffset) o -= kInt8Offset * rt.wacc[0];  // every element of wacc holds the row's sum
     *(f32x4*)(mine + mi * kXchRow + (dt * 16 + 4 * kg) * 4) = o;
   }
   if (kg == 0) {
@@ -817,20 +868,20 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_d128_kernel(Decode
       const bool masked = (tb + kTileTokens > mask_hi_from) || (tb < mask_lo_until);
       // park the tile, then put the next tile's loads in flight while this one is consumed
       if (masked) {
-        st[0].template park<true>(tile, 0, tb, it.len, geom);
-        st[1].template park<true>(tile, 1, tb + 16, it.len, geom);
+        st[0].template park<true>(tile, 0, tb, it.len, p.scale_log2, geom);
+        st[1].template park<true>(tile, 1, tb + 16, it.len, p.scale_log2, geom);
       } else {
-        st[0].template park<false>(tile, 0, tb, it.len, geom);
-        st[1].template park<false>(tile, 1, tb + 16, it.len, geom);
+        st[0].template park<false>(tile, 0, tb, it.len, p.scale_log2, geom);
+        st[1].template park<false>(tile, 1, tb + 16, it.len, p.scale_log2, geom);
       }
       if (tb + kTileTokens < w_end) {
         st[0].issue(p, it, tb + kTileTokens, geom);
         st[1].issue(p, it, tb + kTileTokens + 16, geom);
       }
       if (masked) {
-        rt.template attend<true>(tile, tb, it.len, p.scale_log2);
+        rt.template attend<true>(tile, tb, p.scale_log2);
       } else {
-        rt.template attend<false>(tile, tb, it.len, p.scale_log2);
+        rt.template attend<false>(tile, tb, p.scale_log2);
       }
     }
   }
@@ -885,18 +936,18 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_d128_rows32_kernel
     const bool masked = (tb + kTileTokens > mask_hi_from) || (tb < mask_lo_until);
     if (live) {
       if (masked) {
-        m.template park<true>(tile, rs, tb + 16 * rs, it.len, geom);
+        m.template park<true>(tile, rs, tb + 16 * rs, it.len, p.scale_log2, geom);
       } else {
-        m.template park<false>(tile, rs, tb + 16 * rs, it.len, geom);
+        m.template park<false>(tile, rs, tb + 16 * rs, it.len, p.scale_log2, geom);
       }
       issue(m, tb + 2 * kTileTokens);
     }
     __syncthreads();  // both halves of tile i are parked; everyone is done with tile i-1
     if (live) {
       if (masked) {
-        rt.template attend<true>(tile, tb, it.len, p.scale_log2);
+        rt.template attend<true>(tile, tb, p.scale_log2);
       } else {
-        rt.template attend<false>(tile, tb, it.len, p.scale_log2);
+        rt.template attend<false>(tile, tb, p.scale_log2);
       }
     }
   };
