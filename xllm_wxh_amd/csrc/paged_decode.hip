@@ -199,6 +199,8 @@ struct Item {
   int t_end;    // one past the last token of the chunk (<= len)
   const int32_t* ids;  // block list of the sequence
   int nblk;     // valid entries in ids (>= 1)
+  int64_t head_off;     // hk * stride_head (cache elements)
+  int64_t sc_head_off;  // hk * sc_stride_head (scale elements)
 };
 
 __device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it) {
@@ -221,6 +223,8 @@ __device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it)
   }
   it.nblk = (it.len + p.block_size - 1) >> p.log2_bs;
   if (it.nblk < 1) it.nblk = 1;
+  it.head_off = (int64_t)it.hk * p.stride_head;
+  it.sc_head_off = (int64_t)it.hk * p.sc_stride_head;
   return true;
 }
 
@@ -332,22 +336,31 @@ __device__ inline uint32_t swz_v(int row, int piece) {
   return (uint32_t)(row * 256 + ((piece ^ (((row & 7) << 1) | ((row >> 3) & 1))) << 4));
 }
 
+// Physical block of token `tok` (any token up to the end of the chunk's last tile: the index is
+// clamped to the sequence's block list).  The id comes back through a scalar load; callers fetch it
+// a tile ahead of the loads that need it, so that its latency is off the critical path.
+__device__ inline int block_of(const DecodeParams& p, const Item& it, int tok) {
+  int bi = tok >> p.log2_bs;
+  bi = bi < it.nblk ? bi : it.nblk - 1;
+  return __builtin_amdgcn_readfirstlane(it.ids[bi]);
+}
+
 // Uniform (scalar-register) part of the addresses of 16 consecutive tokens starting at `tok`
-// (a multiple of 16, so they lie in one block): element offset of (block, kv head, slot) in the
-// cache and in the scale tensors.
+// (a multiple of 16, so they lie in one block, `blk`): element offset of (block, kv head, slot) in
+// the cache and in the scale tensors.  The host admits only caches whose block and slot strides are
+// below 2^31 elements to these kernels, so 32 x 32 -> 64 bit products suffice.
 struct HalfBase {
   int64_t elem;
   int64_t scale;
 };
 
-__device__ inline HalfBase half_base(const DecodeParams& p, const Item& it, int tok) {
-  int bi = tok >> p.log2_bs;
-  bi = bi < it.nblk ? bi : it.nblk - 1;
-  const int64_t blk = __builtin_amdgcn_readfirstlane(it.ids[bi]);
-  const int64_t slot = tok & (p.block_size - 1);
+__device__ inline HalfBase half_base(const DecodeParams& p, const Item& it, int tok, int blk) {
+  const uint32_t slot = (uint32_t)(tok & (p.block_size - 1));
   HalfBase b;
-  b.elem = blk * p.stride_block + (int64_t)it.hk * p.stride_head + slot * p.stride_slot;
-  b.scale = blk * p.sc_stride_block + (int64_t)it.hk * p.sc_stride_head + slot * p.sc_stride_slot;
+  b.elem = (int64_t)((uint64_t)(uint32_t)blk * (uint32_t)p.stride_block) + it.head_off +
+           (int64_t)(slot * (uint32_t)p.stride_slot);
+  b.scale = (int64_t)((uint64_t)(uint32_t)blk * (uint32_t)p.sc_stride_block) + it.sc_head_off +
+            (int64_t)(slot * (uint32_t)p.sc_stride_slot);
   return b;
 }
 
@@ -386,8 +399,8 @@ struct KvHalf<XLLM_HIP_BF16> {
   u32x4 k[4];
   u32x4 v[4];
 
-  __device__ inline void issue(const DecodeParams& p, const Item& it, int tok, const Geom& g) {
-    const HalfBase b = half_base(p, it, tok);
+  __device__ inline void issue(const DecodeParams& p, const Item& it, int tok, int blk, const Geom& g) {
+    const HalfBase b = half_base(p, it, tok, blk);
     const uint8_t* kb = p.k_cache + b.elem * 2;
     const uint8_t* vb = p.v_cache + b.elem * 2;
     const int64_t step = 4 * p.stride_slot * 2;  // four rows further, in bytes (uniform)
@@ -511,8 +524,8 @@ struct KvHalfQuant {
   u32x4 v[2];
   float sc;
 
-  __device__ inline void issue(const DecodeParams& p, const Item& it, int tok, const Geom& g) {
-    const HalfBase b = half_base(p, it, tok);
+  __device__ inline void issue(const DecodeParams& p, const Item& it, int tok, int blk, const Geom& g) {
+    const HalfBase b = half_base(p, it, tok, blk);
     const uint8_t* kb = p.k_cache + b.elem;
     const uint8_t* vb = p.v_cache + b.elem;
 #pragma unroll
@@ -862,10 +875,17 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_d128_kernel(Decode
   KvHalf<KV_DT> st[2];  // the two 16-token halves of the tile in flight
 
   if (w_begin < w_end) {
-    st[0].issue(p, it, w_begin, geom);
-    st[1].issue(p, it, w_begin + 16, geom);
+    st[0].issue(p, it, w_begin, block_of(p, it, w_begin), geom);
+    st[1].issue(p, it, w_begin + 16, block_of(p, it, w_begin + 16), geom);
+    // block ids of the next tile's halves, fetched one tile before the loads that use them
+    int blk0 = block_of(p, it, w_begin + kTileTokens);
+    int blk1 = block_of(p, it, w_begin + kTileTokens + 16);
     for (int tb = w_begin; tb < w_end; tb += kTileTokens) {
       const bool masked = (tb + kTileTokens > mask_hi_from) || (tb < mask_lo_until);
+      // The scalar loads of the ids go out before the tile is parked: they share a counter with the
+      // LDS traffic, so the next wait on LDS also waits for them.
+      const int nblk0 = block_of(p, it, tb + 2 * kTileTokens);
+      const int nblk1 = block_of(p, it, tb + 2 * kTileTokens + 16);
       // park the tile, then put the next tile's loads in flight while this one is consumed
       if (masked) {
         st[0].template park<true>(tile, 0, tb, it.len, p.scale_log2, geom);
@@ -875,9 +895,11 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_d128_kernel(Decode
         st[1].template park<false>(tile, 1, tb + 16, it.len, p.scale_log2, geom);
       }
       if (tb + kTileTokens < w_end) {
-        st[0].issue(p, it, tb + kTileTokens, geom);
-        st[1].issue(p, it, tb + kTileTokens + 16, geom);
+        st[0].issue(p, it, tb + kTileTokens, blk0, geom);
+        st[1].issue(p, it, tb + kTileTokens + 16, blk1, geom);
       }
+      blk0 = nblk0;
+      blk1 = nblk1;
       if (masked) {
         rt.template attend<true>(tile, tb, p.scale_log2);
       } else {
@@ -926,11 +948,15 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_d128_rows32_kernel
   // flight per CU to cover the HBM latency.)
   KvHalf<KV_DT> mine[2];  // the 16 tokens this wave fetches: rows 16*rs .. of the tile
 
-  auto issue = [&](KvHalf<KV_DT>& m, int tb) {
-    if (tb < w_end) m.issue(p, it, tb + 16 * rs, geom);
+  auto issue = [&](KvHalf<KV_DT>& m, int blk, int tb) {
+    if (tb < w_end) m.issue(p, it, tb + 16 * rs, blk, geom);
   };
-  auto step = [&](KvHalf<KV_DT>& m, int i) {
+  // `blk`: block id of the half this wave fetches two tiles on; replaced by that of the tile four
+  // on.  The scalar load goes out before the tile is parked: it shares a counter with the LDS
+  // traffic, so the wait before the barrier also waits for it.
+  auto step = [&](KvHalf<KV_DT>& m, int& blk, int i) {
     const int tb = w_begin + i * kTileTokens;
+    const int nblk = block_of(p, it, tb + 4 * kTileTokens + 16 * rs);
     const bool live = tb < w_end;
     uint8_t* tile = tiles + (i & 1) * kLdsTile;
     const bool masked = (tb + kTileTokens > mask_hi_from) || (tb < mask_lo_until);
@@ -940,8 +966,9 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_d128_rows32_kernel
       } else {
         m.template park<false>(tile, rs, tb + 16 * rs, it.len, p.scale_log2, geom);
       }
-      issue(m, tb + 2 * kTileTokens);
+      issue(m, blk, tb + 2 * kTileTokens);
     }
+    blk = nblk;
     __syncthreads();  // both halves of tile i are parked; everyone is done with tile i-1
     if (live) {
       if (masked) {
@@ -951,11 +978,13 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_d128_rows32_kernel
       }
     }
   };
-  issue(mine[0], w_begin);
-  issue(mine[1], w_begin + kTileTokens);
+  issue(mine[0], block_of(p, it, w_begin + 16 * rs), w_begin);
+  issue(mine[1], block_of(p, it, w_begin + kTileTokens + 16 * rs), w_begin + kTileTokens);
+  int blk_a = block_of(p, it, w_begin + 2 * kTileTokens + 16 * rs);
+  int blk_b = block_of(p, it, w_begin + 3 * kTileTokens + 16 * rs);
   for (int i = 0; i < iters; i += 2) {
-    step(mine[0], i);
-    if (i + 1 < iters) step(mine[1], i + 1);
+    step(mine[0], blk_a, i);
+    if (i + 1 < iters) step(mine[1], blk_b, i + 1);
   }
   __syncthreads();  // all tiles consumed before the buffers are reused for the exchange
   finish_item<KV_DT, TW>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, rs, tw, lane);
@@ -1105,14 +1134,16 @@ static Variant pick_variant(const xllm_hip_kv_cache* c, const xllm_hip_decode_ar
     const bool strides_ok = c->stride_block % vec == 0 && c->stride_head % vec == 0 && c->stride_slot % vec == 0 &&
                             a->q_token_stride % 8 == 0;
     const bool ptrs_ok = aligned16(c->k_cache) && aligned16(c->v_cache) && aligned16(a->q);
+    const int64_t lim32 = (int64_t)1 << 31;  // the kernels form block and slot offsets from 32-bit factors
     bool scales_ok = true;
     if (eb == 1) {
-      scales_ok = c->k_scale != nullptr && c->v_scale != nullptr &&
-                  (c->scale_stride_slot != 1 ||
-                   (c->scale_stride_block % 4 == 0 && c->scale_stride_head % 4 == 0 && aligned16(c->k_scale) &&
-                    aligned16(c->v_scale)));
+      scales_ok = c->k_scale != nullptr && c->v_scale != nullptr && c->scale_stride_block >= 0 &&
+                  c->scale_stride_block < lim32 && c->scale_stride_slot >= 0 &&
+                  c->scale_stride_slot * c->block_size < lim32;
     }
-    if (strides_ok && ptrs_ok && scales_ok) return kMfmaD128;
+    const bool range_ok = c->stride_block >= 0 && c->stride_block < lim32 && c->stride_slot >= 0 &&
+                          c->stride_slot * c->block_size < lim32;
+    if (strides_ok && range_ok && ptrs_ok && scales_ok) return kMfmaD128;
   }
   if (c->head_dim <= 256 && is_pow2(c->block_size)) return kGeneric;
   return kNone;
