@@ -54,9 +54,10 @@ def build_pools(w, torch, ops, num_blocks, npools, device):
     gen.manual_seed(1234)
     shape = (num_blocks, w.num_kv_heads, w.block_size, w.head_dim)
     for _ in range(npools):
-        if w.kv_dtype == "bf16":
-            k = torch.randn(shape, device=device, dtype=torch.bfloat16, generator=gen) * w.value_std
-            v = torch.randn(shape, device=device, dtype=torch.bfloat16, generator=gen) * w.value_std
+        if w.kv_dtype in ("bf16", "fp32"):
+            dt = torch.bfloat16 if w.kv_dtype == "bf16" else torch.float32
+            k = torch.randn(shape, device=device, dtype=dt, generator=gen) * w.value_std
+            v = torch.randn(shape, device=device, dtype=dt, generator=gen) * w.value_std
             pools.append((k, v, None, None))
             continue
         cdt = torch.int8 if w.kv_dtype == "int8" else torch.float8_e4m3fn
@@ -107,17 +108,14 @@ def main():
                           "bytes_written_per_launch": src.numel() * 2, "launches": 10}))
         return
     w = workloads.WORKLOADS[args.workload]
-    if w.kv_dtype == "fp32":
-        sys.stderr.write("workload %s is the CPU-reference case; pick a GPU workload\n" % w.name)
-        sys.exit(2)
-
+    io_dtype = torch.float32 if w.kv_dtype == "fp32" else torch.bfloat16  # query, output, new K/V rows
     seq_lens = workloads.make_seq_lens(w, seed=0)
     table, num_blocks, lists = workloads.make_block_tables(w, seq_lens, seed=0)
     pools = build_pools(w, torch, ops, num_blocks, args.pools, device)
     T = w.batch * w.q_per_seq
     gen = torch.Generator(device=device)
     gen.manual_seed(99)
-    q = torch.randn(T, w.num_q_heads, w.head_dim, device=device, dtype=torch.bfloat16, generator=gen)
+    q = torch.randn(T, w.num_q_heads, w.head_dim, device=device, dtype=io_dtype, generator=gen)
     out = torch.empty_like(q)
     block_table = torch.from_numpy(table).to(device)
     seq_lens_d = torch.from_numpy(seq_lens).to(device)
@@ -159,7 +157,7 @@ def main():
     kern_avg_us = sum(kern_us) / len(kern_us)
 
     # the step's KV write, timed on its own
-    src_dt = torch.bfloat16
+    src_dt = io_dtype
     new_k = torch.randn(T, w.num_kv_heads, w.head_dim, device=device, dtype=src_dt, generator=gen)
     new_v = torch.randn(T, w.num_kv_heads, w.head_dim, device=device, dtype=src_dt, generator=gen)
     slots = torch.from_numpy(workloads.decode_slots(w, seq_lens, lists)).to(device)
@@ -186,6 +184,9 @@ def main():
     achieved_gbps = alg_bytes / us_per_step / 1e3
     kern_gbps = alg_bytes / kern_avg_us / 1e3
 
+    rows_per_kv_head = w.q_per_seq * (w.num_q_heads // w.num_kv_heads)
+    kernel_name = ("decode_generic_kernel" if variant != "mfma_d128" else
+                   "decode_mfma_d128_kernel" if rows_per_kv_head <= 16 else "decode_mfma_d128_rows32_kernel")
     traffic = None
     tpath = os.path.join(REPO, "profiles", "hbm_traffic.json")
     if os.path.exists(tpath):
@@ -202,7 +203,7 @@ def main():
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16" if w.kv_dtype == "bf16" else "bf16 (KV %s)" % w.kv_dtype,
+        "dtype": w.kv_dtype if w.kv_dtype in ("bf16", "fp32") else "bf16 (KV %s)" % w.kv_dtype,
         "data": "synthetic",
         "config": {
             "workload": w.name,
@@ -226,7 +227,7 @@ def main():
         "kv_write_us": round(kv_write_us, 2),
         "roofline": {
             "bound": "hbm",
-            "kernel": "decode_mfma_d128_kernel" if variant == "mfma_d128" else "decode_generic_kernel",
+            "kernel": kernel_name,
             "achieved": round(kern_gbps, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
@@ -283,7 +284,8 @@ def cpu_baseline(w, torch, pool, q, block_table, seq_lens, out, step, args):
     ref = run()  # warm-up, also the check below
     times = []
     t_start = time.perf_counter()
-    while len(times) < 3 and (time.perf_counter() - t_start) < args.cpu_seconds:
+    runs = 20 if w.kv_dtype == "fp32" else 3
+    while len(times) < runs and (time.perf_counter() - t_start) < args.cpu_seconds:
         t0 = time.perf_counter()
         run()
         times.append(time.perf_counter() - t0)
