@@ -262,6 +262,46 @@ int xllm_hip_csr_to_block_table(const int32_t* kv_indptr,
                                 int32_t* seq_lens,
                                 xllm_hip_stream_t stream);
 
+/*
+ * Batched block swap — KVCache::swap_blocks
+ * (xllm/core/framework/kv_cache/kv_cache.cpp:104-125; called per layer from
+ * xllm/core/runtime/worker_impl.cpp:584-606 with int64 index tensors): for every pair i the whole
+ * block src_blocks[i] of K, of V and, for a quantised cache, of both scale tensors is copied to
+ * block dst_blocks[i].  The reference gathers all sources first (index_select) and scatters
+ * afterwards (index_copy_), so a block that is both a destination and a source still supplies its
+ * old contents.  With a staging buffer of xllm_hip_swap_blocks_staging_bytes(cache, num_pairs)
+ * bytes (16-byte aligned) this call does exactly that, in two launches.  With staging == NULL it
+ * copies in place in one pass, which is the same result whenever no destination block is also a
+ * source (the block manager hands out fresh blocks as destinations).  Pairs with an id outside
+ * [0, num_blocks) are skipped (the reference would throw).  Duplicate destinations: one of the
+ * writers wins per 16-byte piece, as with index_copy_.
+ */
+size_t xllm_hip_swap_blocks_staging_bytes(const xllm_hip_kv_cache* cache, int64_t num_pairs);
+int xllm_hip_swap_blocks(const xllm_hip_kv_cache* cache,
+                         const int64_t* src_blocks,
+                         const int64_t* dst_blocks,
+                         int64_t num_pairs,
+                         void* staging,
+                         size_t staging_bytes,
+                         xllm_hip_stream_t stream);
+
+/*
+ * One-to-many block copy in the form the batch builder emits for the block-copy kernel
+ * (xllm/core/framework/batch/batch_input_builder.cpp:691-720; fields
+ * xllm/core/framework/model/model_input_params.h:542-545; consumed by
+ * xllm/models/llm/npu/llm_model_base.h:69-75): source block src_block_indices[g] is copied to the
+ * destination blocks dst_block_indices[cum_sum[g-1] .. cum_sum[g]) (cum_sum[-1] = 0), for
+ * g < num_groups; num_dst = cum_sum[num_groups-1].  K, V and the scale tensors move together.
+ * Destinations must not be sources of the same call.
+ */
+int xllm_hip_copy_blocks(const xllm_hip_kv_cache* cache,
+                         const int32_t* src_block_indices,
+                         const int32_t* dst_block_indices,
+                         const int32_t* cum_sum,
+                         int32_t num_groups,
+                         int32_t num_dst,
+                         xllm_hip_stream_t stream);
+
 /* Message of the last non-OK status returned on this host thread ("" if none). */
 const char* xllm_hip_last_error(void);
 

@@ -27,6 +27,11 @@ tree); how each one is pinned is listed beside it:
       xllm/core/runtime/cuda_graph_executor_test.cpp:150-151.  Absolute FlashInfer/tmo outputs:
       PARITY UNPINNED (tolerance only).
   lse_combine                            xllm/core/kernels/cuda/xattention/lse_combine.cu:61-73
+  swap_blocks                            xllm/core/framework/kv_cache/kv_cache.cpp:104-125
+  build_block_copy_groups / copy_blocks  xllm/core/framework/batch/batch_input_builder.cpp:691-720,
+      xllm/models/llm/npu/llm_model_base.h:69-75; pinned by brute force on tiny caches (element
+      loops), by the gather-before-scatter property on a chain a->b, b->c, and by the group arrays
+      expanding back to the transfer list they came from.
   quantize_per_token_head / quant_to_paged_cache
       scale and saturation conventions of xllm/core/kernels/cuda/fp8_quant_utils.cuh:38-53,112-131;
       the int8 rounding of `tmo::quant_to_paged_cache` (xllm/core/kernels/mlu/attention.cpp:50-59) is
@@ -213,6 +218,57 @@ def reshape_paged_cache(slot_ids, keys, values, key_cache, value_cache, layout="
     kc[blk, :, off, :] = keys
     if values is not None:
         _hnd_view(value_cache, layout)[blk, :, off, :] = values
+
+
+# ---- whole-block movement ----------------------------------------------------------------
+
+
+def swap_blocks(arrays, src, dst):
+    """KVCache::swap_blocks (xllm/core/framework/kv_cache/kv_cache.cpp:104-125): for every array whose
+    first dimension is the block (key cache, value cache, and the scale tensors when defined),
+    `selected = index_select(array, 0, src)` and then `array.index_copy_(0, dst, selected)` — all
+    sources are read before any destination is written.  In place; `arrays` is an iterable."""
+    src = np.asarray(src, dtype=np.int64)
+    dst = np.asarray(dst, dtype=np.int64)
+    for a in arrays:
+        if a is None:
+            continue
+        selected = a[src].copy()
+        a[dst] = selected
+
+
+def build_block_copy_groups(pairs):
+    """The (src_block_indices, dst_block_indices, cum_sum) arrays the batch builder derives from
+    its (src, dst) transfer list (xllm/core/framework/batch/batch_input_builder.cpp:691-720): pairs
+    sorted by source, one source entry per distinct source, cum_sum[g] = number of destinations up to
+    and including group g.  (std::sort there is not stable; this port keeps ties in input order.)"""
+    pairs = sorted(pairs, key=lambda sd: sd[0])
+    if not pairs:
+        return [], [], []
+    src_indices, dst_indices, cum_sum = [pairs[0][0]], [pairs[0][1]], []
+    current = pairs[0][0]
+    for i in range(1, len(pairs)):
+        dst_indices.append(pairs[i][1])
+        if pairs[i][0] != current:
+            src_indices.append(pairs[i][0])
+            cum_sum.append(i)
+            current = pairs[i][0]
+    cum_sum.append(len(pairs))
+    return src_indices, dst_indices, cum_sum
+
+
+def copy_blocks(arrays, src_block_indices, dst_block_indices, cum_sum):
+    """What the block-copy step does with those arrays (call site
+    xllm/models/llm/npu/llm_model_base.h:69-75): block src_block_indices[g] is copied to every block
+    in dst_block_indices[cum_sum[g-1]:cum_sum[g]].  Literal loops."""
+    for a in arrays:
+        if a is None:
+            continue
+        begin = 0
+        for g, src in enumerate(src_block_indices):
+            for i in range(begin, cum_sum[g]):
+                a[dst_block_indices[i]] = a[src]
+            begin = cum_sum[g]
 
 
 # ---- quantisers ------------------------------------------------------------------------

@@ -155,3 +155,30 @@ def test_cpp_ops_match_python_ops(gpu, shim):
                           torch.from_numpy(indices).to(gpu), torch.from_numpy(last).to(gpu), -1, case.scale, out_c)
     torch.cuda.synchronize()
     assert torch.equal(out_c, ref)
+
+
+@pytest.mark.gpu
+def test_kv_cache_swap_blocks_and_copy_blocks(gpu, shim):
+    import numpy as np
+    from oracle import paged_kv_oracle as orc
+
+    print("case shim swap_blocks / copy_blocks", flush=True)
+    g = torch.Generator().manual_seed(4)
+    k = torch.randint(-128, 128, (12, 2, 16, 128), generator=g, dtype=torch.int8)
+    v = torch.randint(-128, 128, (12, 2, 16, 128), generator=g, dtype=torch.int8)
+    ks, vs = torch.rand(12, 2, 16, generator=g), torch.rand(12, 2, 16, generator=g)
+    kv = shim.KVCache(k.to(gpu), v.to(gpu), ks.to(gpu), vs.to(gpu))
+    src, dst = [0, 3, 5], [3, 5, 7]  # a chain: each destination must receive the old source
+    ref = [t.numpy().copy() for t in (k, v, ks, vs)]
+    orc.swap_blocks(ref, src, dst)
+    kv.swap_blocks(torch.tensor(src, device=gpu), torch.tensor(dst, device=gpu))
+    got = [kv.get_k_cache(), kv.get_v_cache(), kv.get_k_cache_scale(), kv.get_v_cache_scale()]
+    for a, b in zip(got, ref):
+        assert np.array_equal(a.cpu().numpy(), b)
+    s, d, c = orc.build_block_copy_groups([(1, 8), (1, 9), (2, 10)])
+    orc.copy_blocks(ref, s, d, c)
+    i32 = dict(dtype=torch.int32, device=gpu)
+    shim.copy_blocks(got[0], got[1], got[2], got[3], torch.tensor(s, **i32), torch.tensor(d, **i32),
+                     torch.tensor(c, **i32))
+    for a, b in zip(got, ref):
+        assert np.array_equal(a.cpu().numpy(), b)

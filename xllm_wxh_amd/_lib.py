@@ -34,6 +34,9 @@ EXPORTED_SYMBOLS = (
     "xllm_hip_paged_decode_run_timed",
     "xllm_hip_paged_decode",
     "xllm_hip_csr_to_block_table",
+    "xllm_hip_swap_blocks_staging_bytes",
+    "xllm_hip_swap_blocks",
+    "xllm_hip_copy_blocks",
     "xllm_hip_last_error",
     "xllm_hip_abi_version",
     "xllm_hip_paged_decode_variant",
@@ -129,6 +132,12 @@ def load():
     lib.xllm_hip_paged_decode_run_timed.restype = ctypes.c_int
     lib.xllm_hip_csr_to_block_table.argtypes = [vp, vp, vp, i32, i32, vp, i64, i32, vp, vp]
     lib.xllm_hip_csr_to_block_table.restype = ctypes.c_int
+    lib.xllm_hip_swap_blocks_staging_bytes.argtypes = [P(KvCacheDesc), i64]
+    lib.xllm_hip_swap_blocks_staging_bytes.restype = ctypes.c_size_t
+    lib.xllm_hip_swap_blocks.argtypes = [P(KvCacheDesc), vp, vp, i64, vp, ctypes.c_size_t, vp]
+    lib.xllm_hip_swap_blocks.restype = ctypes.c_int
+    lib.xllm_hip_copy_blocks.argtypes = [P(KvCacheDesc), vp, vp, vp, i32, i32, vp]
+    lib.xllm_hip_copy_blocks.restype = ctypes.c_int
     lib.xllm_hip_last_error.argtypes = []
     lib.xllm_hip_last_error.restype = ctypes.c_char_p
     lib.xllm_hip_abi_version.argtypes = []

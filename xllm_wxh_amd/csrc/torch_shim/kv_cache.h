@@ -6,6 +6,8 @@
 
 #include <optional>
 
+#include "ops_api.h"
+
 namespace xllm {
 
 class KVCache final {
@@ -39,6 +41,13 @@ class KVCache final {
   }
 
   bool empty() const { return !key_cache_.defined() || !value_cache_.defined(); }
+
+  // Batched block copy src_tensor[i] -> dst_tensor[i] over K, V and the scales, sources read first
+  // (xllm/core/framework/kv_cache/kv_cache.cpp:104-125).
+  void swap_blocks(torch::Tensor& src_tensor, torch::Tensor& dst_tensor) {
+    kernel::hip::swap_blocks(key_cache_, value_cache_, get_k_cache_scale(), get_v_cache_scale(), src_tensor,
+                             dst_tensor);
+  }
 
  private:
   torch::Tensor key_cache_;

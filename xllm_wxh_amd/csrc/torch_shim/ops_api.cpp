@@ -256,5 +256,45 @@ void batch_decode_csr(torch::Tensor query,
   run_decode(cache, a, query);
 }
 
+void swap_blocks(const torch::Tensor& k_cache,
+                 const torch::Tensor& v_cache,
+                 const std::optional<torch::Tensor>& k_cache_scale,
+                 const std::optional<torch::Tensor>& v_cache_scale,
+                 const torch::Tensor& src,
+                 const torch::Tensor& dst) {
+  TORCH_CHECK(src.defined() && dst.defined() && src.scalar_type() == torch::kLong &&
+                  dst.scalar_type() == torch::kLong && src.is_cuda() && dst.is_cuda(),
+              "swap_blocks takes int64 index tensors on the GPU");
+  TORCH_CHECK(src.numel() == dst.numel(), "src and dst must name the same number of blocks");
+  const int64_t n = src.numel();
+  if (n == 0) return;
+  xllm_hip_kv_cache cache = make_cache(k_cache, v_cache, k_cache_scale, v_cache_scale);
+  const torch::Tensor s = src.contiguous(), d = dst.contiguous();
+  const size_t bytes = xllm_hip_swap_blocks_staging_bytes(&cache, n);
+  torch::Tensor staging =
+      torch::empty({(int64_t)bytes}, torch::TensorOptions().dtype(torch::kUInt8).device(k_cache.device()));
+  check_status(xllm_hip_swap_blocks(&cache, s.data_ptr<int64_t>(), d.data_ptr<int64_t>(), n, staging.data_ptr(), bytes,
+                                    current_stream(k_cache)));
+}
+
+void copy_blocks(const torch::Tensor& k_cache,
+                 const torch::Tensor& v_cache,
+                 const std::optional<torch::Tensor>& k_cache_scale,
+                 const std::optional<torch::Tensor>& v_cache_scale,
+                 const torch::Tensor& src_block_indices,
+                 const torch::Tensor& dst_block_indices,
+                 const torch::Tensor& cum_sum) {
+  for (const torch::Tensor* t : {&src_block_indices, &dst_block_indices, &cum_sum}) {
+    TORCH_CHECK(t->defined() && t->scalar_type() == torch::kInt && t->is_cuda(),
+                "copy_blocks takes int32 index tensors on the GPU");
+  }
+  TORCH_CHECK(src_block_indices.numel() == cum_sum.numel(), "one cum_sum entry per source block");
+  if (src_block_indices.numel() == 0 || dst_block_indices.numel() == 0) return;
+  xllm_hip_kv_cache cache = make_cache(k_cache, v_cache, k_cache_scale, v_cache_scale);
+  const torch::Tensor s = src_block_indices.contiguous(), d = dst_block_indices.contiguous(), c = cum_sum.contiguous();
+  check_status(xllm_hip_copy_blocks(&cache, s.data_ptr<int32_t>(), d.data_ptr<int32_t>(), c.data_ptr<int32_t>(),
+                                    (int32_t)s.numel(), (int32_t)d.numel(), current_stream(k_cache)));
+}
+
 }  // namespace hip
 }  // namespace xllm::kernel

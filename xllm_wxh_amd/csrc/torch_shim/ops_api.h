@@ -62,6 +62,27 @@ void batch_decode_csr(torch::Tensor query,
                       torch::Tensor output,
                       std::optional<torch::Tensor>& output_lse);
 
+// Whole-block movement inside one layer's cache (K, V and the scale tensors together).
+// swap_blocks: what KVCache::swap_blocks does (xllm/core/framework/kv_cache/kv_cache.cpp:104-125):
+// blocks src[i] -> dst[i], int64 index tensors on the device, all sources read before any
+// destination is written (a staging tensor is allocated for the call, as index_select does).
+void swap_blocks(const torch::Tensor& k_cache,
+                 const torch::Tensor& v_cache,
+                 const std::optional<torch::Tensor>& k_cache_scale,
+                 const std::optional<torch::Tensor>& v_cache_scale,
+                 const torch::Tensor& src,
+                 const torch::Tensor& dst);
+// copy_blocks: the block-copy step on the batch builder's arrays
+// (xllm/core/framework/batch/batch_input_builder.cpp:691-720, xllm/models/llm/npu/llm_model_base.h:69-75):
+// block src_block_indices[g] -> blocks dst_block_indices[cum_sum[g-1] .. cum_sum[g]), int32 tensors.
+void copy_blocks(const torch::Tensor& k_cache,
+                 const torch::Tensor& v_cache,
+                 const std::optional<torch::Tensor>& k_cache_scale,
+                 const std::optional<torch::Tensor>& v_cache_scale,
+                 const torch::Tensor& src_block_indices,
+                 const torch::Tensor& dst_block_indices,
+                 const torch::Tensor& cum_sum);
+
 // Scratch of the decode kernels for this device, grown on demand — the role of the reference's
 // FlashinferWorkspace singleton (xllm/core/layers/cuda/flashinfer_workspace.cpp:24-38).
 torch::Tensor decode_workspace(const torch::Device& device, size_t bytes);

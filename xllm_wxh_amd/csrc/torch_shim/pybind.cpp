@@ -51,7 +51,9 @@ PYBIND11_MODULE(_xllm_hip_torch, m) {
       .def("get_v_cache", &KVCache::get_v_cache)
       .def("get_k_cache_scale", &KVCache::get_k_cache_scale)
       .def("get_v_cache_scale", &KVCache::get_v_cache_scale)
-      .def("empty", &KVCache::empty);
+      .def("empty", &KVCache::empty)
+      .def("swap_blocks", [](KVCache& self, torch::Tensor src, torch::Tensor dst) { self.swap_blocks(src, dst); });
+  m.def("copy_blocks", &xllm::kernel::hip::copy_blocks);
 
   py::class_<AttentionMetadata>(m, "AttentionMetadata")
       .def(py::init<>())

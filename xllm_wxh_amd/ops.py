@@ -329,3 +329,40 @@ def csr_to_block_table(paged_kv_indptr, paged_kv_indices, paged_kv_last_page_len
         _ptr(paged_kv_indptr), _ptr(paged_kv_indices), _ptr(paged_kv_last_page_len), batch, block_size,
         _ptr(table), table.stride(0), max_blocks_per_seq, _ptr(seq_lens), _stream()))
     return table, seq_lens
+
+
+def swap_blocks(k_cache, v_cache, src_tensor, dst_tensor, k_cache_scale=None, v_cache_scale=None, *,
+                kv_layout="HND", exact=True):
+    """KVCache::swap_blocks (xllm/core/framework/kv_cache/kv_cache.cpp:104-125): copy whole blocks
+    src_tensor[i] -> dst_tensor[i] (int64 index tensors on the device) of K, V and the scale tensors.
+    exact=True gathers every source before any destination is written, as index_select followed by
+    index_copy_ does (a staging buffer is allocated for the call); exact=False copies in one pass and
+    needs destinations that are not sources of the same call."""
+    lib = _lib.load()
+    _require(src_tensor.dtype == torch.int64 and dst_tensor.dtype == torch.int64, "block indices must be int64")
+    _require(src_tensor.is_cuda and dst_tensor.is_cuda, "block indices must live on the GPU")
+    _require(src_tensor.numel() == dst_tensor.numel(), "src and dst must name the same number of blocks")
+    src, dst = src_tensor.contiguous(), dst_tensor.contiguous()
+    desc = _cache_desc(k_cache, v_cache, k_cache_scale, v_cache_scale, kv_layout)
+    n = src.numel()
+    staging, nbytes = None, 0
+    if exact and n > 0:
+        nbytes = lib.xllm_hip_swap_blocks_staging_bytes(ctypes.byref(desc), n)
+        staging = torch.empty(nbytes, dtype=torch.uint8, device=k_cache.device)
+    _lib.check(lib.xllm_hip_swap_blocks(ctypes.byref(desc), _ptr(src), _ptr(dst), n,
+                                        _ptr(staging) if staging is not None else None, nbytes, _stream()))
+
+
+def copy_blocks(k_cache, v_cache, src_block_indices, dst_block_indices, cum_sum, k_cache_scale=None,
+                v_cache_scale=None, *, kv_layout="HND"):
+    """The block-copy step of a forward pass (xllm/models/llm/npu/llm_model_base.h:69-75) on the
+    arrays the batch builder emits (xllm/core/framework/batch/batch_input_builder.cpp:691-720):
+    source block src_block_indices[g] goes to destinations dst_block_indices[cum_sum[g-1]:cum_sum[g]]."""
+    lib = _lib.load()
+    for t in (src_block_indices, dst_block_indices, cum_sum):
+        _require(t.dtype == torch.int32 and t.is_cuda, "block-copy index tensors must be int32 on the GPU")
+    _require(src_block_indices.numel() == cum_sum.numel(), "one cum_sum entry per source block")
+    desc = _cache_desc(k_cache, v_cache, k_cache_scale, v_cache_scale, kv_layout)
+    _lib.check(lib.xllm_hip_copy_blocks(ctypes.byref(desc), _ptr(src_block_indices.contiguous()),
+                                        _ptr(dst_block_indices.contiguous()), _ptr(cum_sum.contiguous()),
+                                        src_block_indices.numel(), dst_block_indices.numel(), _stream()))
