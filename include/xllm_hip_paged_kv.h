@@ -263,6 +263,56 @@ int xllm_hip_csr_to_block_table(const int32_t* kv_indptr,
                                 xllm_hip_stream_t stream);
 
 /*
+ * The step in front of the KV write, fused with it: per-head RMSNorm of the query and key heads
+ * (optional), rotary position embedding of both, and the scatter of the new K and V rows into the
+ * paged cache, in one pass over the fused qkv buffer
+ * (call sites: xllm/core/layers/common/qwen2_attention.cpp:147-189 — fused_qk_norm_rope or
+ * q_norm/k_norm + rotary_emb, then AttentionImpl::forward's cache write).
+ *
+ * Norm and rotation follow xllm::kernel::cuda::fused_qk_norm_rope
+ * (xllm/core/kernels/cuda/cuda_ops_api.h:227-241, kernel fused_qknorm_rope.cu:70-262): per head,
+ *   x_d <- x_d * rsqrt(mean_d(x_d^2) + eps) * weight_d        (skipped when q_weight == NULL)
+ *   pairs (j, j + rotary_dim/2) [interleave: (2j, 2j+1)], frequency j, position pos = positions[t]:
+ *   x' = x cos - y sin,  y' = y cos + x sin,   cos = cache[pos][j], sin = cache[pos][rotary_dim/2 + j]
+ * in float with one rounding to the element type at the end; elements beyond rotary_dim pass
+ * through.  round_each_op != 0 rounds to the element type after the norm, after each product and
+ * after the sum instead, which is what xllm::kernel::cuda::rotary_embedding computes on scalar_t
+ * operands (xllm/core/kernels/cuda/rope.cu:26-52, used when the fused kernel is not).
+ * q and k heads are rewritten in place in qkv.  positions outside [0, max_position) are clamped
+ * (the reference would read outside the table).
+ *
+ * With cache != NULL the rotated K heads and the V heads of every token are then written to
+ * slot_mapping[t] exactly as xllm_hip_reshape_paged_cache (cache->dtype == dtype) or
+ * xllm_hip_quant_to_paged_cache (INT8 / FP8_E4M3 cache) would write them from the updated buffer;
+ * num_k_heads and num_v_heads must equal cache->num_kv_heads.  cache == NULL: norm and rotation only.
+ */
+typedef struct xllm_hip_rope_args {
+  void* qkv;            /* [num_tokens, (Hq + Hk + Hv) * head_dim], last dimension contiguous */
+  int64_t token_stride; /* elements between consecutive tokens */
+  int64_t num_tokens;
+  int32_t dtype;        /* BF16 / FP16 / FP32: qkv and the norm weights */
+  int32_t num_q_heads;
+  int32_t num_k_heads;
+  int32_t num_v_heads;
+  int32_t head_dim;     /* <= 512 */
+  int32_t rotary_dim;   /* even, <= head_dim */
+  const void* q_weight; /* [head_dim] or NULL (no norm; then k_weight is NULL too) */
+  const void* k_weight;
+  float eps;
+  int32_t cos_sin_dtype;     /* BF16 / FP16 / FP32 */
+  const void* cos_sin_cache; /* [max_position, rotary_dim] */
+  int64_t max_position;
+  const int64_t* positions;  /* [num_tokens] */
+  int32_t interleave;        /* 0: NeoX pairs (j, j + rotary_dim/2); 1: GPT-J pairs (2j, 2j+1) */
+  int32_t round_each_op;
+} xllm_hip_rope_args;
+
+int xllm_hip_rope_kv_write(const xllm_hip_rope_args* args,
+                           const xllm_hip_kv_cache* cache,
+                           const int32_t* slot_mapping,
+                           xllm_hip_stream_t stream);
+
+/*
  * Batched block swap — KVCache::swap_blocks
  * (xllm/core/framework/kv_cache/kv_cache.cpp:104-125; called per layer from
  * xllm/core/runtime/worker_impl.cpp:584-606 with int64 index tensors): for every pair i the whole

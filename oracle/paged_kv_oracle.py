@@ -27,6 +27,13 @@ tree); how each one is pinned is listed beside it:
       xllm/core/runtime/cuda_graph_executor_test.cpp:150-151.  Absolute FlashInfer/tmo outputs:
       PARITY UNPINNED (tolerance only).
   lse_combine                            xllm/core/kernels/cuda/xattention/lse_combine.cu:61-73
+  fused_qk_norm_rope / rope_pairs        xllm/core/kernels/cuda/fused_qknorm_rope.cu:70-262, rope.cu:26-52
+      pinned by the torch formula the reference's own test checks its kernel against
+      (xllm/core/kernels/cuda/fused_qknorm_rope_test.cpp:28-109, at that test's shapes and tolerances),
+      by torch.nn.functional.rms_norm, by complex multiplication (x + iy) e^{i theta}, and by the
+      identity at cos = 1, sin = 0.  The last bit of the float arithmetic of the CUDA kernels
+      (summation order, fused multiply-adds) is PARITY UNPINNED: outputs are compared within one unit
+      in the last place of the element type; the round-each-operation form without norm is exact.
   swap_blocks                            xllm/core/framework/kv_cache/kv_cache.cpp:104-125
   build_block_copy_groups / copy_blocks  xllm/core/framework/batch/batch_input_builder.cpp:691-720,
       xllm/models/llm/npu/llm_model_base.h:69-75; pinned by brute force on tiny caches (element
@@ -218,6 +225,66 @@ def reshape_paged_cache(slot_ids, keys, values, key_cache, value_cache, layout="
     kc[blk, :, off, :] = keys
     if values is not None:
         _hnd_view(value_cache, layout)[blk, :, off, :] = values
+
+
+# ---- per-head RMSNorm + rotary embedding -------------------------------------------------
+
+
+def round_to_dtype(x, kind):
+    """float64/float32 array -> the nearest value of kind ('bf16' | 'fp16' | 'fp32'), round half to
+    even, returned as float64."""
+    x = np.asarray(x, dtype=np.float64)
+    if kind == "fp32":
+        return x.astype(np.float32).astype(np.float64)
+    if kind == "fp16":
+        return x.astype(np.float16).astype(np.float64)
+    f = x.astype(np.float32)  # double rounding is harmless here: inputs are products of short mantissas
+    u = f.view(np.uint32).astype(np.uint64)
+    u = (u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000
+    return u.astype(np.uint32).view(np.float32).astype(np.float64)
+
+
+def rope_pairs(rotary_dim, interleaved):
+    """Index arrays (x_idx, y_idx) of the rotated pairs, frequency j = position in the arrays:
+    NeoX (j, j + rotary_dim/2), GPT-J (2j, 2j + 1) — xllm/core/kernels/cuda/rope.cu:33-46."""
+    half = rotary_dim // 2
+    j = np.arange(half)
+    return (2 * j, 2 * j + 1) if interleaved else (j, j + half)
+
+
+def fused_qk_norm_rope(qkv, num_heads_q, num_heads_k, num_heads_v, head_dim, eps, q_weight, k_weight,
+                       cos_sin_cache, interleaved, position_ids, kind, round_each_op=False):
+    """Restatement of fused_qknorm_rope_kernel (xllm/core/kernels/cuda/fused_qknorm_rope.cu:70-262): for
+    every q and k head x <- x * rsqrt(mean(x^2) + eps) * weight (skipped when the weights are None),
+    then x' = x cos - y sin, y' = y cos + x sin on the pairs of rope_pairs with cos = cache[pos, j],
+    sin = cache[pos, rotary_dim/2 + j]; elements beyond rotary_dim and the v heads pass through; one
+    rounding to `kind` at the end.  round_each_op=True rounds after the norm, after each product and
+    after the sum instead: arithmetic on scalar_t operands as in rope.cu:49-52.  Computed in float64;
+    qkv is [tokens, (Hq+Hk+Hv)*head_dim] holding values of `kind`.  Returns a new float64 array."""
+    out = np.array(qkv, dtype=np.float64, copy=True)
+    T = out.shape[0]
+    R = cos_sin_cache.shape[1]
+    half = R // 2
+    xi, yi = rope_pairs(R, interleaved)
+    pos = np.asarray(position_ids, dtype=np.int64)
+    cos = np.asarray(cos_sin_cache, dtype=np.float64)[pos][:, :half]
+    sin = np.asarray(cos_sin_cache, dtype=np.float64)[pos][:, half:R]
+    rd = (lambda a: round_to_dtype(a, kind)) if round_each_op else (lambda a: a)
+    if round_each_op:
+        cos, sin = rd(cos), rd(sin)
+    for hh in range(num_heads_q + num_heads_k):
+        w = q_weight if hh < num_heads_q else k_weight
+        x = out[:, hh * head_dim:(hh + 1) * head_dim]
+        if w is not None:
+            rms = 1.0 / np.sqrt((x * x).mean(axis=1, keepdims=True) + eps)
+            x = rd(x * (rms * np.asarray(w, dtype=np.float64)[None, :]))
+        a, b = x[:, xi], x[:, yi]
+        na = rd(rd(a * cos) - rd(b * sin))
+        nb = rd(rd(b * cos) + rd(a * sin))
+        x = x.copy()
+        x[:, xi], x[:, yi] = na, nb
+        out[:, hh * head_dim:(hh + 1) * head_dim] = round_to_dtype(x, kind)
+    return out
 
 
 # ---- whole-block movement ----------------------------------------------------------------

@@ -182,3 +182,62 @@ def test_kv_cache_swap_blocks_and_copy_blocks(gpu, shim):
                      torch.tensor(c, **i32))
     for a, b in zip(got, ref):
         assert np.array_equal(a.cpu().numpy(), b)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("norm", [True, False])
+def test_attention_impl_forward_qkv_equals_separate_steps(gpu, shim, norm):
+    """forward_qkv (norm + rotation + KV write in one launch, then decode) gives bit for bit what the
+    separate operators give: fused_qk_norm_rope / rotary_embedding on the buffer, then forward."""
+    from xllm_wxh_amd import ops
+
+    print("case shim forward_qkv", norm, flush=True)
+    B, Hq, Hkv, D, bs, nblocks = 6, 32, 8, 128, 16, 64
+    lens = np.array([33, 1, 200, 64, 17, 300], np.int32)
+    rng = np.random.default_rng(9)
+    need = (lens + bs - 1) // bs
+    perm = rng.permutation(nblocks - 1) + 1
+    lists, o = [], 0
+    for b in range(B):
+        lists.append(perm[o:o + need[b]].astype(np.int32))
+        o += int(need[b])
+    table = orc.pad_block_tables(lists)
+    slots = np.array([orc.kv_cache_slots(lists[b], bs, int(lens[b]) - 1, int(lens[b]))[0] for b in range(B)], np.int32)
+    g = torch.Generator().manual_seed(6)
+    kc = torch.randn(nblocks, Hkv, bs, D, generator=g).to(torch.bfloat16)
+    vc = torch.randn(nblocks, Hkv, bs, D, generator=g).to(torch.bfloat16)
+    qkv = torch.randn(B, (Hq + 2 * Hkv) * D, generator=g).to(torch.bfloat16)
+    qw = torch.randn(D, generator=g).to(torch.bfloat16).to(gpu) if norm else None
+    kw = torch.randn(D, generator=g).to(torch.bfloat16).to(gpu) if norm else None
+    theta = torch.rand(512, D // 2, generator=g) * 6.283
+    cos_sin = torch.cat([torch.cos(theta), torch.sin(theta)], 1).to(torch.bfloat16).to(gpu)
+    pos = torch.from_numpy(lens.astype(np.int64) - 1).to(gpu)
+    i32 = lambda a: torch.tensor(np.asarray(a), dtype=torch.int32, device=gpu)
+    cu_kv = np.concatenate([[0], np.cumsum(lens)])
+    md = shim.build_decode_metadata(i32(np.arange(B + 1)), i32(cu_kv), i32(slots), i32(table), 1, int(lens.max()),
+                                    int(lens.sum()))
+    attn = shim.AttentionImpl(Hq, D, 1.0 / float(np.sqrt(D)), Hkv, -1)
+
+    a = qkv.to(gpu)
+    cache_a = shim.KVCache(kc.to(gpu), vc.to(gpu))
+    if norm:
+        shim.fused_qk_norm_rope(a, Hq, Hkv, Hkv, D, 1e-6, qw, kw, cos_sin, False, pos)
+    else:
+        shim.rotary_embedding(pos, a[:, : Hq * D], a[:, Hq * D:(Hq + Hkv) * D], cos_sin, True)
+    out_a, _ = attn.forward(md, a[:, : Hq * D], a[:, Hq * D:(Hq + Hkv) * D], a[:, (Hq + Hkv) * D:], cache_a)
+
+    b = qkv.to(gpu)
+    cache_b = shim.KVCache(kc.to(gpu), vc.to(gpu))
+    out_b, _ = attn.forward_qkv(md, pos, b, cos_sin, False, qw, kw, 1e-6, cache_b)
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+    assert torch.equal(cache_a.get_k_cache(), cache_b.get_k_cache())
+    assert torch.equal(cache_a.get_v_cache(), cache_b.get_v_cache())
+    assert torch.equal(out_a, out_b)
+    # and the rotation is the oracle's
+    want = orc.fused_qk_norm_rope(qkv.float().numpy(), Hq, Hkv, Hkv, D, 1e-6,
+                                  qw.float().cpu().numpy() if norm else None,
+                                  kw.float().cpu().numpy() if norm else None, cos_sin.float().cpu().numpy(), False,
+                                  pos.cpu().numpy(), "bf16", round_each_op=not norm)
+    got = b.float().cpu().numpy()
+    assert np.all(np.abs(got - want) <= 2.0 ** -7 * np.abs(want) + 1e-30)

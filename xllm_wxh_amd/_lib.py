@@ -34,6 +34,7 @@ EXPORTED_SYMBOLS = (
     "xllm_hip_paged_decode_run_timed",
     "xllm_hip_paged_decode",
     "xllm_hip_csr_to_block_table",
+    "xllm_hip_rope_kv_write",
     "xllm_hip_swap_blocks_staging_bytes",
     "xllm_hip_swap_blocks",
     "xllm_hip_copy_blocks",
@@ -92,6 +93,31 @@ class DecodeArgs(ctypes.Structure):
     ]
 
 
+class RopeArgs(ctypes.Structure):
+    """struct xllm_hip_rope_args"""
+
+    _fields_ = [
+        ("qkv", ctypes.c_void_p),
+        ("token_stride", ctypes.c_int64),
+        ("num_tokens", ctypes.c_int64),
+        ("dtype", ctypes.c_int32),
+        ("num_q_heads", ctypes.c_int32),
+        ("num_k_heads", ctypes.c_int32),
+        ("num_v_heads", ctypes.c_int32),
+        ("head_dim", ctypes.c_int32),
+        ("rotary_dim", ctypes.c_int32),
+        ("q_weight", ctypes.c_void_p),
+        ("k_weight", ctypes.c_void_p),
+        ("eps", ctypes.c_float),
+        ("cos_sin_dtype", ctypes.c_int32),
+        ("cos_sin_cache", ctypes.c_void_p),
+        ("max_position", ctypes.c_int64),
+        ("positions", ctypes.c_void_p),
+        ("interleave", ctypes.c_int32),
+        ("round_each_op", ctypes.c_int32),
+    ]
+
+
 class XllmHipError(RuntimeError):
     def __init__(self, status, message):
         self.status = status
@@ -132,6 +158,8 @@ def load():
     lib.xllm_hip_paged_decode_run_timed.restype = ctypes.c_int
     lib.xllm_hip_csr_to_block_table.argtypes = [vp, vp, vp, i32, i32, vp, i64, i32, vp, vp]
     lib.xllm_hip_csr_to_block_table.restype = ctypes.c_int
+    lib.xllm_hip_rope_kv_write.argtypes = [P(RopeArgs), P(KvCacheDesc), vp, vp]
+    lib.xllm_hip_rope_kv_write.restype = ctypes.c_int
     lib.xllm_hip_swap_blocks_staging_bytes.argtypes = [P(KvCacheDesc), i64]
     lib.xllm_hip_swap_blocks_staging_bytes.restype = ctypes.c_size_t
     lib.xllm_hip_swap_blocks.argtypes = [P(KvCacheDesc), vp, vp, i64, vp, ctypes.c_size_t, vp]

@@ -48,6 +48,36 @@ std::tuple<torch::Tensor, std::optional<torch::Tensor>> AttentionImpl::forward(
   return {output.view({-1, num_heads_ * head_size_}), output_lse};
 }
 
+std::tuple<torch::Tensor, std::optional<torch::Tensor>> AttentionImpl::forward_qkv(
+    const AttentionMetadata& attn_metadata, const torch::Tensor& positions, torch::Tensor& qkv,
+    const torch::Tensor& cos_sin_cache, bool interleaved, const std::optional<torch::Tensor>& q_norm_weight,
+    const std::optional<torch::Tensor>& k_norm_weight, double eps, KVCache& kv_cache) {
+  std::optional<torch::Tensor> output_lse = std::nullopt;
+  const int64_t q_size = num_heads_ * head_size_;
+  torch::Tensor output = torch::empty({qkv.size(0), q_size}, qkv.options());
+  if (attn_metadata.is_dummy || attn_metadata.max_seq_len == 0) {
+    return {output, output_lse};
+  }
+  TORCH_CHECK(!attn_metadata.is_prefill && !attn_metadata.is_chunked_prefill,
+              "the HIP backend implements the decode path only (prefill is served elsewhere)");
+  TORCH_CHECK(qkv.dim() == 2 && qkv.size(1) == (num_heads_ + 2 * num_kv_heads_) * head_size_,
+              "qkv must be [tokens, (num_heads + 2 * num_kv_heads) * head_size]");
+  torch::Tensor k_cache = kv_cache.get_k_cache();
+  torch::Tensor v_cache = kv_cache.get_v_cache();
+  std::optional<torch::Tensor> k_cache_scale = kv_cache.get_k_cache_scale();
+  std::optional<torch::Tensor> v_cache_scale = kv_cache.get_v_cache_scale();
+  // the fused CUDA kernel serves 1-D positions with the norm weights; without them the reference
+  // rotates with rope.cu, whose arithmetic rounds every operation
+  const bool with_norm = q_norm_weight.has_value() && q_norm_weight->defined();
+  torch::Tensor pos = positions.to(torch::kLong).contiguous();
+  xllm::kernel::hip::rope_kv_write(qkv, num_heads_, num_kv_heads_, head_size_, q_norm_weight, k_norm_weight, eps,
+                                   cos_sin_cache, interleaved, /*round_each_op=*/!with_norm, pos, k_cache, v_cache,
+                                   k_cache_scale, v_cache_scale, attn_metadata.slot_mapping);
+  torch::Tensor query = qkv.slice(/*dim=*/-1, 0, q_size);
+  decoder_forward(attn_metadata, query, output, k_cache, v_cache, k_cache_scale, v_cache_scale);
+  return {output, output_lse};
+}
+
 void AttentionImpl::decoder_forward(const AttentionMetadata& attn_metadata, torch::Tensor& query,
                                     torch::Tensor& output, const torch::Tensor& k_cache,
                                     const torch::Tensor& v_cache, const std::optional<torch::Tensor>& k_cache_scale,

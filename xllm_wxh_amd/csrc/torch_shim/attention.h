@@ -25,6 +25,21 @@ class AttentionImpl {
                                                                    torch::Tensor& value,
                                                                    KVCache& kv_cache);
 
+  // The same step fed from the fused qkv buffer before norm and rotation — what
+  // Qwen2AttentionImpl::forward does between the qkv projection and the output projection
+  // (xllm/core/layers/common/qwen2_attention.cpp:147-189): one launch for q/k norm (when the weights
+  // are given), rotary embedding and the KV write, then the decode.  qkv [T, (Hq + 2 Hkv) * D] is
+  // updated in place; returns (output [T, Hq*D], lse = nullopt).
+  std::tuple<torch::Tensor, std::optional<torch::Tensor>> forward_qkv(const AttentionMetadata& attn_metadata,
+                                                                       const torch::Tensor& positions,
+                                                                       torch::Tensor& qkv,
+                                                                       const torch::Tensor& cos_sin_cache,
+                                                                       bool interleaved,
+                                                                       const std::optional<torch::Tensor>& q_norm_weight,
+                                                                       const std::optional<torch::Tensor>& k_norm_weight,
+                                                                       double eps,
+                                                                       KVCache& kv_cache);
+
  private:
   void decoder_forward(const AttentionMetadata& attn_metadata,
                        torch::Tensor& query,

@@ -256,6 +256,88 @@ void batch_decode_csr(torch::Tensor query,
   run_decode(cache, a, query);
 }
 
+namespace {
+
+void rope_call(torch::Tensor& qkv, int64_t hq, int64_t hk, int64_t hv, int64_t head_dim, double eps,
+               const std::optional<torch::Tensor>& q_weight, const std::optional<torch::Tensor>& k_weight,
+               const torch::Tensor& cos_sin_cache, bool interleaved, bool round_each_op,
+               const torch::Tensor& position_ids, const xllm_hip_kv_cache* cache, const torch::Tensor* slot_mapping) {
+  TORCH_CHECK(qkv.is_cuda() && qkv.dim() == 2 && qkv.stride(1) == 1, "qkv must be a 2-D GPU tensor, rows contiguous");
+  TORCH_CHECK(position_ids.scalar_type() == torch::kLong && position_ids.dim() == 1 && position_ids.is_contiguous() &&
+                  position_ids.numel() == qkv.size(0),
+              "position_ids must be contiguous int64 [num_tokens]");
+  TORCH_CHECK(cos_sin_cache.dim() == 2 && cos_sin_cache.is_contiguous(),
+              "cos_sin_cache must be contiguous [max_position, rotary_dim]");
+  xllm_hip_rope_args a{};
+  a.qkv = qkv.data_ptr();
+  a.token_stride = qkv.stride(0);
+  a.num_tokens = qkv.size(0);
+  a.dtype = dtype_code(qkv);
+  a.num_q_heads = (int32_t)hq;
+  a.num_k_heads = (int32_t)hk;
+  a.num_v_heads = (int32_t)hv;
+  a.head_dim = (int32_t)head_dim;
+  a.rotary_dim = (int32_t)cos_sin_cache.size(1);
+  if (q_weight.has_value() && q_weight->defined()) {
+    TORCH_CHECK(k_weight.has_value() && k_weight->defined(), "q_weight and k_weight go together");
+    for (const torch::Tensor* w : {&*q_weight, &*k_weight}) {
+      TORCH_CHECK(w->scalar_type() == qkv.scalar_type() && w->dim() == 1 && w->numel() == head_dim &&
+                      w->is_contiguous(),
+                  "norm weights must be [head_dim] of qkv's dtype");
+    }
+    a.q_weight = q_weight->data_ptr();
+    a.k_weight = k_weight->data_ptr();
+  }
+  a.eps = (float)eps;
+  a.cos_sin_dtype = dtype_code(cos_sin_cache);
+  a.cos_sin_cache = cos_sin_cache.data_ptr();
+  a.max_position = cos_sin_cache.size(0);
+  a.positions = position_ids.data_ptr<int64_t>();
+  a.interleave = interleaved ? 1 : 0;
+  a.round_each_op = round_each_op ? 1 : 0;
+  const int32_t* slots = nullptr;
+  if (cache != nullptr) {
+    TORCH_CHECK(slot_mapping->scalar_type() == torch::kInt && slot_mapping->is_contiguous() &&
+                    slot_mapping->numel() == qkv.size(0),
+                "slot_mapping must be contiguous int32 [num_tokens]");
+    slots = slot_mapping->data_ptr<int32_t>();
+  }
+  check_status(xllm_hip_rope_kv_write(&a, cache, slots, current_stream(qkv)));
+}
+
+}  // namespace
+
+void fused_qk_norm_rope(torch::Tensor& qkv, int64_t num_heads_q, int64_t num_heads_k, int64_t num_heads_v,
+                        int64_t head_dim, double eps, const torch::Tensor& q_weight, const torch::Tensor& k_weight,
+                        const torch::Tensor& cos_sin_cache, bool interleaved, const torch::Tensor& position_ids) {
+  rope_call(qkv, num_heads_q, num_heads_k, num_heads_v, head_dim, eps, q_weight, k_weight, cos_sin_cache, interleaved,
+            false, position_ids, nullptr, nullptr);
+}
+
+void rotary_embedding(torch::Tensor& positions, torch::Tensor& query, std::optional<torch::Tensor> key,
+                      torch::Tensor& cos_sin_cache, bool is_neox) {
+  const int64_t head_size = cos_sin_cache.size(-1);  // as the reference derives it (rope.cu:169)
+  auto one = [&](torch::Tensor t) {
+    torch::Tensor flat = t.dim() == 3 ? t.view({t.size(0), -1}) : t;
+    TORCH_CHECK(flat.size(1) % head_size == 0, "hidden size is not a multiple of head_size");
+    rope_call(flat, flat.size(1) / head_size, 0, 0, head_size, 0.0, std::nullopt, std::nullopt, cos_sin_cache,
+              !is_neox, true, positions, nullptr, nullptr);
+  };
+  one(query);
+  if (key.has_value() && key->defined()) one(*key);
+}
+
+void rope_kv_write(torch::Tensor& qkv, int64_t num_heads_q, int64_t num_heads_kv, int64_t head_dim,
+                   const std::optional<torch::Tensor>& q_weight, const std::optional<torch::Tensor>& k_weight, double eps,
+                   const torch::Tensor& cos_sin_cache, bool interleaved, bool round_each_op,
+                   const torch::Tensor& position_ids, const torch::Tensor& k_cache, const torch::Tensor& v_cache,
+                   const std::optional<torch::Tensor>& k_cache_scale, const std::optional<torch::Tensor>& v_cache_scale,
+                   const torch::Tensor& slot_mapping) {
+  xllm_hip_kv_cache cache = make_cache(k_cache, v_cache, k_cache_scale, v_cache_scale);
+  rope_call(qkv, num_heads_q, num_heads_kv, num_heads_kv, head_dim, eps, q_weight, k_weight, cos_sin_cache, interleaved,
+            round_each_op, position_ids, &cache, &slot_mapping);
+}
+
 void swap_blocks(const torch::Tensor& k_cache,
                  const torch::Tensor& v_cache,
                  const std::optional<torch::Tensor>& k_cache_scale,

@@ -62,6 +62,49 @@ void batch_decode_csr(torch::Tensor query,
                       torch::Tensor output,
                       std::optional<torch::Tensor>& output_lse);
 
+// xllm::kernel::cuda::fused_qk_norm_rope (xllm/core/kernels/cuda/cuda_ops_api.h:227-241): per-head RMSNorm
+// and rotary embedding of the q and k heads of the fused buffer, in place.
+void fused_qk_norm_rope(torch::Tensor& qkv,
+                        int64_t num_heads_q,
+                        int64_t num_heads_k,
+                        int64_t num_heads_v,
+                        int64_t head_dim,
+                        double eps,
+                        const torch::Tensor& q_weight,
+                        const torch::Tensor& k_weight,
+                        const torch::Tensor& cos_sin_cache,
+                        bool interleaved,
+                        const torch::Tensor& position_ids);
+
+// xllm::kernel::cuda::rotary_embedding (xllm/core/kernels/cuda/rope.cu:152-249): rotation of query
+// [tokens, heads * head_size] and, if given, key, in place, every operation rounded to the element type.
+void rotary_embedding(torch::Tensor& positions,
+                      torch::Tensor& query,
+                      std::optional<torch::Tensor> key,
+                      torch::Tensor& cos_sin_cache,
+                      bool is_neox);
+
+// Steps 2-5 of Qwen2AttentionImpl::forward up to the attention call
+// (xllm/core/layers/common/qwen2_attention.cpp:147-189) in one launch: norm (when the weights are
+// given) and rotation of q and k in place in qkv, then the KV write of the rotated k and of v through
+// slot_mapping — quantising iff the scale tensors are given.
+void rope_kv_write(torch::Tensor& qkv,
+                   int64_t num_heads_q,
+                   int64_t num_heads_kv,
+                   int64_t head_dim,
+                   const std::optional<torch::Tensor>& q_weight,
+                   const std::optional<torch::Tensor>& k_weight,
+                   double eps,
+                   const torch::Tensor& cos_sin_cache,
+                   bool interleaved,
+                   bool round_each_op,
+                   const torch::Tensor& position_ids,
+                   const torch::Tensor& k_cache,
+                   const torch::Tensor& v_cache,
+                   const std::optional<torch::Tensor>& k_cache_scale,
+                   const std::optional<torch::Tensor>& v_cache_scale,
+                   const torch::Tensor& slot_mapping);
+
 // Whole-block movement inside one layer's cache (K, V and the scale tensors together).
 // swap_blocks: what KVCache::swap_blocks does (xllm/core/framework/kv_cache/kv_cache.cpp:104-125):
 // blocks src[i] -> dst[i], int64 index tensors on the device, all sources read before any

@@ -75,5 +75,21 @@ PYBIND11_MODULE(_xllm_hip_torch, m) {
   py::class_<AttentionImpl>(m, "AttentionImpl")
       .def(py::init<int64_t, int64_t, float, int64_t, int64_t>())
       .def("forward", [](AttentionImpl& self, const AttentionMetadata& md, torch::Tensor query, torch::Tensor key,
-                         torch::Tensor value, KVCache& kv) { return self.forward(md, query, key, value, kv); });
+                         torch::Tensor value, KVCache& kv) { return self.forward(md, query, key, value, kv); })
+      .def("forward_qkv", [](AttentionImpl& self, const AttentionMetadata& md, torch::Tensor positions,
+                             torch::Tensor qkv, torch::Tensor cos_sin_cache, bool interleaved,
+                             std::optional<torch::Tensor> q_norm_weight, std::optional<torch::Tensor> k_norm_weight,
+                             double eps, KVCache& kv) {
+        return self.forward_qkv(md, positions, qkv, cos_sin_cache, interleaved, q_norm_weight, k_norm_weight, eps, kv);
+      });
+  m.def("fused_qk_norm_rope", [](torch::Tensor qkv, int64_t hq, int64_t hk, int64_t hv, int64_t head_dim, double eps,
+                                 torch::Tensor q_weight, torch::Tensor k_weight, torch::Tensor cos_sin_cache,
+                                 bool interleaved, torch::Tensor position_ids) {
+    xllm::kernel::hip::fused_qk_norm_rope(qkv, hq, hk, hv, head_dim, eps, q_weight, k_weight, cos_sin_cache, interleaved,
+                                          position_ids);
+  });
+  m.def("rotary_embedding", [](torch::Tensor positions, torch::Tensor query, std::optional<torch::Tensor> key,
+                               torch::Tensor cos_sin_cache, bool is_neox) {
+    xllm::kernel::hip::rotary_embedding(positions, query, key, cos_sin_cache, is_neox);
+  });
 }

@@ -366,3 +366,65 @@ def copy_blocks(k_cache, v_cache, src_block_indices, dst_block_indices, cum_sum,
     _lib.check(lib.xllm_hip_copy_blocks(ctypes.byref(desc), _ptr(src_block_indices.contiguous()),
                                         _ptr(dst_block_indices.contiguous()), _ptr(cum_sum.contiguous()),
                                         src_block_indices.numel(), dst_block_indices.numel(), _stream()))
+
+
+def _rope_call(qkv, num_q, num_k, num_v, head_dim, eps, q_weight, k_weight, cos_sin_cache, interleaved, positions,
+               round_each_op, cache_desc=None, slot_mapping=None):
+    lib = _lib.load()
+    _require(qkv.is_cuda and qkv.dim() == 2 and qkv.stride(1) == 1, "qkv must be a 2-D GPU tensor, rows contiguous")
+    _require(positions.dtype == torch.int64 and positions.dim() == 1 and positions.is_contiguous(),
+             "position_ids must be a contiguous 1-D int64 tensor")
+    _require(positions.numel() == qkv.size(0), "one position per token")
+    _require(cos_sin_cache.dim() == 2 and cos_sin_cache.is_contiguous(), "cos_sin_cache must be [max_position, rotary_dim]")
+    a = _lib.RopeArgs()
+    a.qkv, a.token_stride, a.num_tokens = qkv.data_ptr(), qkv.stride(0), qkv.size(0)
+    a.dtype = _dtype_code(qkv)
+    a.num_q_heads, a.num_k_heads, a.num_v_heads, a.head_dim = num_q, num_k, num_v, head_dim
+    a.rotary_dim = cos_sin_cache.size(1)
+    if q_weight is not None:
+        for w in (q_weight, k_weight):
+            _require(w.dtype == qkv.dtype and w.dim() == 1 and w.numel() == head_dim and w.is_contiguous(),
+                     "norm weights must be [head_dim] of qkv's dtype")
+        a.q_weight, a.k_weight = q_weight.data_ptr(), k_weight.data_ptr()
+    a.eps = eps
+    a.cos_sin_dtype, a.cos_sin_cache, a.max_position = _dtype_code(cos_sin_cache), cos_sin_cache.data_ptr(), \
+        cos_sin_cache.size(0)
+    a.positions = positions.data_ptr()
+    a.interleave, a.round_each_op = int(bool(interleaved)), int(bool(round_each_op))
+    _lib.check(lib.xllm_hip_rope_kv_write(ctypes.byref(a), ctypes.byref(cache_desc) if cache_desc is not None else None,
+                                          _ptr(slot_mapping), _stream()))
+
+
+def fused_qk_norm_rope(qkv, num_heads_q, num_heads_k, num_heads_v, head_dim, eps, q_weight, k_weight, cos_sin_cache,
+                       interleaved, position_ids):
+    """xllm::kernel::cuda::fused_qk_norm_rope (xllm/core/kernels/cuda/cuda_ops_api.h:227-241): per-head
+    RMSNorm + rotary embedding of the q and k heads of the fused buffer, in place."""
+    _rope_call(qkv, num_heads_q, num_heads_k, num_heads_v, head_dim, eps, q_weight, k_weight, cos_sin_cache,
+               interleaved, position_ids, False)
+
+
+def rotary_embedding(positions, query, key, cos_sin_cache, is_neox):
+    """xllm::kernel::cuda::rotary_embedding (xllm/core/kernels/cuda/rope.cu:152-249): rotation of query
+    [tokens, heads * head_size] and, if given, key, in place, every operation rounded to the element
+    type.  head_size is the last dimension of cos_sin_cache... as in the reference (rope.cu:169)."""
+    head_size = cos_sin_cache.size(-1)
+    for t in (query, key):
+        if t is None:
+            continue
+        flat = t.view(t.size(0), -1) if t.dim() == 3 else t
+        _require(flat.size(1) % head_size == 0, "hidden size is not a multiple of head_size")
+        heads = flat.size(1) // head_size
+        _rope_call(flat, heads, 0, 0, head_size, 0.0, None, None, cos_sin_cache, not is_neox, positions, True)
+
+
+def rope_kv_write(qkv, num_heads_q, num_heads_kv, head_dim, cos_sin_cache, position_ids, k_cache, v_cache,
+                  slot_mapping, *, q_weight=None, k_weight=None, eps=1e-6, interleaved=False, round_each_op=False,
+                  k_cache_scale=None, v_cache_scale=None, kv_layout="HND"):
+    """Norm (optional) + rotary embedding of q and k in place, then the KV write of the rotated k and of
+    v through slot_mapping (quantising iff scales are given) — one launch for the steps 2-5 of
+    Qwen2AttentionImpl::forward up to the attention call (xllm/core/layers/common/qwen2_attention.cpp:147-189)."""
+    desc = _cache_desc(k_cache, v_cache, k_cache_scale, v_cache_scale, kv_layout)
+    _require(slot_mapping.dtype == torch.int32 and slot_mapping.is_contiguous() and
+             slot_mapping.numel() == qkv.size(0), "slot_mapping must be contiguous int32, one entry per token")
+    _rope_call(qkv, num_heads_q, num_heads_kv, num_heads_kv, head_dim, eps, q_weight, k_weight, cos_sin_cache,
+               interleaved, position_ids, round_each_op, desc, slot_mapping)
