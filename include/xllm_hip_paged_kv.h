@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define XLLM_HIP_ABI_VERSION 1
+#define XLLM_HIP_ABI_VERSION 2
 
 /* A hipStream_t, passed as an opaque pointer so that C callers need no HIP headers. */
 typedef void* xllm_hip_stream_t;
@@ -144,6 +144,14 @@ int xllm_hip_quant_to_paged_cache(const xllm_hip_kv_cache* cache,
  * the cache) and token j sees seq_lens[b] - (n-1-j) keys, which is what the
  * reference expresses by expanding every draft token into its own decode row
  * with its own kv length (xllm/core/runtime/speculative_worker_impl.cpp:230-243).
+ * With q_indptr != NULL the sequences carry different numbers of query tokens — a chunked-prefill or
+ * mixed step (xllm/core/layers/cuda/flashinfer_attention.cpp:224-284, q_cu_seq_lens / qo_indptr of
+ * xllm/core/layers/common/attention_metadata.h): the tokens of sequence b are rows
+ * q_indptr[b] .. q_indptr[b+1] of q/out, n_b = q_indptr[b+1] - q_indptr[b] of them, again the LAST
+ * n_b tokens of the sequence, token j seeing seq_lens[b] - (n_b-1-j) keys (causal, aligned to the end
+ * of the kv range).  q_per_seq must then be at least max_b n_b (the reference's max_query_len); it
+ * sizes the launch and the workspace, and tokens beyond it are ignored.  Above 128 query rows per kv
+ * head (q_per_seq * num_q_heads / num_kv_heads) sequences are never split into chunks.
  *
  * The block list of sequence b is given in one of two forms:
  *   block_table form (mlu_ops_api.h:130-131): block_table != NULL, row b starts at
@@ -189,6 +197,9 @@ typedef struct xllm_hip_decode_args {
    * >= every kv length; total_kv_len (0 = unknown) only tunes the split. */
   int32_t max_seq_len;
   int64_t total_kv_len;
+  /* Query token offsets [batch+1] for sequences with different numbers of query tokens; NULL: every
+   * sequence has q_per_seq of them. */
+  const int32_t* q_indptr;
 } xllm_hip_decode_args;
 
 /*

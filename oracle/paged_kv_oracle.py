@@ -26,6 +26,8 @@ tree); how each one is pinned is listed beside it:
       agreement with scipy/torch softmax, split-merge identity) and by the reference's invariant
       xllm/core/runtime/cuda_graph_executor_test.cpp:150-151.  Absolute FlashInfer/tmo outputs:
       PARITY UNPINNED (tolerance only).
+  paged_decode_ragged                    per-sequence query counts (chunked prefill, flashinfer_attention.cpp:224-284):
+      one paged_decode call per sequence, so it inherits those pins.
   lse_combine                            xllm/core/kernels/cuda/xattention/lse_combine.cu:61-73
   fused_qk_norm_rope / rope_pairs        xllm/core/kernels/cuda/fused_qknorm_rope.cu:70-262, rope.cu:26-52
       pinned by the torch formula the reference's own test checks its kernel against
@@ -530,6 +532,23 @@ def paged_decode(q, k_cache, v_cache, block_table, seq_lens, scale, q_per_seq=1,
         o = np.einsum("jkgt,ktd->jkgd", p, V)
         out[b * n:(b + 1) * n] = o.reshape(n, Hq, D)
         lse2[b * n:(b + 1) * n] = l2.reshape(n, Hq)
+    return out, lse2
+
+
+def paged_decode_ragged(q, k_cache, v_cache, block_table, seq_lens, q_indptr, scale, **kw):
+    """Sequences with different numbers of query tokens (a chunked-prefill or mixed step,
+    xllm/core/layers/cuda/flashinfer_attention.cpp:224-284 with the causal mask): sequence b owns rows
+    q_indptr[b]:q_indptr[b+1] of q, the last n_b tokens of its kv range, token j seeing
+    seq_lens[b] - (n_b - 1 - j) keys.  One paged_decode call per sequence."""
+    q = np.asarray(q)
+    out = np.zeros(q.shape, np.float64)
+    lse2 = np.full(q.shape[:2], -np.inf, np.float64)
+    for b in range(len(q_indptr) - 1):
+        q0, q1 = int(q_indptr[b]), int(q_indptr[b + 1])
+        if q1 <= q0:
+            continue
+        o, l = paged_decode(q[q0:q1], k_cache, v_cache, [block_table[b]], [seq_lens[b]], scale, q_per_seq=q1 - q0, **kw)
+        out[q0:q1], lse2[q0:q1] = o, l
     return out, lse2
 
 

@@ -49,7 +49,11 @@ def test_struct_sizes_match_the_header_layout():
     assert _lib.DecodeArgs.q_dtype.offset == 40
     assert _lib.DecodeArgs.block_table.offset == 64
     assert _lib.DecodeArgs.max_seq_len.offset == 120
-    assert ctypes.sizeof(_lib.DecodeArgs) == 136
+    assert _lib.DecodeArgs.q_indptr.offset == 136
+    assert ctypes.sizeof(_lib.DecodeArgs) == 144
+    # xllm_hip_rope_args: ptr, 2 i64, 6 i32, 2 ptr, f32 + i32, ptr, i64, ptr, 2 i32
+    assert _lib.RopeArgs.q_weight.offset == 48 and _lib.RopeArgs.cos_sin_cache.offset == 72
+    assert ctypes.sizeof(_lib.RopeArgs) == 104
 
 
 def test_workspace_bytes_is_a_pure_size_function(lib):

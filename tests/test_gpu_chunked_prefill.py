@@ -1,0 +1,85 @@
+"""Sequences with different numbers of query tokens (chunked prefill / mixed steps) over the paged
+cache, through the C ABI, against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import paged_kv_oracle as orc
+from tests.helpers import Case
+from xllm_wxh_amd import ops
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(c, q_counts, max_q, **kw):
+    q_indptr = np.concatenate([[0], np.cumsum(q_counts)]).astype(np.int32)
+    T = int(q_indptr[-1])
+    g = torch.Generator().manual_seed(77)
+    q = torch.randn(T, c.Hq, c.D, generator=g).to(torch.bfloat16 if c.qdt == "bf16" else torch.float32)
+    qd = q.to(c.q.device)
+    out = torch.full_like(qd, 7.0)
+    lse = torch.full((T, c.Hq), 3.0, dtype=torch.float32, device=qd.device)
+    ops.batch_decode(qd, c.k_cache, out, c.block_table, c.seq_lens, c.v_cache, lse, None, c.k_scale, c.v_scale,
+                     scale=c.scale, return_lse=True, kv_cache_quant_bit_size=8 if c.k_scale is not None else -1,
+                     q_per_seq=max_q, q_indptr=torch.from_numpy(q_indptr).to(qd.device), **kw)
+    torch.cuda.synchronize()
+    ref, ref_lse = orc.paged_decode_ragged(q.float().numpy(), c.k_ref, c.v_ref, c.table, c.lens, q_indptr, c.scale,
+                                           window_left=kw.get("window_size_left", -1))
+    return out.float().cpu().numpy(), lse.cpu().numpy(), ref, ref_lse, q_indptr
+
+
+@pytest.mark.parametrize("kv", ["bf16", "fp8", "int8"])
+@pytest.mark.parametrize("Hq,Hkv", [(32, 8), (64, 8), (8, 8)])
+def test_mixed_step_matches_oracle(gpu, kv, Hq, Hkv):
+    """A mixed step: decode sequences (1 token), speculative verify (4) and prefill chunks (up to 70
+    tokens, some reaching back to the start of the sequence) in one call."""
+    print("case mixed step", kv, Hq, Hkv, flush=True)
+    lens = [300, 70, 33, 1, 129, 4096, 64, 40]
+    q_counts = [1, 70, 4, 1, 17, 64, 0, 40]   # 70 == len and 40 == len: the whole sequence is the chunk
+    c = Case(len(lens), Hq, Hkv, 128, 16, lens, kv=kv, seed=21)
+    out, lse, ref, ref_lse, q_indptr = _run(c, q_counts, max(q_counts))
+    err = float(np.abs(out - ref).max())
+    print("   err %.3e" % err, flush=True)
+    assert err <= c.tol
+    fin = np.isfinite(ref_lse)
+    assert np.allclose(lse[fin], ref_lse[fin], atol=2e-2 if kv == "bf16" else 5e-2)
+
+
+def test_chunk_equals_expanded_decode_rows(gpu):
+    """The reference's equivalence (xllm/core/runtime/speculative_worker_impl.cpp:230-243): a chunk of n
+    tokens gives what n separate decode rows with kv lengths L-n+1 .. L over the same blocks give."""
+    print("case chunk vs expanded rows", flush=True)
+    L, n, Hq, Hkv = 777, 48, 32, 8
+    c = Case(1, Hq, Hkv, 128, 16, [L], seed=5)
+    out, lse, ref, _, _ = _run(c, [n], n)
+    qd = torch.randn(n, Hq, 128, generator=torch.Generator().manual_seed(77)).to(torch.bfloat16).to(c.q.device)
+    rows = torch.empty_like(qd)
+    table = c.block_table.expand(n, -1).contiguous()
+    lens = torch.arange(L - n + 1, L + 1, dtype=torch.int32, device=qd.device)
+    ops.batch_decode(qd, c.k_cache, rows, table, lens, c.v_cache, scale=c.scale)
+    torch.cuda.synchronize()
+    assert float(np.abs(rows.float().cpu().numpy() - out).max()) <= 1.2e-2
+    assert float(np.abs(out - ref).max()) <= c.tol
+
+
+def test_prefill_sized_chunks_and_edge_cases(gpu):
+    print("case prefill chunks", flush=True)
+    # 512-token chunks at g = 4: 2048 rows per kv head = 64 row groups, never split
+    lens = [2048, 512, 700]
+    q_counts = [512, 512, 188]
+    c = Case(3, 32, 8, 128, 128, lens, seed=9)
+    out, lse, ref, ref_lse, q_indptr = _run(c, q_counts, 512)
+    assert float(np.abs(out - ref).max()) <= c.tol
+    # counts above q_per_seq are cut to it (documented); rows of other sequences are unaffected
+    c2 = Case(2, 32, 8, 128, 16, [100, 90], seed=10)
+    out2, _, ref2, _, ind2 = _run(c2, [8, 3], 4)
+    assert float(np.abs(out2[ind2[1]:] - ref2[ind2[1]:]).max()) <= c2.tol
+    assert np.all(out2[4:8] == 7.0)  # tokens 4..7 of sequence 0 were ignored
+    # sliding window together with a chunk
+    c3 = Case(2, 32, 8, 128, 16, [500, 64], seed=11)
+    out3, _, ref3, _, _ = _run(c3, [33, 64], 64, window_size_left=100)
+    assert float(np.abs(out3 - ref3).max()) <= c3.tol
+    # the generic kernel (fp32, head_dim 64) takes the same arguments
+    c4 = Case(3, 14, 2, 64, 16, [50, 333, 20], kv="fp32", qdt="fp32", seed=12)
+    out4, _, ref4, _, _ = _run(c4, [5, 40, 20], 40)
+    assert float(np.abs(out4 - ref4).max()) <= 1e-4

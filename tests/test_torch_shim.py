@@ -128,9 +128,6 @@ def test_attention_impl_write_then_attend(gpu, shim, kv):
     out2, _ = attn.forward(md, qkv_d[:, : Hq * D], qkv_d[:, Hq * D:(Hq + Hkv) * D], qkv_d[:, (Hq + Hkv) * D:], cache)
     assert tuple(out2.shape) == (B, Hq * D)
     md.is_dummy = False
-    md.is_prefill = True
-    with pytest.raises(RuntimeError, match="decode path only"):
-        attn.forward(md, qkv_d[:, : Hq * D], qkv_d[:, Hq * D:(Hq + Hkv) * D], qkv_d[:, (Hq + Hkv) * D:], cache)
 
 
 @pytest.mark.gpu
@@ -241,3 +238,58 @@ def test_attention_impl_forward_qkv_equals_separate_steps(gpu, shim, norm):
                                   pos.cpu().numpy(), "bf16", round_each_op=not norm)
     got = b.float().cpu().numpy()
     assert np.all(np.abs(got - want) <= 2.0 ** -7 * np.abs(want) + 1e-30)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kv", ["bf16", "int8"])
+def test_attention_impl_chunked_prefill_step(gpu, shim, kv):
+    """A mixed step through AttentionImpl::forward: prefill chunks of different sizes and decode tokens,
+    the new K/V written through slot_mapping first, then attended from the (quantised) cache."""
+    print("case shim chunked prefill", kv, flush=True)
+    Hq, Hkv, D, bs = 32, 8, 128, 16
+    lens = np.array([200, 48, 1000, 7], np.int32)      # kv lengths including this step's tokens
+    q_counts = np.array([40, 48, 1, 7], np.int32)
+    B, T = len(lens), int(q_counts.sum())
+    rng = np.random.default_rng(13)
+    need = (lens + bs - 1) // bs
+    nblocks = int(need.sum()) + 2
+    perm = rng.permutation(nblocks - 1) + 1
+    lists, o = [], 0
+    for b in range(B):
+        lists.append(perm[o:o + need[b]].astype(np.int32))
+        o += int(need[b])
+    table = orc.pad_block_tables(lists)
+    slots = np.concatenate([orc.kv_cache_slots(lists[b], bs, int(lens[b] - q_counts[b]), int(lens[b]))
+                            for b in range(B)]).astype(np.int32)
+    g = torch.Generator().manual_seed(8)
+    kf = torch.randn(nblocks, Hkv, bs, D, generator=g)
+    vf = torch.randn(nblocks, Hkv, bs, D, generator=g)
+    qkv = torch.randn(T, (Hq + 2 * Hkv) * D, generator=g).to(torch.bfloat16)
+    q, k, v = qkv[:, : Hq * D], qkv[:, Hq * D:(Hq + Hkv) * D], qkv[:, (Hq + Hkv) * D:]
+    k_new, v_new = k.float().numpy().reshape(T, Hkv, D), v.float().numpy().reshape(T, Hkv, D)
+    if kv == "bf16":
+        kc, vc = kf.to(torch.bfloat16), vf.to(torch.bfloat16)
+        k_ref, v_ref = kc.float().numpy(), vc.float().numpy()
+        orc.reshape_paged_cache(slots, k_new, v_new, k_ref, v_ref, "HND")
+        cache = shim.KVCache(kc.to(gpu), vc.to(gpu))
+    else:
+        qk, sk = orc.quantize_per_token_head(kf.numpy(), "int8")
+        qv, sv = orc.quantize_per_token_head(vf.numpy(), "int8")
+        cache = shim.KVCache(torch.from_numpy(qk.copy()).to(gpu), torch.from_numpy(qv.copy()).to(gpu),
+                             torch.from_numpy(sk.copy()).to(gpu), torch.from_numpy(sv.copy()).to(gpu))
+        orc.quant_to_paged_cache(slots, k_new, v_new, qk, qv, sk, sv, "int8", "HND")
+        k_ref, v_ref = orc.dequantize(qk, sk, "int8"), orc.dequantize(qv, sv, "int8")
+    q_indptr = np.concatenate([[0], np.cumsum(q_counts)]).astype(np.int32)
+    scale = 1.0 / float(np.sqrt(D))
+    ref, _ = orc.paged_decode_ragged(q.float().numpy().reshape(T, Hq, D), k_ref, v_ref, table, lens, q_indptr, scale)
+    i32 = lambda a: torch.tensor(np.asarray(a), dtype=torch.int32, device=gpu)
+    md = shim.build_decode_metadata(i32(q_indptr), i32(np.concatenate([[0], np.cumsum(lens)])), i32(slots), i32(table),
+                                    int(q_counts.max()), int(lens.max()), int(lens.sum()))
+    md.is_chunked_prefill = True
+    attn = shim.AttentionImpl(Hq, D, scale, Hkv, -1)
+    qkv_d = qkv.to(gpu)
+    out, _ = attn.forward(md, qkv_d[:, : Hq * D], qkv_d[:, Hq * D:(Hq + Hkv) * D], qkv_d[:, (Hq + Hkv) * D:], cache)
+    torch.cuda.synchronize()
+    err = float(np.abs(out.float().cpu().numpy().reshape(T, Hq, D) - ref).max())
+    print("   err %.3e" % err, flush=True)
+    assert err <= (5e-2 if kv == "int8" else 2e-2)

@@ -10,7 +10,7 @@ import os
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG_DIR, "libxllm_hip_paged_kv.so")
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 # xllm_hip_dtype
 BF16, FP16, FP32, FP8_E4M3, INT8 = 0, 1, 2, 3, 4
@@ -90,6 +90,7 @@ class DecodeArgs(ctypes.Structure):
         ("kv_last_page_len", ctypes.c_void_p),
         ("max_seq_len", ctypes.c_int32),
         ("total_kv_len", ctypes.c_int64),
+        ("q_indptr", ctypes.c_void_p),
     ]
 
 

@@ -82,11 +82,19 @@ inline int row_groups(int q_per_seq, int num_q_heads, int num_kv_heads) {
   return (rows + kMaxRowsPerItem - 1) / kMaxRowsPerItem;
 }
 
+// More than four row groups per kv head (over 128 query rows: chunked prefill rather than decode or
+// speculative verify): sequences are never split into chunks.
+constexpr int kMaxRowGroupsForSplit = 4;
+inline bool never_split(int q_per_seq, int num_q_heads, int num_kv_heads) {
+  return row_groups(q_per_seq, num_q_heads, num_kv_heads) > kMaxRowGroupsForSplit;
+}
+
 // Sum_b ceil(L_b / C) <= sum(L)/C + B and C >= sum(L)*Hkv*RG/target, hence the bound below
 // for every target <= kMaxTargetItems.
 inline WorkspaceLayout workspace_layout(int batch, int q_per_seq, int num_q_heads, int num_kv_heads, int head_dim) {
   WorkspaceLayout w;
   w.max_seq_chunks = (int64_t)kMaxTargetItems / num_kv_heads + batch + 1;
+  if (never_split(q_per_seq, num_q_heads, num_kv_heads)) w.max_seq_chunks = batch + 1;
   size_t off = 0;
   w.header = off;
   off += sizeof(PlanHeader);

@@ -38,6 +38,7 @@ struct DecodeParams {
   const int32_t* kv_indptr;  // non-NULL selects the CSR form
   const int32_t* seq_lens;
   const int32_t* kv_last_page_len;
+  const int32_t* q_indptr;  // [batch+1] first query token of each sequence; NULL: n tokens each
   PlanHeader* hdr;
   int32_t* kv_len;
   int32_t* full_prefix;
@@ -56,7 +57,7 @@ struct DecodeParams {
   int64_t sc_stride_slot;
   int64_t bt_stride;
   int32_t batch;
-  int32_t n;  // query tokens per sequence
+  int32_t n;  // query tokens per sequence (the largest count when q_indptr is set)
   int32_t num_q_heads;
   int32_t num_kv_heads;
   int32_t group;  // q heads per kv head
@@ -199,6 +200,8 @@ struct Item {
   int t_end;    // one past the last token of the chunk (<= len)
   const int32_t* ids;  // block list of the sequence
   int nblk;     // valid entries in ids (>= 1)
+  int n;        // query tokens of the sequence
+  int q0;       // index of its first query token
   int64_t head_off;     // hk * stride_head (cache elements)
   int64_t sc_head_off;  // hk * sc_stride_head (scale elements)
 };
@@ -212,6 +215,15 @@ __device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it)
   it.sc = rest / p.num_kv_heads;
   const SeqChunk s = p.seq_chunks[it.sc];
   it.b = s.seq;
+  if (p.q_indptr != nullptr) {
+    it.q0 = p.q_indptr[it.b];
+    const int cnt = p.q_indptr[it.b + 1] - it.q0;
+    it.n = cnt < 0 ? 0 : (cnt > p.n ? p.n : cnt);  // never beyond what the launch and the workspace were sized for
+  } else {
+    it.q0 = it.b * p.n;
+    it.n = p.n;
+  }
+  if (it.rg * kMaxRowsPerItem >= it.n * p.group) return false;  // this sequence has no rows in the group
   it.len = p.kv_len[it.b];
   it.t_begin = s.chunk * hdr.chunk_tokens;
   const long long end = (long long)it.t_begin + hdr.chunk_tokens;
@@ -241,10 +253,16 @@ __global__ void __launch_bounds__(256) decode_merge_kernel(DecodeParams p) {
   const int sub = threadIdx.x & 31;
   if (row >= (int64_t)p.batch * nhq) return;
   const int b = (int)(row / nhq);
+  int q0 = b * p.n, nb = p.n;
+  if (p.q_indptr != nullptr) {
+    q0 = p.q_indptr[b];
+    nb = min(p.n, p.q_indptr[b + 1] - q0);
+  }
   const int cnt = p.num_chunks[b];
   if (p.direct_single && cnt == 1) return;  // already written by the attention kernel
   const int rem = (int)(row - (int64_t)b * nhq);  // j * Hq + head
   const int j = rem / p.num_q_heads;
+  if (j >= nb) return;
   const int head = rem - j * p.num_q_heads;
   const int D = p.head_dim;
   const float neg_inf = -INFINITY;
@@ -275,7 +293,7 @@ __global__ void __launch_bounds__(256) decode_merge_kernel(DecodeParams p) {
     m = m_new;
   }
   const float inv = ssum > 0.0f ? 1.0f / ssum : 0.0f;
-  const int64_t tok = (int64_t)b * p.n + j;
+  const int64_t tok = (int64_t)q0 + j;
   if (p.lse != nullptr && sub == 0) {
     p.lse[tok * p.num_q_heads + head] = ssum > 0.0f ? m + __builtin_amdgcn_logf(ssum) : neg_inf;
   }
@@ -622,12 +640,12 @@ struct RowTile {
     const int mi = lane & 15;  // MFMA row of A / column of B and D
     kg = lane >> 4;            // k-group of the operands; row block of D
     const int row = it.rg * kMaxRowsPerItem + row_in_item + mi;
-    const bool valid = row < p.rows;
+    const bool valid = row < it.n * p.group;
     const int j = valid ? row / p.group : 0;
     const int gq = valid ? row - j * p.group : 0;
-    lim = it.len - (p.n - 1 - j);
+    lim = it.len - (it.n - 1 - j);
     lo = p.window_left >= 0 ? lim - 1 - p.window_left : 0;
-    const uint16_t* qrow = (const uint16_t*)p.q + (int64_t)(it.b * p.n + j) * p.q_token_stride +
+    const uint16_t* qrow = (const uint16_t*)p.q + (int64_t)(it.q0 + j) * p.q_token_stride +
                            (int64_t)(it.hk * p.group + gq) * 128;
     float sq = 0.0f;
 #pragma unroll
@@ -791,12 +809,12 @@ __device__ inline void finish_item(const DecodeParams& p, const Item& it, RowTil
     l_all += wgt[s] * lds_ml[((rs * TW + s) * 16 + col) * 2 + 1];
   }
   const int r = it.rg * kMaxRowsPerItem + rs * 16 + col;
-  if (r >= p.rows) return;
+  if (r >= it.n * p.group) return;
   const int j = r / p.group;
   const int head = it.hk * p.group + (r - j * p.group);
   const float inv = l_all > 0.0f ? 1.0f / l_all : 0.0f;
   const float lse2 = l_all > 0.0f ? m_all + __builtin_amdgcn_logf(l_all) : neg_inf;
-  const int64_t tok = (int64_t)it.b * p.n + j;
+  const int64_t tok = (int64_t)it.q0 + j;
   const int64_t prow = (int64_t)it.sc * nhq + (int64_t)j * p.num_q_heads + head;
   constexpr int kCols = 128 / TW;  // columns this wave finishes: 8 per lane and pass
 #pragma unroll
@@ -838,7 +856,7 @@ __device__ inline void finish_item(const DecodeParams& p, const Item& it, RowTil
 __device__ inline int first_visible_tile(const DecodeParams& p, const Item& it) {
   int t0 = it.t_begin;
   if (p.window_left >= 0) {
-    int first = it.len - p.n - p.window_left;  // window start of the earliest query row
+    int first = it.len - it.n - p.window_left;  // window start of the earliest query row
     first = first > 0 ? first : 0;
     first &= ~(kTileTokens - 1);
     t0 = t0 > first ? t0 : first;
@@ -867,7 +885,7 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_d128_kernel(Decode
   const int share = span > 0 ? (((span + kWaves - 1) / kWaves + kTileTokens - 1) & ~(kTileTokens - 1)) : 0;
   const int w_begin = t0 + wave * share;
   const int w_end = min(it.t_end, w_begin + share);
-  const int mask_hi_from = it.len - (p.n - 1);                                    // tiles reaching past this need masks
+  const int mask_hi_from = it.len - (it.n - 1);                                    // tiles reaching past this need masks
   const int mask_lo_until = p.window_left >= 0 ? it.len - 1 - p.window_left : 0;  // tiles starting below this too
 
   typename KvHalf<KV_DT>::Geom geom;
@@ -938,7 +956,7 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_d128_rows32_kernel
   // Every wave runs the same number of iterations (the barrier is workgroup wide); a wave whose
   // token half is shorter idles through the tail.
   const int iters = share / kTileTokens;
-  const int mask_hi_from = it.len - (p.n - 1);
+  const int mask_hi_from = it.len - (it.n - 1);
   const int mask_lo_until = p.window_left >= 0 ? it.len - 1 - p.window_left : 0;
 
   typename KvHalf<KV_DT>::Geom geom;
@@ -1006,17 +1024,17 @@ __global__ void __launch_bounds__(64) decode_generic_kernel(DecodeParams p) {
   const float neg_inf = -INFINITY;
   const bool quant = KV_DT == XLLM_HIP_FP8_E4M3 || KV_DT == XLLM_HIP_INT8;
   const int nhq = p.n * p.num_q_heads;
-  const int row_end = min(p.rows, (it.rg + 1) * kMaxRowsPerItem);
+  const int row_end = min(it.n * p.group, (it.rg + 1) * kMaxRowsPerItem);
 
   for (int r = it.rg * kMaxRowsPerItem; r < row_end; ++r) {
     const int j = r / p.group;
     const int gq = r - j * p.group;
     const int head = it.hk * p.group + gq;
-    const int64_t qbase = (int64_t)(it.b * p.n + j) * p.q_token_stride + (int64_t)head * D;
+    const int64_t qbase = (int64_t)(it.q0 + j) * p.q_token_stride + (int64_t)head * D;
     __syncthreads();
     for (int d = lane; d < D; d += 64) qs[d] = Elem<Q_DT>::load(p.q, qbase + d) * p.scale_log2;
     __syncthreads();
-    const int lim = it.len - (p.n - 1 - j);
+    const int lim = it.len - (it.n - 1 - j);
     const int lo = p.window_left >= 0 ? lim - 1 - p.window_left : 0;
 
     float m_run = neg_inf, l_run = 0.0f;
@@ -1206,6 +1224,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
     p.kv_indptr = a->kv_indptr;
     p.kv_last_page_len = a->kv_last_page_len;
   }
+  p.q_indptr = a->q_indptr;
   p.hdr = (PlanHeader*)(ws + w.header);
   p.kv_len = (int32_t*)(ws + w.kv_len);
   p.full_prefix = (int32_t*)(ws + w.full_prefix);
@@ -1248,6 +1267,9 @@ static int fill_params(const xllm_hip_kv_cache* c,
                                      p.target_items)) {
     p.fixed_chunk = 1 << 30;
   }
+  // Many query rows per kv head (chunked prefill): the row groups supply the parallelism, and one
+  // partial per chunk and row would be large, so nothing is split.
+  if (never_split(a->q_per_seq, a->num_q_heads, c->num_kv_heads)) p.fixed_chunk = 1 << 30;
   p.q_dtype = a->q_dtype;
   p.scale_log2 = a->sm_scale * 1.4426950408889634f;
   return XLLM_HIP_OK;
@@ -1395,7 +1417,7 @@ extern "C" int xllm_hip_paged_decode_run_timed(const xllm_hip_kv_cache* cache,
   if (ev_end != nullptr && hipEventRecord((hipEvent_t)ev_end, st) != hipSuccess) {
     return fail(XLLM_HIP_RUNTIME_ERROR, "hipEventRecord(ev_end) failed");
   }
-  if (p.fixed_chunk == (1 << 30)) return XLLM_HIP_OK;  // nothing was split: the outputs are final
+  if (p.direct_single && p.fixed_chunk == (1 << 30)) return XLLM_HIP_OK;  // nothing was split: the outputs are final
 
   const int64_t rows = (int64_t)p.batch * p.n * p.num_q_heads;
   const unsigned mgrid = (unsigned)((rows + 7) / 8);

@@ -20,9 +20,6 @@ std::tuple<torch::Tensor, std::optional<torch::Tensor>> AttentionImpl::forward(
   if (attn_metadata.is_dummy || attn_metadata.max_seq_len == 0) {
     return {output.view({-1, num_heads_ * head_size_}), output_lse};
   }
-  TORCH_CHECK(!attn_metadata.is_prefill && !attn_metadata.is_chunked_prefill,
-              "the HIP backend implements the decode path only (prefill is served elsewhere)");
-
   torch::Tensor k_cache = kv_cache.get_k_cache();
   torch::Tensor v_cache = kv_cache.get_v_cache();
   std::optional<torch::Tensor> k_cache_scale = kv_cache.get_k_cache_scale();
@@ -58,8 +55,6 @@ std::tuple<torch::Tensor, std::optional<torch::Tensor>> AttentionImpl::forward_q
   if (attn_metadata.is_dummy || attn_metadata.max_seq_len == 0) {
     return {output, output_lse};
   }
-  TORCH_CHECK(!attn_metadata.is_prefill && !attn_metadata.is_chunked_prefill,
-              "the HIP backend implements the decode path only (prefill is served elsewhere)");
   TORCH_CHECK(qkv.dim() == 2 && qkv.size(1) == (num_heads_ + 2 * num_kv_heads_) * head_size_,
               "qkv must be [tokens, (num_heads + 2 * num_kv_heads) * head_size]");
   torch::Tensor k_cache = kv_cache.get_k_cache();
@@ -83,6 +78,22 @@ void AttentionImpl::decoder_forward(const AttentionMetadata& attn_metadata, torc
                                     const torch::Tensor& v_cache, const std::optional<torch::Tensor>& k_cache_scale,
                                     const std::optional<torch::Tensor>& v_cache_scale) {
   std::optional<torch::Tensor> output_lse = std::nullopt;
+  if (attn_metadata.is_prefill || attn_metadata.is_chunked_prefill) {
+    // Prefill chunks and mixed steps: the step's K/V are in the cache already (write, then attend), so
+    // every sequence attends its cached range with its own number of query tokens
+    // (xllm/core/layers/mlu/attention.cpp:179-250, xllm/core/layers/cuda/flashinfer_attention.cpp:224-284).
+    TORCH_CHECK(attn_metadata.block_table.defined() && attn_metadata.kv_seq_lens.defined() &&
+                    attn_metadata.q_cu_seq_lens.defined(),
+                "prefill over the paged cache needs block_table, kv_seq_lens and q_cu_seq_lens");
+    torch::Tensor q3 = query.view({-1, num_heads_, head_size_});
+    torch::Tensor o3 = output.view({-1, num_heads_, head_size_});
+    xllm::kernel::hip::batch_prefill_paged(q3, k_cache, v_cache, o3, output_lse, attn_metadata.q_cu_seq_lens,
+                                           attn_metadata.kv_seq_lens, k_cache_scale, v_cache_scale,
+                                           attn_metadata.block_table, attn_metadata.max_query_len,
+                                           attn_metadata.max_seq_len, scale_, sliding_window_, false,
+                                           attn_metadata.total_kv_len);
+    return;
+  }
   // One decode row per query token by default (speculative verify arrives expanded into rows,
   // xllm/core/runtime/speculative_worker_impl.cpp:230-243); a batch whose sequences all carry
   // max_query_len > 1 tokens against one block-table row each is the multi-token form.

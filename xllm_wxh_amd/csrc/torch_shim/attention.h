@@ -1,4 +1,5 @@
-// Decode dispatch of the HIP backend: KV write, then paged decode — the role of
+// Attention dispatch of the HIP backend: KV write, then attention over the paged cache (decode,
+// speculative verify, and prefill chunks / mixed steps through the same kernels) — the role of
 // xllm::layer::AttentionImpl (xllm/core/layers/cuda/attention.h:41-46,
 // xllm/core/layers/mlu/attention.h:47-52; same constructor and forward signature on every backend).
 #pragma once

@@ -227,6 +227,53 @@ void batch_decode(const torch::Tensor& query,
   run_decode(cache, a, q3);
 }
 
+void batch_prefill_paged(const torch::Tensor& query, const torch::Tensor& k_cache, const torch::Tensor& v_cache,
+                         torch::Tensor& output, std::optional<torch::Tensor>& output_lse,
+                         const torch::Tensor& q_cu_seq_lens, const torch::Tensor& kv_seq_lens,
+                         const std::optional<torch::Tensor>& k_cache_quant_scale,
+                         const std::optional<torch::Tensor>& v_cache_quant_scale, const torch::Tensor& block_tables,
+                         int64_t max_query_len, int64_t max_seq_len, float scale, int64_t window_size_left,
+                         bool return_lse, int64_t total_kv_len) {
+  TORCH_CHECK(query.dim() == 3 && output.dim() == 3, "query/output must be [tokens, heads, head_dim]");
+  TORCH_CHECK(max_query_len >= 1, "max_query_len must be at least 1");
+  const bool quant = k_cache_quant_scale.has_value();
+  TORCH_CHECK(!quant || v_cache_quant_scale.has_value(), "v_cache_quant_scale is required with k_cache_quant_scale");
+  const xllm_hip_kv_cache cache = make_cache(k_cache, v_cache, k_cache_quant_scale, v_cache_quant_scale);
+  xllm_hip_decode_args a{};
+  torch::Tensor o3 = output;
+  fill_q_out(a, query, o3, 1);
+  TORCH_CHECK(query.size(2) == cache.head_dim, "query head_dim does not match the cache");
+  TORCH_CHECK(q_cu_seq_lens.scalar_type() == torch::kInt && q_cu_seq_lens.is_contiguous() &&
+                  q_cu_seq_lens.numel() >= 1,
+              "q_cu_seq_lens must be contiguous int32 [batch + 1]");
+  a.batch = (int32_t)(q_cu_seq_lens.numel() - 1);
+  a.q_per_seq = (int32_t)max_query_len;
+  a.q_indptr = q_cu_seq_lens.data_ptr<int32_t>();
+  a.sm_scale = scale;
+  a.window_left = (int32_t)window_size_left;
+  TORCH_CHECK(block_tables.scalar_type() == torch::kInt && block_tables.dim() == 2 && block_tables.stride(1) == 1 &&
+                  block_tables.size(0) == a.batch,
+              "block_tables must be int32 [batch, max_blocks]");
+  TORCH_CHECK(kv_seq_lens.scalar_type() == torch::kInt && kv_seq_lens.is_contiguous() && kv_seq_lens.numel() == a.batch,
+              "kv_seq_lens must be contiguous int32 [batch]");
+  a.block_table = block_tables.data_ptr<int32_t>();
+  a.block_table_stride = block_tables.stride(0);
+  a.max_blocks_per_seq = (int32_t)block_tables.size(1);
+  a.seq_lens = kv_seq_lens.data_ptr<int32_t>();
+  a.max_seq_len = (int32_t)max_seq_len;
+  a.total_kv_len = total_kv_len;
+  if (return_lse) {
+    TORCH_CHECK(output_lse.has_value(), "return_lse needs a pre-allocated output_lse");
+  }
+  if (output_lse.has_value() && output_lse->defined()) {
+    TORCH_CHECK(output_lse->scalar_type() == torch::kFloat && output_lse->is_contiguous() &&
+                    output_lse->numel() == query.size(0) * query.size(1),
+                "output_lse must be contiguous float32 [tokens, heads]");
+    a.lse = output_lse->data_ptr<float>();
+  }
+  run_decode(cache, a, query);
+}
+
 void batch_decode_csr(torch::Tensor query,
                       torch::Tensor k_cache,
                       torch::Tensor v_cache,

@@ -48,6 +48,29 @@ void batch_decode(const torch::Tensor& query,
                   int64_t kv_cache_quant_bit_size,
                   int64_t total_kv_len = 0);
 
+// Chunked prefill / mixed steps over the paged cache: the block_tables form of
+// xllm::kernel::mlu::batch_prefill (xllm/core/kernels/mlu/mlu_ops_api.h:103-124, called with the caches
+// as key/value in xllm/core/layers/mlu/attention.cpp:179-250).  query/output: [tokens, Hq, D]; sequence b
+// owns rows q_cu_seq_lens[b] .. q_cu_seq_lens[b+1], the last tokens of its kv_seq_lens[b] cached tokens
+// (already written), causal.  A quantised cache is attended directly (the reference dequantises it to
+// a dense copy first, attention.cpp:182-222).
+void batch_prefill_paged(const torch::Tensor& query,
+                         const torch::Tensor& k_cache,
+                         const torch::Tensor& v_cache,
+                         torch::Tensor& output,
+                         std::optional<torch::Tensor>& output_lse,
+                         const torch::Tensor& q_cu_seq_lens,
+                         const torch::Tensor& kv_seq_lens,
+                         const std::optional<torch::Tensor>& k_cache_quant_scale,
+                         const std::optional<torch::Tensor>& v_cache_quant_scale,
+                         const torch::Tensor& block_tables,
+                         int64_t max_query_len,
+                         int64_t max_seq_len,
+                         float scale,
+                         int64_t window_size_left,
+                         bool return_lse,
+                         int64_t total_kv_len = 0);
+
 // Tensor arguments of xllm::kernel::cuda::batch_decode (xllm/core/kernels/cuda/cuda_ops_api.h:120-136)
 // without the FlashInfer uri / plan / workspaces, which have no counterpart here.
 // query/output: [tokens, Hq, D]; caches in the CUDA backend's NHD shape [blocks, block_size, Hkv, D].

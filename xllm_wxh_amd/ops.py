@@ -185,7 +185,7 @@ def get_workspace(device, nbytes):
 
 
 def _decode_args(query, output, output_lse, block_table, seq_lens, csr, q_per_seq, scale, window_size_left,
-                 max_seq_len, desc, total_kv_len=0):
+                 max_seq_len, desc, total_kv_len=0, q_indptr=None):
     _require(query.dim() in (3, 4), "query must be [tokens, heads, dim] or [batch, q_len, heads, dim]")
     if query.dim() == 4:
         # [batch, q_len, Hq, D] (xllm/core/layers/mlu/attention.cpp:263-264)
@@ -202,13 +202,20 @@ def _decode_args(query, output, output_lse, block_table, seq_lens, csr, q_per_se
     _require(q3.stride(2) == 1 and q3.stride(1) == q3.size(2), "query heads/head_dim must be contiguous")
     _require(o3.stride(2) == 1 and o3.stride(1) == o3.size(2), "output heads/head_dim must be contiguous")
     _require(q3.size(2) == desc.head_dim, "query head_dim %d != cache head_dim %d" % (q3.size(2), desc.head_dim))
-    _require(q3.size(0) % q_per_seq == 0, "query tokens not divisible by q_per_seq")
+    if q_indptr is None:
+        _require(q3.size(0) % q_per_seq == 0, "query tokens not divisible by q_per_seq")
+        batch = q3.size(0) // q_per_seq
+    else:
+        _require(q_indptr.dtype == torch.int32 and q_indptr.is_contiguous() and q_indptr.numel() >= 1,
+                 "q_indptr must be contiguous int32 [batch + 1]")
+        batch = q_indptr.numel() - 1
 
     a = _lib.DecodeArgs()
     a.q, a.out = q3.data_ptr(), o3.data_ptr()
     a.q_token_stride, a.out_token_stride = q3.stride(0), o3.stride(0)
     a.q_dtype = _dtype_code(q3)
-    a.batch = q3.size(0) // q_per_seq
+    a.batch = batch
+    a.q_indptr = q_indptr.data_ptr() if q_indptr is not None else None
     a.q_per_seq = q_per_seq
     a.num_q_heads = q3.size(1)
     a.sm_scale = float(scale)
@@ -264,7 +271,7 @@ def batch_decode(query, k_cache, output, block_table, seq_lens, v_cache=None, ou
                  alibi_slope=None, mask=None, compute_dtype="float", max_seq_len=0, window_size_left=-1,
                  window_size_right=-1, scale=1.0, return_lse=False, kv_cache_quant_bit_size=-1, *,
                  q_per_seq=None, kv_layout="HND", workspace=None, plan=True, run=True, events=None,
-                 total_kv_len=0):
+                 total_kv_len=0, q_indptr=None):
     """Paged decode in the block_table form; positional arguments as in
     xllm::kernel::mlu::batch_decode (xllm/core/kernels/mlu/mlu_ops_api.h:126-145).
 
@@ -274,7 +281,9 @@ def batch_decode(query, k_cache, output, block_table, seq_lens, v_cache=None, ou
     run=False, then reuse it for every layer with plan=False), events (two raw hipEvent_t handles
     recorded just before and just after the attention kernel, for benchmarks), total_kv_len (the
     host-side sum of the kv lengths, AttentionMetadata.total_kv_len in the reference; together with
-    max_seq_len it lets the library drop the merge launch when no sequence needs splitting).
+    max_seq_len it lets the library drop the merge launch when no sequence needs splitting),
+    q_indptr (int32 [batch + 1]: sequences with different numbers of query tokens, the q_cu_seq_lens of
+    a chunked-prefill or mixed step; q_per_seq is then the largest count, max_query_len).
     """
     _require(v_cache is not None, "v_cache is required (MLA-style single-cache decode is outside this path)")
     for name, t in (("q_quant_scale", q_quant_scale), ("out_quant_scale", out_quant_scale),
@@ -292,7 +301,7 @@ def batch_decode(query, k_cache, output, block_table, seq_lens, v_cache=None, ou
     desc = _cache_desc(k_cache, v_cache, k_cache_quant_scale, v_cache_quant_scale, kv_layout)
     args, _keep = _decode_args(query, output, output_lse if return_lse or output_lse is not None else None,
                                block_table, seq_lens, None, q_per_seq, scale, window_size_left, max_seq_len, desc,
-                               total_kv_len)
+                               total_kv_len, q_indptr)
     _run_decode(desc, args, workspace, query.device, plan, run, events)
 
 
