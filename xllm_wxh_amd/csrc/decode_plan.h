@@ -23,8 +23,9 @@ namespace xllm_hip {
 
 constexpr int kTileTokens = 32;       // tokens per MFMA tile; chunk sizes are multiples of it
 constexpr int kMinChunkTokens = 512;  // smallest split worth a partial round trip (128 tokens per wave)
+constexpr int kMinChunkTokensGeneric = 64;  // the one-wave kernel: one 64-token step
 constexpr int kMaxTargetItems = 4096; // upper bound of the split target (sizes the workspace)
-constexpr int kMaxRowsPerItem = 32;   // query rows (g * n) one work item handles
+constexpr int kMaxRowsPerItem = 32;   // query rows (g * n) one work item of the MFMA kernels handles
 
 #if defined(__HIPCC__)
 #define XLLM_HIP_HD __host__ __device__
@@ -37,14 +38,14 @@ constexpr int kMaxRowsPerItem = 32;   // query rows (g * n) one work item handle
 // above 1.5x the mean), because then the items differ in size and the dispatcher needs slack to
 // balance them.  Shared by the device-side plan and by the host's check that nothing is split.
 XLLM_HIP_HD inline int choose_chunk(long long total, long long max_len, int batch, int num_kv_heads,
-                                    int row_groups, int target) {
+                                    int row_groups, int target, int min_chunk) {
   long long t = target;
   if (max_len * batch * 2 > total * 3) t *= 4;
   if (t > kMaxTargetItems) t = kMaxTargetItems;
   const long long work = total * num_kv_heads * row_groups;
   long long c = (work + t - 1) / t;
   c = (c + kTileTokens - 1) / kTileTokens * kTileTokens;
-  if (c < kMinChunkTokens) c = kMinChunkTokens;
+  if (c < min_chunk) c = min_chunk;
   if (c > (1 << 30)) c = 1 << 30;
   return (int)c;
 }
@@ -77,9 +78,9 @@ struct WorkspaceLayout {
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
-inline int row_groups(int q_per_seq, int num_q_heads, int num_kv_heads) {
+inline int row_groups(int q_per_seq, int num_q_heads, int num_kv_heads, int rows_per_item = kMaxRowsPerItem) {
   const int rows = q_per_seq * (num_q_heads / num_kv_heads);
-  return (rows + kMaxRowsPerItem - 1) / kMaxRowsPerItem;
+  return (rows + rows_per_item - 1) / rows_per_item;
 }
 
 // More than four row groups per kv head (over 128 query rows: chunked prefill rather than decode or

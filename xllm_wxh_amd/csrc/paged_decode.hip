@@ -63,6 +63,8 @@ struct DecodeParams {
   int32_t group;  // q heads per kv head
   int32_t rows;   // group * n
   int32_t row_groups;
+  int32_t rows_per_item;  // query rows one work item handles (32 MFMA, 1 generic)
+  int32_t min_chunk;      // smallest chunk the plan may choose
   int32_t head_dim;
   int32_t block_size;
   int32_t log2_bs;
@@ -120,7 +122,7 @@ __global__ void __launch_bounds__(64) decode_plan_kernel(DecodeParams p) {
   // 2. Chunk size.
   const int chunk = p.fixed_chunk > 0
                         ? p.fixed_chunk
-                        : choose_chunk(total, max_len, p.batch, p.num_kv_heads, p.row_groups, p.target_items);
+                        : choose_chunk(total, max_len, p.batch, p.num_kv_heads, p.row_groups, p.target_items, p.min_chunk);
 
   // 3. Prefix sums of the full-chunk and tail-chunk counts (lengths are re-derived rather than
   //    re-read so that no lane depends on another lane's global store).
@@ -223,7 +225,7 @@ __device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it)
     it.q0 = it.b * p.n;
     it.n = p.n;
   }
-  if (it.rg * kMaxRowsPerItem >= it.n * p.group) return false;  // this sequence has no rows in the group
+  if (it.rg * p.rows_per_item >= it.n * p.group) return false;  // this sequence has no rows in the group
   it.len = p.kv_len[it.b];
   it.t_begin = s.chunk * hdr.chunk_tokens;
   const long long end = (long long)it.t_begin + hdr.chunk_tokens;
@@ -1014,9 +1016,42 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_d128_rows32_kernel
 // so that every shape the operators accept is served and as an independent device-side check.
 // ---------------------------------------------------------------------------------
 
+// q . k over one cache row for the lane's token: 16-byte pieces when the rows allow it.
+template <int KV_DT>
+__device__ inline float dot_row(const uint8_t* cache, int64_t row, const float* qs, int D, bool vec_ok) {
+  float dot = 0.0f;
+  constexpr int kPer = KV_DT == XLLM_HIP_FP32 ? 4 : (KV_DT == XLLM_HIP_BF16 || KV_DT == XLLM_HIP_FP16) ? 8 : 16;
+  if (vec_ok) {
+    const u32x4* src = (const u32x4*)(cache + row * (16 / kPer));
+    for (int d = 0; d < D; d += kPer) {
+      const u32x4 raw = src[d / kPer];
+#pragma unroll
+      for (int e = 0; e < kPer; ++e) {
+        float x;
+        if (KV_DT == XLLM_HIP_FP32) {
+          x = __uint_as_float(raw[e]);
+        } else if (KV_DT == XLLM_HIP_BF16) {
+          x = __uint_as_float((e & 1) ? (raw[e >> 1] & 0xffff0000u) : (raw[e >> 1] << 16));
+        } else if (KV_DT == XLLM_HIP_FP16) {
+          const uint16_t h = (uint16_t)((e & 1) ? (raw[e >> 1] >> 16) : (raw[e >> 1] & 0xffffu));
+          x = (float)__builtin_bit_cast(_Float16, h);
+        } else if (KV_DT == XLLM_HIP_INT8) {
+          x = (float)(int8_t)((raw[e >> 2] >> (8 * (e & 3))) & 0xffu);
+        } else {
+          x = fp8_e4m3_to_float((uint8_t)((raw[e >> 2] >> (8 * (e & 3))) & 0xffu));
+        }
+        dot += qs[d + e] * x;
+      }
+    }
+  } else {
+    for (int d = 0; d < D; ++d) dot += qs[d] * Elem<KV_DT>::load(cache, row + d);
+  }
+  return dot;
+}
+
 template <int Q_DT, int KV_DT>
 __global__ void __launch_bounds__(64) decode_generic_kernel(DecodeParams p) {
-  __shared__ float qs[256];
+  __shared__ __attribute__((aligned(16))) float qs[256];
   Item it;
   if (!decode_item(p, blockIdx.x, it)) return;
   const int lane = threadIdx.x;
@@ -1024,9 +1059,13 @@ __global__ void __launch_bounds__(64) decode_generic_kernel(DecodeParams p) {
   const float neg_inf = -INFINITY;
   const bool quant = KV_DT == XLLM_HIP_FP8_E4M3 || KV_DT == XLLM_HIP_INT8;
   const int nhq = p.n * p.num_q_heads;
-  const int row_end = min(it.n * p.group, (it.rg + 1) * kMaxRowsPerItem);
+  const int row_end = min(it.n * p.group, (it.rg + 1) * p.rows_per_item);
+  const int eb = KV_DT == XLLM_HIP_FP32 ? 4 : (KV_DT == XLLM_HIP_BF16 || KV_DT == XLLM_HIP_FP16) ? 2 : 1;
+  // rows start on 16-byte boundaries and hold whole 16-byte pieces
+  const bool vec_ok = (((uintptr_t)p.k_cache | (uintptr_t)(p.stride_block * eb) | (uintptr_t)(p.stride_head * eb) |
+                        (uintptr_t)(p.stride_slot * eb) | (uintptr_t)(D * eb)) & 15) == 0;
 
-  for (int r = it.rg * kMaxRowsPerItem; r < row_end; ++r) {
+  for (int r = it.rg * p.rows_per_item; r < row_end; ++r) {
     const int j = r / p.group;
     const int gq = r - j * p.group;
     const int head = it.hk * p.group + gq;
@@ -1044,14 +1083,13 @@ __global__ void __launch_bounds__(64) decode_generic_kernel(DecodeParams p) {
       const bool vis = tok < it.t_end && tok < lim && tok >= lo;
       float x = neg_inf;
       float vscale = 0.0f;
-      int64_t vrow = 0;
+      int64_t vrow = 0;  // invisible tokens point at the start of the cache and carry weight 0
       if (vis) {
         int bi = tok >> p.log2_bs;
         const int64_t blk = it.ids[bi];
         const int slot = tok & (p.block_size - 1);
         const int64_t row = blk * p.stride_block + (int64_t)it.hk * p.stride_head + (int64_t)slot * p.stride_slot;
-        float dot = 0.0f;
-        for (int d = 0; d < D; ++d) dot += qs[d] * Elem<KV_DT>::load(p.k_cache, row + d);
+        float dot = dot_row<KV_DT>(p.k_cache, row, qs, D, vec_ok);
         if (quant) {
           const int64_t srow = blk * p.sc_stride_block + (int64_t)it.hk * p.sc_stride_head +
                                (int64_t)slot * p.sc_stride_slot;
@@ -1073,15 +1111,26 @@ __global__ void __launch_bounds__(64) decode_generic_kernel(DecodeParams p) {
       const float pw = e * vscale;
 #pragma unroll
       for (int i = 0; i < 4; ++i) o[i] *= alpha;
+      // p . V: lanes are head-dim columns; four tokens per step keep several loads in flight.  A
+      // weight of exactly 0 (masked token) must not meet a garbage value: its row is skipped by select.
       const int cnt = min(64, it.t_end - tb);
-      for (int tt = 0; tt < cnt; ++tt) {
-        const float pt = __shfl(pw, tt);
-        const int64_t row = __shfl(vrow, tt);
-        if (pt != 0.0f) {
+      for (int tt = 0; tt < cnt; tt += 4) {
+        float pt[4];
+        int64_t rw[4];
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int d = lane + 64 * i;
-            if (d < D) o[i] += pt * Elem<KV_DT>::load(p.v_cache, row + d);
+        for (int u = 0; u < 4; ++u) {
+          pt[u] = __shfl(pw, tt + u);  // lanes beyond cnt carry weight 0 and row 0
+          rw[u] = __shfl(vrow, tt + u);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int d = lane + 64 * i;
+          if (d < D) {
+            float v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = Elem<KV_DT>::load(p.v_cache, rw[u] + d);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) o[i] += pt[u] != 0.0f ? pt[u] * v[u] : 0.0f;
           }
         }
       }
@@ -1248,13 +1297,15 @@ static int fill_params(const xllm_hip_kv_cache* c,
   p.num_kv_heads = c->num_kv_heads;
   p.group = a->num_q_heads / c->num_kv_heads;
   p.rows = p.group * p.n;
-  p.row_groups = row_groups(a->q_per_seq, a->num_q_heads, c->num_kv_heads);
+  const Variant variant = pick_variant(c, a);
+  p.rows_per_item = variant == kMfmaD128 ? kMaxRowsPerItem : 1;
+  p.min_chunk = variant == kMfmaD128 ? kMinChunkTokens : kMinChunkTokensGeneric;
+  p.row_groups = row_groups(a->q_per_seq, a->num_q_heads, c->num_kv_heads, p.rows_per_item);
   p.head_dim = c->head_dim;
   p.block_size = c->block_size;
   p.log2_bs = is_pow2(c->block_size) ? ilog2(c->block_size) : 0;
   p.max_blocks_per_seq = a->max_blocks_per_seq;
   p.window_left = a->window_left;
-  const Variant variant = pick_variant(c, a);
   p.target_items = target_items(variant == kMfmaD128);
   // Only the MFMA kernel finishes single-chunk sequences itself.  When the caller's host-side
   // lengths (the reference keeps both in AttentionMetadata) show that the chunk the plan would
@@ -1264,7 +1315,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
   p.fixed_chunk = 0;
   if (p.direct_single && a->max_seq_len > 0 && a->total_kv_len > 0 &&
       a->max_seq_len <= choose_chunk(a->total_kv_len, a->max_seq_len, p.batch, p.num_kv_heads, p.row_groups,
-                                     p.target_items)) {
+                                     p.target_items, p.min_chunk)) {
     p.fixed_chunk = 1 << 30;
   }
   // Many query rows per kv head (chunked prefill): the row groups supply the parallelism, and one
