@@ -43,6 +43,9 @@ def parse_args():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain 1 GiB device-to-device copy a few times and exit: the known-size "
                          "kernel against which the rocprofv3 FETCH_SIZE / WRITE_SIZE counters are scaled")
+    ap.add_argument("--aux", action="store_true",
+                    help="time the kernels around the decode path instead (KV writes, norm + rotary embedding + "
+                         "write, block copy, a chunked-prefill step) and print one JSON line of their own")
     return ap.parse_args()
 
 
@@ -106,6 +109,9 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"copy_calibration": True, "bytes_read_per_launch": src.numel() * 2,
                           "bytes_written_per_launch": src.numel() * 2, "launches": 10}))
+        return
+    if args.aux:
+        print(json.dumps(aux_kernels(torch, ops, device)), flush=True)
         return
     w = workloads.WORKLOADS[args.workload]
     io_dtype = torch.float32 if w.kv_dtype == "fp32" else torch.bfloat16  # query, output, new K/V rows
@@ -244,6 +250,83 @@ def main():
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(w, torch, pools[0], q, block_table, seq_lens, out, step, args)
     print(json.dumps(result), flush=True)
+
+
+def aux_kernels(torch, ops, device):
+    """Average duration (torch events on the launch stream, 50 launches after 5) and algorithmic
+    bandwidth of the kernels around the decode path, Llama-3-8B head shape (32 q / 8 kv heads, D 128)."""
+    Hq, Hkv, D, bs, nb = 32, 8, 128, 16, 40000  # 40000 blocks of 16 tokens: 2.6 GB of bf16 K+V
+    gen = torch.Generator(device=device)
+    gen.manual_seed(5)
+    kc = torch.randn(nb, Hkv, bs, D, device=device, dtype=torch.bfloat16, generator=gen)
+    vc = torch.randn(nb, Hkv, bs, D, device=device, dtype=torch.bfloat16, generator=gen)
+    kq = torch.empty(nb, Hkv, bs, D, device=device, dtype=torch.int8)
+    vq = torch.empty_like(kq)
+    ksc = torch.empty(nb, Hkv, bs, device=device, dtype=torch.float32)
+    vsc = torch.empty_like(ksc)
+    theta = torch.rand(8192, D // 2, device=device, generator=gen) * 6.283
+    cos_sin = torch.cat([torch.cos(theta), torch.sin(theta)], 1).to(torch.bfloat16)
+
+    def timed(fn, n=50):
+        for _ in range(5):
+            fn()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(n):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) * 1e3 / n
+
+    res = {"aux_kernels": True, "shape": "32 q / 8 kv heads, head_dim 128, bf16 activations", "entries": []}
+
+    def add(name, us, nbytes, note=""):
+        res["entries"].append({"kernel": name, "us": round(us, 2), "algorithmic_bytes": int(nbytes),
+                               "gbps": round(nbytes / us / 1e3, 1), "note": note})
+
+    for T in (64, 8192):
+        qkv = torch.randn(T, (Hq + 2 * Hkv) * D, device=device, dtype=torch.bfloat16, generator=gen)
+        key = qkv[:, Hq * D:(Hq + Hkv) * D].view(T, Hkv, D)
+        val = qkv[:, (Hq + Hkv) * D:].view(T, Hkv, D)
+        slots = torch.randperm(nb * bs, device=device, generator=gen)[:T].to(torch.int32)
+        pos = torch.randint(0, 8192, (T,), device=device, generator=gen)
+        p16 = ops.ReshapePagedCacheParams(key=key, value=val, k_cache=kc, v_cache=vc, slot_mapping=slots)
+        p8 = ops.ReshapePagedCacheParams(key=key, value=val, k_cache=kq, v_cache=vq, slot_mapping=slots,
+                                         k_cache_scale=ksc, v_cache_scale=vsc)
+        kvb = T * Hkv * D * 2
+        add("reshape_paged_cache T=%d" % T, timed(lambda: ops.reshape_paged_cache(p16)), 2 * kvb * 2)
+        add("quant_to_paged_cache int8 T=%d" % T, timed(lambda: ops.quant_to_paged_cache(p8)),
+            2 * kvb + 2 * kvb // 2 + 2 * T * Hkv * 4)
+        add("rope_kv_write bf16 cache T=%d" % T,
+            timed(lambda: ops.rope_kv_write(qkv, Hq, Hkv, D, cos_sin, pos, kc, vc, slots, round_each_op=True)),
+            T * ((2 * Hq + 2 * Hkv) * D * 2 + Hkv * D * 2 + 2 * Hkv * D * 2), "q,k read+written, v read, cache written")
+        add("rope_kv_write int8 cache T=%d" % T,
+            timed(lambda: ops.rope_kv_write(qkv, Hq, Hkv, D, cos_sin, pos, kq, vq, slots, round_each_op=True,
+                                            k_cache_scale=ksc, v_cache_scale=vsc)),
+            T * ((2 * Hq + 2 * Hkv) * D * 2 + Hkv * D * 2 + 2 * Hkv * D + 2 * Hkv * 4))
+    for nblk in (64, 4096):
+        perm = torch.randperm(nb, device=device, generator=gen)
+        src, dst = perm[:nblk].contiguous(), perm[nblk:2 * nblk].contiguous()
+        blk_bytes = 2 * Hkv * bs * D * 2
+        add("swap_blocks in place, %d blocks of 16 tokens" % nblk,
+            timed(lambda: ops.swap_blocks(kc, vc, src, dst, exact=False)), 2 * nblk * blk_bytes, "read + write")
+        add("swap_blocks gather-then-scatter, %d blocks" % nblk,
+            timed(lambda: ops.swap_blocks(kc, vc, src, dst, exact=True)), 4 * nblk * blk_bytes,
+            "two passes through a staging buffer allocated per call")
+    # a chunked-prefill step: 4 sequences, 512 new tokens each on top of a 3584-token prefix
+    B, n, L = 4, 512, 4096
+    q = torch.randn(B * n, Hq, D, device=device, dtype=torch.bfloat16, generator=gen)
+    out = torch.empty_like(q)
+    table = torch.randperm(nb, device=device, generator=gen)[: B * (L // bs)].to(torch.int32).view(B, L // bs)
+    lens = torch.full((B,), L, device=device, dtype=torch.int32)
+    q_indptr = (torch.arange(B + 1, device=device) * n).to(torch.int32)
+    us = timed(lambda: ops.batch_decode(q, kc, out, table, lens, vc, scale=D ** -0.5, q_per_seq=n, q_indptr=q_indptr,
+                                        max_seq_len=L, total_kv_len=B * L), n=10)
+    flops = 4.0 * B * Hq * D * sum(L - n + 1 + j for j in range(n))
+    res["entries"].append({"kernel": "chunked prefill through the decode kernel, 4 x 512 tokens on a 3584-token prefix",
+                           "us": round(us, 1), "tflops": round(flops / us / 1e6, 1),
+                           "note": "untuned: every 32 query rows stream the sequence's K/V again"})
+    return res
 
 
 def cpu_baseline(w, torch, pool, q, block_table, seq_lens, out, step, args):
