@@ -931,33 +931,27 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_d128_kernel(Decode
 }
 
 template <int KV_DT>
-__global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_d128_rows32_kernel(DecodeParams p) {
-  constexpr int TW = 2;  // waves per row set = token halves of the item
-  // [token half][buffer]: a tile is parked by the two waves that share the token half while both
-  // still read the previous tile from the other buffer, so one barrier per tile suffices.
-  __shared__ __attribute__((aligned(16))) uint8_t lds_all[TW * 2 * kLdsTile];
-  __shared__ float lds_ml[kWaves * 16 * 2];
+__global__ void __launch_bounds__(128, 2) decode_mfma_d128_rows32_kernel(DecodeParams p) {
+  // A workgroup is one pair of waves: wave w owns query rows 16w .. 16w+15 and fetches rows 16w ..
+  // of every tile.  A tile is parked while both waves still read the previous one from the other
+  // buffer, so one barrier (of two waves) per tile suffices.  Four such workgroups share a CU.
+  __shared__ __attribute__((aligned(16))) uint8_t lds_all[2 * kLdsTile];
+  __shared__ float lds_ml[2 * 16 * 2];
 
   Item it;
   if (!decode_item(p, blockIdx.x, it)) return;
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int rs = wave >> 1;  // row set: query rows 16*rs .. 16*rs+15; also the tile half this wave fetches
-  const int tw = wave & 1;   // token half of the item
+  const int rs = wave;  // row set; also the tile half this wave fetches
   const int lane = threadIdx.x & 63;
-  uint8_t* tiles = lds_all + tw * 2 * kLdsTile;
+  uint8_t* tiles = lds_all;
 
   RowTile<KV_DT> rt;
   rt.init(p, it, 16 * rs, lane);
 
-  const int t0 = first_visible_tile(p, it);
-  const int span = it.t_end - t0;
-  const int share = span > 0 ? (((span + TW - 1) / TW + kTileTokens - 1) & ~(kTileTokens - 1)) : 0;
-  const int w_begin = t0 + tw * share;
-  const int w_end = min(it.t_end, w_begin + share);
-  // Every wave runs the same number of iterations (the barrier is workgroup wide); a wave whose
-  // token half is shorter idles through the tail.
-  const int iters = share / kTileTokens;
+  const int w_begin = first_visible_tile(p, it);
+  const int w_end = it.t_end;
+  const int iters = w_end > w_begin ? (w_end - w_begin + kTileTokens - 1) / kTileTokens : 0;
   const int mask_hi_from = it.len - (it.n - 1);
   const int mask_lo_until = p.window_left >= 0 ? it.len - 1 - p.window_left : 0;
 
@@ -965,7 +959,7 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_d128_rows32_kernel
   geom.init(p, lane);
   // Two register stages, used alternately: the loads of tiles i+1 and i+2 are in flight while tile
   // i is consumed.  (A wave fetches only half a tile, so one stage would leave too few bytes in
-  // flight per CU to cover the HBM latency.)
+  // flight per CU to cover the HBM latency.)  Both waves run the same iterations.
   KvHalf<KV_DT> mine[2];  // the 16 tokens this wave fetches: rows 16*rs .. of the tile
 
   auto issue = [&](KvHalf<KV_DT>& m, int blk, int tb) {
@@ -977,25 +971,20 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_d128_rows32_kernel
   auto step = [&](KvHalf<KV_DT>& m, int& blk, int i) {
     const int tb = w_begin + i * kTileTokens;
     const int nblk = block_of(p, it, tb + 4 * kTileTokens + 16 * rs);
-    const bool live = tb < w_end;
     uint8_t* tile = tiles + (i & 1) * kLdsTile;
     const bool masked = (tb + kTileTokens > mask_hi_from) || (tb < mask_lo_until);
-    if (live) {
-      if (masked) {
-        m.template park<true>(tile, rs, tb + 16 * rs, it.len, p.scale_log2, geom);
-      } else {
-        m.template park<false>(tile, rs, tb + 16 * rs, it.len, p.scale_log2, geom);
-      }
-      issue(m, blk, tb + 2 * kTileTokens);
+    if (masked) {
+      m.template park<true>(tile, rs, tb + 16 * rs, it.len, p.scale_log2, geom);
+    } else {
+      m.template park<false>(tile, rs, tb + 16 * rs, it.len, p.scale_log2, geom);
     }
+    issue(m, blk, tb + 2 * kTileTokens);
     blk = nblk;
-    __syncthreads();  // both halves of tile i are parked; everyone is done with tile i-1
-    if (live) {
-      if (masked) {
-        rt.template attend<true>(tile, tb, p.scale_log2);
-      } else {
-        rt.template attend<false>(tile, tb, p.scale_log2);
-      }
+    __syncthreads();  // both halves of tile i are parked; both waves are done with tile i-1
+    if (masked) {
+      rt.template attend<true>(tile, tb, p.scale_log2);
+    } else {
+      rt.template attend<false>(tile, tb, p.scale_log2);
     }
   };
   issue(mine[0], block_of(p, it, w_begin + 16 * rs), w_begin);
@@ -1007,7 +996,7 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_d128_rows32_kernel
     if (i + 1 < iters) step(mine[1], blk_b, i + 1);
   }
   __syncthreads();  // all tiles consumed before the buffers are reused for the exchange
-  finish_item<KV_DT, TW>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, rs, tw, lane);
+  finish_item<KV_DT, 1>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, rs, 0, lane);
 }
 
 // ---------------------------------------------------------------------------------
@@ -1180,8 +1169,10 @@ enum Variant { kNone = 0, kMfmaD128 = 1, kGeneric = 2 };
 // The generic kernel runs one wave per item.
 constexpr int kNumCUs = 256;
 
-static int target_items(int variant_is_mfma) {
-  int v = variant_is_mfma ? 2 * kNumCUs : 8 * kNumCUs;
+// Work items to aim for: two 4-wave workgroups per CU for the 16-row MFMA kernel, four 2-wave
+// workgroups for the 32-row one, eight single waves for the generic kernel.
+static int target_items(int variant_is_mfma, int rows) {
+  int v = variant_is_mfma ? (rows > 16 ? 4 * kNumCUs : 2 * kNumCUs) : 8 * kNumCUs;
   if (const char* e = getenv("XLLM_HIP_DECODE_TARGET_ITEMS")) {
     const int t = atoi(e);
     if (t > 0) v = t;
@@ -1306,7 +1297,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
   p.log2_bs = is_pow2(c->block_size) ? ilog2(c->block_size) : 0;
   p.max_blocks_per_seq = a->max_blocks_per_seq;
   p.window_left = a->window_left;
-  p.target_items = target_items(variant == kMfmaD128);
+  p.target_items = target_items(variant == kMfmaD128, p.rows);
   // Only the MFMA kernel finishes single-chunk sequences itself.  When the caller's host-side
   // lengths (the reference keeps both in AttentionMetadata) show that the chunk the plan would
   // pick covers the longest sequence, no sequence is split: the plan is told never to split
@@ -1341,7 +1332,7 @@ static void launch_mfma(const DecodeParams& p, unsigned grid, hipStream_t st) {
   if (rows_per_item <= 16) {
     decode_mfma_d128_kernel<KV_DT><<<grid, 64 * kWaves, 0, st>>>(p);
   } else {
-    decode_mfma_d128_rows32_kernel<KV_DT><<<grid, 64 * kWaves, 0, st>>>(p);
+    decode_mfma_d128_rows32_kernel<KV_DT><<<grid, 128, 0, st>>>(p);
   }
 }
 
