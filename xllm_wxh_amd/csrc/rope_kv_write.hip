@@ -8,8 +8,10 @@
 //   call sites                                        xllm/core/layers/common/qwen2_attention.cpp:147-189
 //   cache write                                       the arithmetic of kv_write.hip
 //
-// One wave per (token, head).  The head's values go through LDS once so that a lane can pick up the
-// rotation partner of each of its elements whatever head_dim, rotary_dim and style are.
+// General kernel: one wave per (token, head); the head's values go through LDS once so that a lane
+// can pick up the rotation partner of each of its elements whatever head_dim, rotary_dim and style
+// are.  head_dim 128 with 2-byte elements (every current model on this path) takes a kernel with
+// sixteen lanes per head and 16-byte accesses instead.
 #include "device_utils.h"
 #include "host_utils.h"
 
@@ -212,6 +214,236 @@ __global__ void __launch_bounds__(256) rope_kv_write_kernel(RopeParams p) {
   }
 }
 
+// head_dim 128 with 2-byte elements: sixteen lanes per head, eight consecutive elements (16 bytes)
+// per lane, four heads per wave.  The rotation partner of a lane's elements sits in the lane
+// rotary_dim/16 further (NeoX pairs) or in the lane itself (interleaved pairs).  Same arithmetic as
+// the general kernel except for the order in which the squares are summed.
+template <int G>
+__device__ inline float group_sum(float v) {  // over G consecutive lanes (G a power of two)
+#pragma unroll
+  for (int o = G / 2; o >= 1; o >>= 1) v += __shfl_xor(v, o);
+  return v;
+}
+template <int G>
+__device__ inline float group_max(float v) {
+#pragma unroll
+  for (int o = G / 2; o >= 1; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+  return v;
+}
+
+template <int DT>
+__device__ inline void unpack8(const u32x4 raw, float (&x)[8]) {
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const uint32_t w = raw[e >> 1];
+    if (DT == XLLM_HIP_BF16) {
+      x[e] = __uint_as_float((e & 1) ? (w & 0xffff0000u) : (w << 16));
+    } else {
+      x[e] = (float)__builtin_bit_cast(_Float16, (uint16_t)((e & 1) ? (w >> 16) : (w & 0xffffu)));
+    }
+  }
+}
+template <int DT>
+__device__ inline u32x4 pack8(const float (&x)[8]) {
+  u32x4 r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    uint32_t lo, hi;
+    if (DT == XLLM_HIP_BF16) {
+      lo = float_to_bf16_bits(x[2 * i]);
+      hi = float_to_bf16_bits(x[2 * i + 1]);
+    } else {
+      lo = __builtin_bit_cast(uint16_t, (_Float16)x[2 * i]);
+      hi = __builtin_bit_cast(uint16_t, (_Float16)x[2 * i + 1]);
+    }
+    r[i] = lo | (hi << 16);
+  }
+  return r;
+}
+
+// Eight consecutive cos (or sin) values starting at element `idx` of the table.
+__device__ inline void load8_any(const void* p, int64_t idx, int dtype, float (&o)[8], int count) {
+  if (dtype == XLLM_HIP_FP32) {
+    const f32x4 a = *(const f32x4*)((const float*)p + idx);
+    const f32x4 b = count > 4 ? *(const f32x4*)((const float*)p + idx + 4) : a;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      o[e] = a[e];
+      o[4 + e] = b[e];
+    }
+  } else if (count > 4) {
+    const u32x4 raw = *(const u32x4*)((const uint16_t*)p + idx);
+    if (dtype == XLLM_HIP_BF16) {
+      unpack8<XLLM_HIP_BF16>(raw, o);
+    } else {
+      unpack8<XLLM_HIP_FP16>(raw, o);
+    }
+  } else {
+    const u32x2 r2 = *(const u32x2*)((const uint16_t*)p + idx);
+    const u32x4 raw = {r2[0], r2[1], 0, 0};
+    if (dtype == XLLM_HIP_BF16) {
+      unpack8<XLLM_HIP_BF16>(raw, o);
+    } else {
+      unpack8<XLLM_HIP_FP16>(raw, o);
+    }
+  }
+}
+
+template <int DT, int CACHE>
+__global__ void __launch_bounds__(256) rope_kv_write_d128_kernel(RopeParams p, int cache_vec_ok) {
+  const int sub = threadIdx.x & 15;
+  const int heads = p.num_q_heads + p.num_k_heads + p.num_v_heads;
+  const int64_t unit = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+  const bool live = unit < p.num_tokens * heads;  // idle groups still take part in the shuffles
+  const int64_t t = live ? unit / heads : 0;
+  const int hh = live ? (int)(unit - t * heads) : 0;
+  const bool is_q = hh < p.num_q_heads;
+  const bool is_v = hh >= p.num_q_heads + p.num_k_heads;
+  const int R = p.rotary_dim;
+  const int64_t base = t * p.token_stride + (int64_t)hh * 128 + 8 * sub;
+
+  float x[8];
+  u32x4 raw = {0, 0, 0, 0};
+  if (live) raw = *(const u32x4*)(p.qkv + base * 2);
+  unpack8<DT>(raw, x);
+
+  if (!is_v) {
+    const void* w = is_q ? p.q_weight : p.k_weight;
+    if (w != nullptr) {
+      float ss = 0.0f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += x[e] * x[e];
+      ss = group_sum<16>(ss);
+      const float rms = 1.0f / sqrtf(ss / 128.0f + p.eps);
+      float wv[8];
+      unpack8<DT>(*(const u32x4*)((const uint16_t*)w + 8 * sub), wv);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        x[e] *= rms * wv[e];
+        if (p.per_op) x[e] = rounded<DT>(x[e]);
+      }
+    }
+    int64_t pos = p.positions[t];
+    pos = pos < 0 ? 0 : (pos >= p.max_position ? p.max_position - 1 : pos);
+    const int half = R >> 1;
+    const int hl = R >> 4;  // lanes per half of the rotated range
+    float y[8];             // rotation partners
+    float c[8], sn[8];
+    bool first[8];
+    const bool rotates = 8 * sub < R;
+    if (p.interleave) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        y[e] = x[e ^ 1];
+        first[e] = (e & 1) == 0;
+      }
+      float c4[8], s4[8];
+      const int64_t f0 = pos * R + (rotates ? 4 * sub : 0);
+      load8_any(p.cos_sin, f0, p.cos_sin_dtype, c4, 4);
+      load8_any(p.cos_sin, f0 + half, p.cos_sin_dtype, s4, 4);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        c[e] = c4[e >> 1];
+        sn[e] = s4[e >> 1];
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        y[e] = __shfl_xor(x[e], hl);
+        first[e] = sub < hl;
+      }
+      const int fl = rotates ? (sub < hl ? sub : sub - hl) : 0;
+      load8_any(p.cos_sin, pos * R + 8 * fl, p.cos_sin_dtype, c, 8);
+      load8_any(p.cos_sin, pos * R + half + 8 * fl, p.cos_sin_dtype, sn, 8);
+    }
+    if (rotates) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float a = x[e], b = y[e];
+        if (p.per_op) {
+          const float cc = rounded<DT>(c[e]), ss2 = rounded<DT>(sn[e]);
+          const float ac = rounded<DT>(a * cc), bs = rounded<DT>(b * ss2);
+          x[e] = rounded<DT>(first[e] ? ac - bs : ac + bs);
+        } else {
+          x[e] = first[e] ? a * c[e] - b * sn[e] : b * sn[e] + a * c[e];
+        }
+      }
+    }
+    const u32x4 packed = pack8<DT>(x);
+    if (live) *(u32x4*)(p.qkv + base * 2) = packed;
+    unpack8<DT>(packed, x);  // the cache receives what a reader of qkv would see
+  }
+
+  if (CACHE == kNoCache) return;
+  int64_t slot = -1;
+  if (live && !is_q) slot = p.slots[t];
+  const bool writes = slot >= 0 && slot < p.num_slots;
+  const int64_t block = writes ? slot / p.block_size : 0;
+  const int64_t off = writes ? slot % p.block_size : 0;
+  const int h = is_v ? hh - p.num_q_heads - p.num_k_heads : hh - p.num_q_heads;
+  const int64_t row = block * p.stride_block + (int64_t)h * p.stride_head + off * p.stride_slot + 8 * sub;
+  uint8_t* cache = is_v ? p.v_cache : p.k_cache;
+  if (CACHE == kVerbatim) {
+    if (!writes) return;
+    const u32x4 packed = is_v ? raw : pack8<DT>(x);  // value rows are copied bit for bit
+    if (cache_vec_ok) {
+      *(u32x4*)(cache + row * 2) = packed;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ((uint16_t*)cache)[row + e] = (uint16_t)(packed[e >> 1] >> (16 * (e & 1)));
+    }
+    return;
+  }
+  float amax = 0.0f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(x[e]));
+  amax = group_max<16>(amax);
+  if (!writes) return;
+  constexpr float kQmax = CACHE == kInt8 ? 127.0f : 448.0f;
+  constexpr float kMinScale = CACHE == kInt8 ? FLT_EPSILON : 1.0f / (448.0f * 512.0f);
+  const float scale = fmaxf(amax / kQmax, kMinScale);
+  uint32_t q2[2] = {0, 0};
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float yv = x[e] / scale;
+    uint32_t q;
+    if (CACHE == kInt8) {
+      q = (uint8_t)(int8_t)(int)fminf(fmaxf(rintf(yv), -127.0f), 127.0f);
+    } else {
+      q = to_fp8_e4m3(yv);
+    }
+    q2[e >> 2] |= q << (8 * (e & 3));
+  }
+  if (cache_vec_ok) {
+    *(u32x2*)(cache + row) = u32x2{q2[0], q2[1]};
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) cache[row + e] = (uint8_t)(q2[e >> 2] >> (8 * (e & 3)));
+  }
+  if (sub == 0) {
+    float* sc = is_v ? p.v_scale : p.k_scale;
+    sc[block * p.sc_stride_block + (int64_t)h * p.sc_stride_head + off * p.sc_stride_slot] = scale;
+  }
+}
+
+template <int DT>
+static void launch_rope_d128(int cache_kind, const RopeParams& p, int cache_vec_ok, unsigned grid, hipStream_t st) {
+  switch (cache_kind) {
+    case kNoCache:
+      rope_kv_write_d128_kernel<DT, kNoCache><<<grid, 256, 0, st>>>(p, cache_vec_ok);
+      break;
+    case kVerbatim:
+      rope_kv_write_d128_kernel<DT, kVerbatim><<<grid, 256, 0, st>>>(p, cache_vec_ok);
+      break;
+    case kInt8:
+      rope_kv_write_d128_kernel<DT, kInt8><<<grid, 256, 0, st>>>(p, cache_vec_ok);
+      break;
+    default:
+      rope_kv_write_d128_kernel<DT, kFp8><<<grid, 256, 0, st>>>(p, cache_vec_ok);
+      break;
+  }
+}
+
 template <int DT>
 static void launch_rope(int cache_kind, const RopeParams& p, unsigned grid, hipStream_t st) {
   switch (cache_kind) {
@@ -313,8 +545,37 @@ extern "C" int xllm_hip_rope_kv_write(const xllm_hip_rope_args* a,
   }
   const int64_t units = a->num_tokens * (a->num_q_heads + a->num_k_heads + a->num_v_heads);
   XLLM_HIP_REQUIRE((units + 3) / 4 <= 0x7fffffff, "too many (token, head) pairs: %lld", (long long)units);
-  const unsigned grid = (unsigned)((units + 3) / 4);
   hipStream_t st = (hipStream_t)stream;
+  // The 16-lanes-per-head kernel: head_dim 128, 2-byte elements, rotary_dim a power of two from 16
+  // (so that the rotation partner is a fixed lane away), everything it reads on 16-byte boundaries.
+  // Whether it is used never depends on the cache, so a call with and one without a cache compute
+  // identical values; a cache whose rows are not 16-byte aligned is written element by element.
+  const int cs_eb = elem_bytes(a->cos_sin_dtype);
+  const bool d128 = a->head_dim == 128 && (a->dtype == XLLM_HIP_BF16 || a->dtype == XLLM_HIP_FP16) &&
+                    (a->rotary_dim == 16 || a->rotary_dim == 32 || a->rotary_dim == 64 || a->rotary_dim == 128) &&
+                    (((uintptr_t)a->qkv | (uintptr_t)a->q_weight | (uintptr_t)a->k_weight |
+                      (uintptr_t)a->cos_sin_cache) & 15) == 0 &&
+                    a->token_stride % 8 == 0 && (a->rotary_dim / 2 * cs_eb) % (a->interleave ? 8 : 16) == 0 &&
+                    (a->rotary_dim * cs_eb) % 16 == 0;
+  if (d128) {
+    int cache_vec_ok = 0;
+    if (cache != nullptr) {
+      const int ceb = elem_bytes(cache->dtype);
+      const int need = ceb == 1 ? 8 : 16;  // bytes a lane stores at once
+      cache_vec_ok = (((uintptr_t)cache->k_cache | (uintptr_t)cache->v_cache | (uintptr_t)(cache->stride_block * ceb) |
+                       (uintptr_t)(cache->stride_head * ceb) | (uintptr_t)(cache->stride_slot * ceb)) &
+                      (uintptr_t)(need - 1)) == 0;
+    }
+    XLLM_HIP_REQUIRE((units + 15) / 16 <= 0x7fffffff, "too many (token, head) pairs: %lld", (long long)units);
+    const unsigned g16 = (unsigned)((units + 15) / 16);
+    if (a->dtype == XLLM_HIP_BF16) {
+      launch_rope_d128<XLLM_HIP_BF16>(kind, p, cache_vec_ok, g16, st);
+    } else {
+      launch_rope_d128<XLLM_HIP_FP16>(kind, p, cache_vec_ok, g16, st);
+    }
+    return check_launch("rope_kv_write_d128_kernel");
+  }
+  const unsigned grid = (unsigned)((units + 3) / 4);
   switch (a->dtype) {
     case XLLM_HIP_BF16:
       launch_rope<XLLM_HIP_BF16>(kind, p, grid, st);
