@@ -200,8 +200,92 @@ extern "C" int xllm_hip_reshape_paged_cache(const xllm_hip_kv_cache* cache,
   return check_launch("reshape_paged_cache_kernel");
 }
 
+// head_dim 128 on aligned rows: sixteen lanes per (token, head, K|V), eight consecutive elements per
+// lane (one 16-byte load for 2-byte sources, two for fp32), one 8-byte store.  Same arithmetic as
+// above (a maximum does not depend on the order it is taken in).
+template <int SRC_DT, int DST_DT>
+__global__ void __launch_bounds__(256) quant_to_paged_cache_d128_kernel(KvWriteParams p) {
+  const int sub = threadIdx.x & 15;
+  const int64_t pair = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+  const bool live = pair < p.num_tokens * p.num_kv_heads;  // idle groups still take part in the shuffles
+  const bool is_v = blockIdx.y != 0;
+  const int64_t t = live ? pair / p.num_kv_heads : 0;
+  const int h = live ? (int)(pair - t * p.num_kv_heads) : 0;
+  const int64_t slot = live ? (int64_t)p.slots[t] : -1;
+  const bool writes = slot >= 0 && slot < p.num_slots;
+  const int64_t block = writes ? slot / p.block_size : 0;
+  const int64_t off = writes ? slot % p.block_size : 0;
+  const uint8_t* src = is_v ? p.value : p.key;
+  const int64_t src_base = t * (is_v ? p.value_token_stride : p.key_token_stride) + (int64_t)h * 128 + 8 * sub;
+  float x[8];
+  if (SRC_DT == XLLM_HIP_FP32) {
+    const f32x4 a = *(const f32x4*)(src + src_base * 4);
+    const f32x4 b = *(const f32x4*)(src + src_base * 4 + 16);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      x[e] = a[e];
+      x[4 + e] = b[e];
+    }
+  } else {
+    const u32x4 raw = *(const u32x4*)(src + src_base * 2);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const uint32_t w = raw[e >> 1];
+      if (SRC_DT == XLLM_HIP_BF16) {
+        x[e] = __uint_as_float((e & 1) ? (w & 0xffff0000u) : (w << 16));
+      } else {
+        x[e] = (float)__builtin_bit_cast(_Float16, (uint16_t)((e & 1) ? (w >> 16) : (w & 0xffffu)));
+      }
+    }
+  }
+  float amax = 0.0f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(x[e]));
+#pragma unroll
+  for (int o = 8; o >= 1; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+  if (!writes) return;
+  constexpr float kQmax = DST_DT == XLLM_HIP_INT8 ? 127.0f : 448.0f;
+  constexpr float kMinScale = DST_DT == XLLM_HIP_INT8 ? FLT_EPSILON : 1.0f / (448.0f * 512.0f);
+  const float scale = fmaxf(amax / kQmax, kMinScale);
+  uint32_t q2[2] = {0, 0};
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float y = x[e] / scale;
+    uint32_t q;
+    if (DST_DT == XLLM_HIP_INT8) {
+      q = (uint8_t)(int8_t)(int)fminf(fmaxf(rintf(y), -127.0f), 127.0f);
+    } else {
+      q = float_to_fp8_e4m3(y);
+    }
+    q2[e >> 2] |= q << (8 * (e & 3));
+  }
+  uint8_t* dst = (is_v ? p.v_cache : p.k_cache) + block * p.stride_block + (int64_t)h * p.stride_head +
+                 off * p.stride_slot + 8 * sub;
+  *(u32x2*)dst = u32x2{q2[0], q2[1]};
+  if (sub == 0) {
+    float* sc = is_v ? p.v_scale : p.k_scale;
+    sc[block * p.scale_stride_block + (int64_t)h * p.scale_stride_head + off * p.scale_stride_slot] = scale;
+  }
+}
+
 template <int SRC_DT>
 static void launch_quant(int dst_dtype, const KvWriteParams& p, dim3 grid, hipStream_t st) {
+  const int seb = SRC_DT == XLLM_HIP_FP32 ? 4 : 2;
+  const bool d128 = p.head_dim == 128 &&
+                    (((uintptr_t)p.key | (uintptr_t)p.value | (uintptr_t)(p.key_token_stride * seb) |
+                      (uintptr_t)(p.value_token_stride * seb)) & 15) == 0 &&
+                    (((uintptr_t)p.k_cache | (uintptr_t)p.v_cache | (uintptr_t)p.stride_block | (uintptr_t)p.stride_head |
+                      (uintptr_t)p.stride_slot) & 7) == 0;
+  if (d128) {
+    const int64_t pairs = p.num_tokens * p.num_kv_heads;
+    const dim3 g16((unsigned)((pairs + 15) / 16), grid.y);
+    if (dst_dtype == XLLM_HIP_INT8) {
+      quant_to_paged_cache_d128_kernel<SRC_DT, XLLM_HIP_INT8><<<g16, 256, 0, st>>>(p);
+    } else {
+      quant_to_paged_cache_d128_kernel<SRC_DT, XLLM_HIP_FP8_E4M3><<<g16, 256, 0, st>>>(p);
+    }
+    return;
+  }
   if (dst_dtype == XLLM_HIP_INT8) {
     quant_to_paged_cache_kernel<SRC_DT, XLLM_HIP_INT8><<<grid, 256, 0, st>>>(p);
   } else {
