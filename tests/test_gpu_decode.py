@@ -60,6 +60,28 @@ def test_mfma_decode_matches_oracle(gpu, shape, kv):
     _check(case)
 
 
+@pytest.mark.parametrize("kv", ["fp16", "fp8", "int8"])
+@pytest.mark.parametrize("shape", [SHAPES[1], SHAPES[2], SHAPES[7], SHAPES[9]],
+                         ids=lambda s: "B%d_Hq%d_n%d_L%d" % (s[0], s[1], s[6], max(s[5])))
+def test_mfma_decode_fp16_queries(gpu, shape, kv):
+    """fp16 queries and outputs: the MFMA kernels compute in fp16 (an fp16 cache as it is, e4m3 and
+    int8 caches converted exactly)."""
+    B, Hq, Hkv, D, bs, lens, n = shape
+    print("case mfma fp16", shape, kv, flush=True)
+    case = Case(B, Hq, Hkv, D, bs, lens, n=n, kv=kv, qdt="fp16", seed=12)
+    assert case.variant() == "mfma_d128"
+    out, _ = _check(case)
+    assert out.dtype == torch.float16
+
+
+def test_mixed_16_bit_types_take_the_generic_kernel(gpu):
+    print("case mixed 16-bit", flush=True)
+    for kv, qdt in (("bf16", "fp16"), ("fp16", "bf16")):
+        case = Case(2, 8, 2, 128, 16, [100, 33], kv=kv, qdt=qdt, seed=13)
+        assert case.variant() == "generic"
+        _check(case)
+
+
 @pytest.mark.parametrize("kv,qdt", [("bf16", "bf16"), ("fp32", "fp32"), ("fp16", "fp16"), ("fp8", "bf16"), ("int8", "bf16")])
 @pytest.mark.parametrize("shape", [
     (2, 14, 2, 64, 16, [300, 17], 1),

@@ -311,7 +311,7 @@ __global__ void __launch_bounds__(256) decode_merge_kernel(DecodeParams p) {
 }
 
 // ---------------------------------------------------------------------------------
-// MFMA kernels, head_dim 128, bf16 queries.  One workgroup of four waves per work item.
+// MFMA kernels, head_dim 128, bf16 or fp16 queries.  One workgroup of four waves per work item.
 //
 // A tile is 32 tokens.  Its K and V rows are fetched with fully coalesced 16-byte loads, parked
 // in LDS (row-major, 16-byte pieces XOR-swizzled by row so that every access pattern below is
@@ -384,15 +384,21 @@ __device__ inline HalfBase half_base(const DecodeParams& p, const Item& it, int 
   return b;
 }
 
+// Template tag of the MFMA kernels: the cache dtype, plus kQF16 when the queries (and outputs) are
+// fp16 rather than bf16.  An fp16 cache implies fp16 queries.
+constexpr int kQF16 = 64;
+constexpr int kv_of(int kt) { return kt & (kQF16 - 1); }
+constexpr bool qf16_of(int kt) { return (kt & kQF16) != 0 || kv_of(kt) == XLLM_HIP_FP16; }
+constexpr bool quant_of(int kt) { return kv_of(kt) == XLLM_HIP_FP8_E4M3 || kv_of(kt) == XLLM_HIP_INT8; }
+
 // KvHalf<KV>: the registers that hold 16 tokens (half a tile) of K and V in flight, the per-lane
 // geometry of their loads, and how they are parked in rows 16*h .. 16*h+15 of an LDS tile.
 template <int KV_DT>
 struct KvHalf;
 
-// bf16 cache: 8 loads of 16 bytes per lane (4 K + 4 V); a load instruction covers 4 rows:
+// bf16 / fp16 cache: 8 loads of 16 bytes per lane (4 K + 4 V); a load instruction covers 4 rows:
 // lane = (row-in-load, piece).
-template <>
-struct KvHalf<XLLM_HIP_BF16> {
+struct KvHalf16 {
   // Row 4j + lrow differs from row lrow only in bits the lane does not own, so its swizzled LDS
   // offset is the offset of row lrow with a j-dependent constant XORed in (plus j KiB): one register
   // per array instead of one per row.
@@ -443,13 +449,18 @@ struct KvHalf<XLLM_HIP_BF16> {
     }
   }
 };
+template <>
+struct KvHalf<XLLM_HIP_BF16> : KvHalf16 {};
+template <>
+struct KvHalf<XLLM_HIP_FP16> : KvHalf16 {};
 
-// The 16-bit type the MFMAs compute in.  bf16 and e4m3 caches use bf16 (both convert exactly).  An
-// int8 cache uses fp16, because a byte u = x + 128 becomes the fp16 number 1024 + u by a byte
-// permute alone (0x6400 | u), 0.75 instructions per element instead of 1.75 through float; the
-// kernel takes the offset 1152 = 1024 + 128 back out of the scores and of the output.
-template <int KV_DT>
-struct Mma {
+// The 16-bit type the MFMAs compute in: that of the queries (bf16 and e4m3 cache values convert to
+// either exactly) — except that an int8 cache always uses fp16, because a byte u = x + 128 becomes
+// the fp16 number 1024 + u by a byte permute alone (0x6400 | u), 0.75 instructions per element
+// instead of 1.75 through float; the kernel takes the offset 1152 = 1024 + 128 back out of the scores
+// and of the output, and bf16 queries are converted once per work item.
+template <bool F16>
+struct MmaOps {
   typedef bf16x8 Op;
   __device__ static inline f32x4 run(Op a, Op b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
@@ -459,7 +470,7 @@ struct Mma {
   }
 };
 template <>
-struct Mma<XLLM_HIP_INT8> {
+struct MmaOps<true> {
   typedef f16x8 Op;
   __device__ static inline f32x4 run(Op a, Op b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
@@ -468,6 +479,9 @@ struct Mma<XLLM_HIP_INT8> {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, f16x2));
   }
 };
+constexpr bool f16_ops(int kt) { return kv_of(kt) == XLLM_HIP_INT8 || qf16_of(kt); }
+template <int KV_DT>
+struct Mma : MmaOps<f16_ops(KV_DT)> {};
 constexpr float kInt8Offset = 1152.0f;
 
 // Convert 16 quantised bytes to 16 numbers of the MFMA operand type (two 16-byte pieces).
@@ -476,7 +490,10 @@ __device__ inline void dequant16(const u32x4 raw, u32x4& lo, u32x4& hi) {
   uint32_t o[8];
 #pragma unroll
   for (int w = 0; w < 4; ++w) {
-    if (KV_DT == XLLM_HIP_FP8_E4M3) {
+    if (kv_of(KV_DT) == XLLM_HIP_FP8_E4M3 && f16_ops(KV_DT)) {
+      o[2 * w] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(raw[w], 1.0f, false));
+      o[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(raw[w], 1.0f, true));
+    } else if (kv_of(KV_DT) == XLLM_HIP_FP8_E4M3) {
       o[2 * w] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)raw[w], 1.0f, false));
       o[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)raw[w], 1.0f, true));
     } else {
@@ -586,6 +603,10 @@ template <>
 struct KvHalf<XLLM_HIP_FP8_E4M3> : KvHalfQuant<XLLM_HIP_FP8_E4M3> {};
 template <>
 struct KvHalf<XLLM_HIP_INT8> : KvHalfQuant<XLLM_HIP_INT8> {};
+template <>
+struct KvHalf<XLLM_HIP_FP8_E4M3 | kQF16> : KvHalfQuant<XLLM_HIP_FP8_E4M3 | kQF16> {};
+template <>
+struct KvHalf<XLLM_HIP_INT8 | kQF16> : KvHalfQuant<XLLM_HIP_INT8 | kQF16> {};
 
 // max / sum over the four lanes (kg = 0..3) that share a query row: lanes l, l^16, l^32, l^48.
 // v_permlane16_swap exchanges the odd 16-lane rows of its first operand with the even rows of its
@@ -617,13 +638,13 @@ __device__ inline float kg_sum(float v) {
 // State of one wave's tile of 16 query rows, and the attention over one parked tile.
 template <int KV_DT>
 struct RowTile {
-  static constexpr bool kQuant = KV_DT != XLLM_HIP_BF16;
+  static constexpr bool kQuant = quant_of(KV_DT);
   // int8 rows sit in LDS as x + 1152.  With K' = K + 1152 and V' = V + 1152:
   //   q.K  = q.K' - 1152 * sum_d q_d                     the constant is the MFMA's initial C operand
   //   sum_t w_t V_t = sum_t w_t V'_t - 1152 * sum_t w_t   sum_t w_t comes from one more MFMA whose A
   //                                                       operand is all ones (wacc)
   // Rows zeroed because they lie past the sequence end carry weight 0 in both sums.
-  static constexpr bool kOffset = KV_DT == XLLM_HIP_INT8;
+  static constexpr bool kOffset = kv_of(KV_DT) == XLLM_HIP_INT8;
   typedef typename Mma<KV_DT>::Op Op;
 
   Op qf[4];        // Q^T fragments (B operand) of the lane's query row
@@ -654,17 +675,17 @@ struct RowTile {
     for (int c = 0; c < 4; ++c) {
       u32x4 raw = {0, 0, 0, 0};
       if (valid) raw = *(const u32x4*)(qrow + c * 32 + kg * 8);
-      const bf16x8 qb = __builtin_bit_cast(bf16x8, raw);
-      if constexpr (kOffset) {
-        // bf16 -> fp16 is exact for magnitudes in [2^-14, 65504]; smaller ones lose low bits only
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const _Float16 hq = (_Float16)(float)qb[e];
-          qf[c][e] = hq;
-          sq += (float)hq;
-        }
+      if constexpr (qf16_of(KV_DT) || !f16_ops(KV_DT)) {
+        qf[c] = __builtin_bit_cast(Op, raw);  // the queries already have the operand type
       } else {
-        qf[c] = __builtin_bit_cast(Op, qb);
+        // bf16 -> fp16 is exact for magnitudes in [2^-14, 65504]; smaller ones lose low bits only
+        const bf16x8 qb = __builtin_bit_cast(bf16x8, raw);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qf[c][e] = (_Float16)(float)qb[e];
+      }
+      if constexpr (kOffset) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sq += (float)qf[c][e];
       }
     }
     s_init = kOffset ? -kInt8Offset * kg_sum(sq) : 0.0f;
@@ -779,7 +800,7 @@ struct RowTile {
 template <int KV_DT, int TW>
 __device__ inline void finish_item(const DecodeParams& p, const Item& it, RowTile<KV_DT>& rt, uint8_t* xch_base,
                                    int xch_stride, float* lds_ml, int wave, int rs, int tw, int lane) {
-  constexpr bool kOffset = KV_DT == XLLM_HIP_INT8;
+  constexpr bool kOffset = kv_of(KV_DT) == XLLM_HIP_INT8;
   const float neg_inf = -INFINITY;
   const int mi = lane & 15, kg = lane >> 4;
   const int nhq = p.n * p.num_q_heads;
@@ -832,13 +853,13 @@ __device__ inline void finish_item(const DecodeParams& p, const Item& it, RowTil
     o_lo *= inv;
     o_hi *= inv;
     if (single) {
-      bf16x8 ob;
+      typename MmaOps<qf16_of(KV_DT)>::Op ob;  // the output has the queries' type
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        ob[e] = (__bf16)o_lo[e];
-        ob[4 + e] = (__bf16)o_hi[e];
+        ob[e] = (decltype(ob[0] + ob[0]))o_lo[e];
+        ob[4 + e] = (decltype(ob[0] + ob[0]))o_hi[e];
       }
-      *(bf16x8*)((uint16_t*)p.out + tok * p.out_token_stride + (int64_t)head * 128 + d0) = ob;
+      *(decltype(ob)*)((uint16_t*)p.out + tok * p.out_token_stride + (int64_t)head * 128 + d0) = ob;
     } else {
       float* po = p.partial_out + prow * 128 + d0;
       *(f32x4*)(po) = o_lo;
@@ -1184,9 +1205,11 @@ static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
 static Variant pick_variant(const xllm_hip_kv_cache* c, const xllm_hip_decode_args* a) {
   const int eb = elem_bytes(c->dtype);
-  const bool kv_ok = c->dtype == XLLM_HIP_BF16 || c->dtype == XLLM_HIP_FP8_E4M3 || c->dtype == XLLM_HIP_INT8;
+  // 16-bit queries; a 16-bit cache must have the queries' type
+  const bool q16 = a->q_dtype == XLLM_HIP_BF16 || a->q_dtype == XLLM_HIP_FP16;
+  const bool kv_ok = q16 && (c->dtype == a->q_dtype || c->dtype == XLLM_HIP_FP8_E4M3 || c->dtype == XLLM_HIP_INT8);
   const bool force_generic = getenv("XLLM_HIP_DECODE_FORCE_GENERIC") != nullptr;
-  if (!force_generic && c->head_dim == 128 && a->q_dtype == XLLM_HIP_BF16 && kv_ok && c->block_size >= 16 &&
+  if (!force_generic && c->head_dim == 128 && kv_ok && c->block_size >= 16 &&
       is_pow2(c->block_size)) {
     const int vec = 16 / eb;  // elements per 16-byte load
     const bool strides_ok = c->stride_block % vec == 0 && c->stride_head % vec == 0 && c->stride_slot % vec == 0 &&
@@ -1429,15 +1452,27 @@ extern "C" int xllm_hip_paged_decode_run_timed(const xllm_hip_kv_cache* cache,
     return fail(XLLM_HIP_RUNTIME_ERROR, "hipEventRecord(ev_begin) failed");
   }
   if (v == kMfmaD128) {
+    const bool qf16 = args->q_dtype == XLLM_HIP_FP16;
     switch (cache->dtype) {
       case XLLM_HIP_BF16:
         launch_mfma<XLLM_HIP_BF16>(p, grid, st);
         break;
+      case XLLM_HIP_FP16:
+        launch_mfma<XLLM_HIP_FP16>(p, grid, st);
+        break;
       case XLLM_HIP_FP8_E4M3:
-        launch_mfma<XLLM_HIP_FP8_E4M3>(p, grid, st);
+        if (qf16) {
+          launch_mfma<XLLM_HIP_FP8_E4M3 | kQF16>(p, grid, st);
+        } else {
+          launch_mfma<XLLM_HIP_FP8_E4M3>(p, grid, st);
+        }
         break;
       default:
-        launch_mfma<XLLM_HIP_INT8>(p, grid, st);
+        if (qf16) {
+          launch_mfma<XLLM_HIP_INT8 | kQF16>(p, grid, st);
+        } else {
+          launch_mfma<XLLM_HIP_INT8>(p, grid, st);
+        }
         break;
     }
   } else {
