@@ -73,6 +73,8 @@ struct DecodeParams {
   int32_t target_items;
   int32_t fixed_chunk;    // > 0: chunk size chosen on the host (1 << 30 = never split)
   int32_t direct_single;  // the attention kernel writes the output rows of single-chunk sequences itself
+  int32_t implicit_plan;  // nothing is split and nothing is merged: item = (sequence, kv head, row group),
+                          // lengths come straight from the inputs and no plan kernel runs
   int32_t q_dtype;
   float scale_log2;  // sm_scale * log2(e)
 };
@@ -209,14 +211,22 @@ struct Item {
 };
 
 __device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it) {
-  const PlanHeader hdr = *p.hdr;
-  if (item_id >= hdr.total_items) return false;
   it.rg = item_id % p.row_groups;
   const int rest = item_id / p.row_groups;
   it.hk = rest % p.num_kv_heads;
   it.sc = rest / p.num_kv_heads;
-  const SeqChunk s = p.seq_chunks[it.sc];
-  it.b = s.seq;
+  int chunk = 0, chunk_tokens = 1 << 30;
+  if (p.implicit_plan) {
+    if (it.sc >= p.batch) return false;
+    it.b = it.sc;
+  } else {
+    const PlanHeader hdr = *p.hdr;
+    if (item_id >= hdr.total_items) return false;
+    const SeqChunk s = p.seq_chunks[it.sc];
+    it.b = s.seq;
+    chunk = s.chunk;
+    chunk_tokens = hdr.chunk_tokens;
+  }
   if (p.q_indptr != nullptr) {
     it.q0 = p.q_indptr[it.b];
     const int cnt = p.q_indptr[it.b + 1] - it.q0;
@@ -226,9 +236,20 @@ __device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it)
     it.n = p.n;
   }
   if (it.rg * p.rows_per_item >= it.n * p.group) return false;  // this sequence has no rows in the group
-  it.len = p.kv_len[it.b];
-  it.t_begin = s.chunk * hdr.chunk_tokens;
-  const long long end = (long long)it.t_begin + hdr.chunk_tokens;
+  if (p.implicit_plan) {
+    int len;
+    if (p.kv_indptr != nullptr) {
+      const int nb = p.kv_indptr[it.b + 1] - p.kv_indptr[it.b];
+      len = nb > 0 ? (nb - 1) * p.block_size + p.kv_last_page_len[it.b] : 0;
+    } else {
+      len = p.seq_lens[it.b];
+    }
+    it.len = len > 0 ? len : 0;
+  } else {
+    it.len = p.kv_len[it.b];
+  }
+  it.t_begin = chunk * chunk_tokens;
+  const long long end = (long long)it.t_begin + chunk_tokens;
   it.t_end = end < it.len ? (int)end : it.len;
   if (p.kv_indptr != nullptr) {
     it.ids = p.block_ids + p.kv_indptr[it.b];
@@ -804,7 +825,7 @@ __device__ inline void finish_item(const DecodeParams& p, const Item& it, RowTil
   const float neg_inf = -INFINITY;
   const int mi = lane & 15, kg = lane >> 4;
   const int nhq = p.n * p.num_q_heads;
-  const bool single = p.direct_single != 0 && p.num_chunks[it.b] == 1;
+  const bool single = p.implicit_plan != 0 || (p.direct_single != 0 && p.num_chunks[it.b] == 1);
   const float l = kg_sum(rt.l_run);
   uint8_t* mine = xch_base + wave * xch_stride;
 #pragma unroll
@@ -1335,6 +1356,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
   // Many query rows per kv head (chunked prefill): the row groups supply the parallelism, and one
   // partial per chunk and row would be large, so nothing is split.
   if (never_split(a->q_per_seq, a->num_q_heads, c->num_kv_heads)) p.fixed_chunk = 1 << 30;
+  p.implicit_plan = p.direct_single && p.fixed_chunk == (1 << 30) ? 1 : 0;
   p.q_dtype = a->q_dtype;
   p.scale_log2 = a->sm_scale * 1.4426950408889634f;
   return XLLM_HIP_OK;
@@ -1416,7 +1438,7 @@ extern "C" int xllm_hip_paged_decode_plan(const xllm_hip_kv_cache* cache,
                                           xllm_hip_stream_t stream) {
   DecodeParams p;
   if (int s = fill_params(cache, args, workspace, workspace_bytes, p)) return s;
-  if (p.batch == 0) return XLLM_HIP_OK;
+  if (p.batch == 0 || p.implicit_plan) return XLLM_HIP_OK;  // an unsplit step needs no schedule
   decode_plan_kernel<<<1, 64, 0, (hipStream_t)stream>>>(p);
   return check_launch("decode_plan_kernel");
 }
@@ -1494,7 +1516,7 @@ extern "C" int xllm_hip_paged_decode_run_timed(const xllm_hip_kv_cache* cache,
   if (ev_end != nullptr && hipEventRecord((hipEvent_t)ev_end, st) != hipSuccess) {
     return fail(XLLM_HIP_RUNTIME_ERROR, "hipEventRecord(ev_end) failed");
   }
-  if (p.direct_single && p.fixed_chunk == (1 << 30)) return XLLM_HIP_OK;  // nothing was split: the outputs are final
+  if (p.implicit_plan) return XLLM_HIP_OK;  // nothing was split: the outputs are final
 
   const int64_t rows = (int64_t)p.batch * p.n * p.num_q_heads;
   const unsigned mgrid = (unsigned)((rows + 7) / 8);
