@@ -403,3 +403,28 @@ def test_decode_step_replays_under_hip_graph(gpu):
         assert torch.equal(k_after, k_cache)
         # some unrelated eager work between replays
         _ = (k_cache[:8].float() @ torch.ones(D, 4, device=gpu)).sum().item()
+
+
+@pytest.mark.parametrize("kv", ["bf16", "int8"])
+def test_long_context_single_sequence(gpu, kv):
+    """131072 cached tokens in one sequence: 64 chunks per kv head, merged."""
+    print("case long context", kv, flush=True)
+    case = Case(1, 32, 8, 128, 128, [131072], kv=kv, seed=31, std=0.5)
+    out, _ = _check(case)
+    out_h, _ = case.run(hints=True)
+    assert torch.equal(out, out_h)
+
+
+def test_large_batch_of_short_sequences(gpu):
+    """3000 sequences (the plan walks the batch 64 at a time), lengths 1..200, some empty."""
+    print("case large batch", flush=True)
+    rng = np.random.default_rng(3)
+    lens = rng.integers(1, 200, size=3000).astype(np.int32)
+    lens[::97] = 0
+    case = Case(3000, 32, 8, 128, 16, lens, seed=32)
+    ref, _ = case.oracle()
+    for hints in (False, True):
+        out, _ = case.run(hints=hints)
+        assert not torch.isnan(out.float()).any()
+        assert max_abs_err(out, ref) <= REG_TOL
+        assert float(out[::97].float().abs().max()) == 0.0  # empty sequences give zeros
