@@ -43,6 +43,8 @@ def parse_args():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain 1 GiB device-to-device copy a few times and exit: the known-size "
                          "kernel against which the rocprofv3 FETCH_SIZE / WRITE_SIZE counters are scaled")
+    ap.add_argument("--settle-ms", type=float, default=150.0,
+                    help="untimed steps run for this long before the warm-up steps (clock and TLB settling)")
     ap.add_argument("--aux", action="store_true",
                     help="time the kernels around the decode path instead (KV writes, norm + rotary embedding + "
                          "write, block copy, a chunked-prefill step) and print one JSON line of their own")
@@ -146,6 +148,15 @@ def main():
         b.record()
     handles = [(a.cuda_event, b.cuda_event) for a, b in ev]
 
+    # Let clocks and address translation settle first: right after the pools are generated the first
+    # ~100 launches of a step run up to 30 % slower than the steady state a serving loop sees.
+    t_settle = time.perf_counter()
+    i = 0
+    while (time.perf_counter() - t_settle) * 1e3 < args.settle_ms:
+        step(i)
+        i += 1
+        if i % 16 == 0:
+            torch.cuda.synchronize()
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()

@@ -97,6 +97,11 @@ __device__ inline void wave_scan2(int& a, int& b, int lane) {
 
 __global__ void __launch_bounds__(64) decode_plan_kernel(DecodeParams p) {
   const int lane = threadIdx.x;
+  // tails by size class: how many there are, then how many have been placed
+  __shared__ int tail_hist[64];
+  __shared__ int tail_fill[64];
+  tail_hist[lane] = 0;
+  tail_fill[lane] = 0;
 
   // 1. kv lengths, their sum and their maximum.
   long long total = 0;
@@ -138,6 +143,9 @@ __global__ void __launch_bounds__(64) decode_plan_kernel(DecodeParams p) {
     }
     return len > 0 ? len : 0;
   };
+  // The tail chunks differ in size.  They are dispatched after the (equal) full chunks, longest
+  // first — in 64 size classes — so that the launch ends with the shortest work items.
+  auto tail_class = [&](int tail_len) { return (int)(((long long)tail_len * 64) / chunk); };  // tail_len < chunk
   int total_full = 0, total_tail = 0;
   for (int base = 0; base < p.batch; base += 64) {
     const int b = base + lane;
@@ -146,17 +154,30 @@ __global__ void __launch_bounds__(64) decode_plan_kernel(DecodeParams p) {
       const int len = length_of(b);
       nf = len / chunk;
       nt = ((len - nf * chunk) > 0 || len == 0) ? 1 : 0;  // an empty sequence keeps one (empty) chunk: it writes zeros
+      if (nt) atomicAdd(&tail_hist[tail_class(len - nf * chunk)], 1);
     }
     int sf = nf, st = nt;
     wave_scan2(sf, st, lane);
     if (b < p.batch) {
       p.full_prefix[b] = total_full + sf - nf;
-      p.tail_prefix[b] = total_tail + st - nt;
       p.num_chunks[b] = nf + nt;
     }
     total_full += __shfl(sf, 63);
     total_tail += __shfl(st, 63);
   }
+  // first slot of size class `lane`: the number of tails in larger classes
+  int class_start = 0;
+  {
+    const int mine = tail_hist[lane];
+    int incl = mine;  // inclusive scan from the top: lanes 63, 62, ...
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int up = __shfl_down(incl, o);
+      if (lane + o < 64) incl += up;
+    }
+    class_start = incl - mine;
+  }
+  tail_hist[lane] = class_start;  // reused as the class offsets
   if (lane == 0) {
     p.full_prefix[p.batch] = total_full;
     p.tail_prefix[p.batch] = total_tail;
@@ -168,22 +189,27 @@ __global__ void __launch_bounds__(64) decode_plan_kernel(DecodeParams p) {
     *p.hdr = h;
   }
 
-  // 4. Chunk table: full chunks first, then the tails.
+  // 4. Chunk table: full chunks first, then the tails by decreasing size class.
   int run_full = 0, run_tail = 0;
   for (int base = 0; base < p.batch; base += 64) {
     const int b = base + lane;
-    int nf = 0, nt = 0;
+    int nf = 0, nt = 0, len_b = 0;
     if (b < p.batch) {
-      const int len = length_of(b);
-      nf = len / chunk;
-      nt = ((len - nf * chunk) > 0 || len == 0) ? 1 : 0;  // an empty sequence keeps one (empty) chunk: it writes zeros
+      len_b = length_of(b);
+      nf = len_b / chunk;
+      nt = ((len_b - nf * chunk) > 0 || len_b == 0) ? 1 : 0;  // an empty sequence keeps one (empty) chunk: it writes zeros
     }
     int sf = nf, st = nt;
     wave_scan2(sf, st, lane);
     if (b < p.batch) {
       const int f0 = run_full + sf - nf;
       for (int ci = 0; ci < nf; ++ci) p.seq_chunks[f0 + ci] = SeqChunk{b, ci};
-      if (nt) p.seq_chunks[total_full + run_tail + st - nt] = SeqChunk{b, nf};
+      if (nt) {
+        const int cls = tail_class(len_b - nf * chunk);
+        const int slot = tail_hist[cls] + atomicAdd(&tail_fill[cls], 1);
+        p.tail_prefix[b] = slot;
+        p.seq_chunks[total_full + slot] = SeqChunk{b, nf};
+      }
     }
     run_full += __shfl(sf, 63);
     run_tail += __shfl(st, 63);
