@@ -34,13 +34,15 @@ constexpr int kMaxRowsPerItem = 32;   // query rows (g * n) one work item of the
 #endif
 
 // Chunk size for a batch whose kv lengths sum to `total` with maximum `max_len`: split so that
-// about `target` work items exist — four times as many when the batch is ragged (longest sequence
-// above 1.5x the mean), because then the items differ in size and the dispatcher needs slack to
-// balance them.  Shared by the device-side plan and by the host's check that nothing is split.
+// about `target` work items exist — a quarter more when the batch is ragged (longest sequence above
+// 1.5x the mean): the tail chunks then differ in size, and although they are dispatched longest
+// first a little slack helps the last ones pack.  (Measured on the ragged workload: 512 to 900
+// items are equally good, 2000 items cost 4 %.)  Shared by the device-side plan and by the host's
+// check that nothing is split.
 XLLM_HIP_HD inline int choose_chunk(long long total, long long max_len, int batch, int num_kv_heads,
                                     int row_groups, int target, int min_chunk) {
   long long t = target;
-  if (max_len * batch * 2 > total * 3) t *= 4;
+  if (max_len * batch * 2 > total * 3) t += t / 4;
   if (t > kMaxTargetItems) t = kMaxTargetItems;
   const long long work = total * num_kv_heads * row_groups;
   long long c = (work + t - 1) / t;

@@ -1392,7 +1392,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
 static int64_t max_items(const DecodeParams& p) {
   const int64_t per = (int64_t)p.num_kv_heads * p.row_groups;
   if (p.fixed_chunk == (1 << 30)) return (int64_t)p.batch * per;
-  int64_t t = 4 * (int64_t)p.target_items;  // choose_chunk may quadruple the target
+  int64_t t = 2 * (int64_t)p.target_items;  // choose_chunk may raise the target (by a quarter)
   if (t > kMaxTargetItems) t = kMaxTargetItems;
   return (t / per + p.batch + 1) * per;
 }
