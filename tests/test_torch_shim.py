@@ -293,3 +293,71 @@ def test_attention_impl_chunked_prefill_step(gpu, shim, kv):
     err = float(np.abs(out.float().cpu().numpy().reshape(T, Hq, D) - ref).max())
     print("   err %.3e" % err, flush=True)
     assert err <= (5e-2 if kv == "int8" else 2e-2)
+
+
+@pytest.mark.gpu
+def test_forward_qkv_replays_under_hip_graph(gpu, shim):
+    """AttentionImpl::forward_qkv (norm + rotation + KV write, then decode) captured in a HIP graph and
+    replayed on changing persistent inputs; total_kv_len = 0 in the metadata keeps host-side lengths
+    out of the captured kernel choice.  Every replay is compared with an eager call."""
+    print("case shim graph", flush=True)
+    B, Hq, Hkv, D, bs, max_blocks = 4, 32, 8, 128, 16, 260
+    nblocks = B * max_blocks + 1
+    g = torch.Generator().manual_seed(61)
+    perm = (torch.randperm(nblocks - 1, generator=g) + 1).to(torch.int32)
+    table_full = perm[: B * max_blocks].view(B, max_blocks)
+    k_cache = torch.randn(nblocks, Hkv, bs, D, generator=g).to(torch.bfloat16).to(gpu)
+    v_cache = torch.randn(nblocks, Hkv, bs, D, generator=g).to(torch.bfloat16).to(gpu)
+    theta = torch.rand(8192, D // 2, generator=g) * 6.283
+    cos_sin = torch.cat([torch.cos(theta), torch.sin(theta)], 1).to(torch.bfloat16).to(gpu)
+    # persistent inputs
+    qkv = torch.zeros(B, (Hq + 2 * Hkv) * D, dtype=torch.bfloat16, device=gpu)
+    qkv_src = torch.zeros_like(qkv)
+    positions = torch.zeros(B, dtype=torch.int64, device=gpu)
+    slots = torch.zeros(B, dtype=torch.int32, device=gpu)
+    kv_cu = torch.zeros(B + 1, dtype=torch.int32, device=gpu)
+    q_cu = torch.arange(B + 1, dtype=torch.int32, device=gpu)
+    block_table = table_full.to(gpu).contiguous()
+    md = shim.build_decode_metadata(q_cu, kv_cu, slots, block_table, 1, max_blocks * bs, 0)
+    kv_seq_lens = torch.ones(B, dtype=torch.int32, device=gpu)
+    md.kv_seq_lens = kv_seq_lens  # persistent, refreshed in place before every replay
+    attn = shim.AttentionImpl(Hq, D, 1.0 / float(np.sqrt(D)), Hkv, -1)
+    cache = shim.KVCache(k_cache, v_cache)
+
+    def load_inputs(lens, seed):
+        gg = torch.Generator().manual_seed(seed)
+        qkv_src.copy_(torch.randn(B, (Hq + 2 * Hkv) * D, generator=gg).to(torch.bfloat16))
+        lens_t = torch.tensor(lens, dtype=torch.int32)
+        pos = lens_t - 1
+        blk = table_full[torch.arange(B), (pos // bs).long()]
+        slots.copy_((blk * bs + pos % bs).to(torch.int32))
+        positions.copy_(pos.to(torch.int64))
+        kv_seq_lens.copy_(lens_t)
+
+    def step():
+        qkv.copy_(qkv_src)  # forward_qkv rotates in place
+        return attn.forward_qkv(md, positions, qkv, cos_sin, False, None, None, 0.0, cache)[0]
+
+    load_inputs([100, 20, 4000, 1], 0)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_graph = step()
+    for it, lens in enumerate(([100, 20, 4000, 1], [4100, 3, 17, 2048], [5, 5, 5, 5])):
+        load_inputs(lens, 20 + it)
+        k_before, v_before = k_cache.clone(), v_cache.clone()
+        graph.replay()
+        torch.cuda.synchronize()
+        got, k_after = out_graph.clone(), k_cache.clone()
+        k_cache.copy_(k_before)
+        v_cache.copy_(v_before)
+        eager = step()
+        torch.cuda.synchronize()
+        assert torch.equal(got, eager), "replay %d differs from eager" % it
+        assert torch.equal(k_after, k_cache)
+        _ = (k_cache[:8].float() @ torch.ones(D, 4, device=gpu)).sum().item()
