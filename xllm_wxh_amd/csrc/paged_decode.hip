@@ -1,14 +1,16 @@
 // Paged-attention decode for gfx950 (MI355X): split-KV ("flash decoding") over
-// block_tables / seq_lens with GQA, bf16 / fp8-e4m3 / int8 KV caches.
+// block_tables / seq_lens with GQA, bf16 / fp16 / fp8-e4m3 / int8 KV caches, one or several query
+// tokens per sequence (decode, speculative verify, prefill chunks).
 //
 // Launches per call, none of which reads anything back to the host:
 //   decode_plan_kernel   kv lengths -> chunk size, chunk table (one wave; once per step)
-//   decode_*_kernel      one workgroup per (sequence chunk, kv head, row group): its waves split
-//                        the chunk, stream its K and V once and combine their results through
-//                        LDS; a sequence that is a single chunk gets its output rows written
-//                        directly, otherwise a normalised partial + log2-sum-exp is written
-//   decode_merge_kernel  combines the partials of the sequences that were split; skipped when
-//                        the host-side length hints show that no sequence is split
+//   decode_*_kernel      one workgroup per (sequence chunk, kv head, row group): its waves stream
+//                        the chunk's K and V once; a sequence that is a single chunk gets its
+//                        output rows written directly, otherwise a normalised partial +
+//                        log2-sum-exp is written
+//   decode_merge_kernel  combines the partials of the sequences that were split
+// When the host-side length hints show that no sequence needs splitting, only the middle one is
+// launched: a work item is then (sequence, kv head, row group) and needs no schedule.
 //
 // Semantics follow the reference's decode operators: head map kv = h / (Hq/Hkv)
 // and fp32 softmax as in xllm/core/layers/cuda/flashinfer_attention.cpp:61-88, the
@@ -358,7 +360,7 @@ __global__ void __launch_bounds__(256) decode_merge_kernel(DecodeParams p) {
 }
 
 // ---------------------------------------------------------------------------------
-// MFMA kernels, head_dim 128, bf16 or fp16 queries.  One workgroup of four waves per work item.
+// MFMA kernels, head_dim 128, bf16 or fp16 queries.  One workgroup per work item.
 //
 // A tile is 32 tokens.  Its K and V rows are fetched with fully coalesced 16-byte loads, parked
 // in LDS (row-major, 16-byte pieces XOR-swizzled by row so that every access pattern below is
@@ -370,21 +372,20 @@ __global__ void __launch_bounds__(256) decode_merge_kernel(DecodeParams p) {
 // softmax statistics are per-lane scalars.  Query rows r = j*g + gq (draft token j, head gq of
 // the group) fill the 16 columns of an MFMA tile; a wave owns one such tile of rows.
 //
-// decode_mfma_d128_kernel        up to 16 rows per item: the four waves take a quarter of the
-//                                item's tokens each, stage their tiles privately and meet only
+// decode_mfma_d128_kernel        up to 16 rows per item, four waves: each takes a quarter of the
+//                                item's tokens, stages its tiles privately, and they meet only
 //                                at the end.
-// decode_mfma_d128_rows32_kernel up to 32 rows per item: waves 0-1 own rows 0-15, waves 2-3 rows
-//                                16-31; a wave of each pair takes half of the tokens and the two
-//                                waves that share tokens also share the LDS tile — each fetches
-//                                and parks 16 of its 32 rows, then both read all of it — so K and
-//                                V still cross HBM once.
+// decode_mfma_d128_rows32_kernel up to 32 rows per item, two waves: wave w owns rows 16w .. 16w+15,
+//                                both walk all tokens of the item and share the LDS tile — each
+//                                fetches and parks 16 of its 32 rows, then both read all of it —
+//                                so K and V still cross HBM once.
 // ---------------------------------------------------------------------------------
 
 constexpr int kLdsK = 0;
 constexpr int kLdsV = 8192;
 constexpr int kLdsSc = 16384;    // per-token factors of a quantised tile: three arrays of 32 floats
 constexpr int kLdsTile = 16768;  // one 32-token tile of K and V as 16-bit numbers, plus the factors
-constexpr int kWaves = 4;        // waves per work item
+constexpr int kWaves = 4;        // waves per work item of the 16-row kernel
 constexpr int kXchRow = 528;     // bytes per query row in the end-of-item exchange (128 floats + 16 pad)
 
 __device__ inline u32x4 ldg_stream(const void* p) {
