@@ -336,7 +336,17 @@ def aux_kernels(torch, ops, device):
     flops = 4.0 * B * Hq * D * sum(L - n + 1 + j for j in range(n))
     res["entries"].append({"kernel": "chunked prefill through the decode kernel, 4 x 512 tokens on a 3584-token prefix",
                            "us": round(us, 1), "tflops": round(flops / us / 1e6, 1),
-                           "note": "untuned: every 32 query rows stream the sequence's K/V again"})
+                           "note": "every 32 query rows stream the sequence's K/V again, from the L2 of their XCD"})
+    # speculative verify with 64 query rows per kv head (64 q heads, 8 draft tokens): two row groups
+    B, n, L, Hq2 = 32, 8, 8192, 64
+    q = torch.randn(B * n, Hq2, D, device=device, dtype=torch.bfloat16, generator=gen)
+    out = torch.empty_like(q)
+    table = torch.randperm(nb, device=device, generator=gen)[: B * (L // bs)].to(torch.int32).view(B, L // bs)
+    lens = torch.full((B,), L, device=device, dtype=torch.int32)
+    us = timed(lambda: ops.batch_decode(q, kc, out, table, lens, vc, scale=D ** -0.5, q_per_seq=n, max_seq_len=L,
+                                        total_kv_len=B * L), n=20)
+    add("verify, 64 rows per kv head (2 row groups), 32 x 8192 tokens bf16", us, B * L * Hkv * D * 2 * 2,
+        "K/V bytes counted once; the second row group is meant to hit the XCD's L2")
     return res
 
 

@@ -238,9 +238,22 @@ struct Item {
   int64_t sc_head_off;  // hk * sc_stride_head (scale elements)
 };
 
+constexpr int kXcds = 8;  // workgroup x runs on XCD x % 8, each with its own L2
+
 __device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it) {
-  it.rg = item_id % p.row_groups;
-  const int rest = item_id / p.row_groups;
+  // With several row groups the same K/V is streamed once per group.  Consecutive workgroup ids land
+  // on different XCDs, so the groups of one (sequence chunk, kv head) are given ids that are
+  // congruent mod 8 and consecutive on that XCD: they then run there at about the same time and all
+  // but the first find the K/V in that XCD's L2.
+  int rest;
+  if (p.row_groups > 1) {
+    const int on_xcd = item_id / kXcds;
+    it.rg = on_xcd % p.row_groups;
+    rest = (on_xcd / p.row_groups) * kXcds + item_id % kXcds;
+  } else {
+    it.rg = 0;
+    rest = item_id;
+  }
   it.hk = rest % p.num_kv_heads;
   it.sc = rest / p.num_kv_heads;
   int chunk = 0, chunk_tokens = 1 << 30;
@@ -249,7 +262,7 @@ __device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it)
     it.b = it.sc;
   } else {
     const PlanHeader hdr = *p.hdr;
-    if (item_id >= hdr.total_items) return false;
+    if (rest * p.row_groups >= hdr.total_items) return false;
     const SeqChunk s = p.seq_chunks[it.sc];
     it.b = s.seq;
     chunk = s.chunk;
@@ -1392,10 +1405,15 @@ static int fill_params(const xllm_hip_kv_cache* c,
 // Upper bound of the work-item count for any lengths (see workspace_layout).
 static int64_t max_items(const DecodeParams& p) {
   const int64_t per = (int64_t)p.num_kv_heads * p.row_groups;
-  if (p.fixed_chunk == (1 << 30)) return (int64_t)p.batch * per;
-  int64_t t = 2 * (int64_t)p.target_items;  // choose_chunk may raise the target (by a quarter)
-  if (t > kMaxTargetItems) t = kMaxTargetItems;
-  return (t / per + p.batch + 1) * per;
+  int64_t seq_chunks = p.batch;
+  if (p.fixed_chunk != (1 << 30)) {
+    int64_t t = 2 * (int64_t)p.target_items;  // choose_chunk may raise the target (by a quarter)
+    if (t > kMaxTargetItems) t = kMaxTargetItems;
+    seq_chunks = t / per + p.batch + 1;
+  }
+  int64_t pairs = seq_chunks * p.num_kv_heads;  // (sequence chunk, kv head)
+  if (p.row_groups > 1) pairs = (pairs + kXcds - 1) / kXcds * kXcds;  // see decode_item
+  return pairs * p.row_groups;
 }
 
 template <int KV_DT>
