@@ -65,6 +65,7 @@ struct DecodeParams {
   int32_t group;  // q heads per kv head
   int32_t rows;   // group * n
   int32_t row_groups;
+  int32_t cluster;        // neighbouring work items kept on one XCD (see decode_item)
   int32_t rows_per_item;  // query rows one work item handles (32 MFMA, 1 generic)
   int32_t min_chunk;      // smallest chunk the plan may choose
   int32_t head_dim;
@@ -241,19 +242,19 @@ struct Item {
 constexpr int kXcds = 8;  // workgroup x runs on XCD x % 8, each with its own L2
 
 __device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it) {
-  // With several row groups the same K/V is streamed once per group.  Consecutive workgroup ids land
-  // on different XCDs, so the groups of one (sequence chunk, kv head) are given ids that are
-  // congruent mod 8 and consecutive on that XCD: they then run there at about the same time and all
-  // but the first find the K/V in that XCD's L2.
-  int rest;
-  if (p.row_groups > 1) {
+  // Work items in their natural order are (sequence chunk, kv head, row group), row group fastest.
+  // Some neighbours in that order read the same memory: the row groups of one (chunk, kv head) stream
+  // the same K/V, and with small blocks the scale rows of neighbouring kv heads share cache lines.
+  // Consecutive workgroup ids land on different XCDs, so a cluster of `p.cluster` neighbours is
+  // given ids that are congruent mod 8 and consecutive on that XCD: its members then run there at
+  // about the same time, and all but the first find the shared lines in that XCD's L2.
+  int linear = item_id;
+  if (p.cluster > 1) {
     const int on_xcd = item_id / kXcds;
-    it.rg = on_xcd % p.row_groups;
-    rest = (on_xcd / p.row_groups) * kXcds + item_id % kXcds;
-  } else {
-    it.rg = 0;
-    rest = item_id;
+    linear = ((on_xcd / p.cluster) * kXcds + item_id % kXcds) * p.cluster + on_xcd % p.cluster;
   }
+  it.rg = linear % p.row_groups;
+  const int rest = linear / p.row_groups;
   it.hk = rest % p.num_kv_heads;
   it.sc = rest / p.num_kv_heads;
   int chunk = 0, chunk_tokens = 1 << 30;
@@ -1397,6 +1398,14 @@ static int fill_params(const xllm_hip_kv_cache* c,
   // partial per chunk and row would be large, so nothing is split.
   if (never_split(a->q_per_seq, a->num_q_heads, c->num_kv_heads)) p.fixed_chunk = 1 << 30;
   p.implicit_plan = p.direct_single && p.fixed_chunk == (1 << 30) ? 1 : 0;
+  // XCD clusters: the row groups of a (chunk, kv head); and, for a quantised cache whose scale rows
+  // are shorter than a 128-byte line and contiguous over the heads, the heads that share a line.
+  int heads_per_line = 1;
+  if (quant && c->scale_stride_slot == 1 && c->scale_stride_head == c->block_size && c->block_size * 4 < 128) {
+    heads_per_line = 128 / (c->block_size * 4);
+    while (heads_per_line > 1 && c->num_kv_heads % heads_per_line != 0) heads_per_line >>= 1;
+  }
+  p.cluster = p.row_groups * heads_per_line;
   p.q_dtype = a->q_dtype;
   p.scale_log2 = a->sm_scale * 1.4426950408889634f;
   return XLLM_HIP_OK;
@@ -1411,9 +1420,12 @@ static int64_t max_items(const DecodeParams& p) {
     if (t > kMaxTargetItems) t = kMaxTargetItems;
     seq_chunks = t / per + p.batch + 1;
   }
-  int64_t pairs = seq_chunks * p.num_kv_heads;  // (sequence chunk, kv head)
-  if (p.row_groups > 1) pairs = (pairs + kXcds - 1) / kXcds * kXcds;  // see decode_item
-  return pairs * p.row_groups;
+  int64_t items = seq_chunks * per;
+  if (p.cluster > 1) {  // whole clusters, eight at a time (see decode_item)
+    const int64_t clusters = (items + p.cluster - 1) / p.cluster;
+    items = (clusters + kXcds - 1) / kXcds * kXcds * p.cluster;
+  }
+  return items;
 }
 
 template <int KV_DT>
