@@ -111,6 +111,10 @@ def test_variant_selection_is_host_only(lib):
     assert lib.xllm_hip_paged_decode_variant(ctypes.byref(desc), ctypes.byref(args)) == b"mfma_d128"
     desc.head_dim = 64
     assert lib.xllm_hip_paged_decode_variant(ctypes.byref(desc), ctypes.byref(args)) == b"generic"
+    # head_dim 64 with contiguous tokens and blocks of at least 32 tokens has an MFMA path of its own
+    desc.block_size, desc.stride_block, desc.stride_head, desc.stride_slot = 32, 8 * 32 * 64, 32 * 64, 64
+    assert lib.xllm_hip_paged_decode_variant(ctypes.byref(desc), ctypes.byref(args)) == b"mfma_d64"
+    desc.block_size, desc.stride_block, desc.stride_head, desc.stride_slot = 16, 8 * 16 * 128, 16 * 128, 128
     desc.head_dim, desc.dtype = 128, _lib.FP32
     assert lib.xllm_hip_paged_decode_variant(ctypes.byref(desc), ctypes.byref(args)) == b"generic"
     desc.head_dim = 512

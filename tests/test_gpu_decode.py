@@ -74,6 +74,48 @@ def test_mfma_decode_fp16_queries(gpu, shape, kv):
     assert out.dtype == torch.float16
 
 
+SHAPES_D64 = [
+    # B, Hq, Hkv, D, bs, lens, n
+    (4, 32, 8, 64, 32, [1, 2, 63, 65], 1),          # odd lengths: the second token of the last row is masked
+    (3, 32, 8, 64, 32, [4096, 777, 128], 1),        # chunk boundaries of the split
+    (3, 14, 2, 64, 128, [4097, 129, 64], 1),        # g = 7
+    (2, 64, 8, 64, 64, [3001, 517], 4),             # 32 query rows per kv head: the two-wave kernel
+    (2, 64, 4, 64, 32, [700, 91], 4),               # two row groups
+    (3, 32, 8, 64, 32, [5, 2, 3], 2),               # draft tokens at the very start of a sequence
+]
+
+
+@pytest.mark.parametrize("kv,qdt", [("bf16", "bf16"), ("fp8", "bf16"), ("int8", "bf16"), ("fp16", "fp16"), ("int8", "fp16")])
+@pytest.mark.parametrize("shape", SHAPES_D64, ids=lambda s: "B%d_Hq%d_Hkv%d_bs%d_n%d_L%d" % (s[0], s[1], s[2], s[4], s[6], max(s[5])))
+def test_mfma_decode_head_dim_64(gpu, shape, kv, qdt):
+    """head_dim 64 runs on the MFMA kernels with two tokens per tile row."""
+    B, Hq, Hkv, D, bs, lens, n = shape
+    print("case mfma d64", shape, kv, qdt, flush=True)
+    case = Case(B, Hq, Hkv, D, bs, lens, n=n, kv=kv, qdt=qdt, seed=21)
+    assert case.variant() == "mfma_d64"
+    _check(case)
+
+
+def test_head_dim_64_falls_back_when_tokens_are_not_contiguous(gpu):
+    print("case d64 layouts", flush=True)
+    # NHD with several kv heads: a token's row is followed by the other heads' rows
+    case = Case(2, 8, 2, 64, 32, [100, 33], layout="NHD", seed=22)
+    assert case.variant() == "generic"
+    _check(case)
+    # block_size 16: half a tile would straddle two blocks
+    case = Case(2, 8, 2, 64, 16, [100, 33], seed=22)
+    assert case.variant() == "generic"
+    _check(case)
+
+
+def test_head_dim_64_sliding_window(gpu):
+    print("case d64 window", flush=True)
+    for kv in ("bf16", "int8"):
+        case = Case(2, 32, 8, 64, 32, [3000, 517], n=2, kv=kv, seed=23)
+        assert case.variant() == "mfma_d64"
+        _check(case, window_left=301)
+
+
 def test_mixed_16_bit_types_take_the_generic_kernel(gpu):
     print("case mixed 16-bit", flush=True)
     for kv, qdt in (("bf16", "fp16"), ("fp16", "bf16")):

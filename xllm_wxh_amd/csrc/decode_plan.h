@@ -21,7 +21,7 @@
 
 namespace xllm_hip {
 
-constexpr int kTileTokens = 32;       // tokens per MFMA tile; chunk sizes are multiples of it
+constexpr int kTileTokens = 32;       // rows per MFMA tile (one token each, two at head_dim 64); chunk sizes are multiples of a tile
 constexpr int kMinChunkTokens = 512;  // smallest split worth a partial round trip (128 tokens per wave)
 constexpr int kMinChunkTokensGeneric = 64;  // the one-wave kernel: one 64-token step
 constexpr int kMaxTargetItems = 4096; // upper bound of the split target (sizes the workspace)
@@ -40,13 +40,13 @@ constexpr int kMaxRowsPerItem = 32;   // query rows (g * n) one work item of the
 // items are equally good, 2000 items cost 4 %.)  Shared by the device-side plan and by the host's
 // check that nothing is split.
 XLLM_HIP_HD inline int choose_chunk(long long total, long long max_len, int batch, int num_kv_heads,
-                                    int row_groups, int target, int min_chunk) {
+                                    int row_groups, int target, int min_chunk, int tile = kTileTokens) {
   long long t = target;
   if (max_len * batch * 2 > total * 3) t += t / 4;
   if (t > kMaxTargetItems) t = kMaxTargetItems;
   const long long work = total * num_kv_heads * row_groups;
   long long c = (work + t - 1) / t;
-  c = (c + kTileTokens - 1) / kTileTokens * kTileTokens;
+  c = (c + tile - 1) / tile * tile;
   if (c < min_chunk) c = min_chunk;
   if (c > (1 << 30)) c = 1 << 30;
   return (int)c;

@@ -69,6 +69,8 @@ struct DecodeParams {
   int32_t rows_per_item;  // query rows one work item handles (32 MFMA, 1 generic)
   int32_t min_chunk;      // smallest chunk the plan may choose
   int32_t head_dim;
+  int32_t tok;          // tokens per 256-byte LDS row of the MFMA kernels: 1 (head_dim 128) or 2 (head_dim 64)
+  int32_t tile_tokens;  // tokens per tile: 32 * tok; chunk sizes are multiples of it
   int32_t block_size;
   int32_t log2_bs;
   int32_t max_blocks_per_seq;
@@ -132,7 +134,8 @@ __global__ void __launch_bounds__(64) decode_plan_kernel(DecodeParams p) {
   // 2. Chunk size.
   const int chunk = p.fixed_chunk > 0
                         ? p.fixed_chunk
-                        : choose_chunk(total, max_len, p.batch, p.num_kv_heads, p.row_groups, p.target_items, p.min_chunk);
+                        : choose_chunk(total, max_len, p.batch, p.num_kv_heads, p.row_groups, p.target_items, p.min_chunk,
+                                       p.tile_tokens);
 
   // 3. Prefix sums of the full-chunk and tail-chunk counts (lengths are re-derived rather than
   //    re-read so that no lane depends on another lane's global store).
@@ -397,8 +400,8 @@ __global__ void __launch_bounds__(256) decode_merge_kernel(DecodeParams p) {
 
 constexpr int kLdsK = 0;
 constexpr int kLdsV = 8192;
-constexpr int kLdsSc = 16384;    // per-token factors of a quantised tile: three arrays of 32 floats
-constexpr int kLdsTile = 16768;  // one 32-token tile of K and V as 16-bit numbers, plus the factors
+constexpr int kLdsSc = 16384;    // per-token factors of a quantised tile: three arrays of up to 64 floats
+constexpr int kLdsTile = 17152;  // one tile of K and V as 16-bit numbers (32 rows of 256 bytes each), plus the factors
 constexpr int kWaves = 4;        // waves per work item of the 16-row kernel
 constexpr int kXchRow = 528;     // bytes per query row in the end-of-item exchange (128 floats + 16 pad)
 
@@ -469,10 +472,14 @@ struct KvHalf16 {
     uint32_t wk;     // LDS offset of K row lrow, piece
     uint32_t wv;     // LDS offset of V row lrow, piece
     int lrow;
+    int tok;         // tokens per row
+    int second;      // 1 if this lane's piece belongs to the second token of its row
     __device__ inline void init(const DecodeParams& p, int lane) {
       lrow = lane >> 4;
       const int piece = lane & 15;
-      g_off = (uint32_t)((lrow * p.stride_slot + piece * 8) * 2);
+      tok = p.tok;
+      second = tok == 2 && piece >= 8 ? 1 : 0;
+      g_off = (uint32_t)((lrow * p.stride_slot * p.tok + piece * 8) * 2);
       wk = kLdsK + swz_k(lrow, piece);
       wv = kLdsV + swz_v(lrow, piece);
     }
@@ -491,7 +498,7 @@ struct KvHalf16 {
     const HalfBase b = half_base(p, it, tok, blk);
     const uint8_t* kb = p.k_cache + b.elem * 2;
     const uint8_t* vb = p.v_cache + b.elem * 2;
-    const int64_t step = 4 * p.stride_slot * 2;  // four rows further, in bytes (uniform)
+    const int64_t step = 4 * p.stride_slot * p.tok * 2;  // four rows further, in bytes (uniform)
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       k[j] = ldg_stream(kb + j * step + g.g_off);
@@ -505,7 +512,7 @@ struct KvHalf16 {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       u32x4 vv = v[j];
-      if (MASKED && tok + 4 * j + g.lrow >= len) vv = u32x4{0, 0, 0, 0};
+      if (MASKED && tok + g.tok * (4 * j + g.lrow) + g.second >= len) vv = u32x4{0, 0, 0, 0};
       *(u32x4*)(tile + g.k_row(j, h)) = k[j];
       *(u32x4*)(tile + g.v_row(j, h)) = vv;
     }
@@ -592,24 +599,33 @@ struct KvHalfQuant {
     uint32_t wv;      // LDS offset of V row vrow, piece 2 * chunk
     uint32_t sc_g;    // byte offset of this lane's scale from the scale of the first of the 16 tokens
     uint32_t sc_lds;  // where kscl / lv is parked (before adding 64 bytes for the second half of the tile)
+    uint32_t sc_half; // bytes between the two halves of a tile in each scale array
+    uint32_t sc_next; // bytes from one scale array to the next
     int vrow;
-    int sc_tok;       // token (of the 16) whose scale this lane carries
-    bool sc_on;       // lanes 0..31 carry a scale
+    int tok;          // tokens per row
+    int second;       // 1 if this lane's chunk belongs to the second token of its row
+    int sc_tok;       // token (of the 16 * tok) whose scale this lane carries
+    bool sc_on;       // lanes 0 .. 32 * tok - 1 carry a scale: first the K scales, then the V scales
     bool sc_is_v;
     __device__ inline void init(const DecodeParams& p, int lane) {
       const int chunk = 4 * ((lane >> 3) & 1) + (lane & 3);
       const int pair = (lane >> 2) & 1;
       const int krow = 2 * (lane >> 4) + pair;  // rows r, r+1 alternate between quads (krow < 8)
       vrow = (lane >> 4) + 8 * pair;            // rows r, r+8 alternate between quads (vrow & 7 < 4)
-      gk_off = (uint32_t)(krow * p.stride_slot + chunk * 16);
-      gv_off = (uint32_t)(vrow * p.stride_slot + chunk * 16);
+      tok = p.tok;
+      second = tok == 2 && chunk >= 4 ? 1 : 0;
+      gk_off = (uint32_t)(krow * p.stride_slot * p.tok + chunk * 16);
+      gv_off = (uint32_t)(vrow * p.stride_slot * p.tok + chunk * 16);
       wk = kLdsK + swz_k(krow, 2 * chunk);
       wv = kLdsV + swz_v(vrow, 2 * chunk);
-      sc_tok = lane & 15;
+      const int per_half = 16 * p.tok;  // tokens per half tile
+      sc_tok = lane % per_half;
       sc_g = (uint32_t)(sc_tok * p.sc_stride_slot * 4);
-      sc_is_v = ((lane >> 4) & 1) != 0;
-      sc_lds = kLdsSc + (sc_is_v ? 128 : 0) + sc_tok * 4;
-      sc_on = lane < 32;
+      sc_is_v = ((lane / per_half) & 1) != 0;
+      sc_on = lane < 2 * per_half;
+      sc_half = (uint32_t)(per_half * 4);
+      sc_next = 2 * sc_half;
+      sc_lds = kLdsSc + (sc_is_v ? sc_next : 0) + sc_tok * 4;
     }
     // K row krow + 8j: swizzle adds 8; V row vrow + 4j: swizzle adds 8; second piece: XOR 1.
     __device__ inline uint32_t k_row(int j, int hi, int h) const {
@@ -629,8 +645,8 @@ struct KvHalfQuant {
     const uint8_t* vb = p.v_cache + b.elem;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      k[j] = ldg_stream(kb + j * 8 * p.stride_slot + g.gk_off);
-      v[j] = ldg_stream(vb + j * 4 * p.stride_slot + g.gv_off);
+      k[j] = ldg_stream(kb + j * 8 * p.stride_slot * p.tok + g.gk_off);
+      v[j] = ldg_stream(vb + j * 4 * p.stride_slot * p.tok + g.gv_off);
     }
     const float* sb = (g.sc_is_v ? p.v_scale : p.k_scale) + b.scale;
     if (g.sc_on) sc = *(const float*)((const uint8_t*)sb + g.sc_g);
@@ -643,7 +659,7 @@ struct KvHalfQuant {
       u32x4 klo, khi, vlo, vhi;
       dequant16<KV_DT>(k[j], klo, khi);
       dequant16<KV_DT>(v[j], vlo, vhi);
-      if (MASKED && tok + g.vrow + 4 * j >= len) vlo = vhi = u32x4{0, 0, 0, 0};
+      if (MASKED && tok + g.tok * (g.vrow + 4 * j) + g.second >= len) vlo = vhi = u32x4{0, 0, 0, 0};
       *(u32x4*)(tile + g.k_row(j, 0, h)) = klo;
       *(u32x4*)(tile + g.k_row(j, 1, h)) = khi;
       *(u32x4*)(tile + g.v_row(j, 0, h)) = vlo;
@@ -656,8 +672,8 @@ struct KvHalfQuant {
       float a = g.sc_is_v ? __builtin_amdgcn_logf(vs) : sc * scale_log2;
       float r = __builtin_amdgcn_rcpf(vs);
       if (MASKED && tok + g.sc_tok >= len) a = r = 0.0f;  // slots past the end may hold anything
-      *(float*)(tile + g.sc_lds + h * 64) = a;
-      if (g.sc_is_v) *(float*)(tile + g.sc_lds + 128 + h * 64) = r;
+      *(float*)(tile + g.sc_lds + h * g.sc_half) = a;
+      if (g.sc_is_v) *(float*)(tile + g.sc_lds + g.sc_next + h * g.sc_half) = r;
     }
   }
 };
@@ -698,7 +714,16 @@ __device__ inline float kg_sum(float v) {
 }
 
 // State of one wave's tile of 16 query rows, and the attention over one parked tile.
-template <int KV_DT>
+//
+// TOK = 1: head_dim 128, an LDS row is one token.  TOK = 2: head_dim 64 with the tokens of a block
+// contiguous in memory; an LDS row is then two consecutive tokens (the same 256 bytes), so loads,
+// parking and swizzles are those of head_dim 128, and the MFMAs split the row again:
+//   scores of the first  token of row t:  K chunks 0, 1 of the row against the query's two chunks
+//   scores of the second token of row t:  K chunks 2, 3 against the same query chunks
+//   head-dim tiles 0..3 of V^T are the first token's values, tiles 4..7 the second's, so they take
+//   the first / second tokens' weights as B operand and the two halves of O^T are added at the end.
+// A tile is 32 rows either way, i.e. 32 * TOK tokens.
+template <int KV_DT, int TOK>
 struct RowTile {
   static constexpr bool kQuant = quant_of(KV_DT);
   // int8 rows sit in LDS as x + 1152.  With K' = K + 1152 and V' = V + 1152:
@@ -707,10 +732,12 @@ struct RowTile {
   //                                                       operand is all ones (wacc)
   // Rows zeroed because they lie past the sequence end carry weight 0 in both sums.
   static constexpr bool kOffset = kv_of(KV_DT) == XLLM_HIP_INT8;
+  static constexpr int kD = 128 / TOK;   // head_dim
+  static constexpr int kQC = 4 / TOK;    // 32-element chunks of a query row
   typedef typename Mma<KV_DT>::Op Op;
 
-  Op qf[4];        // Q^T fragments (B operand) of the lane's query row
-  f32x4 acc[8];    // O^T accumulators: head-dim tile dt, rows 4*kg + rr
+  Op qf[kQC];      // Q^T fragments (B operand) of the lane's query row
+  f32x4 acc[8];    // O^T accumulators: tile dt of the 128 row elements, query rows 4*kg + rr
   f32x4 wacc;      // sum of the weights as the MFMA saw them (int8 only)
   float m_run;     // running maximum of the log2-scaled scores (of score + log2 v_scale if quantised)
   float l_run;     // this lane's share of the softmax denominator
@@ -718,7 +745,7 @@ struct RowTile {
   int lim;         // tokens >= lim are invisible to the row (causal among draft tokens)
   int lo;          // tokens < lo are outside the sliding window
   uint32_t k_off0; // LDS offset of K row mi, piece kg        (piece 4c + kg: XOR c << 6)
-  uint32_t v_off0; // LDS offset of the transpose read, tile 0 (head-dim tile dt: XOR dt << 5)
+  uint32_t v_off0; // LDS offset of the transpose read, tile 0 (tile dt: XOR dt << 5)
   int kg;
 
   __device__ inline void init(const DecodeParams& p, const Item& it, int row_in_item, int lane) {
@@ -731,10 +758,10 @@ struct RowTile {
     lim = it.len - (it.n - 1 - j);
     lo = p.window_left >= 0 ? lim - 1 - p.window_left : 0;
     const uint16_t* qrow = (const uint16_t*)p.q + (int64_t)(it.q0 + j) * p.q_token_stride +
-                           (int64_t)(it.hk * p.group + gq) * 128;
+                           (int64_t)(it.hk * p.group + gq) * kD;
     float sq = 0.0f;
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
+    for (int c = 0; c < kQC; ++c) {
       u32x4 raw = {0, 0, 0, 0};
       if (valid) raw = *(const u32x4*)(qrow + c * 32 + kg * 8);
       if constexpr (qf16_of(KV_DT) || !f16_ops(KV_DT)) {
@@ -757,69 +784,93 @@ struct RowTile {
 #pragma unroll
     for (int dt = 0; dt < 8; ++dt) acc[dt] = f32x4{0, 0, 0, 0};
     k_off0 = kLdsK + swz_k(mi, kg);
-    const int tau = 4 * kg + (mi >> 2);  // token row (within 16) this lane points the transpose read at
+    const int tau = 4 * kg + (mi >> 2);  // row (within 16) this lane points the transpose read at
     v_off0 = kLdsV + swz_v(tau, (mi & 3) >> 1) + (mi & 1) * 8;
   }
 
-  // Attention of the 16 rows over the 32 tokens parked in `tile` (first token tb).
+  // Attention of the 16 query rows over the 32 * TOK tokens parked in `tile` (first token tb).
+  // Score / weight index i = (u * 2 + h) * 4 + rr: token TOK * (16h + 4kg + rr) + u of the tile.
   template <bool MASKED>
   __device__ inline void attend(const uint8_t* tile, int tb, float scale_log2) {
     const float neg_inf = -INFINITY;
-    f32x4 kscl[2], lv[2], rvs[2];  // per-token factors of tokens tb + 16h + 4kg + rr
+    constexpr int kN = 8 * TOK;  // scores per lane
+    float kscl[kN], lv[kN], rvs[kN];
     if (kQuant) {
+      // the factors of tokens TOK * (16h + 4kg) .. + 4 * TOK - 1 are contiguous in each array
+      constexpr int kArr = 32 * TOK * 4;  // bytes per array
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
-        kscl[h] = *(const f32x4*)(tile + kLdsSc + (16 * h + 4 * kg) * 4);
-        lv[h] = *(const f32x4*)(tile + kLdsSc + 128 + (16 * h + 4 * kg) * 4);
-        rvs[h] = *(const f32x4*)(tile + kLdsSc + 256 + (16 * h + 4 * kg) * 4);
+        const int first = TOK * (16 * h + 4 * kg) * 4;
+#pragma unroll
+        for (int v4 = 0; v4 < TOK; ++v4) {
+          const f32x4 a = *(const f32x4*)(tile + kLdsSc + first + 16 * v4);
+          const f32x4 b = *(const f32x4*)(tile + kLdsSc + kArr + first + 16 * v4);
+          const f32x4 c = *(const f32x4*)(tile + kLdsSc + 2 * kArr + first + 16 * v4);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int t = 4 * v4 + e;  // token of the lane's 4 * TOK: row rr = t / TOK, u = t % TOK
+            const int i = ((t % TOK) * 2 + h) * 4 + t / TOK;
+            kscl[i] = a[e];
+            lv[i] = b[e];
+            rvs[i] = c[e];
+          }
+        }
       }
     }
     // ---- S^T = K Q^T ----
-    f32x4 s[2];
-    s[0] = s[1] = f32x4{s_init, s_init, s_init, s_init};
+    f32x4 s[TOK][2];
+#pragma unroll
+    for (int u = 0; u < TOK; ++u) s[u][0] = s[u][1] = f32x4{s_init, s_init, s_init, s_init};
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
       const uint32_t ko = k_off0 ^ (uint32_t)(c << 6);
       const Op kf0 = *(const Op*)(tile + ko);
       const Op kf1 = *(const Op*)(tile + ko + 4096);
-      s[0] = Mma<KV_DT>::run(kf0, qf[c], s[0]);
-      s[1] = Mma<KV_DT>::run(kf1, qf[c], s[1]);
+      s[c / kQC][0] = Mma<KV_DT>::run(kf0, qf[c % kQC], s[c / kQC][0]);
+      s[c / kQC][1] = Mma<KV_DT>::run(kf1, qf[c % kQC], s[c / kQC][1]);
     }
     // ---- online softmax of the lane's query row ----
-    float x[8];
+    float x[kN];
+    float mt = neg_inf;
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
+    for (int u = 0; u < TOK; ++u) {
 #pragma unroll
-      for (int rr = 0; rr < 4; ++rr) {
-        float v = kQuant ? __builtin_fmaf(s[h][rr], kscl[h][rr], lv[h][rr]) : s[h][rr] * scale_log2;
-        if (MASKED) {
-          const int tok = tb + 16 * h + 4 * kg + rr;
-          v = (tok < lim && tok >= lo) ? v : neg_inf;
+      for (int h = 0; h < 2; ++h) {
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+          const int i = (u * 2 + h) * 4 + rr;
+          float v = kQuant ? __builtin_fmaf(s[u][h][rr], kscl[i], lv[i]) : s[u][h][rr] * scale_log2;
+          if (MASKED) {
+            const int tok = tb + TOK * (16 * h + 4 * kg + rr) + u;
+            v = (tok < lim && tok >= lo) ? v : neg_inf;
+          }
+          x[i] = v;
+          mt = fmaxf(mt, v);
         }
-        x[4 * h + rr] = v;
       }
     }
-    const float mt =
-        kg_max(fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7]))));
+    mt = kg_max(mt);
     const float m_new = fmaxf(m_run, mt);
     const float m_safe = m_new == neg_inf ? 0.0f : m_new;
     const bool moved = __builtin_amdgcn_ballot_w64(m_new != m_run) != 0;
     const float alpha = __builtin_amdgcn_exp2f(m_run - m_safe);
     l_run *= alpha;
     m_run = m_new;
-    float w[8];
+    float w[kN];
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-#pragma unroll
-      for (int rr = 0; rr < 4; ++rr) {
-        const float e = __builtin_amdgcn_exp2f(x[4 * h + rr] - m_safe);
-        w[4 * h + rr] = e;
-        l_run = kQuant ? __builtin_fmaf(e, rvs[h][rr], l_run) : l_run + e;
-      }
+    for (int i = 0; i < kN; ++i) {
+      const float e = __builtin_amdgcn_exp2f(x[i] - m_safe);
+      w[i] = e;
+      l_run = kQuant ? __builtin_fmaf(e, rvs[i], l_run) : l_run + e;
     }
-    const u32x4 pw = {Mma<KV_DT>::pack(w[0], w[1]), Mma<KV_DT>::pack(w[2], w[3]), Mma<KV_DT>::pack(w[4], w[5]),
-                      Mma<KV_DT>::pack(w[6], w[7])};
-    const Op pf = __builtin_bit_cast(Op, pw);
+    Op pf[TOK];  // B operand of the second MFMA: k-slot e = 4h + rr
+#pragma unroll
+    for (int u = 0; u < TOK; ++u) {
+      const float* wu = w + 8 * u;
+      const u32x4 pw = {Mma<KV_DT>::pack(wu[0], wu[1]), Mma<KV_DT>::pack(wu[2], wu[3]), Mma<KV_DT>::pack(wu[4], wu[5]),
+                        Mma<KV_DT>::pack(wu[6], wu[7])};
+      pf[u] = __builtin_bit_cast(Op, pw);
+    }
     // ---- O^T = O^T * alpha + V^T P^T ----
     // The accumulators need rescaling only when some row's maximum moved, which becomes rare a few
     // tiles into a sequence.  Both variants of the product are written out, so that each path ends
@@ -833,7 +884,7 @@ struct RowTile {
   }
 
   template <bool RESCALE>
-  __device__ inline void accumulate(const uint8_t* tile, const Op pf, float alpha) {
+  __device__ inline void accumulate(const uint8_t* tile, const Op (&pf)[TOK], float alpha) {
 #pragma unroll
     for (int dt = 0; dt < 8; ++dt) {
       const uint32_t vo = v_off0 ^ (uint32_t)(dt << 5);
@@ -844,25 +895,28 @@ struct RowTile {
       const Op vf = __builtin_bit_cast(Op, __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7));
       f32x4 c = acc[dt];
       if (RESCALE) c *= alpha;
-      acc[dt] = Mma<KV_DT>::run(vf, pf, c);
+      acc[dt] = Mma<KV_DT>::run(vf, pf[dt * TOK / 8], c);
     }
     if (kOffset) {
       const u32x4 ones = {0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u};  // fp16 1.0
       f32x4 c = wacc;
       if (RESCALE) c *= alpha;
-      wacc = Mma<KV_DT>::run(__builtin_bit_cast(Op, ones), pf, c);
+#pragma unroll
+      for (int u = 0; u < TOK; ++u) c = Mma<KV_DT>::run(__builtin_bit_cast(Op, ones), pf[u], c);
+      wacc = c;
     }
   }
 };
 
 // End of an item: the TW waves that share a set of 16 query rows exchange (m, l, acc) through LDS
-// (each wave's own 16 KiB region `xch_base + wave * xch_stride`), then each finishes 128/TW columns:
+// (each wave's own 16 KiB region `xch_base + wave * xch_stride`), then each finishes head_dim/TW columns:
 // a sequence that is a single chunk gets its bf16 output rows (and LSE) written directly, a split
 // sequence a normalised fp32 partial and its log2-sum-exp.  All waves of the workgroup must call it.
-template <int KV_DT, int TW>
-__device__ inline void finish_item(const DecodeParams& p, const Item& it, RowTile<KV_DT>& rt, uint8_t* xch_base,
+template <int KV_DT, int TOK, int TW>
+__device__ inline void finish_item(const DecodeParams& p, const Item& it, RowTile<KV_DT, TOK>& rt, uint8_t* xch_base,
                                    int xch_stride, float* lds_ml, int wave, int rs, int tw, int lane) {
   constexpr bool kOffset = kv_of(KV_DT) == XLLM_HIP_INT8;
+  constexpr int kD = 128 / TOK;
   const float neg_inf = -INFINITY;
   const int mi = lane & 15, kg = lane >> 4;
   const int nhq = p.n * p.num_q_heads;
@@ -870,8 +924,9 @@ __device__ inline void finish_item(const DecodeParams& p, const Item& it, RowTil
   const float l = kg_sum(rt.l_run);
   uint8_t* mine = xch_base + wave * xch_stride;
 #pragma unroll
-  for (int dt = 0; dt < 8; ++dt) {
+  for (int dt = 0; dt < 8 / TOK; ++dt) {
     f32x4 o = rt.acc[dt];
+    if (TOK == 2) o += rt.acc[dt + 4];  // the two tokens of a row accumulated into separate tiles
     if (kOffset) o -= kInt8Offset * rt.wacc[0];  // every element of wacc holds the row's sum
     *(f32x4*)(mine + mi * kXchRow + (dt * 16 + 4 * kg) * 4) = o;
   }
@@ -901,9 +956,11 @@ __device__ inline void finish_item(const DecodeParams& p, const Item& it, RowTil
   const float lse2 = l_all > 0.0f ? m_all + __builtin_amdgcn_logf(l_all) : neg_inf;
   const int64_t tok = (int64_t)it.q0 + j;
   const int64_t prow = (int64_t)it.sc * nhq + (int64_t)j * p.num_q_heads + head;
-  constexpr int kCols = 128 / TW;  // columns this wave finishes: 8 per lane and pass
+  constexpr int kCols = kD / TW;  // columns this wave finishes: 8 per lane and pass
+  constexpr int kPasses = kCols >= 32 ? kCols / 32 : 1;
+  if (kCols < 32 && 8 * kg >= kCols) return;
 #pragma unroll
-  for (int pass = 0; pass < kCols / 32; ++pass) {
+  for (int pass = 0; pass < kPasses; ++pass) {
     const int d0 = kCols * tw + 32 * pass + 8 * kg;
     f32x4 o_lo = {0, 0, 0, 0}, o_hi = {0, 0, 0, 0};
 #pragma unroll
@@ -921,9 +978,9 @@ __device__ inline void finish_item(const DecodeParams& p, const Item& it, RowTil
         ob[e] = (decltype(ob[0] + ob[0]))o_lo[e];
         ob[4 + e] = (decltype(ob[0] + ob[0]))o_hi[e];
       }
-      *(decltype(ob)*)((uint16_t*)p.out + tok * p.out_token_stride + (int64_t)head * 128 + d0) = ob;
+      *(decltype(ob)*)((uint16_t*)p.out + tok * p.out_token_stride + (int64_t)head * kD + d0) = ob;
     } else {
-      float* po = p.partial_out + prow * 128 + d0;
+      float* po = p.partial_out + prow * kD + d0;
       *(f32x4*)(po) = o_lo;
       *(f32x4*)(po + 4) = o_hi;
     }
@@ -943,16 +1000,19 @@ __device__ inline int first_visible_tile(const DecodeParams& p, const Item& it) 
   if (p.window_left >= 0) {
     int first = it.len - it.n - p.window_left;  // window start of the earliest query row
     first = first > 0 ? first : 0;
-    first &= ~(kTileTokens - 1);
+    first &= ~(p.tile_tokens - 1);
     t0 = t0 > first ? t0 : first;
   }
   return t0;
 }
 
-template <int KV_DT>
+template <int KV_DT, int TOK>
 __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_d128_kernel(DecodeParams p) {
   __shared__ __attribute__((aligned(16))) uint8_t lds_all[kWaves * kLdsTile];
   __shared__ float lds_ml[kWaves * 16 * 2];  // (running max, denominator) per wave and query row
+
+  constexpr int kT = 32 * TOK;  // tokens per tile
+  constexpr int kH = 16 * TOK;  // tokens per half tile
 
   Item it;
   if (!decode_item(p, blockIdx.x, it)) return;
@@ -961,13 +1021,13 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_d128_kernel(Decode
   const int lane = threadIdx.x & 63;
   uint8_t* tile = lds_all + wave * kLdsTile;  // this wave's private K/V tile
 
-  RowTile<KV_DT> rt;
+  RowTile<KV_DT, TOK> rt;
   rt.init(p, it, 0, lane);
 
   // This wave's share of the item's tokens.
   const int t0 = first_visible_tile(p, it);
   const int span = it.t_end - t0;
-  const int share = span > 0 ? (((span + kWaves - 1) / kWaves + kTileTokens - 1) & ~(kTileTokens - 1)) : 0;
+  const int share = span > 0 ? (((span + kWaves - 1) / kWaves + kT - 1) & ~(kT - 1)) : 0;
   const int w_begin = t0 + wave * share;
   const int w_end = min(it.t_end, w_begin + share);
   const int mask_hi_from = it.len - (it.n - 1);                                    // tiles reaching past this need masks
@@ -975,31 +1035,31 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_d128_kernel(Decode
 
   typename KvHalf<KV_DT>::Geom geom;
   geom.init(p, lane);
-  KvHalf<KV_DT> st[2];  // the two 16-token halves of the tile in flight
+  KvHalf<KV_DT> st[2];  // the two halves (16 rows each) of the tile in flight
 
   if (w_begin < w_end) {
     st[0].issue(p, it, w_begin, block_of(p, it, w_begin), geom);
-    st[1].issue(p, it, w_begin + 16, block_of(p, it, w_begin + 16), geom);
+    st[1].issue(p, it, w_begin + kH, block_of(p, it, w_begin + kH), geom);
     // block ids of the next tile's halves, fetched one tile before the loads that use them
-    int blk0 = block_of(p, it, w_begin + kTileTokens);
-    int blk1 = block_of(p, it, w_begin + kTileTokens + 16);
-    for (int tb = w_begin; tb < w_end; tb += kTileTokens) {
-      const bool masked = (tb + kTileTokens > mask_hi_from) || (tb < mask_lo_until);
+    int blk0 = block_of(p, it, w_begin + kT);
+    int blk1 = block_of(p, it, w_begin + kT + kH);
+    for (int tb = w_begin; tb < w_end; tb += kT) {
+      const bool masked = (tb + kT > mask_hi_from) || (tb < mask_lo_until);
       // The scalar loads of the ids go out before the tile is parked: they share a counter with the
       // LDS traffic, so the next wait on LDS also waits for them.
-      const int nblk0 = block_of(p, it, tb + 2 * kTileTokens);
-      const int nblk1 = block_of(p, it, tb + 2 * kTileTokens + 16);
+      const int nblk0 = block_of(p, it, tb + 2 * kT);
+      const int nblk1 = block_of(p, it, tb + 2 * kT + kH);
       // park the tile, then put the next tile's loads in flight while this one is consumed
       if (masked) {
         st[0].template park<true>(tile, 0, tb, it.len, p.scale_log2, geom);
-        st[1].template park<true>(tile, 1, tb + 16, it.len, p.scale_log2, geom);
+        st[1].template park<true>(tile, 1, tb + kH, it.len, p.scale_log2, geom);
       } else {
         st[0].template park<false>(tile, 0, tb, it.len, p.scale_log2, geom);
-        st[1].template park<false>(tile, 1, tb + 16, it.len, p.scale_log2, geom);
+        st[1].template park<false>(tile, 1, tb + kH, it.len, p.scale_log2, geom);
       }
-      if (tb + kTileTokens < w_end) {
-        st[0].issue(p, it, tb + kTileTokens, blk0, geom);
-        st[1].issue(p, it, tb + kTileTokens + 16, blk1, geom);
+      if (tb + kT < w_end) {
+        st[0].issue(p, it, tb + kT, blk0, geom);
+        st[1].issue(p, it, tb + kT + kH, blk1, geom);
       }
       blk0 = nblk0;
       blk1 = nblk1;
@@ -1010,16 +1070,19 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_d128_kernel(Decode
       }
     }
   }
-  finish_item<KV_DT, kWaves>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, 0, wave, lane);
+  finish_item<KV_DT, TOK, kWaves>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, 0, wave, lane);
 }
 
-template <int KV_DT>
+template <int KV_DT, int TOK>
 __global__ void __launch_bounds__(128, 2) decode_mfma_d128_rows32_kernel(DecodeParams p) {
   // A workgroup is one pair of waves: wave w owns query rows 16w .. 16w+15 and fetches rows 16w ..
   // of every tile.  A tile is parked while both waves still read the previous one from the other
   // buffer, so one barrier (of two waves) per tile suffices.  Four such workgroups share a CU.
   __shared__ __attribute__((aligned(16))) uint8_t lds_all[2 * kLdsTile];
   __shared__ float lds_ml[2 * 16 * 2];
+
+  constexpr int kT = 32 * TOK;  // tokens per tile
+  constexpr int kH = 16 * TOK;  // tokens per half tile
 
   Item it;
   if (!decode_item(p, blockIdx.x, it)) return;
@@ -1029,12 +1092,12 @@ __global__ void __launch_bounds__(128, 2) decode_mfma_d128_rows32_kernel(DecodeP
   const int lane = threadIdx.x & 63;
   uint8_t* tiles = lds_all;
 
-  RowTile<KV_DT> rt;
+  RowTile<KV_DT, TOK> rt;
   rt.init(p, it, 16 * rs, lane);
 
   const int w_begin = first_visible_tile(p, it);
   const int w_end = it.t_end;
-  const int iters = w_end > w_begin ? (w_end - w_begin + kTileTokens - 1) / kTileTokens : 0;
+  const int iters = w_end > w_begin ? (w_end - w_begin + kT - 1) / kT : 0;
   const int mask_hi_from = it.len - (it.n - 1);
   const int mask_lo_until = p.window_left >= 0 ? it.len - 1 - p.window_left : 0;
 
@@ -1043,25 +1106,25 @@ __global__ void __launch_bounds__(128, 2) decode_mfma_d128_rows32_kernel(DecodeP
   // Two register stages, used alternately: the loads of tiles i+1 and i+2 are in flight while tile
   // i is consumed.  (A wave fetches only half a tile, so one stage would leave too few bytes in
   // flight per CU to cover the HBM latency.)  Both waves run the same iterations.
-  KvHalf<KV_DT> mine[2];  // the 16 tokens this wave fetches: rows 16*rs .. of the tile
+  KvHalf<KV_DT> mine[2];  // the 16 rows this wave fetches: rows 16*rs .. of the tile
 
   auto issue = [&](KvHalf<KV_DT>& m, int blk, int tb) {
-    if (tb < w_end) m.issue(p, it, tb + 16 * rs, blk, geom);
+    if (tb < w_end) m.issue(p, it, tb + kH * rs, blk, geom);
   };
   // `blk`: block id of the half this wave fetches two tiles on; replaced by that of the tile four
   // on.  The scalar load goes out before the tile is parked: it shares a counter with the LDS
   // traffic, so the wait before the barrier also waits for it.
   auto step = [&](KvHalf<KV_DT>& m, int& blk, int i) {
-    const int tb = w_begin + i * kTileTokens;
-    const int nblk = block_of(p, it, tb + 4 * kTileTokens + 16 * rs);
+    const int tb = w_begin + i * kT;
+    const int nblk = block_of(p, it, tb + 4 * kT + kH * rs);
     uint8_t* tile = tiles + (i & 1) * kLdsTile;
-    const bool masked = (tb + kTileTokens > mask_hi_from) || (tb < mask_lo_until);
+    const bool masked = (tb + kT > mask_hi_from) || (tb < mask_lo_until);
     if (masked) {
-      m.template park<true>(tile, rs, tb + 16 * rs, it.len, p.scale_log2, geom);
+      m.template park<true>(tile, rs, tb + kH * rs, it.len, p.scale_log2, geom);
     } else {
-      m.template park<false>(tile, rs, tb + 16 * rs, it.len, p.scale_log2, geom);
+      m.template park<false>(tile, rs, tb + kH * rs, it.len, p.scale_log2, geom);
     }
-    issue(m, blk, tb + 2 * kTileTokens);
+    issue(m, blk, tb + 2 * kT);
     blk = nblk;
     __syncthreads();  // both halves of tile i are parked; both waves are done with tile i-1
     if (masked) {
@@ -1070,16 +1133,16 @@ __global__ void __launch_bounds__(128, 2) decode_mfma_d128_rows32_kernel(DecodeP
       rt.template attend<false>(tile, tb, p.scale_log2);
     }
   };
-  issue(mine[0], block_of(p, it, w_begin + 16 * rs), w_begin);
-  issue(mine[1], block_of(p, it, w_begin + kTileTokens + 16 * rs), w_begin + kTileTokens);
-  int blk_a = block_of(p, it, w_begin + 2 * kTileTokens + 16 * rs);
-  int blk_b = block_of(p, it, w_begin + 3 * kTileTokens + 16 * rs);
+  issue(mine[0], block_of(p, it, w_begin + kH * rs), w_begin);
+  issue(mine[1], block_of(p, it, w_begin + kT + kH * rs), w_begin + kT);
+  int blk_a = block_of(p, it, w_begin + 2 * kT + kH * rs);
+  int blk_b = block_of(p, it, w_begin + 3 * kT + kH * rs);
   for (int i = 0; i < iters; i += 2) {
     step(mine[0], blk_a, i);
     if (i + 1 < iters) step(mine[1], blk_b, i + 1);
   }
   __syncthreads();  // all tiles consumed before the buffers are reused for the exchange
-  finish_item<KV_DT, 1>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, rs, 0, lane);
+  finish_item<KV_DT, TOK, 1>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, rs, 0, lane);
 }
 
 // ---------------------------------------------------------------------------------
@@ -1245,7 +1308,8 @@ __global__ void __launch_bounds__(256) csr_to_block_table_kernel(const int32_t* 
 // Host side.
 // ---------------------------------------------------------------------------------
 
-enum Variant { kNone = 0, kMfmaD128 = 1, kGeneric = 2 };
+enum Variant { kNone = 0, kMfmaD128 = 1, kGeneric = 2, kMfmaD64 = 3 };
+static bool is_mfma(Variant v) { return v == kMfmaD128 || v == kMfmaD64; }
 
 // Split target: about this many work items (workgroups) per launch.  A workgroup of the MFMA kernel
 // is four waves, one per SIMD of a CU, and two workgroups fit on a CU (256 VGPRs, < 80 KiB of LDS).
@@ -1271,8 +1335,11 @@ static Variant pick_variant(const xllm_hip_kv_cache* c, const xllm_hip_decode_ar
   const bool q16 = a->q_dtype == XLLM_HIP_BF16 || a->q_dtype == XLLM_HIP_FP16;
   const bool kv_ok = q16 && (c->dtype == a->q_dtype || c->dtype == XLLM_HIP_FP8_E4M3 || c->dtype == XLLM_HIP_INT8);
   const bool force_generic = getenv("XLLM_HIP_DECODE_FORCE_GENERIC") != nullptr;
-  if (!force_generic && c->head_dim == 128 && kv_ok && c->block_size >= 16 &&
-      is_pow2(c->block_size)) {
+  // head_dim 64 rides on the head_dim-128 kernels with two tokens per tile row: the tokens of a
+  // block must then be contiguous, and half a tile (32 tokens) must lie in one block.
+  const bool d128 = c->head_dim == 128 && c->block_size >= 16;
+  const bool d64 = c->head_dim == 64 && c->block_size >= 32 && c->stride_slot == 64;
+  if (!force_generic && (d128 || d64) && kv_ok && is_pow2(c->block_size)) {
     const int vec = 16 / eb;  // elements per 16-byte load
     const bool strides_ok = c->stride_block % vec == 0 && c->stride_head % vec == 0 && c->stride_slot % vec == 0 &&
                             a->q_token_stride % 8 == 0;
@@ -1286,7 +1353,7 @@ static Variant pick_variant(const xllm_hip_kv_cache* c, const xllm_hip_decode_ar
     }
     const bool range_ok = c->stride_block >= 0 && c->stride_block < lim32 && c->stride_slot >= 0 &&
                           c->stride_slot * c->block_size < lim32;
-    if (strides_ok && range_ok && ptrs_ok && scales_ok) return kMfmaD128;
+    if (strides_ok && range_ok && ptrs_ok && scales_ok) return d128 ? kMfmaD128 : kMfmaD64;
   }
   if (c->head_dim <= 256 && is_pow2(c->block_size)) return kGeneric;
   return kNone;
@@ -1374,24 +1441,26 @@ static int fill_params(const xllm_hip_kv_cache* c,
   p.group = a->num_q_heads / c->num_kv_heads;
   p.rows = p.group * p.n;
   const Variant variant = pick_variant(c, a);
-  p.rows_per_item = variant == kMfmaD128 ? kMaxRowsPerItem : 1;
-  p.min_chunk = variant == kMfmaD128 ? kMinChunkTokens : kMinChunkTokensGeneric;
+  p.rows_per_item = is_mfma(variant) ? kMaxRowsPerItem : 1;
+  p.min_chunk = is_mfma(variant) ? kMinChunkTokens : kMinChunkTokensGeneric;
+  p.tok = variant == kMfmaD64 ? 2 : 1;
+  p.tile_tokens = kTileTokens * p.tok;
   p.row_groups = row_groups(a->q_per_seq, a->num_q_heads, c->num_kv_heads, p.rows_per_item);
   p.head_dim = c->head_dim;
   p.block_size = c->block_size;
   p.log2_bs = is_pow2(c->block_size) ? ilog2(c->block_size) : 0;
   p.max_blocks_per_seq = a->max_blocks_per_seq;
   p.window_left = a->window_left;
-  p.target_items = target_items(variant == kMfmaD128, p.rows);
+  p.target_items = target_items(is_mfma(variant), p.rows);
   // Only the MFMA kernel finishes single-chunk sequences itself.  When the caller's host-side
   // lengths (the reference keeps both in AttentionMetadata) show that the chunk the plan would
   // pick covers the longest sequence, no sequence is split: the plan is told never to split
   // (which stays correct even if the hints were wrong) and the merge launch is dropped.
-  p.direct_single = variant == kMfmaD128 ? 1 : 0;
+  p.direct_single = is_mfma(variant) ? 1 : 0;
   p.fixed_chunk = 0;
   if (p.direct_single && a->max_seq_len > 0 && a->total_kv_len > 0 &&
       a->max_seq_len <= choose_chunk(a->total_kv_len, a->max_seq_len, p.batch, p.num_kv_heads, p.row_groups,
-                                     p.target_items, p.min_chunk)) {
+                                     p.target_items, p.min_chunk, p.tile_tokens)) {
     p.fixed_chunk = 1 << 30;
   }
   // Many query rows per kv head (chunked prefill): the row groups supply the parallelism, and one
@@ -1428,13 +1497,22 @@ static int64_t max_items(const DecodeParams& p) {
   return items;
 }
 
-template <int KV_DT>
-static void launch_mfma(const DecodeParams& p, unsigned grid, hipStream_t st) {
+template <int KV_DT, int TOK>
+static void launch_mfma_tok(const DecodeParams& p, unsigned grid, hipStream_t st) {
   const int rows_per_item = p.rows < kMaxRowsPerItem ? p.rows : kMaxRowsPerItem;
   if (rows_per_item <= 16) {
-    decode_mfma_d128_kernel<KV_DT><<<grid, 64 * kWaves, 0, st>>>(p);
+    decode_mfma_d128_kernel<KV_DT, TOK><<<grid, 64 * kWaves, 0, st>>>(p);
   } else {
-    decode_mfma_d128_rows32_kernel<KV_DT><<<grid, 128, 0, st>>>(p);
+    decode_mfma_d128_rows32_kernel<KV_DT, TOK><<<grid, 128, 0, st>>>(p);
+  }
+}
+
+template <int KV_DT>
+static void launch_mfma(const DecodeParams& p, unsigned grid, hipStream_t st) {
+  if (p.tok == 2) {
+    launch_mfma_tok<KV_DT, 2>(p, grid, st);
+  } else {
+    launch_mfma_tok<KV_DT, 1>(p, grid, st);
   }
 }
 
@@ -1481,6 +1559,8 @@ extern "C" const char* xllm_hip_paged_decode_variant(const xllm_hip_kv_cache* ca
   switch (pick_variant(cache, args)) {
     case kMfmaD128:
       return "mfma_d128";
+    case kMfmaD64:
+      return "mfma_d64";
     case kGeneric:
       return "generic";
     default:
@@ -1530,7 +1610,7 @@ extern "C" int xllm_hip_paged_decode_run_timed(const xllm_hip_kv_cache* cache,
   if (ev_begin != nullptr && hipEventRecord((hipEvent_t)ev_begin, st) != hipSuccess) {
     return fail(XLLM_HIP_RUNTIME_ERROR, "hipEventRecord(ev_begin) failed");
   }
-  if (v == kMfmaD128) {
+  if (is_mfma(v)) {
     const bool qf16 = args->q_dtype == XLLM_HIP_FP16;
     switch (cache->dtype) {
       case XLLM_HIP_BF16:
