@@ -202,7 +202,7 @@ def main():
     kern_gbps = alg_bytes / kern_avg_us / 1e3
 
     rows_per_kv_head = w.q_per_seq * (w.num_q_heads // w.num_kv_heads)
-    kernel_name = ("decode_generic_kernel" if variant != "mfma_d128" else
+    kernel_name = ("decode_generic_kernel" if not variant.startswith("mfma") else
                    "decode_mfma_d128_kernel" if rows_per_kv_head <= 16 else "decode_mfma_d128_rows32_kernel")
     traffic = None
     tpath = os.path.join(REPO, "profiles", "hbm_traffic.json")

@@ -370,7 +370,7 @@ const char* xllm_hip_last_error(void);
 int xllm_hip_abi_version(void);
 
 /* Name of the kernel variant xllm_hip_paged_decode_run would pick for these
- * arguments ("mfma_d128", "generic", ... or "" if unsupported); host-only, launches nothing. */
+ * arguments ("mfma_d128", "mfma_d64", "generic", or "" if unsupported); host-only, launches nothing. */
 const char* xllm_hip_paged_decode_variant(const xllm_hip_kv_cache* cache,
                                           const xllm_hip_decode_args* args);
 
