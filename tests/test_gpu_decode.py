@@ -96,14 +96,18 @@ def test_mfma_decode_head_dim_64(gpu, shape, kv, qdt):
     _check(case)
 
 
-def test_head_dim_64_falls_back_when_tokens_are_not_contiguous(gpu):
-    print("case d64 layouts", flush=True)
-    # NHD with several kv heads: a token's row is followed by the other heads' rows
-    case = Case(2, 8, 2, 64, 32, [100, 33], layout="NHD", seed=22)
-    assert case.variant() == "generic"
+@pytest.mark.parametrize("kv", ["bf16", "fp8", "int8"])
+def test_head_dim_64_nhd_layout(gpu, kv):
+    """NHD: the two tokens of a tile row are not adjacent in memory."""
+    print("case d64 nhd", kv, flush=True)
+    case = Case(3, 16, 4, 64, 32, [700, 33, 64], layout="NHD", kv=kv, seed=22)
+    assert case.variant() == "mfma_d64"
     _check(case)
-    # block_size 16: half a tile would straddle two blocks
-    case = Case(2, 8, 2, 64, 16, [100, 33], seed=22)
+
+
+def test_head_dim_64_small_blocks_take_the_generic_kernel(gpu):
+    print("case d64 bs16", flush=True)
+    case = Case(2, 8, 2, 64, 16, [100, 33], seed=22)  # half a tile would straddle two blocks
     assert case.variant() == "generic"
     _check(case)
 

@@ -479,7 +479,7 @@ struct KvHalf16 {
       const int piece = lane & 15;
       tok = p.tok;
       second = tok == 2 && piece >= 8 ? 1 : 0;
-      g_off = (uint32_t)((lrow * p.stride_slot * p.tok + piece * 8) * 2);
+      g_off = (uint32_t)(((lrow * p.tok + second) * p.stride_slot + (piece & (16 / p.tok - 1)) * 8) * 2);
       wk = kLdsK + swz_k(lrow, piece);
       wv = kLdsV + swz_v(lrow, piece);
     }
@@ -614,8 +614,9 @@ struct KvHalfQuant {
       vrow = (lane >> 4) + 8 * pair;            // rows r, r+8 alternate between quads (vrow & 7 < 4)
       tok = p.tok;
       second = tok == 2 && chunk >= 4 ? 1 : 0;
-      gk_off = (uint32_t)(krow * p.stride_slot * p.tok + chunk * 16);
-      gv_off = (uint32_t)(vrow * p.stride_slot * p.tok + chunk * 16);
+      const int in_tok = (chunk & (8 / p.tok - 1)) * 16;  // byte within the token's row
+      gk_off = (uint32_t)((krow * p.tok + second) * p.stride_slot + in_tok);
+      gv_off = (uint32_t)((vrow * p.tok + second) * p.stride_slot + in_tok);
       wk = kLdsK + swz_k(krow, 2 * chunk);
       wv = kLdsV + swz_v(vrow, 2 * chunk);
       const int per_half = 16 * p.tok;  // tokens per half tile
@@ -715,9 +716,9 @@ __device__ inline float kg_sum(float v) {
 
 // State of one wave's tile of 16 query rows, and the attention over one parked tile.
 //
-// TOK = 1: head_dim 128, an LDS row is one token.  TOK = 2: head_dim 64 with the tokens of a block
-// contiguous in memory; an LDS row is then two consecutive tokens (the same 256 bytes), so loads,
-// parking and swizzles are those of head_dim 128, and the MFMAs split the row again:
+// TOK = 1: head_dim 128, an LDS row is one token.  TOK = 2: head_dim 64; an LDS row is then two
+// consecutive tokens (its first eight 16-byte pieces from one, the rest from the next), so parking
+// and swizzles are those of head_dim 128, and the MFMAs split the row again:
 //   scores of the first  token of row t:  K chunks 0, 1 of the row against the query's two chunks
 //   scores of the second token of row t:  K chunks 2, 3 against the same query chunks
 //   head-dim tiles 0..3 of V^T are the first token's values, tiles 4..7 the second's, so they take
@@ -1335,10 +1336,10 @@ static Variant pick_variant(const xllm_hip_kv_cache* c, const xllm_hip_decode_ar
   const bool q16 = a->q_dtype == XLLM_HIP_BF16 || a->q_dtype == XLLM_HIP_FP16;
   const bool kv_ok = q16 && (c->dtype == a->q_dtype || c->dtype == XLLM_HIP_FP8_E4M3 || c->dtype == XLLM_HIP_INT8);
   const bool force_generic = getenv("XLLM_HIP_DECODE_FORCE_GENERIC") != nullptr;
-  // head_dim 64 rides on the head_dim-128 kernels with two tokens per tile row: the tokens of a
-  // block must then be contiguous, and half a tile (32 tokens) must lie in one block.
+  // head_dim 64 rides on the head_dim-128 kernels with two tokens per tile row: half a tile
+  // (32 tokens) must then lie in one block.
   const bool d128 = c->head_dim == 128 && c->block_size >= 16;
-  const bool d64 = c->head_dim == 64 && c->block_size >= 32 && c->stride_slot == 64;
+  const bool d64 = c->head_dim == 64 && c->block_size >= 32;
   if (!force_generic && (d128 || d64) && kv_ok && is_pow2(c->block_size)) {
     const int vec = 16 / eb;  // elements per 16-byte load
     const bool strides_ok = c->stride_block % vec == 0 && c->stride_head % vec == 0 && c->stride_slot % vec == 0 &&
