@@ -324,6 +324,22 @@ def aux_kernels(torch, ops, device):
         add("swap_blocks gather-then-scatter, %d blocks" % nblk,
             timed(lambda: ops.swap_blocks(kc, vc, src, dst, exact=True)), 4 * nblk * blk_bytes,
             "two passes through a staging buffer allocated per call")
+    # sequences read back out of the cache: 32 sequences of 4096 tokens
+    B, L = 32, 4096
+    table = torch.randperm(nb, device=device, generator=gen)[: B * (L // bs)].to(torch.int32).view(B, L // bs)
+    lens = torch.full((B,), L, device=device, dtype=torch.int32)
+    dk = torch.empty(B * L, Hkv, D, device=device, dtype=torch.bfloat16)
+    dv = torch.empty_like(dk)
+    kvb = B * L * Hkv * D * 2  # elements of K and V
+    add("reshape_from_cache bf16, 32 x 4096 tokens", timed(lambda: ops.reshape_from_cache(dk, dv, kc, vc, lens, L, None, table)),
+        2 * kvb * 2, "read + write")
+    ops.quant_to_paged_cache(ops.ReshapePagedCacheParams(
+        key=dk[:4096], value=dv[:4096], k_cache=kq, v_cache=vq, k_cache_scale=ksc, v_cache_scale=vsc,
+        slot_mapping=torch.arange(4096, device=device, dtype=torch.int32)))
+    add("dequant_from_paged_cache int8 -> bf16, 32 x 4096 tokens",
+        timed(lambda: ops.dequant_from_paged_cache(dk, dv, kq, vq, ksc, vsc, lens, L, None, table)),
+        kvb + B * L * Hkv * 4 * 2 + kvb * 2, "1-byte cache and scales read, bf16 written")
+    del dk, dv
     # a chunked-prefill step: 4 sequences, 512 new tokens each on top of a 3584-token prefix
     B, n, L = 4, 512, 4096
     q = torch.randn(B * n, Hq, D, device=device, dtype=torch.bfloat16, generator=gen)

@@ -366,6 +366,43 @@ int xllm_hip_copy_blocks(const xllm_hip_kv_cache* cache,
 /* Message of the last non-OK status returned on this host thread ("" if none). */
 const char* xllm_hip_last_error(void);
 
+/*
+ * Sequences read back out of the paged cache into dense tensors: the paged mode of
+ * xllm::kernel::reshape_from_cache (xllm/core/kernels/ops_api.cpp:182-196, arguments
+ * xllm/core/kernels/param.h:160-215, xllm/core/kernels/mlu/mlu_ops_api.h:56-64) and
+ * xllm::kernel::dequant_from_paged_cache (xllm/core/kernels/ops_api.cpp:214-232,
+ * xllm/core/kernels/mlu/mlu_ops_api.h:79-101; run before a chunked-prefill step over a quantised
+ * cache, xllm/core/layers/mlu/attention.cpp:179-214).  For every sequence b < batch and token
+ * t < context_lengths[b]:
+ *   pos = (cache_seq_offset ? cache_seq_offset[b] : 0) + t
+ *   blk = block_tables[b * block_table_stride + pos / block_size],  slot = pos % block_size
+ *   row = (context_seq_offset ? context_seq_offset[b] : context_lengths[0] + .. + context_lengths[b-1]) + t
+ *   key_out[row][h][d] = k_cache[blk][slot][h][d]            (same for value_out; NULL: keys only)
+ * key_out/value_out are [rows, num_kv_heads, head_dim] with a free token stride (elements).
+ * out_dtype == cache->dtype copies the elements verbatim (any dtype).  For an FP8_E4M3/INT8 cache
+ * out_dtype BF16/FP16/FP32 dequantises: (float)q * scale, rounded once to out_dtype, where the scale
+ * is the cache's per-(block, head, slot) one (quant_mode 1, per token) or k_scale/v_scale read as
+ * a dense [num_kv_heads, head_dim] array (quant_mode 0, per channel).  max_context_len bounds
+ * context_lengths (it sizes the grid; longer sequences are cut there).  Tokens whose block index
+ * lies beyond max_blocks_per_seq or whose block id is outside [0, num_blocks) are skipped.
+ */
+int xllm_hip_gather_from_cache(const xllm_hip_kv_cache* cache,
+                               void* key_out,
+                               void* value_out,
+                               int32_t out_dtype,
+                               int64_t key_token_stride,
+                               int64_t value_token_stride,
+                               const int32_t* context_lengths,
+                               const int32_t* context_seq_offset,
+                               const int32_t* cache_seq_offset,
+                               const int32_t* block_tables,
+                               int64_t block_table_stride,
+                               int32_t max_blocks_per_seq,
+                               int32_t batch,
+                               int32_t max_context_len,
+                               int32_t quant_mode,
+                               xllm_hip_stream_t stream);
+
 /* XLLM_HIP_ABI_VERSION the library was built with. */
 int xllm_hip_abi_version(void);
 

@@ -41,6 +41,13 @@ tree); how each one is pinned is listed beside it:
       xllm/models/llm/npu/llm_model_base.h:69-75; pinned by brute force on tiny caches (element
       loops), by the gather-before-scatter property on a chain a->b, b->c, and by the group arrays
       expanding back to the transfer list they came from.
+  reshape_from_cache / dequant_from_paged_cache
+      argument contract of xllm/core/kernels/param.h:160-215 and xllm/core/kernels/mlu/mlu_ops_api.h:56-101,
+      call site xllm/core/layers/mlu/attention.cpp:179-214; the bodies live in the closed `tmo`
+      library: PARITY UNPINNED beyond the documented contract.  Pinned by literal loops on tiny
+      caches, by the round trips reshape_paged_cache -> reshape_from_cache = identity and
+      quant_to_paged_cache -> dequant_from_paged_cache = dequantize(quantize(x)), and by agreement
+      with gather_sequence (the gather the attention oracle itself uses).
   quantize_per_token_head / quant_to_paged_cache
       scale and saturation conventions of xllm/core/kernels/cuda/fp8_quant_utils.cuh:38-53,112-131;
       the int8 rounding of `tmo::quant_to_paged_cache` (xllm/core/kernels/mlu/attention.cpp:50-59) is
@@ -338,6 +345,58 @@ def copy_blocks(arrays, src_block_indices, dst_block_indices, cum_sum):
             for i in range(begin, cum_sum[g]):
                 a[dst_block_indices[i]] = a[src]
             begin = cum_sum[g]
+
+
+# ---- sequences read back out of the cache -------------------------------------------------
+
+
+def reshape_from_cache(key_cache, value_cache, context_lengths, block_tables, context_seq_offset=None,
+                       cache_seq_offset=None, total_rows=None, layout="HND", fill=0):
+    """Paged mode of xllm::kernel::reshape_from_cache (xllm/core/kernels/param.h:160-201,
+    xllm/core/kernels/mlu/mlu_ops_api.h:56-64): token t of sequence b, stored at cache position
+    cache_seq_offset[b] + t (block block_tables[b][pos // bs], slot pos % bs), goes to output row
+    context_seq_offset[b] + t; without context_seq_offset the sequences are packed in order.
+    Returns (key [rows, H, D], value or None); rows no sequence covers hold `fill`.  Literal loops."""
+    kc = _hnd_view(key_cache, layout)
+    vc = _hnd_view(value_cache, layout) if value_cache is not None else None
+    bs = kc.shape[2]
+    lens = [int(x) for x in context_lengths]
+    if context_seq_offset is None:
+        context_seq_offset = np.concatenate([[0], np.cumsum(lens)[:-1]]) if lens else []
+    if total_rows is None:
+        total_rows = max([int(o) + n for o, n in zip(context_seq_offset, lens)], default=0)
+    key = np.full((total_rows, kc.shape[1], kc.shape[3]), fill, dtype=kc.dtype)
+    value = np.full((total_rows, vc.shape[1], vc.shape[3]), fill, dtype=vc.dtype) if vc is not None else None
+    for b, n in enumerate(lens):
+        start = int(cache_seq_offset[b]) if cache_seq_offset is not None else 0
+        for t in range(n):
+            pos = start + t
+            blk = int(block_tables[b][pos // bs])
+            key[int(context_seq_offset[b]) + t] = kc[blk, :, pos % bs, :]
+            if vc is not None:
+                value[int(context_seq_offset[b]) + t] = vc[blk, :, pos % bs, :]
+    return key, value
+
+
+def dequant_from_paged_cache(key_cache, value_cache, key_scale, value_scale, context_lengths, block_tables, kind,
+                             out_kind="fp32", quant_mode=1, context_seq_offset=None, total_rows=None):
+    """xllm::kernel::dequant_from_paged_cache (xllm/core/kernels/mlu/mlu_ops_api.h:79-101; HND cache,
+    call site xllm/core/layers/mlu/attention.cpp:196-214): the gather of reshape_from_cache applied to
+    the dequantised cache, (float)q * scale rounded once to the output type.  quant_mode 1: one scale
+    per (block, head, slot); quant_mode 0: one per (head, channel), scale arrays [H, D].
+    Returns float32 arrays holding values of `out_kind` ("fp32", "bf16", "fp16")."""
+    def dense(cache, scale):
+        if cache is None:
+            return None
+        if kind == "int8":
+            f = np.asarray(cache, np.int8).astype(np.float32)
+        else:
+            f = e4m3fn_to_float(np.asarray(cache).view(np.uint8))
+        sc = np.asarray(scale, np.float32)
+        f = f * (sc[..., None] if quant_mode == 1 else sc[None, :, None, :])
+        return round_to_dtype(f.astype(np.float32), out_kind).astype(np.float32)
+    return reshape_from_cache(dense(key_cache, key_scale), dense(value_cache, value_scale), context_lengths,
+                              block_tables, context_seq_offset=context_seq_offset, total_rows=total_rows)
 
 
 # ---- quantisers ------------------------------------------------------------------------

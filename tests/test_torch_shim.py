@@ -182,6 +182,50 @@ def test_kv_cache_swap_blocks_and_copy_blocks(gpu, shim):
 
 
 @pytest.mark.gpu
+def test_reshape_from_cache_and_dequant_from_paged_cache_params(gpu, shim):
+    """The ReshapeFromCacheParams operators give what the Python mirrors give (those are checked
+    bit-exactly against the oracle)."""
+    from xllm_wxh_amd import ops
+
+    print("case shim reshape_from_cache / dequant_from_paged_cache", flush=True)
+    g = torch.Generator().manual_seed(6)
+    k = torch.randint(-128, 128, (12, 2, 16, 128), generator=g, dtype=torch.int8).to(gpu)
+    v = torch.randint(-128, 128, (12, 2, 16, 128), generator=g, dtype=torch.int8).to(gpu)
+    ks, vs = torch.rand(12, 2, 16, generator=g).to(gpu), torch.rand(12, 2, 16, generator=g).to(gpu)
+    lens = torch.tensor([40, 7], dtype=torch.int32, device=gpu)
+    bt = torch.tensor([[3, 9, 1], [5, 0, 0]], dtype=torch.int32, device=gpu)
+
+    p = shim.ReshapeFromCacheParams()
+    p.key = torch.zeros(47, 2, 128, dtype=torch.bfloat16, device=gpu)
+    p.value = torch.zeros_like(p.key)
+    p.key_cache, p.value_cache = k, v
+    p.key_cache_quant_scale, p.value_cache_quant_scale = ks, vs
+    p.context_lengths, p.max_context_len, p.block_tables = lens, 40, bt
+    shim.dequant_from_paged_cache(p)
+    want_k, want_v = torch.zeros_like(p.key), torch.zeros_like(p.key)
+    ops.dequant_from_paged_cache(want_k, want_v, k, v, ks, vs, lens, 40, None, bt)
+    assert torch.equal(p.key, want_k) and torch.equal(p.value, want_v)
+    assert p.key.abs().sum() > 0
+
+    r = shim.ReshapeFromCacheParams()
+    r.key = torch.zeros(47, 2, 128, dtype=torch.int8, device=gpu)
+    r.key_cache = k
+    r.context_lengths, r.max_context_len, r.block_tables = lens, 40, bt
+    shim.reshape_from_cache(r)
+    want = torch.zeros_like(r.key)
+    ops.reshape_from_cache(want, None, k, None, lens, 40, None, bt)
+    assert torch.equal(r.key, want)
+    assert torch.equal(r.key[40:47], k[5, :, :7].permute(1, 0, 2))
+
+    r.block_tables = None  # the linear mode is refused, as is a dequant without scales
+    with pytest.raises(RuntimeError):
+        shim.reshape_from_cache(r)
+    p.key_cache_quant_scale = None
+    with pytest.raises(RuntimeError):
+        shim.dequant_from_paged_cache(p)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("norm", [True, False])
 def test_attention_impl_forward_qkv_equals_separate_steps(gpu, shim, norm):
     """forward_qkv (norm + rotation + KV write in one launch, then decode) gives bit for bit what the

@@ -38,6 +38,7 @@ EXPORTED_SYMBOLS = (
     "xllm_hip_swap_blocks_staging_bytes",
     "xllm_hip_swap_blocks",
     "xllm_hip_copy_blocks",
+    "xllm_hip_gather_from_cache",
     "xllm_hip_last_error",
     "xllm_hip_abi_version",
     "xllm_hip_paged_decode_variant",
@@ -167,6 +168,9 @@ def load():
     lib.xllm_hip_swap_blocks.restype = ctypes.c_int
     lib.xllm_hip_copy_blocks.argtypes = [P(KvCacheDesc), vp, vp, vp, i32, i32, vp]
     lib.xllm_hip_copy_blocks.restype = ctypes.c_int
+    lib.xllm_hip_gather_from_cache.argtypes = [P(KvCacheDesc), vp, vp, i32, i64, i64, vp, vp, vp, vp, i64, i32, i32,
+                                               i32, i32, vp]
+    lib.xllm_hip_gather_from_cache.restype = ctypes.c_int
     lib.xllm_hip_last_error.argtypes = []
     lib.xllm_hip_last_error.restype = ctypes.c_char_p
     lib.xllm_hip_abi_version.argtypes = []

@@ -15,7 +15,7 @@ CSRC_DIR = os.path.join(PKG_DIR, "csrc")
 LIB_NAME = "libxllm_hip_paged_kv.so"
 LIB_PATH = os.path.join(PKG_DIR, LIB_NAME)
 
-HIP_SOURCES = ["kv_write.hip", "block_move.hip", "rope_kv_write.hip", "paged_decode.hip", "c_abi_misc.hip"]
+HIP_SOURCES = ["kv_write.hip", "block_move.hip", "gather_from_cache.hip", "rope_kv_write.hip", "paged_decode.hip", "c_abi_misc.hip"]
 
 # -packed-fp32-ops is switched off: the compiler then never forms v_pk_*_f32.
 HIPCC_FLAGS = [

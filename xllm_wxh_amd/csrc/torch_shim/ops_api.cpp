@@ -124,6 +124,81 @@ void quant_to_paged_cache(ReshapePagedCacheParams& params) {
                                              dtype_code(params.key), current_stream(params.key)));
 }
 
+namespace {
+
+void gather_from_cache(ReshapeFromCacheParams& p, bool dequant) {
+  TORCH_CHECK(p.key.defined() && p.key_cache.defined() && p.context_lengths.defined(),
+              "key, key_cache and context_lengths are required");
+  TORCH_CHECK(p.block_tables.has_value() && p.block_tables->defined() && p.block_tables->dim() == 2,
+              "block_tables [batch, max_blocks] is required (the linear cache mode is not part of the paged path)");
+  TORCH_CHECK(p.key.dim() == 3 && p.key.stride(-1) == 1 && p.key.stride(-2) == p.key.size(-1),
+              "key must be [total_length, num_kv_heads, head_dim], contiguous in its last two dimensions");
+  const bool has_v = p.value.has_value() && p.value->defined();
+  if (has_v) {
+    TORCH_CHECK(p.value_cache.has_value() && p.value_cache->defined(), "value given without value_cache");
+    TORCH_CHECK(p.value->dim() == 3 && p.value->scalar_type() == p.key.scalar_type() &&
+                    p.value->size(1) == p.key.size(1) && p.value->size(2) == p.key.size(2) &&
+                    p.value->stride(-1) == 1 && p.value->stride(-2) == p.value->size(-1),
+                "value must match key in dtype and row shape");
+  }
+  TORCH_CHECK(p.key.size(1) == p.key_cache.size(1) && p.key.size(2) == p.key_cache.size(3),
+              "key heads/head_dim do not match the cache");
+  auto i32 = [](const torch::Tensor& t) { return t.scalar_type() == torch::kInt && t.is_cuda(); };
+  TORCH_CHECK(i32(p.context_lengths) && i32(*p.block_tables) && p.block_tables->stride(1) == 1,
+              "context_lengths and block_tables must be int32 tensors on the GPU");
+  const int64_t batch = p.context_lengths.numel();
+  TORCH_CHECK(p.block_tables->size(0) >= batch, "one block_tables row per sequence");
+  torch::Tensor lens = p.context_lengths.contiguous(), rows, starts;
+  if (p.context_seq_offset.has_value() && p.context_seq_offset->defined()) {
+    TORCH_CHECK(i32(*p.context_seq_offset) && p.context_seq_offset->numel() == batch, "bad context_seq_offset");
+    rows = p.context_seq_offset->contiguous();
+  }
+  if (p.cache_seq_offset.has_value() && p.cache_seq_offset->defined()) {
+    TORCH_CHECK(i32(*p.cache_seq_offset) && p.cache_seq_offset->numel() == batch, "bad cache_seq_offset");
+    starts = p.cache_seq_offset->contiguous();
+  }
+  const std::optional<torch::Tensor> vc = has_v ? p.value_cache : std::nullopt;
+  xllm_hip_kv_cache cache;
+  if (!dequant) {
+    TORCH_CHECK(p.key.scalar_type() == p.key_cache.scalar_type(),
+                "reshape_from_cache copies verbatim: key and key_cache dtypes differ");
+    cache = make_cache(p.key_cache, vc, std::nullopt, std::nullopt);
+  } else {
+    TORCH_CHECK(p.quant_bit == 8, "only 8-bit caches exist on this path");
+    TORCH_CHECK(p.key_cache_quant_scale.has_value() && p.key_cache_quant_scale->defined(),
+                "key_cache_quant_scale is required for dequant_from_paged_cache");
+    TORCH_CHECK(p.key_cache.element_size() == 1 && p.key.element_size() > 1,
+                "dequant_from_paged_cache reads a 1-byte cache into bf16/fp16/fp32 tensors");
+    if (p.quant_mode == 1) {
+      cache = make_cache(p.key_cache, vc, p.key_cache_quant_scale, has_v ? p.value_cache_quant_scale : std::nullopt);
+      TORCH_CHECK(!has_v || cache.v_scale != nullptr, "value needs value_cache_quant_scale");
+    } else {
+      TORCH_CHECK(p.quant_mode == 0, "quant_mode must be 0 (per channel) or 1 (per token)");
+      cache = make_cache(p.key_cache, vc, std::nullopt, std::nullopt);
+      auto channel = [&](const std::optional<torch::Tensor>& s) {
+        TORCH_CHECK(s.has_value() && s->defined() && s->scalar_type() == torch::kFloat && s->is_contiguous() &&
+                        s->dim() == 2 && s->size(0) == cache.num_kv_heads && s->size(1) == cache.head_dim,
+                    "per-channel scales must be contiguous float32 [num_kv_heads, head_dim]");
+        return s->data_ptr<float>();
+      };
+      cache.k_scale = channel(p.key_cache_quant_scale);
+      if (has_v) cache.v_scale = channel(p.value_cache_quant_scale);
+    }
+  }
+  check_status(xllm_hip_gather_from_cache(
+      &cache, p.key.data_ptr(), has_v ? p.value->data_ptr() : nullptr, dtype_code(p.key), p.key.stride(0),
+      has_v ? p.value->stride(0) : 0, lens.data_ptr<int32_t>(), rows.defined() ? rows.data_ptr<int32_t>() : nullptr,
+      starts.defined() ? starts.data_ptr<int32_t>() : nullptr, p.block_tables->data_ptr<int32_t>(),
+      p.block_tables->stride(0), (int32_t)p.block_tables->size(1), (int32_t)batch, (int32_t)p.max_context_len,
+      (int32_t)p.quant_mode, current_stream(p.key)));
+}
+
+}  // namespace
+
+void reshape_from_cache(ReshapeFromCacheParams& params) { gather_from_cache(params, false); }
+
+void dequant_from_paged_cache(ReshapeFromCacheParams& params) { gather_from_cache(params, true); }
+
 namespace hip {
 
 torch::Tensor decode_workspace(const torch::Device& device, size_t bytes) {

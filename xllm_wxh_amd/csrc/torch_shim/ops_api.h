@@ -22,6 +22,13 @@ void reshape_paged_cache(ReshapePagedCacheParams& params);
 // xllm/core/kernels/ops_api.h:35-37 — per-token-per-head quantising KV write (int8 / fp8-e4m3).
 void quant_to_paged_cache(ReshapePagedCacheParams& params);
 
+// xllm/core/kernels/ops_api.h:33 — cached sequences copied verbatim into dense tensors (paged mode).
+void reshape_from_cache(ReshapeFromCacheParams& params);
+
+// xllm/core/kernels/ops_api.h:41 — the same gather out of a quantised cache, dequantising on the way
+// (what xllm/core/layers/mlu/attention.cpp:196-214 runs before a chunked prefill).
+void dequant_from_paged_cache(ReshapeFromCacheParams& params);
+
 namespace hip {
 
 // Argument list of xllm::kernel::mlu::batch_decode (xllm/core/kernels/mlu/mlu_ops_api.h:126-145).

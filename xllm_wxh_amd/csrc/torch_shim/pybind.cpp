@@ -7,6 +7,7 @@
 
 namespace py = pybind11;
 using xllm::KVCache;
+using xllm::kernel::ReshapeFromCacheParams;
 using xllm::kernel::ReshapePagedCacheParams;
 using xllm::layer::AttentionImpl;
 using xllm::layer::AttentionMetadata;
@@ -22,6 +23,23 @@ PYBIND11_MODULE(_xllm_hip_torch, m) {
       .def_readwrite("direction", &ReshapePagedCacheParams::direction)
       .def_readwrite("k_cache_scale", &ReshapePagedCacheParams::k_cache_scale)
       .def_readwrite("v_cache_scale", &ReshapePagedCacheParams::v_cache_scale);
+  py::class_<ReshapeFromCacheParams>(m, "ReshapeFromCacheParams")
+      .def(py::init<>())
+      .def_readwrite("key", &ReshapeFromCacheParams::key)
+      .def_readwrite("value", &ReshapeFromCacheParams::value)
+      .def_readwrite("key_cache", &ReshapeFromCacheParams::key_cache)
+      .def_readwrite("value_cache", &ReshapeFromCacheParams::value_cache)
+      .def_readwrite("context_lengths", &ReshapeFromCacheParams::context_lengths)
+      .def_readwrite("max_context_len", &ReshapeFromCacheParams::max_context_len)
+      .def_readwrite("context_seq_offset", &ReshapeFromCacheParams::context_seq_offset)
+      .def_readwrite("block_tables", &ReshapeFromCacheParams::block_tables)
+      .def_readwrite("cache_seq_offset", &ReshapeFromCacheParams::cache_seq_offset)
+      .def_readwrite("key_cache_quant_scale", &ReshapeFromCacheParams::key_cache_quant_scale)
+      .def_readwrite("value_cache_quant_scale", &ReshapeFromCacheParams::value_cache_quant_scale)
+      .def_readwrite("quant_mode", &ReshapeFromCacheParams::quant_mode)
+      .def_readwrite("quant_bit", &ReshapeFromCacheParams::quant_bit);
+  m.def("reshape_from_cache", &xllm::kernel::reshape_from_cache);
+  m.def("dequant_from_paged_cache", &xllm::kernel::dequant_from_paged_cache);
   m.def("reshape_paged_cache", &xllm::kernel::reshape_paged_cache);
   m.def("quant_to_paged_cache", &xllm::kernel::quant_to_paged_cache);
   m.def("batch_decode",

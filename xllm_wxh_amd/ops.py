@@ -377,6 +377,69 @@ def copy_blocks(k_cache, v_cache, src_block_indices, dst_block_indices, cum_sum,
                                         src_block_indices.numel(), dst_block_indices.numel(), _stream()))
 
 
+def _gather_from_cache(key, value, key_cache, value_cache, key_scale, value_scale, context_lengths, max_context_len,
+                       context_seq_offset, block_tables, cache_seq_offset, quant_mode, kv_layout):
+    lib = _lib.load()
+    _require(key.is_cuda and key.dim() == 3 and key.stride(2) == 1 and key.stride(1) == key.size(2),
+             "key must be a GPU tensor [rows, num_kv_heads, head_dim] with the last two dimensions contiguous")
+    if value is not None:
+        _require(value_cache is not None, "value given without value_cache")
+        _require(value.dtype == key.dtype and value.shape[1:] == key.shape[1:] and value.stride(2) == 1 and
+                 value.stride(1) == value.size(2), "value must match key in dtype and row shape")
+    _require(block_tables is not None and block_tables.dim() == 2, "block_tables [batch, max_blocks] is required "
+             "(the linear cache mode of the reference is not part of the paged path)")
+    for t in (context_lengths, block_tables, context_seq_offset, cache_seq_offset):
+        _require(t is None or (t.dtype == torch.int32 and t.is_cuda), "index tensors must be int32 on the GPU")
+    _require(block_tables.stride(1) == 1, "block_tables rows must be contiguous")
+    batch = context_lengths.numel()
+    _require(block_tables.size(0) >= batch, "one block_tables row per sequence")
+    per_channel = key_scale is not None and quant_mode == 0
+    desc = _cache_desc(key_cache, value_cache if value is not None else None,
+                       None if per_channel else key_scale, None if per_channel else value_scale, kv_layout)
+    if per_channel:
+        for sc in (key_scale, value_scale if value is not None else None):
+            _require(sc is None or (sc.dtype == torch.float32 and sc.is_contiguous() and
+                                    tuple(sc.shape) == (desc.num_kv_heads, desc.head_dim)),
+                     "per-channel scales must be contiguous float32 [num_kv_heads, head_dim]")
+        desc.k_scale = key_scale.data_ptr()
+        desc.v_scale = value_scale.data_ptr() if value is not None and value_scale is not None else None
+    _require(tuple(key.shape[1:]) == (desc.num_kv_heads, desc.head_dim), "key rows do not match the cache")
+    cl = context_lengths.contiguous()
+    cso = context_seq_offset.contiguous() if context_seq_offset is not None else None
+    cao = cache_seq_offset.contiguous() if cache_seq_offset is not None else None
+    _lib.check(lib.xllm_hip_gather_from_cache(
+        ctypes.byref(desc), _ptr(key), _ptr(value) if value is not None else None, _dtype_code(key), key.stride(0),
+        value.stride(0) if value is not None else 0, _ptr(cl), _ptr(cso) if cso is not None else None,
+        _ptr(cao) if cao is not None else None, _ptr(block_tables), block_tables.stride(0), block_tables.size(1),
+        batch, int(max_context_len), int(quant_mode), _stream()))
+
+
+def reshape_from_cache(key, value, key_cache, value_cache, context_lengths, max_context_len, context_seq_offset=None,
+                       block_tables=None, cache_seq_offset=None, *, kv_layout="HND"):
+    """Paged mode of xllm::kernel::mlu::reshape_from_cache (xllm/core/kernels/mlu/mlu_ops_api.h:56-64;
+    fields xllm/core/kernels/param.h:160-201): the cached tokens of every sequence copied verbatim
+    into key/value [rows, num_kv_heads, head_dim] (same dtype as the cache), sequence b starting at
+    row context_seq_offset[b] (default: packed in order)."""
+    _require(key.dtype == key_cache.dtype, "reshape_from_cache copies verbatim: key and key_cache dtypes differ")
+    _gather_from_cache(key, value, key_cache, value_cache, None, None, context_lengths, max_context_len,
+                       context_seq_offset, block_tables, cache_seq_offset, 1, kv_layout)
+
+
+def dequant_from_paged_cache(key, value, key_cache, value_cache, key_cache_quant_scale, value_cache_quant_scale,
+                             context_lengths, max_context_len, context_seq_offset, block_tables, quant_mode=1,
+                             quant_bit=8, *, kv_layout="HND"):
+    """xllm::kernel::mlu::dequant_from_paged_cache (xllm/core/kernels/mlu/mlu_ops_api.h:79-101), the
+    step before a chunked prefill over a quantised cache (xllm/core/layers/mlu/attention.cpp:196-214):
+    key/value [rows, num_kv_heads, head_dim] in bf16/fp16/fp32 receive (float)q * scale.
+    quant_mode 1: scales [num_blocks, num_kv_heads, block_size]; 0: [num_kv_heads, head_dim]."""
+    _require(quant_bit == 8, "only 8-bit caches exist on this path")
+    _require(key_cache.dtype in (torch.int8, torch.float8_e4m3fn, torch.uint8), "key_cache is not quantised")
+    _require(key_cache_quant_scale is not None, "key_cache_quant_scale is required for dequant_from_paged_cache")
+    _require(value is None or value_cache_quant_scale is not None, "value needs value_cache_quant_scale")
+    _gather_from_cache(key, value, key_cache, value_cache, key_cache_quant_scale, value_cache_quant_scale,
+                       context_lengths, max_context_len, context_seq_offset, block_tables, None, quant_mode, kv_layout)
+
+
 def _rope_call(qkv, num_q, num_k, num_v, head_dim, eps, q_weight, k_weight, cos_sin_cache, interleaved, positions,
                round_each_op, cache_desc=None, slot_mapping=None):
     lib = _lib.load()
