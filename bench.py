@@ -350,9 +350,11 @@ def aux_kernels(torch, ops, device):
     us = timed(lambda: ops.batch_decode(q, kc, out, table, lens, vc, scale=D ** -0.5, q_per_seq=n, q_indptr=q_indptr,
                                         max_seq_len=L, total_kv_len=B * L), n=10)
     flops = 4.0 * B * Hq * D * sum(L - n + 1 + j for j in range(n))
-    res["entries"].append({"kernel": "chunked prefill through the decode kernel, 4 x 512 tokens on a 3584-token prefix",
+    res["entries"].append({"kernel": "chunked prefill (128-row kernel), 4 x 512 tokens on a 3584-token prefix, bf16",
                            "us": round(us, 1), "tflops": round(flops / us / 1e6, 1),
-                           "note": "every 32 query rows stream the sequence's K/V again, from the L2 of their XCD"})
+                           "frac_of_mfma_peak": round(flops / us / 1e6 / 2500.0, 3),
+                           "note": "flops of the visible (causal) part only; every 128 query rows stream the "
+                                   "sequence's K/V again, from the L2 of their XCD"})
     # speculative verify with 64 query rows per kv head (64 q heads, 8 draft tokens): two row groups
     B, n, L, Hq2 = 32, 8, 8192, 64
     q = torch.randn(B * n, Hq2, D, device=device, dtype=torch.bfloat16, generator=gen)

@@ -83,3 +83,68 @@ def test_prefill_sized_chunks_and_edge_cases(gpu):
     c4 = Case(3, 14, 2, 64, 16, [50, 333, 20], kv="fp32", qdt="fp32", seed=12)
     out4, _, ref4, _, _ = _run(c4, [5, 40, 20], 40)
     assert float(np.abs(out4 - ref4).max()) <= 1e-4
+
+
+@pytest.mark.parametrize("D,bs,layout", [(128, 16, "HND"), (128, 128, "NHD"), (64, 32, "HND"), (64, 64, "NHD")])
+@pytest.mark.parametrize("qdt", ["bf16", "fp16"])
+def test_many_row_kernel_shapes(gpu, D, bs, layout, qdt):
+    """16-bit caches with more than 64 query rows per kv head take the 128-row kernel (tiles go from
+    global memory straight to LDS): lengths around its tile and buffer counts, chunks that are the
+    whole sequence, a chunk shorter than one row group, sequences without query tokens."""
+    print("case many rows", D, bs, layout, qdt, flush=True)
+    lens = [1, 31, 32, 33, 127, 129, 160, 1000, 97, 2500]
+    q_counts = [1, 31, 32, 33, 100, 129, 0, 300, 97, 257]
+    kv = "bf16" if qdt == "bf16" else "fp16"
+    c = Case(len(lens), 32, 8, D, bs, lens, kv=kv, qdt=qdt, layout=layout, seed=31)
+    q_indptr = np.concatenate([[0], np.cumsum(q_counts)]).astype(np.int32)
+    T = int(q_indptr[-1])
+    dt = torch.bfloat16 if qdt == "bf16" else torch.float16
+    q = torch.randn(T, c.Hq, c.D, generator=torch.Generator().manual_seed(78)).to(dt)
+    qd = q.to(c.q.device)
+    out = torch.full_like(qd, 7.0)
+    lse = torch.full((T, c.Hq), 3.0, dtype=torch.float32, device=qd.device)
+    ops.batch_decode(qd, c.k_cache, out, c.block_table, c.seq_lens, c.v_cache, lse, scale=c.scale, return_lse=True,
+                     q_per_seq=max(q_counts), q_indptr=torch.from_numpy(q_indptr).to(qd.device), kv_layout=layout)
+    torch.cuda.synchronize()
+    ref, ref_lse = orc.paged_decode_ragged(q.float().numpy(), c.k_ref, c.v_ref, c.table, c.lens, q_indptr, c.scale)
+    got = out.float().cpu().numpy()
+    assert not np.isnan(got).any()
+    err = float(np.abs(got - ref).max())
+    print("   err %.3e" % err, flush=True)
+    assert err <= 1.2e-2
+    fin = np.isfinite(ref_lse)
+    assert np.allclose(lse.cpu().numpy()[fin], ref_lse[fin], atol=2e-2)
+
+
+def test_many_row_kernel_split_sequences_and_window(gpu):
+    """65 to 128 rows per kv head: one 128-row item per (sequence, kv head), split into chunks like
+    any decode step when the batch is small; and a sliding window over a chunked step."""
+    print("case many rows split / window", flush=True)
+    c = Case(2, 64, 8, 128, 16, [9000, 700], n=12, seed=32)  # 96 rows; 9000 tokens are split
+    ref, lse_ref = c.oracle()
+    out, lse = c.run()
+    assert float(np.abs(out.float().cpu().numpy() - ref).max()) <= 1.2e-2
+    c = Case(2, 32, 8, 128, 16, [3000, 517], n=40, seed=33)  # 160 rows, window
+    ref, _ = c.oracle(301)
+    out, _ = c.run(301)
+    assert float(np.abs(out.float().cpu().numpy() - ref).max()) <= 1.2e-2
+
+
+def test_garbage_past_the_sequence_end_does_not_reach_the_many_row_kernel(gpu):
+    print("case many rows garbage", flush=True)
+    lens = [45, 200]
+    c = Case(2, 32, 8, 128, 16, lens, n=24, seed=34)
+    ref, _ = c.oracle()
+    # NaN in every slot past the end of each sequence's last block and in unused blocks
+    nan = float("nan")
+    used = torch.zeros(c.k_cache.size(0), 16, dtype=torch.bool)
+    for b, L in enumerate(lens):
+        for t in range(L):
+            used[c.table[b, t // 16], t % 16] = True
+    mask = (~used).to(c.k_cache.device)
+    c.k_cache.permute(0, 2, 1, 3)[mask] = nan
+    c.v_cache.permute(0, 2, 1, 3)[mask] = nan
+    out, _ = c.run()
+    got = out.float().cpu().numpy()
+    assert not np.isnan(got).any()
+    assert float(np.abs(got - ref).max()) <= 1.2e-2

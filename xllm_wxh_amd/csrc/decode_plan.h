@@ -25,7 +25,9 @@ constexpr int kTileTokens = 32;       // rows per MFMA tile (one token each, two
 constexpr int kMinChunkTokens = 512;  // smallest split worth a partial round trip (128 tokens per wave)
 constexpr int kMinChunkTokensGeneric = 64;  // the one-wave kernel: one 64-token step
 constexpr int kMaxTargetItems = 4096; // upper bound of the split target (sizes the workspace)
-constexpr int kMaxRowsPerItem = 32;   // query rows (g * n) one work item of the MFMA kernels handles
+constexpr int kMaxRowsPerItem = 32;   // query rows (g * n) one work item of the MFMA decode kernels handles
+constexpr int kPrefillRowsPerItem = 128;  // ... and of the many-row (prefill) kernel, used above kPrefillMinRows rows
+constexpr int kPrefillMinRows = 64;
 
 #if defined(__HIPCC__)
 #define XLLM_HIP_HD __host__ __device__

@@ -66,7 +66,7 @@ struct DecodeParams {
   int32_t rows;   // group * n
   int32_t row_groups;
   int32_t cluster;        // neighbouring work items kept on one XCD (see decode_item)
-  int32_t rows_per_item;  // query rows one work item handles (32 MFMA, 1 generic)
+  int32_t rows_per_item;  // query rows one work item handles (32 or 128 MFMA, 1 generic)
   int32_t min_chunk;      // smallest chunk the plan may choose
   int32_t head_dim;
   int32_t tok;          // tokens per 256-byte LDS row of the MFMA kernels: 1 (head_dim 128) or 2 (head_dim 64)
@@ -296,6 +296,12 @@ __device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it)
   it.t_begin = chunk * chunk_tokens;
   const long long end = (long long)it.t_begin + chunk_tokens;
   it.t_end = end < it.len ? (int)end : it.len;
+  {  // no row of the item sees beyond the causal limit of its last row
+    const int rows = it.n * p.group;
+    const int last = min((it.rg + 1) * p.rows_per_item, rows) - 1;
+    const int lim = it.len - (it.n - 1 - last / p.group);
+    it.t_end = it.t_end < lim ? it.t_end : lim;
+  }
   if (p.kv_indptr != nullptr) {
     it.ids = p.block_ids + p.kv_indptr[it.b];
   } else {
@@ -428,6 +434,16 @@ __device__ inline int block_of(const DecodeParams& p, const Item& it, int tok) {
   int bi = tok >> p.log2_bs;
   bi = bi < it.nblk ? bi : it.nblk - 1;
   return __builtin_amdgcn_readfirstlane(it.ids[bi]);
+}
+
+// The same through the constant address space, which makes the load a scalar one whatever else the
+// kernel does (after a global-to-LDS load the compiler no longer proves on its own that the table is
+// unchanged, and a vector load here would make its wait cover every tile in flight).  The block
+// lists are never written by these kernels.
+__device__ inline int block_of_const(const DecodeParams& p, const Item& it, int tok) {
+  int bi = tok >> p.log2_bs;
+  bi = bi < it.nblk ? bi : it.nblk - 1;
+  return ((const __attribute__((address_space(4))) int32_t*)it.ids)[bi];
 }
 
 // Uniform (scalar-register) part of the addresses of 16 consecutive tokens starting at `tok`
@@ -752,7 +768,7 @@ struct RowTile {
   __device__ inline void init(const DecodeParams& p, const Item& it, int row_in_item, int lane) {
     const int mi = lane & 15;  // MFMA row of A / column of B and D
     kg = lane >> 4;            // k-group of the operands; row block of D
-    const int row = it.rg * kMaxRowsPerItem + row_in_item + mi;
+    const int row = it.rg * p.rows_per_item + row_in_item + mi;
     const bool valid = row < it.n * p.group;
     const int j = valid ? row / p.group : 0;
     const int gq = valid ? row - j * p.group : 0;
@@ -789,48 +805,53 @@ struct RowTile {
     v_off0 = kLdsV + swz_v(tau, (mi & 3) >> 1) + (mi & 1) * 8;
   }
 
-  // Attention of the 16 query rows over the 32 * TOK tokens parked in `tile` (first token tb).
-  // Score / weight index i = (u * 2 + h) * 4 + rr: token TOK * (16h + 4kg + rr) + u of the tile.
-  template <bool MASKED>
-  __device__ inline void attend(const uint8_t* tile, int tb, float scale_log2) {
-    const float neg_inf = -INFINITY;
-    constexpr int kN = 8 * TOK;  // scores per lane
-    float kscl[kN], lv[kN], rvs[kN];
-    if (kQuant) {
-      // the factors of tokens TOK * (16h + 4kg) .. + 4 * TOK - 1 are contiguous in each array
-      constexpr int kArr = 32 * TOK * 4;  // bytes per array
+  static constexpr int kN = 8 * TOK;  // scores per lane and tile
+  // (per-token factors of a quantised tile travel as three arrays in score order: as one struct
+  // they cost registers to the point of spilling)
+  typedef f32x4 Scores[TOK][2];
+
+  __device__ __forceinline__ void load_factors(const uint8_t* tile, float (&kscl)[kN], float (&lv)[kN], float (&rvs)[kN]) const {
+    if (!kQuant) return;
+    // the factors of tokens TOK * (16h + 4kg) .. + 4 * TOK - 1 are contiguous in each array
+    constexpr int kArr = 32 * TOK * 4;  // bytes per array
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const int first = TOK * (16 * h + 4 * kg) * 4;
+    for (int h = 0; h < 2; ++h) {
+      const int first = TOK * (16 * h + 4 * kg) * 4;
 #pragma unroll
-        for (int v4 = 0; v4 < TOK; ++v4) {
-          const f32x4 a = *(const f32x4*)(tile + kLdsSc + first + 16 * v4);
-          const f32x4 b = *(const f32x4*)(tile + kLdsSc + kArr + first + 16 * v4);
-          const f32x4 c = *(const f32x4*)(tile + kLdsSc + 2 * kArr + first + 16 * v4);
+      for (int v4 = 0; v4 < TOK; ++v4) {
+        const f32x4 a = *(const f32x4*)(tile + kLdsSc + first + 16 * v4);
+        const f32x4 b = *(const f32x4*)(tile + kLdsSc + kArr + first + 16 * v4);
+        const f32x4 c = *(const f32x4*)(tile + kLdsSc + 2 * kArr + first + 16 * v4);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int t = 4 * v4 + e;  // token of the lane's 4 * TOK: row rr = t / TOK, u = t % TOK
-            const int i = ((t % TOK) * 2 + h) * 4 + t / TOK;
-            kscl[i] = a[e];
-            lv[i] = b[e];
-            rvs[i] = c[e];
-          }
+        for (int e = 0; e < 4; ++e) {
+          const int t = 4 * v4 + e;  // token of the lane's 4 * TOK: row rr = t / TOK, u = t % TOK
+          const int i = ((t % TOK) * 2 + h) * 4 + t / TOK;
+          kscl[i] = a[e];
+          lv[i] = b[e];
+          rvs[i] = c[e];
         }
       }
     }
-    // ---- S^T = K Q^T ----
-    f32x4 s[TOK][2];
+  }
+
+  // ---- S^T = K Q^T: chunk c of the rows' 128 elements, K fragments of the tile's two halves ----
+  __device__ __forceinline__ void scores_init(Scores& s) const {
 #pragma unroll
     for (int u = 0; u < TOK; ++u) s[u][0] = s[u][1] = f32x4{s_init, s_init, s_init, s_init};
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const uint32_t ko = k_off0 ^ (uint32_t)(c << 6);
-      const Op kf0 = *(const Op*)(tile + ko);
-      const Op kf1 = *(const Op*)(tile + ko + 4096);
-      s[c / kQC][0] = Mma<KV_DT>::run(kf0, qf[c % kQC], s[c / kQC][0]);
-      s[c / kQC][1] = Mma<KV_DT>::run(kf1, qf[c % kQC], s[c / kQC][1]);
-    }
-    // ---- online softmax of the lane's query row ----
+  }
+  __device__ __forceinline__ void scores_step(int c, const Op& kf0, const Op& kf1, Scores& s) const {
+    s[c / kQC][0] = Mma<KV_DT>::run(kf0, qf[c % kQC], s[c / kQC][0]);
+    s[c / kQC][1] = Mma<KV_DT>::run(kf1, qf[c % kQC], s[c / kQC][1]);
+  }
+
+  // ---- online softmax of the lane's query row over the tile starting at token tb ----
+  // Score / weight index i = (u * 2 + h) * 4 + rr: token TOK * (16h + 4kg + rr) + u of the tile.
+  // Leaves the weights as B operand of the second MFMA (k-slot e = 4h + rr) in pf and the factor
+  // the accumulators are to be scaled by in alpha; returns whether any row's maximum moved.
+  template <bool MASKED>
+  __device__ __forceinline__ bool softmax(const Scores& s, const float (&kscl)[kN], const float (&lv)[kN], const float (&rvs)[kN], int tb, float scale_log2, Op (&pf)[TOK],
+                                 float& alpha) {
+    const float neg_inf = -INFINITY;
     float x[kN];
     float mt = neg_inf;
 #pragma unroll
@@ -854,7 +875,7 @@ struct RowTile {
     const float m_new = fmaxf(m_run, mt);
     const float m_safe = m_new == neg_inf ? 0.0f : m_new;
     const bool moved = __builtin_amdgcn_ballot_w64(m_new != m_run) != 0;
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_safe);
+    alpha = __builtin_amdgcn_exp2f(m_run - m_safe);
     l_run *= alpha;
     m_run = m_new;
     float w[kN];
@@ -864,7 +885,6 @@ struct RowTile {
       w[i] = e;
       l_run = kQuant ? __builtin_fmaf(e, rvs[i], l_run) : l_run + e;
     }
-    Op pf[TOK];  // B operand of the second MFMA: k-slot e = 4h + rr
 #pragma unroll
     for (int u = 0; u < TOK; ++u) {
       const float* wu = w + 8 * u;
@@ -872,7 +892,56 @@ struct RowTile {
                         Mma<KV_DT>::pack(wu[6], wu[7])};
       pf[u] = __builtin_bit_cast(Op, pw);
     }
-    // ---- O^T = O^T * alpha + V^T P^T ----
+    return moved;
+  }
+
+  // ---- O^T = O^T * alpha + V^T P^T, tile dt of the rows' 128 elements ----
+  __device__ __forceinline__ Op v_fragment(const uint8_t* tile, int dt) const {
+    const uint32_t vo = v_off0 ^ (uint32_t)(dt << 5);
+    const s16x4 a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (__attribute__((address_space(3))) s16x4*)(tile + vo));
+    const s16x4 a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (__attribute__((address_space(3))) s16x4*)(tile + vo + 4096));
+    return __builtin_bit_cast(Op, __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7));
+  }
+  template <bool RESCALE>
+  __device__ __forceinline__ void accumulate_step(int dt, const Op& vf, const Op (&pf)[TOK], float alpha) {
+    f32x4 c = acc[dt];
+    if (RESCALE) c *= alpha;
+    acc[dt] = Mma<KV_DT>::run(vf, pf[dt * TOK / 8], c);
+  }
+  template <bool RESCALE>
+  __device__ __forceinline__ void accumulate_weights(const Op (&pf)[TOK], float alpha) {
+    if (!kOffset) return;
+    const u32x4 ones = {0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u};  // fp16 1.0
+    f32x4 c = wacc;
+    if (RESCALE) c *= alpha;
+#pragma unroll
+    for (int u = 0; u < TOK; ++u) c = Mma<KV_DT>::run(__builtin_bit_cast(Op, ones), pf[u], c);
+    wacc = c;
+  }
+  template <bool RESCALE>
+  __device__ __forceinline__ void accumulate(const uint8_t* tile, const Op (&pf)[TOK], float alpha) {
+#pragma unroll
+    for (int dt = 0; dt < 8; ++dt) accumulate_step<RESCALE>(dt, v_fragment(tile, dt), pf, alpha);
+    accumulate_weights<RESCALE>(pf, alpha);
+  }
+
+  // Attention of the 16 query rows over the 32 * TOK tokens parked in `tile` (first token tb).
+  template <bool MASKED>
+  __device__ __forceinline__ void attend(const uint8_t* tile, int tb, float scale_log2) {
+    float kscl[kN], lv[kN], rvs[kN];
+    load_factors(tile, kscl, lv, rvs);
+    Scores s;
+    scores_init(s);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const uint32_t ko = k_off0 ^ (uint32_t)(c << 6);
+      scores_step(c, *(const Op*)(tile + ko), *(const Op*)(tile + ko + 4096), s);
+    }
+    Op pf[TOK];
+    float alpha;
+    const bool moved = softmax<MASKED>(s, kscl, lv, rvs, tb, scale_log2, pf, alpha);
     // The accumulators need rescaling only when some row's maximum moved, which becomes rare a few
     // tiles into a sequence.  Both variants of the product are written out, so that each path ends
     // in the MFMAs that define the accumulators (a branch around the multiplies alone makes the
@@ -883,39 +952,61 @@ struct RowTile {
       accumulate<false>(tile, pf, alpha);
     }
   }
+};
 
-  template <bool RESCALE>
-  __device__ inline void accumulate(const uint8_t* tile, const Op (&pf)[TOK], float alpha) {
+// The same for two row tiles held by one wave (32 query rows): every K and V fragment read from
+// LDS feeds two MFMAs, which is what keeps a prefill-sized step from being bound by LDS bandwidth.
+template <bool MASKED, int KV_DT, int TOK>
+__device__ __forceinline__ void attend_pair(RowTile<KV_DT, TOK> (&rt)[2], const uint8_t* tile, int tb, float scale_log2) {
+  typedef RowTile<KV_DT, TOK> RT;
+  typedef typename RT::Op Op;
+  float kscl[RT::kN], lv[RT::kN], rvs[RT::kN];
+  rt[0].load_factors(tile, kscl, lv, rvs);
+  typename RT::Scores s0, s1;
+  rt[0].scores_init(s0);
+  rt[1].scores_init(s1);
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const uint32_t ko = rt[0].k_off0 ^ (uint32_t)(c << 6);
+    const Op kf0 = *(const Op*)(tile + ko);
+    const Op kf1 = *(const Op*)(tile + ko + 4096);
+    rt[0].scores_step(c, kf0, kf1, s0);
+    rt[1].scores_step(c, kf0, kf1, s1);
+  }
+  Op pf0[TOK], pf1[TOK];
+  float alpha0, alpha1;
+  const bool moved0 = rt[0].template softmax<MASKED>(s0, kscl, lv, rvs, tb, scale_log2, pf0, alpha0);
+  __builtin_amdgcn_sched_barrier(0);  // one softmax at a time: interleaving the two costs registers
+  const bool moved1 = rt[1].template softmax<MASKED>(s1, kscl, lv, rvs, tb, scale_log2, pf1, alpha1);
+  if (moved0 || moved1) {  // the factor of a tile whose maxima stayed is exactly 1
 #pragma unroll
     for (int dt = 0; dt < 8; ++dt) {
-      const uint32_t vo = v_off0 ^ (uint32_t)(dt << 5);
-      const s16x4 a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (__attribute__((address_space(3))) s16x4*)(tile + vo));
-      const s16x4 a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (__attribute__((address_space(3))) s16x4*)(tile + vo + 4096));
-      const Op vf = __builtin_bit_cast(Op, __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7));
-      f32x4 c = acc[dt];
-      if (RESCALE) c *= alpha;
-      acc[dt] = Mma<KV_DT>::run(vf, pf[dt * TOK / 8], c);
+      const Op vf = rt[0].v_fragment(tile, dt);
+      rt[0].template accumulate_step<true>(dt, vf, pf0, alpha0);
+      rt[1].template accumulate_step<true>(dt, vf, pf1, alpha1);
     }
-    if (kOffset) {
-      const u32x4 ones = {0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u};  // fp16 1.0
-      f32x4 c = wacc;
-      if (RESCALE) c *= alpha;
+    rt[0].template accumulate_weights<true>(pf0, alpha0);
+    rt[1].template accumulate_weights<true>(pf1, alpha1);
+  } else {
 #pragma unroll
-      for (int u = 0; u < TOK; ++u) c = Mma<KV_DT>::run(__builtin_bit_cast(Op, ones), pf[u], c);
-      wacc = c;
+    for (int dt = 0; dt < 8; ++dt) {
+      const Op vf = rt[0].v_fragment(tile, dt);
+      rt[0].template accumulate_step<false>(dt, vf, pf0, alpha0);
+      rt[1].template accumulate_step<false>(dt, vf, pf1, alpha1);
     }
+    rt[0].template accumulate_weights<false>(pf0, alpha0);
+    rt[1].template accumulate_weights<false>(pf1, alpha1);
   }
-};
+}
 
 // End of an item: the TW waves that share a set of 16 query rows exchange (m, l, acc) through LDS
 // (each wave's own 16 KiB region `xch_base + wave * xch_stride`), then each finishes head_dim/TW columns:
 // a sequence that is a single chunk gets its bf16 output rows (and LSE) written directly, a split
-// sequence a normalised fp32 partial and its log2-sum-exp.  All waves of the workgroup must call it.
+// sequence a normalised fp32 partial and its log2-sum-exp.  `row_set` says which 16 rows of the item
+// these are.  All waves of the workgroup must call it.
 template <int KV_DT, int TOK, int TW>
 __device__ inline void finish_item(const DecodeParams& p, const Item& it, RowTile<KV_DT, TOK>& rt, uint8_t* xch_base,
-                                   int xch_stride, float* lds_ml, int wave, int rs, int tw, int lane) {
+                                   int xch_stride, float* lds_ml, int wave, int rs, int tw, int lane, int row_set) {
   constexpr bool kOffset = kv_of(KV_DT) == XLLM_HIP_INT8;
   constexpr int kD = 128 / TOK;
   const float neg_inf = -INFINITY;
@@ -949,7 +1040,7 @@ __device__ inline void finish_item(const DecodeParams& p, const Item& it, RowTil
     wgt[s] = __builtin_amdgcn_exp2f(lds_ml[((rs * TW + s) * 16 + col) * 2] - m_safe);
     l_all += wgt[s] * lds_ml[((rs * TW + s) * 16 + col) * 2 + 1];
   }
-  const int r = it.rg * kMaxRowsPerItem + rs * 16 + col;
+  const int r = it.rg * p.rows_per_item + row_set * 16 + col;
   if (r >= it.n * p.group) return;
   const int j = r / p.group;
   const int head = it.hk * p.group + (r - j * p.group);
@@ -1071,7 +1162,7 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_d128_kernel(Decode
       }
     }
   }
-  finish_item<KV_DT, TOK, kWaves>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, 0, wave, lane);
+  finish_item<KV_DT, TOK, kWaves>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, 0, wave, lane, 0);
 }
 
 template <int KV_DT, int TOK>
@@ -1143,7 +1234,165 @@ __global__ void __launch_bounds__(128, 2) decode_mfma_d128_rows32_kernel(DecodeP
     if (i + 1 < iters) step(mine[1], blk_b, i + 1);
   }
   __syncthreads();  // all tiles consumed before the buffers are reused for the exchange
-  finish_item<KV_DT, TOK, 1>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, rs, 0, lane);
+  finish_item<KV_DT, TOK, 1>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, rs, 0, lane, rs);
+}
+
+// Many query rows per kv head (prefill chunks, long verify steps) over a 16-bit cache: a workgroup is
+// four waves and 128 query rows of one (sequence, kv head); wave w owns rows 32w .. 32w+31 as two row
+// tiles, so every K and V fragment it reads from LDS feeds two MFMAs.  All four waves walk the
+// item's tokens together, one tile per step.  The tile needs no conversion, so it goes from global
+// memory straight into LDS (global_load_lds, 16 bytes per lane): no staging registers, no park.
+// Such a load writes the wave's 64 pieces to consecutive LDS addresses, i.e. four whole rows; the
+// swizzle is applied on the global side (lane = (row, position) fetches the piece that belongs at
+// that position).  Wave w fetches rows 8w .. 8w+7 of K and of V.  Four tile buffers rotate: tiles
+// i+1 .. i+3 are in flight while tile i is read.  Each buffer is an LDS array of its own and the
+// loop is unrolled over them, so that the compiler can tell the loads in flight from the buffer
+// being read and does not wait for them.  With causal rows a wave skips the tiles none of its rows
+// can see.  Two such workgroups share a CU.
+constexpr int kPrefillBuffers = 4;
+constexpr int kPrefillTile = 16896;  // 16 KiB of K and V; as the end-of-item exchange 16 rows of kXchRow
+
+#define XLLM_HIP_GLOBAL_TO_LDS_16(gptr, lptr)                                                   \
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gptr),       \
+                                   (__attribute__((address_space(3))) void*)(lptr), 16, 0, 0)
+
+template <int KV_DT, int TOK>
+struct PrefillLoader {
+  int wave, lane;
+
+  // Load q (0, 1) covers rows 4q .. 4q+3 of the wave's eight: token (within the wave's 8 * TOK)
+  // and byte offset of the piece this lane fetches for position lane % 16 of its row.
+  // Recomputed at every use — a few integer operations — rather than held in registers.
+  __device__ inline void piece(int q, bool v, int& tok, int& byte) const {
+    int lane = this->lane;
+    asm volatile("" : "+v"(lane));  // keeps the compiler from hoisting these out of the loop and then spilling them
+    const int row8 = 4 * q + (lane >> 4);
+    const int row = 8 * wave + row8;  // row of the tile
+    const int pos = lane & 15;
+    const int lp = v ? pos ^ (((row & 7) << 1) | ((row >> 3) & 1))  // see swz_v
+                     : pos ^ (row & 15);                             // see swz_k
+    constexpr int kPerTok = 16 / TOK;  // pieces per token
+    tok = row8 * TOK + lp / kPerTok;
+    byte = (lp % kPerTok) * 16;
+  }
+  __device__ inline uint32_t offset(const DecodeParams& p, int q, bool v) const {
+    int tok, byte;
+    piece(q, v, tok, byte);
+    return (uint32_t)(tok * p.stride_slot * 2 + byte);
+  }
+
+  // Loads of the wave's rows of the tile starting at token tb into `buf` (in flight on return).
+  __device__ inline void issue(const DecodeParams& p, const Item& it, int tb, int blk, uint8_t* buf) const {
+    const HalfBase b = half_base(p, it, tb + 8 * TOK * wave, blk);
+    const uint8_t* kb = p.k_cache + b.elem * 2;
+    const uint8_t* vb = p.v_cache + b.elem * 2;
+    uint8_t* kl = buf + kLdsK + 2048 * wave;
+    uint8_t* vl = buf + kLdsV + 2048 * wave;
+    XLLM_HIP_GLOBAL_TO_LDS_16(kb + offset(p, 0, false), kl);
+    XLLM_HIP_GLOBAL_TO_LDS_16(kb + offset(p, 1, false), kl + 1024);
+    XLLM_HIP_GLOBAL_TO_LDS_16(vb + offset(p, 0, true), vl);
+    XLLM_HIP_GLOBAL_TO_LDS_16(vb + offset(p, 1, true), vl + 1024);
+  }
+
+  // Zeros over the V pieces of tokens at or past the sequence end (after the loads have landed):
+  // whatever those slots hold must not reach the MFMA, where even a weight of zero times NaN is NaN.
+  __device__ inline void clear_tail(int tb, int len, uint8_t* buf) const {
+    const int first = tb + 8 * TOK * wave;
+    uint32_t z = 0;
+    asm volatile("" : "+v"(z));  // made here, on the rare path, instead of living in registers through the loop
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      int tok, byte;
+      piece(q, true, tok, byte);
+      if (first + tok >= len) *(u32x4*)(buf + kLdsV + 2048 * wave + 1024 * q + lane * 16) = u32x4{z, z, z, z};
+    }
+  }
+};
+
+template <int KV_DT, int TOK>
+__global__ void __launch_bounds__(256, 2) prefill_mfma_d128_kernel(DecodeParams p) {
+  static_assert(!quant_of(KV_DT), "a 1-byte cache needs converting on the way into LDS");
+  __shared__ __attribute__((aligned(16))) uint8_t buf0[kPrefillTile];
+  __shared__ __attribute__((aligned(16))) uint8_t buf1[kPrefillTile];
+  __shared__ __attribute__((aligned(16))) uint8_t buf2[kPrefillTile];
+  __shared__ __attribute__((aligned(16))) uint8_t buf3[kPrefillTile];
+  __shared__ float lds_ml[4 * 16 * 2];
+  constexpr int kT = 32 * TOK;  // tokens per tile
+
+  Item it;
+  if (!decode_item(p, blockIdx.x, it)) return;
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+
+  RowTile<KV_DT, TOK> rt[2];
+  rt[0].init(p, it, 32 * wave, lane);
+  rt[1].init(p, it, 32 * wave + 16, lane);
+
+  // What this wave's rows can see: row r belongs to query token r / group, which sees the tokens
+  // below lim(j) = len - (n - 1 - j) and, with a sliding window, from lim(j) - 1 - window_left on.
+  const int rows = it.n * p.group;
+  const int r_first = it.rg * p.rows_per_item + 32 * wave;
+  const bool has_rows = r_first < rows;
+  const int r_last = min(r_first + 31, rows - 1);
+  const int lim_first = it.len - (it.n - 1 - r_first / p.group);
+  const int lim_last = has_rows ? it.len - (it.n - 1 - r_last / p.group) : 0;
+  const int lo_first = p.window_left >= 0 ? lim_first - 1 - p.window_left : 0;
+  const int lo_last = p.window_left >= 0 ? lim_last - 1 - p.window_left : 0;
+
+  const int w_begin = first_visible_tile(p, it);
+  const int w_end = it.t_end;
+  const int iters = w_end > w_begin ? (w_end - w_begin + kT - 1) / kT : 0;
+
+  PrefillLoader<KV_DT, TOK> ld;
+  ld.wave = wave;
+  ld.lane = lane;
+  const int mine = 8 * TOK * wave;  // first of the tokens this wave fetches, within a tile
+
+  // Tile i: wait for this wave's share of it (tiles i+1 and i+2 stay in flight), meet the other
+  // waves — their shares have landed too, and everyone is done with tile i-1, whose buffer `next`
+  // is — then put tile i+3 in flight into `next` and attend tile i from `buf`.  Every step issues
+  // its four loads, also past the end of the item (block_of keeps those inside the sequence's
+  // blocks; nobody reads them): the count of loads in flight is then the same on every path, which
+  // is what lets the compiler, too, wait for exactly the buffer it reads.
+  auto step = [&](int i, uint8_t* buf, uint8_t* next, int& blk) {
+    const int tb = w_begin + i * kT;
+    const int nblk = block_of_const(p, it, tb + 4 * kT + mine);
+    // (the builtin, not asm with a memory clobber: after such a clobber the block ids would no
+    // longer come through scalar loads, and a vector load's wait would cover the tiles in flight)
+    __builtin_amdgcn_s_waitcnt(0x0f78);  // vmcnt(8)
+    if (tb + kT > it.len) ld.clear_tail(tb, it.len, buf);
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the zeros above are in LDS
+    __builtin_amdgcn_s_barrier();
+    ld.issue(p, it, tb + 3 * kT, blk, next);
+    blk = nblk;
+    if (!(tb >= lim_last || tb + kT <= lo_first)) {  // else: nothing here for this wave's rows
+      if (tb + kT > lim_first || tb < lo_last) {
+        attend_pair<true>(rt, buf, tb, p.scale_log2);
+      } else {
+        attend_pair<false>(rt, buf, tb, p.scale_log2);
+      }
+    }
+  };
+  ld.issue(p, it, w_begin, block_of_const(p, it, w_begin + mine), buf0);
+  ld.issue(p, it, w_begin + kT, block_of_const(p, it, w_begin + kT + mine), buf1);
+  ld.issue(p, it, w_begin + 2 * kT, block_of_const(p, it, w_begin + 2 * kT + mine), buf2);
+  int blk = block_of_const(p, it, w_begin + 3 * kT + mine);
+  int i = 0;
+  for (; i + 4 <= iters; i += 4) {
+    step(i, buf0, buf3, blk);
+    step(i + 1, buf1, buf0, blk);
+    step(i + 2, buf2, buf1, blk);
+    step(i + 3, buf3, buf2, blk);
+  }
+  if (i < iters) step(i, buf0, buf3, blk);
+  if (i + 1 < iters) step(i + 1, buf1, buf0, blk);
+  if (i + 2 < iters) step(i + 2, buf2, buf1, blk);
+  __syncthreads();  // all tiles consumed before the buffers are reused for the exchange
+  uint8_t* xch = wave == 0 ? buf0 : wave == 1 ? buf1 : wave == 2 ? buf2 : buf3;
+  finish_item<KV_DT, TOK, 1>(p, it, rt[0], xch, 0, lds_ml, wave, wave, 0, lane, 2 * wave);
+  __syncthreads();
+  finish_item<KV_DT, TOK, 1>(p, it, rt[1], xch, 0, lds_ml, wave, wave, 0, lane, 2 * wave + 1);
 }
 
 // ---------------------------------------------------------------------------------
@@ -1317,10 +1566,10 @@ static bool is_mfma(Variant v) { return v == kMfmaD128 || v == kMfmaD64; }
 // The generic kernel runs one wave per item.
 constexpr int kNumCUs = 256;
 
-// Work items to aim for: two 4-wave workgroups per CU for the 16-row MFMA kernel, four 2-wave
-// workgroups for the 32-row one, eight single waves for the generic kernel.
+// Work items to aim for: two 4-wave workgroups per CU for the 16-row and the 128-row MFMA kernels,
+// four 2-wave workgroups for the 32-row one, eight single waves for the generic kernel.
 static int target_items(int variant_is_mfma, int rows) {
-  int v = variant_is_mfma ? (rows > 16 ? 4 * kNumCUs : 2 * kNumCUs) : 8 * kNumCUs;
+  int v = !variant_is_mfma ? 8 * kNumCUs : (rows > 16 && rows <= kPrefillMinRows) ? 4 * kNumCUs : 2 * kNumCUs;
   if (const char* e = getenv("XLLM_HIP_DECODE_TARGET_ITEMS")) {
     const int t = atoi(e);
     if (t > 0) v = t;
@@ -1442,7 +1691,8 @@ static int fill_params(const xllm_hip_kv_cache* c,
   p.group = a->num_q_heads / c->num_kv_heads;
   p.rows = p.group * p.n;
   const Variant variant = pick_variant(c, a);
-  p.rows_per_item = is_mfma(variant) ? kMaxRowsPerItem : 1;
+  // the many-row kernel moves tiles from global memory to LDS as they are: 16-bit caches only
+  p.rows_per_item = !is_mfma(variant) ? 1 : (p.rows > kPrefillMinRows && !quant) ? kPrefillRowsPerItem : kMaxRowsPerItem;
   p.min_chunk = is_mfma(variant) ? kMinChunkTokens : kMinChunkTokensGeneric;
   p.tok = variant == kMfmaD64 ? 2 : 1;
   p.tile_tokens = kTileTokens * p.tok;
@@ -1500,8 +1750,9 @@ static int64_t max_items(const DecodeParams& p) {
 
 template <int KV_DT, int TOK>
 static void launch_mfma_tok(const DecodeParams& p, unsigned grid, hipStream_t st) {
-  const int rows_per_item = p.rows < kMaxRowsPerItem ? p.rows : kMaxRowsPerItem;
-  if (rows_per_item <= 16) {
+  if (p.rows_per_item == kPrefillRowsPerItem) {
+    if constexpr (!quant_of(KV_DT)) prefill_mfma_d128_kernel<KV_DT, TOK><<<grid, 256, 0, st>>>(p);
+  } else if (p.rows <= 16) {
     decode_mfma_d128_kernel<KV_DT, TOK><<<grid, 64 * kWaves, 0, st>>>(p);
   } else {
     decode_mfma_d128_rows32_kernel<KV_DT, TOK><<<grid, 128, 0, st>>>(p);
