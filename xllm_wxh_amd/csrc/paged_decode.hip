@@ -852,6 +852,10 @@ struct RowTile {
   __device__ __forceinline__ bool softmax(const Scores& s, const float (&kscl)[kN], const float (&lv)[kN], const float (&rvs)[kN], int tb, float scale_log2, Op (&pf)[TOK],
                                  float& alpha) {
     const float neg_inf = -INFINITY;
+    // A plain tile of a 16-bit cache: the maximum is taken over the raw scores (the scale is
+    // not negative: the host sends other scales to the generic kernel) and the scale rides in the FMA
+    // that forms the exponent, one operation per score less.
+    constexpr bool kFold = !kQuant && !MASKED;
     float x[kN];
     float mt = neg_inf;
 #pragma unroll
@@ -861,7 +865,8 @@ struct RowTile {
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) {
           const int i = (u * 2 + h) * 4 + rr;
-          float v = kQuant ? __builtin_fmaf(s[u][h][rr], kscl[i], lv[i]) : s[u][h][rr] * scale_log2;
+          float v = kFold ? s[u][h][rr]
+                          : kQuant ? __builtin_fmaf(s[u][h][rr], kscl[i], lv[i]) : s[u][h][rr] * scale_log2;
           if (MASKED) {
             const int tok = tb + TOK * (16 * h + 4 * kg + rr) + u;
             v = (tok < lim && tok >= lo) ? v : neg_inf;
@@ -872,6 +877,7 @@ struct RowTile {
       }
     }
     mt = kg_max(mt);
+    if (kFold) mt *= scale_log2;
     const float m_new = fmaxf(m_run, mt);
     const float m_safe = m_new == neg_inf ? 0.0f : m_new;
     const bool moved = __builtin_amdgcn_ballot_w64(m_new != m_run) != 0;
@@ -881,7 +887,7 @@ struct RowTile {
     float w[kN];
 #pragma unroll
     for (int i = 0; i < kN; ++i) {
-      const float e = __builtin_amdgcn_exp2f(x[i] - m_safe);
+      const float e = __builtin_amdgcn_exp2f(kFold ? __builtin_fmaf(x[i], scale_log2, -m_safe) : x[i] - m_safe);
       w[i] = e;
       l_run = kQuant ? __builtin_fmaf(e, rvs[i], l_run) : l_run + e;
     }
@@ -1589,7 +1595,7 @@ static Variant pick_variant(const xllm_hip_kv_cache* c, const xllm_hip_decode_ar
   // (32 tokens) must then lie in one block.
   const bool d128 = c->head_dim == 128 && c->block_size >= 16;
   const bool d64 = c->head_dim == 64 && c->block_size >= 32;
-  if (!force_generic && (d128 || d64) && kv_ok && is_pow2(c->block_size)) {
+  if (!force_generic && (d128 || d64) && kv_ok && is_pow2(c->block_size) && a->sm_scale >= 0.0f) {
     const int vec = 16 / eb;  // elements per 16-byte load
     const bool strides_ok = c->stride_block % vec == 0 && c->stride_head % vec == 0 && c->stride_slot % vec == 0 &&
                             a->q_token_stride % 8 == 0;
