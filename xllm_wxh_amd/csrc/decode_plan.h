@@ -27,7 +27,7 @@ constexpr int kMinChunkTokensGeneric = 64;  // the one-wave kernel: one 64-token
 constexpr int kMaxTargetItems = 4096; // upper bound of the split target (sizes the workspace)
 constexpr int kMaxRowsPerItem = 32;   // query rows (g * n) one work item of the MFMA decode kernels handles
 constexpr int kPrefillRowsPerItem = 128;  // ... and of the many-row (prefill) kernel, used above kPrefillMinRows rows
-constexpr int kPrefillMinRows = 64;
+constexpr int kPrefillMinRows = 32;
 
 #if defined(__HIPCC__)
 #define XLLM_HIP_HD __host__ __device__
