@@ -409,6 +409,7 @@ constexpr int kLdsV = 8192;
 constexpr int kLdsSc = 16384;    // per-token factors of a quantised tile: three arrays of up to 64 floats
 constexpr int kLdsTile = 17152;  // one tile of K and V as 16-bit numbers (32 rows of 256 bytes each), plus the factors
 constexpr int kWaves = 4;        // waves per work item of the 16-row kernel
+constexpr float kLazyRescale = 8.0f;  // log2 of the largest softmax weight tolerated before the reference maximum moves
 constexpr int kXchRow = 528;     // bytes per query row in the end-of-item exchange (128 floats + 16 pad)
 
 __device__ inline u32x4 ldg_stream(const void* p) {
@@ -756,7 +757,7 @@ struct RowTile {
   Op qf[kQC];      // Q^T fragments (B operand) of the lane's query row
   f32x4 acc[8];    // O^T accumulators: tile dt of the 128 row elements, query rows 4*kg + rr
   f32x4 wacc;      // sum of the weights as the MFMA saw them (int8 only)
-  float m_run;     // running maximum of the log2-scaled scores (of score + log2 v_scale if quantised)
+  float m_run;     // reference point of the exponents: follows the running maximum of the log2-scaled scores (of score + log2 v_scale if quantised) lazily, see softmax
   float l_run;     // this lane's share of the softmax denominator
   float s_init;    // initial value of the score accumulators: -1152 * sum_d q[r][d] (int8), else 0
   int lim;         // tokens >= lim are invisible to the row (causal among draft tokens)
@@ -878,9 +879,16 @@ struct RowTile {
     }
     mt = kg_max(mt);
     if (kFold) mt *= scale_log2;
-    const float m_new = fmaxf(m_run, mt);
+    // The reference point of the exponents follows the running maximum lazily: it moves (for every
+    // row of the tile) only when some row's maximum has grown by more than kLazyRescale, i.e. when
+    // weights above 2^kLazyRescale would appear.  Until then weights may exceed 1 by up to that
+    // factor — harmless for the 16-bit weights (same relative precision) and the fp32 sums — and the
+    // accumulators need no rescaling, which with 16 or 32 rows per wave is otherwise due on most
+    // tiles of the first few thousand tokens.
+    const float m_top = fmaxf(m_run, mt);
+    const bool moved = __builtin_amdgcn_ballot_w64(m_top > m_run + kLazyRescale) != 0;
+    const float m_new = moved ? m_top : m_run;
     const float m_safe = m_new == neg_inf ? 0.0f : m_new;
-    const bool moved = __builtin_amdgcn_ballot_w64(m_new != m_run) != 0;
     alpha = __builtin_amdgcn_exp2f(m_run - m_safe);
     l_run *= alpha;
     m_run = m_new;
