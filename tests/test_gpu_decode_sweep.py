@@ -1,0 +1,45 @@
+"""Seeded random sweep of decode / verify / chunk shapes against the oracle, through the C ABI: every
+kernel variant (16-row, 32-row, 128-row, head_dim 64, generic) under shapes nobody hand-picked."""
+import numpy as np
+import pytest
+import torch
+
+from tests.helpers import Case, lse_err, max_abs_err
+
+pytestmark = pytest.mark.gpu
+
+
+def _random_case(rng):
+    D = int(rng.choice([128, 128, 64]))
+    kv = str(rng.choice(["bf16", "bf16", "fp8", "int8", "fp16"]))
+    qdt = "fp16" if kv == "fp16" or (kv in ("fp8", "int8") and rng.random() < 0.3) else "bf16"
+    bs = int(rng.choice([16, 32, 64, 128]))
+    Hkv = int(rng.choice([1, 2, 4, 8]))
+    g = int(rng.choice([1, 2, 4, 5, 8]))
+    n = int(rng.choice([1, 1, 2, 4, 7, 12, 33]))
+    B = int(rng.integers(1, 6))
+    lens = []
+    for _ in range(B):
+        kind = rng.random()
+        hi = 40 if kind < 0.3 else 700 if kind < 0.8 else 5000
+        lens.append(int(rng.integers(n, max(n + 1, hi))))  # at least n tokens: the chunk is part of the sequence
+    layout = str(rng.choice(["HND", "NHD"]))
+    window = int(rng.choice([-1, -1, -1, 37, 300]))
+    return dict(B=B, Hq=Hkv * g, Hkv=Hkv, D=D, bs=bs, lens=lens, n=n, kv=kv, qdt=qdt, layout=layout), window
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_shapes_match_oracle(gpu, seed):
+    rng = np.random.default_rng(1000 + seed)
+    for rep in range(3):
+        cfg, window = _random_case(rng)
+        print("case sweep", seed, rep, cfg, "window", window, flush=True)
+        c = Case(cfg["B"], cfg["Hq"], cfg["Hkv"], cfg["D"], cfg["bs"], cfg["lens"], n=cfg["n"], kv=cfg["kv"],
+                 qdt=cfg["qdt"], layout=cfg["layout"], seed=seed * 10 + rep)
+        ref, lse_ref = c.oracle(window)
+        out, lse = c.run(window)
+        assert not torch.isnan(out.float()).any()
+        e = max_abs_err(out, ref)
+        print("   variant=%s err=%.3e" % (c.variant(), e), flush=True)
+        assert e <= (2.5e-2 if cfg["kv"] in ("fp8", "int8") else 1.2e-2), (cfg, window, e)
+        assert lse_err(lse, lse_ref) <= 1e-4
