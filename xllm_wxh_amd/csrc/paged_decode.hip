@@ -1388,20 +1388,22 @@ __global__ void __launch_bounds__(256, 2) prefill_mfma_d128_kernel(DecodeParams 
       }
     }
   };
-  ld.issue(p, it, w_begin, block_of_const(p, it, w_begin + mine), buf0);
-  ld.issue(p, it, w_begin + kT, block_of_const(p, it, w_begin + kT + mine), buf1);
-  ld.issue(p, it, w_begin + 2 * kT, block_of_const(p, it, w_begin + 2 * kT + mine), buf2);
-  int blk = block_of_const(p, it, w_begin + 3 * kT + mine);
-  int i = 0;
-  for (; i + 4 <= iters; i += 4) {
-    step(i, buf0, buf3, blk);
-    step(i + 1, buf1, buf0, blk);
-    step(i + 2, buf2, buf1, blk);
-    step(i + 3, buf3, buf2, blk);
+  if (iters > 0) {  // (an item without visible tokens touches no block: its table row may hold anything)
+    ld.issue(p, it, w_begin, block_of_const(p, it, w_begin + mine), buf0);
+    ld.issue(p, it, w_begin + kT, block_of_const(p, it, w_begin + kT + mine), buf1);
+    ld.issue(p, it, w_begin + 2 * kT, block_of_const(p, it, w_begin + 2 * kT + mine), buf2);
+    int blk = block_of_const(p, it, w_begin + 3 * kT + mine);
+    int i = 0;
+    for (; i + 4 <= iters; i += 4) {
+      step(i, buf0, buf3, blk);
+      step(i + 1, buf1, buf0, blk);
+      step(i + 2, buf2, buf1, blk);
+      step(i + 3, buf3, buf2, blk);
+    }
+    if (i < iters) step(i, buf0, buf3, blk);
+    if (i + 1 < iters) step(i + 1, buf1, buf0, blk);
+    if (i + 2 < iters) step(i + 2, buf2, buf1, blk);
   }
-  if (i < iters) step(i, buf0, buf3, blk);
-  if (i + 1 < iters) step(i + 1, buf1, buf0, blk);
-  if (i + 2 < iters) step(i + 2, buf2, buf1, blk);
   __syncthreads();  // all tiles consumed before the buffers are reused for the exchange
   uint8_t* xch = wave == 0 ? buf0 : wave == 1 ? buf1 : wave == 2 ? buf2 : buf3;
   finish_item<KV_DT, TOK, 1>(p, it, rt[0], xch, 0, lds_ml, wave, wave, 0, lane, 2 * wave);
