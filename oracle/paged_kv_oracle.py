@@ -24,8 +24,14 @@ tree); how each one is pinned is listed beside it:
       library, neither of which is in the reference tree: pinned by mathematics (kv_len 1 gives the
       value row, identical keys give the mean of values, block-table permutation invariance,
       agreement with scipy/torch softmax, split-merge identity) and by the reference's invariant
-      xllm/core/runtime/cuda_graph_executor_test.cpp:150-151.  Absolute FlashInfer/tmo outputs:
-      PARITY UNPINNED (tolerance only).
+      xllm/core/runtime/cuda_graph_executor_test.cpp:150-151.  The int8 decode (with seeded_tensor,
+      the rotary embedding and the scale layout [block, head, slot]) is also pinned by the reference's
+      one numeric known answer that crosses it: the output statistics of
+      Qwen2AttentionTest.QuantizedKVCacheDecodeTest (xllm/core/layers/common/tests/qwen2_attention_tests.cpp:
+      500-578), reproduced to 0.1 % of the sum where the reference allows 1 %
+      (tests/test_oracle_qwen2_int8_decode_kat.py; its softmaxes are one-hot, so it pins the token
+      and head indexing and the dequantisation, not the softmax arithmetic).  Absolute FlashInfer
+      outputs and the low-order bits of tmo's: PARITY UNPINNED (tolerance only).
   paged_decode_ragged                    per-sequence query counts (chunked prefill, flashinfer_attention.cpp:224-284):
       one paged_decode call per sequence, so it inherits those pins.
   lse_combine                            xllm/core/kernels/cuda/xattention/lse_combine.cu:61-73
