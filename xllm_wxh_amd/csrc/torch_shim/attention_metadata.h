@@ -6,6 +6,8 @@
 
 #include <torch/torch.h>
 
+#include "host_index.h"
+
 namespace xllm::layer {
 
 struct AttentionMetadata {
@@ -50,6 +52,24 @@ inline AttentionMetadata build_decode_metadata(const torch::Tensor& q_cu_seq_len
   m.q_seq_lens = torch::diff(q_cu_seq_lens).contiguous();
   m.is_dummy = q_max_seq_len == 0;
   if (m.is_dummy) m.slot_mapping = torch::tensor({1}, new_cache_slots.options());
+  return m;
+}
+
+// The same from the host-side batch arrays: their int32 tensors are created on `device` the way
+// BatchInputBuilder::state_to_forward_input (xllm/core/framework/batch/batch_input_builder.cpp:500-560)
+// creates them (block tables padded with 0), CSR arrays included.
+inline AttentionMetadata build_decode_metadata(const host_index::DecodeBatchInputs& in, const torch::Device& device) {
+  auto i32 = [&](const std::vector<int32_t>& v) {
+    return torch::tensor(v, torch::TensorOptions().dtype(torch::kInt32)).to(device);
+  };
+  int32_t max_blocks = 0;
+  const std::vector<int32_t> flat = in.pad_block_tables(max_blocks);
+  torch::Tensor table = i32(flat).view({(int64_t)in.num_sequences(), (int64_t)max_blocks});
+  AttentionMetadata m = build_decode_metadata(i32(in.q_seq_lens), i32(in.kv_seq_lens), i32(in.new_cache_slots), table,
+                                              in.q_max_seq_len, in.kv_max_seq_len, in.total_kv_len());
+  m.paged_kv_indptr = i32(in.paged_kv_indptr);
+  m.paged_kv_indices = i32(in.paged_kv_indices);
+  m.paged_kv_last_page_len = i32(in.paged_kv_last_page_len);
   return m;
 }
 

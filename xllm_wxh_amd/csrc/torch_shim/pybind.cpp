@@ -88,7 +88,49 @@ PYBIND11_MODULE(_xllm_hip_torch, m) {
       .def_readwrite("paged_kv_indptr", &AttentionMetadata::paged_kv_indptr)
       .def_readwrite("paged_kv_indices", &AttentionMetadata::paged_kv_indices)
       .def_readwrite("paged_kv_last_page_len", &AttentionMetadata::paged_kv_last_page_len);
-  m.def("build_decode_metadata", &xllm::layer::build_decode_metadata);
+  m.def("build_decode_metadata",
+        py::overload_cast<const torch::Tensor&, const torch::Tensor&, const torch::Tensor&, const torch::Tensor&, int64_t,
+                          int64_t, int64_t>(&xllm::layer::build_decode_metadata));
+  m.def("build_decode_metadata", [](const xllm::host_index::DecodeBatchInputs& in, const std::string& device) {
+    return xllm::layer::build_decode_metadata(in, torch::Device(device));
+  });
+
+  // host-side index producers
+  namespace hi = xllm::host_index;
+  m.def("kv_cache_slots", &hi::kv_cache_slots);
+  m.def("calc_slot_id", &hi::calc_slot_id);
+  m.def("calc_kv_len", &hi::calc_kv_len);
+  py::class_<hi::DecodeBatchInputs>(m, "DecodeBatchInputs")
+      .def(py::init<int32_t>())
+      .def("add_sequence", &hi::DecodeBatchInputs::add_sequence)
+      .def("pad_decode_batch", &hi::DecodeBatchInputs::pad_decode_batch)
+      .def("num_sequences", &hi::DecodeBatchInputs::num_sequences)
+      .def("total_kv_len", &hi::DecodeBatchInputs::total_kv_len)
+      .def("padded_block_tables",
+           [](const hi::DecodeBatchInputs& self) {
+             int32_t width = 0;
+             const std::vector<int32_t> flat = self.pad_block_tables(width);
+             std::vector<std::vector<int32_t>> rows(self.block_tables.size());
+             for (size_t b = 0; b < rows.size(); ++b) rows[b].assign(flat.begin() + b * width, flat.begin() + (b + 1) * width);
+             return rows;
+           })
+      .def_readonly("positions", &hi::DecodeBatchInputs::positions)
+      .def_readonly("new_cache_slots", &hi::DecodeBatchInputs::new_cache_slots)
+      .def_readonly("q_seq_lens", &hi::DecodeBatchInputs::q_seq_lens)
+      .def_readonly("kv_seq_lens", &hi::DecodeBatchInputs::kv_seq_lens)
+      .def_readonly("paged_kv_indptr", &hi::DecodeBatchInputs::paged_kv_indptr)
+      .def_readonly("paged_kv_indices", &hi::DecodeBatchInputs::paged_kv_indices)
+      .def_readonly("paged_kv_last_page_len", &hi::DecodeBatchInputs::paged_kv_last_page_len)
+      .def_readonly("write_block_ids", &hi::DecodeBatchInputs::write_block_ids)
+      .def_readonly("q_max_seq_len", &hi::DecodeBatchInputs::q_max_seq_len)
+      .def_readonly("kv_max_seq_len", &hi::DecodeBatchInputs::kv_max_seq_len);
+  py::class_<hi::ExpandedDecodeRows>(m, "ExpandedDecodeRows")
+      .def_readonly("positions", &hi::ExpandedDecodeRows::positions)
+      .def_readonly("new_cache_slots", &hi::ExpandedDecodeRows::new_cache_slots)
+      .def_readonly("kv_seq_lens", &hi::ExpandedDecodeRows::kv_seq_lens)
+      .def_readonly("block_tables", &hi::ExpandedDecodeRows::block_tables)
+      .def_readonly("kv_max_seq_len", &hi::ExpandedDecodeRows::kv_max_seq_len);
+  m.def("expand_decode_rows", &hi::expand_decode_rows);
 
   py::class_<AttentionImpl>(m, "AttentionImpl")
       .def(py::init<int64_t, int64_t, float, int64_t, int64_t>())
