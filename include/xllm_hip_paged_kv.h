@@ -407,7 +407,7 @@ int xllm_hip_gather_from_cache(const xllm_hip_kv_cache* cache,
 int xllm_hip_abi_version(void);
 
 /* Name of the kernel variant xllm_hip_paged_decode_run would pick for these
- * arguments ("mfma_d128", "mfma_d64", "generic", or "" if unsupported); host-only, launches nothing. */
+ * arguments ("mfma_d128", "mfma_d64", "mfma_d256", "generic", or "" if unsupported); host-only, launches nothing. */
 const char* xllm_hip_paged_decode_variant(const xllm_hip_kv_cache* cache,
                                           const xllm_hip_decode_args* args);
 

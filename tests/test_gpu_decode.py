@@ -105,6 +105,51 @@ def test_head_dim_64_nhd_layout(gpu, kv):
     _check(case)
 
 
+SHAPES_D256 = [
+    # B, Hq, Hkv, D, bs, lens, n
+    (4, 16, 4, 256, 16, [1, 15, 16, 17], 1),         # sequence ends inside and at the edge of a 16-token tile
+    (3, 32, 8, 256, 16, [4096, 777, 128], 1),        # chunk boundaries of the split
+    (3, 14, 2, 256, 128, [4097, 129, 64], 1),        # g = 7
+    (2, 8, 8, 256, 64, [300, 17], 1),                # MHA, g = 1
+    (2, 64, 8, 256, 64, [3001, 517], 4),             # 32 query rows per kv head: the two-wave kernel
+    (2, 64, 4, 256, 32, [700, 91], 4),               # two row groups
+    (3, 32, 8, 256, 32, [5, 2, 3], 2),               # draft tokens at the very start of a sequence
+    (2, 32, 8, 256, 16, [600, 90], 40),              # a prefill chunk: row groups of 32
+]
+
+
+@pytest.mark.parametrize("kv,qdt", [("bf16", "bf16"), ("fp8", "bf16"), ("int8", "bf16"), ("fp16", "fp16"), ("int8", "fp16")])
+@pytest.mark.parametrize("shape", SHAPES_D256, ids=lambda s: "B%d_Hq%d_Hkv%d_bs%d_n%d_L%d" % (s[0], s[1], s[2], s[4], s[6], max(s[5])))
+def test_mfma_decode_head_dim_256(gpu, shape, kv, qdt):
+    """head_dim 256 runs on the MFMA kernels with two tile rows per token (16-token tiles)."""
+    B, Hq, Hkv, D, bs, lens, n = shape
+    print("case mfma d256", shape, kv, qdt, flush=True)
+    case = Case(B, Hq, Hkv, D, bs, lens, n=n, kv=kv, qdt=qdt, seed=31)
+    assert case.variant() == "mfma_d256"
+    _check(case)
+
+
+@pytest.mark.parametrize("kv", ["bf16", "fp8", "int8"])
+def test_head_dim_256_nhd_layout_and_window(gpu, kv):
+    print("case d256 nhd", kv, flush=True)
+    case = Case(3, 16, 4, 256, 32, [700, 33, 64], layout="NHD", kv=kv, seed=32)
+    assert case.variant() == "mfma_d256"
+    _check(case)
+    case = Case(2, 32, 8, 256, 32, [3000, 517], n=2, kv=kv, seed=33)
+    _check(case, window_left=301)
+
+
+def test_head_dim_256_equals_generic_kernel(gpu, monkeypatch):
+    print("case d256 vs generic", flush=True)
+    case = Case(3, 32, 8, 256, 16, [1500, 40, 333], kv="int8", seed=34)
+    out, lse = case.run()
+    monkeypatch.setenv("XLLM_HIP_DECODE_FORCE_GENERIC", "1")
+    assert case.variant() == "generic"
+    out_g, lse_g = case.run()
+    assert max_abs_err(out, out_g.float().cpu().numpy()) <= 2e-2
+    assert float((lse - lse_g).abs().max()) <= 1e-4
+
+
 def test_head_dim_64_small_blocks_take_the_generic_kernel(gpu):
     print("case d64 bs16", flush=True)
     case = Case(2, 8, 2, 64, 16, [100, 33], seed=22)  # half a tile would straddle two blocks

@@ -1,5 +1,5 @@
 """Seeded random sweep of decode / verify / chunk shapes against the oracle, through the C ABI: every
-kernel variant (16-row, 32-row, 128-row, head_dim 64, generic) under shapes nobody hand-picked."""
+kernel variant (16-row, 32-row, 128-row, head_dim 64 and 256, generic) under shapes nobody hand-picked."""
 import numpy as np
 import pytest
 import torch
@@ -10,7 +10,7 @@ pytestmark = pytest.mark.gpu
 
 
 def _random_case(rng):
-    D = int(rng.choice([128, 128, 64]))
+    D = int(rng.choice([128, 128, 64, 256]))
     kv = str(rng.choice(["bf16", "bf16", "fp8", "int8", "fp16"]))
     qdt = "fp16" if kv == "fp16" or (kv in ("fp8", "int8") and rng.random() < 0.3) else "bf16"
     bs = int(rng.choice([16, 32, 64, 128]))

@@ -174,6 +174,9 @@ SMALL = {
     "cfg3_ragged_b256": dict(batch=24, seq_len_max=6000),
     "cfg4_fp8_qwen3_32b": dict(batch=4, seq_len=2048),
     "cfg5_int8_spec_verify": dict(batch=2, seq_len=4096),
+    "aux_d256_bf16_b64_ctx4k": dict(batch=5, seq_len=4096),
+    "aux_d256_fp8_b64_ctx8k": dict(batch=3, seq_len=2048),
+    "aux_d256_int8_spec_verify": dict(batch=2, seq_len=4096),
 }
 
 
@@ -193,7 +196,7 @@ def test_workload_reduced_size_full_check(gpu, name):
         assert err <= tol
 
 
-FULL = [n for n in workloads.WORKLOADS if n != "cfg1_cpu_fp32"]
+FULL = [n for n in workloads.WORKLOADS if n.startswith("cfg") and n != "cfg1_cpu_fp32"]
 
 
 @pytest.mark.parametrize("name", FULL)

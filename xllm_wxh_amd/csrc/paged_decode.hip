@@ -69,8 +69,9 @@ struct DecodeParams {
   int32_t rows_per_item;  // query rows one work item handles (32 or 128 MFMA, 1 generic)
   int32_t min_chunk;      // smallest chunk the plan may choose
   int32_t head_dim;
-  int32_t tok;          // tokens per 256-byte LDS row of the MFMA kernels: 1 (head_dim 128) or 2 (head_dim 64)
-  int32_t tile_tokens;  // tokens per tile: 32 * tok; chunk sizes are multiples of it
+  int32_t tok;          // tokens per 256-byte LDS row of the MFMA kernels: 1 (head_dim 128), 2 (head_dim 64),
+                        // 0 (head_dim 256: a token is two rows, one in each half of the tile)
+  int32_t tile_tokens;  // tokens per tile: 32 * tok (16 at head_dim 256); chunk sizes are multiples of it
   int32_t block_size;
   int32_t log2_bs;
   int32_t max_blocks_per_seq;
@@ -410,7 +411,6 @@ constexpr int kLdsSc = 16384;    // per-token factors of a quantised tile: three
 constexpr int kLdsTile = 17152;  // one tile of K and V as 16-bit numbers (32 rows of 256 bytes each), plus the factors
 constexpr int kWaves = 4;        // waves per work item of the 16-row kernel
 constexpr float kLazyRescale = 8.0f;  // log2 of the largest softmax weight tolerated before the reference maximum moves
-constexpr int kXchRow = 528;     // bytes per query row in the end-of-item exchange (128 floats + 16 pad)
 
 __device__ inline u32x4 ldg_stream(const void* p) {
   return __builtin_nontemporal_load((const u32x4*)p);
@@ -494,9 +494,9 @@ struct KvHalf16 {
     __device__ inline void init(const DecodeParams& p, int lane) {
       lrow = lane >> 4;
       const int piece = lane & 15;
-      tok = p.tok;
+      tok = p.tok == 0 ? 1 : p.tok;  // head_dim 256: rows are tokens here too; `plane` picks the half of the token
       second = tok == 2 && piece >= 8 ? 1 : 0;
-      g_off = (uint32_t)(((lrow * p.tok + second) * p.stride_slot + (piece & (16 / p.tok - 1)) * 8) * 2);
+      g_off = (uint32_t)(((lrow * tok + second) * p.stride_slot + (piece & (16 / tok - 1)) * 8) * 2);
       wk = kLdsK + swz_k(lrow, piece);
       wv = kLdsV + swz_v(lrow, piece);
     }
@@ -511,11 +511,12 @@ struct KvHalf16 {
   u32x4 k[4];
   u32x4 v[4];
 
-  __device__ inline void issue(const DecodeParams& p, const Item& it, int tok, int blk, const Geom& g) {
+  // `plane` (head_dim 256 only): 0 = elements 0..127 of the 16 tokens, 1 = elements 128..255.
+  __device__ inline void issue(const DecodeParams& p, const Item& it, int tok, int blk, const Geom& g, int plane = 0) {
     const HalfBase b = half_base(p, it, tok, blk);
-    const uint8_t* kb = p.k_cache + b.elem * 2;
-    const uint8_t* vb = p.v_cache + b.elem * 2;
-    const int64_t step = 4 * p.stride_slot * p.tok * 2;  // four rows further, in bytes (uniform)
+    const uint8_t* kb = p.k_cache + b.elem * 2 + plane * 256;
+    const uint8_t* vb = p.v_cache + b.elem * 2 + plane * 256;
+    const int64_t step = 4 * p.stride_slot * g.tok * 2;  // four rows further, in bytes (uniform)
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       k[j] = ldg_stream(kb + j * step + g.g_off);
@@ -551,6 +552,12 @@ struct MmaOps {
   __device__ static inline f32x4 run(Op a, Op b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
   }
+  // K = 16: the first four elements of each operand
+  __device__ static inline f32x4 run16(Op a, Op b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(
+        __builtin_bit_cast(s16x4, __builtin_shufflevector(a, a, 0, 1, 2, 3)),
+        __builtin_bit_cast(s16x4, __builtin_shufflevector(b, b, 0, 1, 2, 3)), c, 0, 0, 0);
+  }
   __device__ static inline uint32_t pack(float a, float b) {
     return __builtin_bit_cast(uint32_t, bf16x2{(__bf16)a, (__bf16)b});
   }
@@ -560,6 +567,10 @@ struct MmaOps<true> {
   typedef f16x8 Op;
   __device__ static inline f32x4 run(Op a, Op b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+  __device__ static inline f32x4 run16(Op a, Op b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_shufflevector(a, a, 0, 1, 2, 3),
+                                                 __builtin_shufflevector(b, b, 0, 1, 2, 3), c, 0, 0, 0);
   }
   __device__ static inline uint32_t pack(float a, float b) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, f16x2));
@@ -629,14 +640,14 @@ struct KvHalfQuant {
       const int pair = (lane >> 2) & 1;
       const int krow = 2 * (lane >> 4) + pair;  // rows r, r+1 alternate between quads (krow < 8)
       vrow = (lane >> 4) + 8 * pair;            // rows r, r+8 alternate between quads (vrow & 7 < 4)
-      tok = p.tok;
+      tok = p.tok == 0 ? 1 : p.tok;  // head_dim 256: rows are tokens here too; `plane` picks the half of the token
       second = tok == 2 && chunk >= 4 ? 1 : 0;
-      const int in_tok = (chunk & (8 / p.tok - 1)) * 16;  // byte within the token's row
-      gk_off = (uint32_t)((krow * p.tok + second) * p.stride_slot + in_tok);
-      gv_off = (uint32_t)((vrow * p.tok + second) * p.stride_slot + in_tok);
+      const int in_tok = (chunk & (8 / tok - 1)) * 16;  // byte within the token's row
+      gk_off = (uint32_t)((krow * tok + second) * p.stride_slot + in_tok);
+      gv_off = (uint32_t)((vrow * tok + second) * p.stride_slot + in_tok);
       wk = kLdsK + swz_k(krow, 2 * chunk);
       wv = kLdsV + swz_v(vrow, 2 * chunk);
-      const int per_half = 16 * p.tok;  // tokens per half tile
+      const int per_half = 16 * tok;  // tokens per half tile
       sc_tok = lane % per_half;
       sc_g = (uint32_t)(sc_tok * p.sc_stride_slot * 4);
       sc_is_v = ((lane / per_half) & 1) != 0;
@@ -657,14 +668,17 @@ struct KvHalfQuant {
   u32x4 v[2];
   float sc;
 
-  __device__ inline void issue(const DecodeParams& p, const Item& it, int tok, int blk, const Geom& g) {
+  // `plane` (head_dim 256 only): 0 = elements 0..127 of the 16 tokens, 1 = elements 128..255.  Both
+  // planes carry the tokens' scales (the second copy comes from the cache and lands in the unused
+  // half of the factor arrays).
+  __device__ inline void issue(const DecodeParams& p, const Item& it, int tok, int blk, const Geom& g, int plane = 0) {
     const HalfBase b = half_base(p, it, tok, blk);
-    const uint8_t* kb = p.k_cache + b.elem;
-    const uint8_t* vb = p.v_cache + b.elem;
+    const uint8_t* kb = p.k_cache + b.elem + plane * 128;
+    const uint8_t* vb = p.v_cache + b.elem + plane * 128;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      k[j] = ldg_stream(kb + j * 8 * p.stride_slot * p.tok + g.gk_off);
-      v[j] = ldg_stream(vb + j * 4 * p.stride_slot * p.tok + g.gv_off);
+      k[j] = ldg_stream(kb + j * 8 * p.stride_slot * g.tok + g.gk_off);
+      v[j] = ldg_stream(vb + j * 4 * p.stride_slot * g.tok + g.gv_off);
     }
     const float* sb = (g.sc_is_v ? p.v_scale : p.k_scale) + b.scale;
     if (g.sc_on) sc = *(const float*)((const uint8_t*)sb + g.sc_g);
@@ -741,6 +755,16 @@ __device__ inline float kg_sum(float v) {
 //   head-dim tiles 0..3 of V^T are the first token's values, tiles 4..7 the second's, so they take
 //   the first / second tokens' weights as B operand and the two halves of O^T are added at the end.
 // A tile is 32 rows either way, i.e. 32 * TOK tokens.
+// TOK = 0: head_dim 256.  A token is two rows: row t of the tile's first half holds its elements
+// 0..127, row t of the second half (row 16 + t) its elements 128..255, so a tile is 16 tokens.  The
+// K fragments of the two halves then meet the query's chunks 0..3 and 4..7 and add up to one score
+// tile; the V^T tiles of the first half are head-dim tiles 0..7 and those of the second 8..15, each
+// against the 16 tokens' weights with the K = 16 form of the MFMA.
+constexpr int tile_tokens_of(int tok) { return tok == 0 ? 16 : 32 * tok; }
+constexpr int half_tokens_of(int tok) { return 16 * tok; }  // tokens between the tile's two halves (none at head_dim 256)
+constexpr int head_dim_of(int tok) { return tok == 0 ? 256 : 128 / tok; }
+constexpr int xch_row_bytes(int tok) { return head_dim_of(tok) * 4 + 16; }  // a query row in the end-of-item exchange
+
 template <int KV_DT, int TOK>
 struct RowTile {
   static constexpr bool kQuant = quant_of(KV_DT);
@@ -750,12 +774,15 @@ struct RowTile {
   //                                                       operand is all ones (wacc)
   // Rows zeroed because they lie past the sequence end carry weight 0 in both sums.
   static constexpr bool kOffset = kv_of(KV_DT) == XLLM_HIP_INT8;
-  static constexpr int kD = 128 / TOK;   // head_dim
-  static constexpr int kQC = 4 / TOK;    // 32-element chunks of a query row
+  static constexpr int kD = head_dim_of(TOK);
+  static constexpr int kQC = kD / 32;    // 32-element chunks of a query row
+  static constexpr int kDT = TOK == 0 ? 16 : 8;  // O^T accumulator tiles
+  static constexpr int kU = TOK == 2 ? 2 : 1;    // tokens per row
+  static constexpr int kHalves = TOK == 0 ? 1 : 2;  // halves of the tile that hold different tokens
   typedef typename Mma<KV_DT>::Op Op;
 
   Op qf[kQC];      // Q^T fragments (B operand) of the lane's query row
-  f32x4 acc[8];    // O^T accumulators: tile dt of the 128 row elements, query rows 4*kg + rr
+  f32x4 acc[kDT];  // O^T accumulators: tile dt of the row elements, query rows 4*kg + rr
   f32x4 wacc;      // sum of the weights as the MFMA saw them (int8 only)
   float m_run;     // reference point of the exponents: follows the running maximum of the log2-scaled scores (of score + log2 v_scale if quantised) lazily, see softmax
   float l_run;     // this lane's share of the softmax denominator
@@ -800,33 +827,33 @@ struct RowTile {
     l_run = 0.0f;
     wacc = f32x4{0, 0, 0, 0};
 #pragma unroll
-    for (int dt = 0; dt < 8; ++dt) acc[dt] = f32x4{0, 0, 0, 0};
+    for (int dt = 0; dt < kDT; ++dt) acc[dt] = f32x4{0, 0, 0, 0};
     k_off0 = kLdsK + swz_k(mi, kg);
     const int tau = 4 * kg + (mi >> 2);  // row (within 16) this lane points the transpose read at
     v_off0 = kLdsV + swz_v(tau, (mi & 3) >> 1) + (mi & 1) * 8;
   }
 
-  static constexpr int kN = 8 * TOK;  // scores per lane and tile
+  static constexpr int kN = 4 * kU * kHalves;  // scores per lane and tile
   // (per-token factors of a quantised tile travel as three arrays in score order: as one struct
   // they cost registers to the point of spilling)
-  typedef f32x4 Scores[TOK][2];
+  typedef f32x4 Scores[kU][2];  // head_dim 256: the two halves' shares of one score tile
 
   __device__ __forceinline__ void load_factors(const uint8_t* tile, float (&kscl)[kN], float (&lv)[kN], float (&rvs)[kN]) const {
     if (!kQuant) return;
-    // the factors of tokens TOK * (16h + 4kg) .. + 4 * TOK - 1 are contiguous in each array
-    constexpr int kArr = 32 * TOK * 4;  // bytes per array
+    // the factors of tokens kU * (16h + 4kg) .. + 4 * kU - 1 are contiguous in each array
+    constexpr int kArr = 32 * kU * 4;  // bytes per array
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int first = TOK * (16 * h + 4 * kg) * 4;
+    for (int h = 0; h < kHalves; ++h) {
+      const int first = kU * (16 * h + 4 * kg) * 4;
 #pragma unroll
-      for (int v4 = 0; v4 < TOK; ++v4) {
+      for (int v4 = 0; v4 < kU; ++v4) {
         const f32x4 a = *(const f32x4*)(tile + kLdsSc + first + 16 * v4);
         const f32x4 b = *(const f32x4*)(tile + kLdsSc + kArr + first + 16 * v4);
         const f32x4 c = *(const f32x4*)(tile + kLdsSc + 2 * kArr + first + 16 * v4);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const int t = 4 * v4 + e;  // token of the lane's 4 * TOK: row rr = t / TOK, u = t % TOK
-          const int i = ((t % TOK) * 2 + h) * 4 + t / TOK;
+          const int t = 4 * v4 + e;  // token of the lane's 4 * kU: row rr = t / kU, u = t % kU
+          const int i = ((t % kU) * kHalves + h) * 4 + t / kU;
           kscl[i] = a[e];
           lv[i] = b[e];
           rvs[i] = c[e];
@@ -838,19 +865,25 @@ struct RowTile {
   // ---- S^T = K Q^T: chunk c of the rows' 128 elements, K fragments of the tile's two halves ----
   __device__ __forceinline__ void scores_init(Scores& s) const {
 #pragma unroll
-    for (int u = 0; u < TOK; ++u) s[u][0] = s[u][1] = f32x4{s_init, s_init, s_init, s_init};
+    for (int u = 0; u < kU; ++u) s[u][0] = s[u][1] = f32x4{s_init, s_init, s_init, s_init};
+    if (TOK == 0) s[0][1] = f32x4{0, 0, 0, 0};  // the halves are added: the offset term enters once
   }
   __device__ __forceinline__ void scores_step(int c, const Op& kf0, const Op& kf1, Scores& s) const {
-    s[c / kQC][0] = Mma<KV_DT>::run(kf0, qf[c % kQC], s[c / kQC][0]);
-    s[c / kQC][1] = Mma<KV_DT>::run(kf1, qf[c % kQC], s[c / kQC][1]);
+    if constexpr (TOK == 0) {
+      s[0][0] = Mma<KV_DT>::run(kf0, qf[c], s[0][0]);
+      s[0][1] = Mma<KV_DT>::run(kf1, qf[4 + c], s[0][1]);
+    } else {
+      s[c / kQC][0] = Mma<KV_DT>::run(kf0, qf[c % kQC], s[c / kQC][0]);
+      s[c / kQC][1] = Mma<KV_DT>::run(kf1, qf[c % kQC], s[c / kQC][1]);
+    }
   }
 
   // ---- online softmax of the lane's query row over the tile starting at token tb ----
-  // Score / weight index i = (u * 2 + h) * 4 + rr: token TOK * (16h + 4kg + rr) + u of the tile.
+  // Score / weight index i = (u * kHalves + h) * 4 + rr: token kU * (16h + 4kg + rr) + u of the tile.
   // Leaves the weights as B operand of the second MFMA (k-slot e = 4h + rr) in pf and the factor
   // the accumulators are to be scaled by in alpha; returns whether any row's maximum moved.
   template <bool MASKED>
-  __device__ __forceinline__ bool softmax(const Scores& s, const float (&kscl)[kN], const float (&lv)[kN], const float (&rvs)[kN], int tb, float scale_log2, Op (&pf)[TOK],
+  __device__ __forceinline__ bool softmax(const Scores& s, const float (&kscl)[kN], const float (&lv)[kN], const float (&rvs)[kN], int tb, float scale_log2, Op (&pf)[kU],
                                  float& alpha) {
     const float neg_inf = -INFINITY;
     // A plain tile of a 16-bit cache: the maximum is taken over the raw scores (the scale is
@@ -860,16 +893,16 @@ struct RowTile {
     float x[kN];
     float mt = neg_inf;
 #pragma unroll
-    for (int u = 0; u < TOK; ++u) {
+    for (int u = 0; u < kU; ++u) {
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {
+      for (int h = 0; h < kHalves; ++h) {
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) {
-          const int i = (u * 2 + h) * 4 + rr;
-          float v = kFold ? s[u][h][rr]
-                          : kQuant ? __builtin_fmaf(s[u][h][rr], kscl[i], lv[i]) : s[u][h][rr] * scale_log2;
+          const int i = (u * kHalves + h) * 4 + rr;
+          const float raw = TOK == 0 ? s[0][0][rr] + s[0][1][rr] : s[u][h][rr];
+          float v = kFold ? raw : kQuant ? __builtin_fmaf(raw, kscl[i], lv[i]) : raw * scale_log2;
           if (MASKED) {
-            const int tok = tb + TOK * (16 * h + 4 * kg + rr) + u;
+            const int tok = tb + kU * (16 * h + 4 * kg + rr) + u;
             v = (tok < lim && tok >= lo) ? v : neg_inf;
           }
           x[i] = v;
@@ -899,45 +932,64 @@ struct RowTile {
       w[i] = e;
       l_run = kQuant ? __builtin_fmaf(e, rvs[i], l_run) : l_run + e;
     }
+    if constexpr (TOK == 0) {  // four weights: the B operand of the K = 16 MFMA
+      const u32x4 pw = {Mma<KV_DT>::pack(w[0], w[1]), Mma<KV_DT>::pack(w[2], w[3]), 0u, 0u};
+      pf[0] = __builtin_bit_cast(Op, pw);
+    } else {
 #pragma unroll
-    for (int u = 0; u < TOK; ++u) {
-      const float* wu = w + 8 * u;
-      const u32x4 pw = {Mma<KV_DT>::pack(wu[0], wu[1]), Mma<KV_DT>::pack(wu[2], wu[3]), Mma<KV_DT>::pack(wu[4], wu[5]),
-                        Mma<KV_DT>::pack(wu[6], wu[7])};
-      pf[u] = __builtin_bit_cast(Op, pw);
+      for (int u = 0; u < kU; ++u) {
+        const float* wu = w + 8 * u;
+        const u32x4 pw = {Mma<KV_DT>::pack(wu[0], wu[1]), Mma<KV_DT>::pack(wu[2], wu[3]),
+                          Mma<KV_DT>::pack(wu[4], wu[5]), Mma<KV_DT>::pack(wu[6], wu[7])};
+        pf[u] = __builtin_bit_cast(Op, pw);
+      }
     }
     return moved;
   }
 
   // ---- O^T = O^T * alpha + V^T P^T, tile dt of the rows' 128 elements ----
   __device__ __forceinline__ Op v_fragment(const uint8_t* tile, int dt) const {
-    const uint32_t vo = v_off0 ^ (uint32_t)(dt << 5);
-    const s16x4 a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-        (__attribute__((address_space(3))) s16x4*)(tile + vo));
-    const s16x4 a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-        (__attribute__((address_space(3))) s16x4*)(tile + vo + 4096));
-    return __builtin_bit_cast(Op, __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7));
+    const uint32_t vo = v_off0 ^ (uint32_t)((dt & 7) << 5);
+    if constexpr (TOK == 0) {  // tile dt of the 16 tokens: from the first half (dt < 8) or the second
+      const s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (__attribute__((address_space(3))) s16x4*)(tile + vo + (dt >> 3) * 4096));
+      return __builtin_bit_cast(Op, __builtin_shufflevector(a, a, 0, 1, 2, 3, 0, 1, 2, 3));
+    } else {
+      const s16x4 a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (__attribute__((address_space(3))) s16x4*)(tile + vo));
+      const s16x4 a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (__attribute__((address_space(3))) s16x4*)(tile + vo + 4096));
+      return __builtin_bit_cast(Op, __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7));
+    }
   }
   template <bool RESCALE>
-  __device__ __forceinline__ void accumulate_step(int dt, const Op& vf, const Op (&pf)[TOK], float alpha) {
+  __device__ __forceinline__ void accumulate_step(int dt, const Op& vf, const Op (&pf)[kU], float alpha) {
     f32x4 c = acc[dt];
     if (RESCALE) c *= alpha;
-    acc[dt] = Mma<KV_DT>::run(vf, pf[dt * TOK / 8], c);
+    if constexpr (TOK == 0) {
+      acc[dt] = Mma<KV_DT>::run16(vf, pf[0], c);
+    } else {
+      acc[dt] = Mma<KV_DT>::run(vf, pf[dt * kU / 8], c);
+    }
   }
   template <bool RESCALE>
-  __device__ __forceinline__ void accumulate_weights(const Op (&pf)[TOK], float alpha) {
+  __device__ __forceinline__ void accumulate_weights(const Op (&pf)[kU], float alpha) {
     if (!kOffset) return;
     const u32x4 ones = {0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u};  // fp16 1.0
     f32x4 c = wacc;
     if (RESCALE) c *= alpha;
+    if constexpr (TOK == 0) {
+      c = Mma<KV_DT>::run16(__builtin_bit_cast(Op, ones), pf[0], c);
+    } else {
 #pragma unroll
-    for (int u = 0; u < TOK; ++u) c = Mma<KV_DT>::run(__builtin_bit_cast(Op, ones), pf[u], c);
+      for (int u = 0; u < kU; ++u) c = Mma<KV_DT>::run(__builtin_bit_cast(Op, ones), pf[u], c);
+    }
     wacc = c;
   }
   template <bool RESCALE>
-  __device__ __forceinline__ void accumulate(const uint8_t* tile, const Op (&pf)[TOK], float alpha) {
+  __device__ __forceinline__ void accumulate(const uint8_t* tile, const Op (&pf)[kU], float alpha) {
 #pragma unroll
-    for (int dt = 0; dt < 8; ++dt) accumulate_step<RESCALE>(dt, v_fragment(tile, dt), pf, alpha);
+    for (int dt = 0; dt < kDT; ++dt) accumulate_step<RESCALE>(dt, v_fragment(tile, dt), pf, alpha);
     accumulate_weights<RESCALE>(pf, alpha);
   }
 
@@ -953,7 +1005,7 @@ struct RowTile {
       const uint32_t ko = k_off0 ^ (uint32_t)(c << 6);
       scores_step(c, *(const Op*)(tile + ko), *(const Op*)(tile + ko + 4096), s);
     }
-    Op pf[TOK];
+    Op pf[kU];
     float alpha;
     const bool moved = softmax<MASKED>(s, kscl, lv, rvs, tb, scale_log2, pf, alpha);
     // The accumulators need rescaling only when some row's maximum moved, which becomes rare a few
@@ -987,7 +1039,7 @@ __device__ __forceinline__ void attend_pair(RowTile<KV_DT, TOK> (&rt)[2], const 
     rt[0].scores_step(c, kf0, kf1, s0);
     rt[1].scores_step(c, kf0, kf1, s1);
   }
-  Op pf0[TOK], pf1[TOK];
+  Op pf0[RT::kU], pf1[RT::kU];
   float alpha0, alpha1;
   const bool moved0 = rt[0].template softmax<MASKED>(s0, kscl, lv, rvs, tb, scale_log2, pf0, alpha0);
   __builtin_amdgcn_sched_barrier(0);  // one softmax at a time: interleaving the two costs registers
@@ -1014,7 +1066,7 @@ __device__ __forceinline__ void attend_pair(RowTile<KV_DT, TOK> (&rt)[2], const 
 }
 
 // End of an item: the TW waves that share a set of 16 query rows exchange (m, l, acc) through LDS
-// (each wave's own 16 KiB region `xch_base + wave * xch_stride`), then each finishes head_dim/TW columns:
+// (each wave's own region `xch_base + wave * xch_stride` of 16 rows of head_dim floats + 16 bytes), then each finishes head_dim/TW columns:
 // a sequence that is a single chunk gets its bf16 output rows (and LSE) written directly, a split
 // sequence a normalised fp32 partial and its log2-sum-exp.  `row_set` says which 16 rows of the item
 // these are.  All waves of the workgroup must call it.
@@ -1022,7 +1074,8 @@ template <int KV_DT, int TOK, int TW>
 __device__ inline void finish_item(const DecodeParams& p, const Item& it, RowTile<KV_DT, TOK>& rt, uint8_t* xch_base,
                                    int xch_stride, float* lds_ml, int wave, int rs, int tw, int lane, int row_set) {
   constexpr bool kOffset = kv_of(KV_DT) == XLLM_HIP_INT8;
-  constexpr int kD = 128 / TOK;
+  constexpr int kD = head_dim_of(TOK);
+  constexpr int kXchRow = xch_row_bytes(TOK);
   const float neg_inf = -INFINITY;
   const int mi = lane & 15, kg = lane >> 4;
   const int nhq = p.n * p.num_q_heads;
@@ -1030,7 +1083,7 @@ __device__ inline void finish_item(const DecodeParams& p, const Item& it, RowTil
   const float l = kg_sum(rt.l_run);
   uint8_t* mine = xch_base + wave * xch_stride;
 #pragma unroll
-  for (int dt = 0; dt < 8 / TOK; ++dt) {
+  for (int dt = 0; dt < kD / 16; ++dt) {
     f32x4 o = rt.acc[dt];
     if (TOK == 2) o += rt.acc[dt + 4];  // the two tokens of a row accumulated into separate tiles
     if (kOffset) o -= kInt8Offset * rt.wacc[0];  // every element of wacc holds the row's sum
@@ -1113,12 +1166,14 @@ __device__ inline int first_visible_tile(const DecodeParams& p, const Item& it) 
 }
 
 template <int KV_DT, int TOK>
-__global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_d128_kernel(DecodeParams p) {
+__global__ void __launch_bounds__(64 * kWaves, TOK == 0 ? 1 : 2) decode_mfma_d128_kernel(DecodeParams p) {
   __shared__ __attribute__((aligned(16))) uint8_t lds_all[kWaves * kLdsTile];
   __shared__ float lds_ml[kWaves * 16 * 2];  // (running max, denominator) per wave and query row
 
-  constexpr int kT = 32 * TOK;  // tokens per tile
-  constexpr int kH = 16 * TOK;  // tokens per half tile
+  constexpr int kT = tile_tokens_of(TOK);  // tokens per tile
+  constexpr int kH = half_tokens_of(TOK);  // tokens from the tile's first half to its second
+  constexpr int kP1 = TOK == 0 ? 1 : 0;    // head_dim 256: the second half is the same tokens' second plane
+  static_assert(16 * xch_row_bytes(TOK) <= kLdsTile, "the end-of-item exchange must fit a wave's tile");
 
   Item it;
   if (!decode_item(p, blockIdx.x, it)) return;
@@ -1141,38 +1196,55 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_d128_kernel(Decode
 
   typename KvHalf<KV_DT>::Geom geom;
   geom.init(p, lane);
-  KvHalf<KV_DT> st[2];  // the two halves (16 rows each) of the tile in flight
+  // Register stages: the tiles in flight while one is consumed.  (Two stages for the 1-byte caches of
+  // head_dim 256, which run one wave per SIMD and so have few bytes in flight per CU, were slower:
+  // 458 against 367 us on 64 x 8192 tokens of fp8 — the registers they take are paid for in copies
+  // between the two register files.)
+  constexpr int kDepth = 1;
+  KvHalf<KV_DT> st[kDepth][2];  // per stage: the two halves (16 rows each) of a tile
+  int blk[kDepth][2];           // block ids of the halves each stage loads next, fetched a round earlier
 
+  // Tile at tb: park it from its stage, put the tile kDepth further in flight into the same stage,
+  // attend.  The scalar loads of the ids go out before the tile is parked: they share a counter with
+  // the LDS traffic, so the next wait on LDS also waits for them.
+  auto step = [&](KvHalf<KV_DT> (&s)[2], int (&b)[2], int tb) {
+    const bool masked = (tb + kT > mask_hi_from) || (tb < mask_lo_until);
+    const int nblk0 = block_of(p, it, tb + 2 * kDepth * kT);
+    const int nblk1 = block_of(p, it, tb + 2 * kDepth * kT + kH);
+    if (masked) {
+      s[0].template park<true>(tile, 0, tb, it.len, p.scale_log2, geom);
+      s[1].template park<true>(tile, 1, tb + kH, it.len, p.scale_log2, geom);
+    } else {
+      s[0].template park<false>(tile, 0, tb, it.len, p.scale_log2, geom);
+      s[1].template park<false>(tile, 1, tb + kH, it.len, p.scale_log2, geom);
+    }
+    if (tb + kDepth * kT < w_end) {
+      s[0].issue(p, it, tb + kDepth * kT, b[0], geom);
+      s[1].issue(p, it, tb + kDepth * kT + kH, b[1], geom, kP1);
+    }
+    b[0] = nblk0;
+    b[1] = nblk1;
+    if (masked) {
+      rt.template attend<true>(tile, tb, p.scale_log2);
+    } else {
+      rt.template attend<false>(tile, tb, p.scale_log2);
+    }
+  };
   if (w_begin < w_end) {
-    st[0].issue(p, it, w_begin, block_of(p, it, w_begin), geom);
-    st[1].issue(p, it, w_begin + kH, block_of(p, it, w_begin + kH), geom);
-    // block ids of the next tile's halves, fetched one tile before the loads that use them
-    int blk0 = block_of(p, it, w_begin + kT);
-    int blk1 = block_of(p, it, w_begin + kT + kH);
-    for (int tb = w_begin; tb < w_end; tb += kT) {
-      const bool masked = (tb + kT > mask_hi_from) || (tb < mask_lo_until);
-      // The scalar loads of the ids go out before the tile is parked: they share a counter with the
-      // LDS traffic, so the next wait on LDS also waits for them.
-      const int nblk0 = block_of(p, it, tb + 2 * kT);
-      const int nblk1 = block_of(p, it, tb + 2 * kT + kH);
-      // park the tile, then put the next tile's loads in flight while this one is consumed
-      if (masked) {
-        st[0].template park<true>(tile, 0, tb, it.len, p.scale_log2, geom);
-        st[1].template park<true>(tile, 1, tb + kH, it.len, p.scale_log2, geom);
-      } else {
-        st[0].template park<false>(tile, 0, tb, it.len, p.scale_log2, geom);
-        st[1].template park<false>(tile, 1, tb + kH, it.len, p.scale_log2, geom);
+#pragma unroll
+    for (int d = 0; d < kDepth; ++d) {
+      const int tb = w_begin + d * kT;
+      if (tb < w_end) {
+        st[d][0].issue(p, it, tb, block_of(p, it, tb), geom);
+        st[d][1].issue(p, it, tb + kH, block_of(p, it, tb + kH), geom, kP1);
       }
-      if (tb + kT < w_end) {
-        st[0].issue(p, it, tb + kT, blk0, geom);
-        st[1].issue(p, it, tb + kT + kH, blk1, geom);
-      }
-      blk0 = nblk0;
-      blk1 = nblk1;
-      if (masked) {
-        rt.template attend<true>(tile, tb, p.scale_log2);
-      } else {
-        rt.template attend<false>(tile, tb, p.scale_log2);
+      blk[d][0] = block_of(p, it, tb + kDepth * kT);
+      blk[d][1] = block_of(p, it, tb + kDepth * kT + kH);
+    }
+    for (int tb = w_begin; tb < w_end; tb += kDepth * kT) {
+      step(st[0], blk[0], tb);
+      if constexpr (kDepth > 1) {
+        if (tb + kT < w_end) step(st[1], blk[1], tb + kT);
       }
     }
   }
@@ -1180,15 +1252,17 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_d128_kernel(Decode
 }
 
 template <int KV_DT, int TOK>
-__global__ void __launch_bounds__(128, 2) decode_mfma_d128_rows32_kernel(DecodeParams p) {
+__global__ void __launch_bounds__(128, TOK == 0 ? 1 : 2) decode_mfma_d128_rows32_kernel(DecodeParams p) {
   // A workgroup is one pair of waves: wave w owns query rows 16w .. 16w+15 and fetches rows 16w ..
   // of every tile.  A tile is parked while both waves still read the previous one from the other
   // buffer, so one barrier (of two waves) per tile suffices.  Four such workgroups share a CU.
   __shared__ __attribute__((aligned(16))) uint8_t lds_all[2 * kLdsTile];
   __shared__ float lds_ml[2 * 16 * 2];
 
-  constexpr int kT = 32 * TOK;  // tokens per tile
-  constexpr int kH = 16 * TOK;  // tokens per half tile
+  constexpr int kT = tile_tokens_of(TOK);  // tokens per tile
+  constexpr int kH = half_tokens_of(TOK);  // tokens from the tile's first half to its second
+  constexpr int kP1 = TOK == 0 ? 1 : 0;    // head_dim 256: the second half is the same tokens' second plane
+  static_assert(16 * xch_row_bytes(TOK) <= kLdsTile, "the end-of-item exchange must fit a wave's tile");
 
   Item it;
   if (!decode_item(p, blockIdx.x, it)) return;
@@ -1209,20 +1283,23 @@ __global__ void __launch_bounds__(128, 2) decode_mfma_d128_rows32_kernel(DecodeP
 
   typename KvHalf<KV_DT>::Geom geom;
   geom.init(p, lane);
-  // Two register stages, used alternately: the loads of tiles i+1 and i+2 are in flight while tile
-  // i is consumed.  (A wave fetches only half a tile, so one stage would leave too few bytes in
-  // flight per CU to cover the HBM latency.)  Both waves run the same iterations.
-  KvHalf<KV_DT> mine[2];  // the 16 rows this wave fetches: rows 16*rs .. of the tile
+  // kDepth register stages, used in turn: the loads of tiles i+1 .. i+kDepth are in flight while tile
+  // i is consumed (a wave fetches only half a tile, so one stage would leave too few bytes in flight
+  // per CU to cover the HBM latency; four stages for head_dim 256, which runs one wave per SIMD,
+  // were slower than two).  Both waves run the same iterations.
+  constexpr int kDepth = 2;
+  KvHalf<KV_DT> mine[kDepth];  // the 16 rows this wave fetches: rows 16*rs .. of the tile
+  int blk[kDepth];             // block id of the half each stage loads next, fetched a round earlier
 
-  auto issue = [&](KvHalf<KV_DT>& m, int blk, int tb) {
-    if (tb < w_end) m.issue(p, it, tb + kH * rs, blk, geom);
+  auto issue = [&](KvHalf<KV_DT>& m, int b, int tb) {
+    if (tb < w_end) m.issue(p, it, tb + kH * rs, b, geom, kP1 * rs);
   };
-  // `blk`: block id of the half this wave fetches two tiles on; replaced by that of the tile four
-  // on.  The scalar load goes out before the tile is parked: it shares a counter with the LDS
-  // traffic, so the wait before the barrier also waits for it.
-  auto step = [&](KvHalf<KV_DT>& m, int& blk, int i) {
+  // `b`: block id of the half this wave fetches kDepth tiles on; replaced by that of the tile
+  // 2 * kDepth on.  The scalar load goes out before the tile is parked: it shares a counter with the
+  // LDS traffic, so the wait before the barrier also waits for it.
+  auto step = [&](KvHalf<KV_DT>& m, int& b, int i) {
     const int tb = w_begin + i * kT;
-    const int nblk = block_of(p, it, tb + 4 * kT + kH * rs);
+    const int nblk = block_of(p, it, tb + 2 * kDepth * kT + kH * rs);
     uint8_t* tile = tiles + (i & 1) * kLdsTile;
     const bool masked = (tb + kT > mask_hi_from) || (tb < mask_lo_until);
     if (masked) {
@@ -1230,8 +1307,8 @@ __global__ void __launch_bounds__(128, 2) decode_mfma_d128_rows32_kernel(DecodeP
     } else {
       m.template park<false>(tile, rs, tb + kH * rs, it.len, p.scale_log2, geom);
     }
-    issue(m, blk, tb + 2 * kT);
-    blk = nblk;
+    issue(m, b, tb + kDepth * kT);
+    b = nblk;
     __syncthreads();  // both halves of tile i are parked; both waves are done with tile i-1
     if (masked) {
       rt.template attend<true>(tile, tb, p.scale_log2);
@@ -1239,13 +1316,18 @@ __global__ void __launch_bounds__(128, 2) decode_mfma_d128_rows32_kernel(DecodeP
       rt.template attend<false>(tile, tb, p.scale_log2);
     }
   };
-  issue(mine[0], block_of(p, it, w_begin + kH * rs), w_begin);
-  issue(mine[1], block_of(p, it, w_begin + kT + kH * rs), w_begin + kT);
-  int blk_a = block_of(p, it, w_begin + 2 * kT + kH * rs);
-  int blk_b = block_of(p, it, w_begin + 3 * kT + kH * rs);
-  for (int i = 0; i < iters; i += 2) {
-    step(mine[0], blk_a, i);
-    if (i + 1 < iters) step(mine[1], blk_b, i + 1);
+#pragma unroll
+  for (int d = 0; d < kDepth; ++d) {
+    issue(mine[d], block_of(p, it, w_begin + d * kT + kH * rs), w_begin + d * kT);
+    blk[d] = block_of(p, it, w_begin + (kDepth + d) * kT + kH * rs);
+  }
+  for (int i = 0; i < iters; i += kDepth) {
+    step(mine[0], blk[0], i);
+    if (i + 1 < iters) step(mine[1], blk[1], i + 1);
+    if constexpr (kDepth > 2) {
+      if (i + 2 < iters) step(mine[2], blk[2], i + 2);
+      if (i + 3 < iters) step(mine[3], blk[3], i + 3);
+    }
   }
   __syncthreads();  // all tiles consumed before the buffers are reused for the exchange
   finish_item<KV_DT, TOK, 1>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, rs, 0, lane, rs);
@@ -1264,7 +1346,7 @@ __global__ void __launch_bounds__(128, 2) decode_mfma_d128_rows32_kernel(DecodeP
 // being read and does not wait for them.  With causal rows a wave skips the tiles none of its rows
 // can see.  Two such workgroups share a CU.
 constexpr int kPrefillBuffers = 4;
-constexpr int kPrefillTile = 16896;  // 16 KiB of K and V; as the end-of-item exchange 16 rows of kXchRow
+constexpr int kPrefillTile = 16896;  // 16 KiB of K and V; as the end-of-item exchange 16 rows of 528 bytes
 
 #define XLLM_HIP_GLOBAL_TO_LDS_16(gptr, lptr)                                                   \
   __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gptr),       \
@@ -1331,6 +1413,7 @@ __global__ void __launch_bounds__(256, 2) prefill_mfma_d128_kernel(DecodeParams 
   __shared__ __attribute__((aligned(16))) uint8_t buf2[kPrefillTile];
   __shared__ __attribute__((aligned(16))) uint8_t buf3[kPrefillTile];
   __shared__ float lds_ml[4 * 16 * 2];
+  static_assert(TOK != 0, "head_dim 256 does not fit two row tiles per wave");
   constexpr int kT = 32 * TOK;  // tokens per tile
 
   Item it;
@@ -1574,8 +1657,8 @@ __global__ void __launch_bounds__(256) csr_to_block_table_kernel(const int32_t* 
 // Host side.
 // ---------------------------------------------------------------------------------
 
-enum Variant { kNone = 0, kMfmaD128 = 1, kGeneric = 2, kMfmaD64 = 3 };
-static bool is_mfma(Variant v) { return v == kMfmaD128 || v == kMfmaD64; }
+enum Variant { kNone = 0, kMfmaD128 = 1, kGeneric = 2, kMfmaD64 = 3, kMfmaD256 = 4 };
+static bool is_mfma(Variant v) { return v == kMfmaD128 || v == kMfmaD64 || v == kMfmaD256; }
 
 // Split target: about this many work items (workgroups) per launch.  A workgroup of the MFMA kernel
 // is four waves, one per SIMD of a CU, and two workgroups fit on a CU (256 VGPRs, < 80 KiB of LDS).
@@ -1584,8 +1667,9 @@ constexpr int kNumCUs = 256;
 
 // Work items to aim for: two 4-wave workgroups per CU for the 16-row and the 128-row MFMA kernels,
 // four 2-wave workgroups for the 32-row one, eight single waves for the generic kernel.
-static int target_items(int variant_is_mfma, int rows) {
+static int target_items(int variant_is_mfma, int rows, bool one_wave_per_simd) {
   int v = !variant_is_mfma ? 8 * kNumCUs : (rows > 16 && rows <= kPrefillMinRows) ? 4 * kNumCUs : 2 * kNumCUs;
+  if (one_wave_per_simd) v /= 2;  // head_dim 256: half as many workgroups fit a CU
   if (const char* e = getenv("XLLM_HIP_DECODE_TARGET_ITEMS")) {
     const int t = atoi(e);
     if (t > 0) v = t;
@@ -1603,9 +1687,11 @@ static Variant pick_variant(const xllm_hip_kv_cache* c, const xllm_hip_decode_ar
   const bool force_generic = getenv("XLLM_HIP_DECODE_FORCE_GENERIC") != nullptr;
   // head_dim 64 rides on the head_dim-128 kernels with two tokens per tile row: half a tile
   // (32 tokens) must then lie in one block.
+  // head_dim 256 rides on them with two tile rows per token: a tile is 16 tokens.
   const bool d128 = c->head_dim == 128 && c->block_size >= 16;
   const bool d64 = c->head_dim == 64 && c->block_size >= 32;
-  if (!force_generic && (d128 || d64) && kv_ok && is_pow2(c->block_size) && a->sm_scale >= 0.0f) {
+  const bool d256 = c->head_dim == 256 && c->block_size >= 16;
+  if (!force_generic && (d128 || d64 || d256) && kv_ok && is_pow2(c->block_size) && a->sm_scale >= 0.0f) {
     const int vec = 16 / eb;  // elements per 16-byte load
     const bool strides_ok = c->stride_block % vec == 0 && c->stride_head % vec == 0 && c->stride_slot % vec == 0 &&
                             a->q_token_stride % 8 == 0;
@@ -1619,7 +1705,7 @@ static Variant pick_variant(const xllm_hip_kv_cache* c, const xllm_hip_decode_ar
     }
     const bool range_ok = c->stride_block >= 0 && c->stride_block < lim32 && c->stride_slot >= 0 &&
                           c->stride_slot * c->block_size < lim32;
-    if (strides_ok && range_ok && ptrs_ok && scales_ok) return d128 ? kMfmaD128 : kMfmaD64;
+    if (strides_ok && range_ok && ptrs_ok && scales_ok) return d128 ? kMfmaD128 : d64 ? kMfmaD64 : kMfmaD256;
   }
   if (c->head_dim <= 256 && is_pow2(c->block_size)) return kGeneric;
   return kNone;
@@ -1708,17 +1794,20 @@ static int fill_params(const xllm_hip_kv_cache* c,
   p.rows = p.group * p.n;
   const Variant variant = pick_variant(c, a);
   // the many-row kernel moves tiles from global memory to LDS as they are: 16-bit caches only
-  p.rows_per_item = !is_mfma(variant) ? 1 : (p.rows > kPrefillMinRows && !quant) ? kPrefillRowsPerItem : kMaxRowsPerItem;
+  // (nor does head_dim 256: two row tiles of 256 elements per wave do not fit the registers)
+  p.rows_per_item = !is_mfma(variant) ? 1
+                    : (p.rows > kPrefillMinRows && !quant && variant != kMfmaD256) ? kPrefillRowsPerItem
+                                                                                   : kMaxRowsPerItem;
   p.min_chunk = is_mfma(variant) ? kMinChunkTokens : kMinChunkTokensGeneric;
-  p.tok = variant == kMfmaD64 ? 2 : 1;
-  p.tile_tokens = kTileTokens * p.tok;
+  p.tok = variant == kMfmaD64 ? 2 : variant == kMfmaD256 ? 0 : 1;
+  p.tile_tokens = variant == kMfmaD256 ? kTileTokens / 2 : kTileTokens * p.tok;
   p.row_groups = row_groups(a->q_per_seq, a->num_q_heads, c->num_kv_heads, p.rows_per_item);
   p.head_dim = c->head_dim;
   p.block_size = c->block_size;
   p.log2_bs = is_pow2(c->block_size) ? ilog2(c->block_size) : 0;
   p.max_blocks_per_seq = a->max_blocks_per_seq;
   p.window_left = a->window_left;
-  p.target_items = target_items(is_mfma(variant), p.rows);
+  p.target_items = target_items(is_mfma(variant), p.rows, variant == kMfmaD256);
   // Only the MFMA kernel finishes single-chunk sequences itself.  When the caller's host-side
   // lengths (the reference keeps both in AttentionMetadata) show that the chunk the plan would
   // pick covers the longest sequence, no sequence is split: the plan is told never to split
@@ -1767,7 +1856,7 @@ static int64_t max_items(const DecodeParams& p) {
 template <int KV_DT, int TOK>
 static void launch_mfma_tok(const DecodeParams& p, unsigned grid, hipStream_t st) {
   if (p.rows_per_item == kPrefillRowsPerItem) {
-    if constexpr (!quant_of(KV_DT)) prefill_mfma_d128_kernel<KV_DT, TOK><<<grid, 256, 0, st>>>(p);
+    if constexpr (!quant_of(KV_DT) && TOK != 0) prefill_mfma_d128_kernel<KV_DT, TOK><<<grid, 256, 0, st>>>(p);
   } else if (p.rows <= 16) {
     decode_mfma_d128_kernel<KV_DT, TOK><<<grid, 64 * kWaves, 0, st>>>(p);
   } else {
@@ -1779,6 +1868,8 @@ template <int KV_DT>
 static void launch_mfma(const DecodeParams& p, unsigned grid, hipStream_t st) {
   if (p.tok == 2) {
     launch_mfma_tok<KV_DT, 2>(p, grid, st);
+  } else if (p.tok == 0) {
+    launch_mfma_tok<KV_DT, 0>(p, grid, st);
   } else {
     launch_mfma_tok<KV_DT, 1>(p, grid, st);
   }
@@ -1829,6 +1920,8 @@ extern "C" const char* xllm_hip_paged_decode_variant(const xllm_hip_kv_cache* ca
       return "mfma_d128";
     case kMfmaD64:
       return "mfma_d64";
+    case kMfmaD256:
+      return "mfma_d256";
     case kGeneric:
       return "generic";
     default:

@@ -68,6 +68,20 @@ WORKLOADS = {
         name="cfg5_int8_spec_verify", batch=32, num_q_heads=64, num_kv_heads=8, head_dim=128, block_size=128,
         q_per_seq=4, kv_dtype="int8", seq_len_kind="fixed", seq_len=32768,
         description="int8 KV speculative verify: 64q/8kv, D=128, bs=128, B=32, L=32768, 4 causal draft tokens"),
+    # Shapes beside the five configurations above, measured the same way (head_dim 256 as in Gemma-2 /
+    # Qwen3-Next attention layers).
+    "aux_d256_bf16_b64_ctx4k": DecodeWorkload(
+        name="aux_d256_bf16_b64_ctx4k", batch=64, num_q_heads=16, num_kv_heads=8, head_dim=256, block_size=16,
+        seq_len_kind="fixed", seq_len=4096, value_std=0.5,
+        description="head_dim 256 decode: bf16, 16q/8kv, D=256, bs=16, B=64, L=4096"),
+    "aux_d256_fp8_b64_ctx8k": DecodeWorkload(
+        name="aux_d256_fp8_b64_ctx8k", batch=64, num_q_heads=32, num_kv_heads=8, head_dim=256, block_size=16,
+        kv_dtype="fp8", seq_len_kind="fixed", seq_len=8192,
+        description="head_dim 256 decode over an fp8-e4m3 cache: 32q/8kv, D=256, bs=16, B=64, L=8192"),
+    "aux_d256_int8_spec_verify": DecodeWorkload(
+        name="aux_d256_int8_spec_verify", batch=32, num_q_heads=64, num_kv_heads=8, head_dim=256, block_size=128,
+        q_per_seq=4, kv_dtype="int8", seq_len_kind="fixed", seq_len=16384,
+        description="head_dim 256 speculative verify over an int8 cache: 64q/8kv, D=256, bs=128, B=32, L=16384, 4 draft tokens"),
 }
 
 
