@@ -318,14 +318,20 @@ __device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it)
 // ---------------------------------------------------------------------------------
 // Merge of the sequences that were split into several chunks:
 //   out = sum_i 2^(lse_i - lse) * partial_i,   lse = log2 sum_i 2^lse_i
-// in one pass over the partials with a running maximum.  32 threads per output row.
+// One wave per output row.  First the row's log-sum-exps, one chunk per lane, give the maximum and
+// the denominator by wave reductions; then the partials are summed with their weights, the lanes
+// covering the row's columns and the loads of several chunks in flight at a time — a long sequence
+// of a small batch has hundreds of chunks per row, and a chunk-by-chunk running maximum would
+// serialise that many memory latencies.
 // ---------------------------------------------------------------------------------
 
+constexpr int kMergeRowsPerBlock = 4;
+
 template <int Q_DT>
-__global__ void __launch_bounds__(256) decode_merge_kernel(DecodeParams p) {
+__global__ void __launch_bounds__(64 * kMergeRowsPerBlock) decode_merge_kernel(DecodeParams p) {
   const int nhq = p.n * p.num_q_heads;
-  const int64_t row = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 5);
-  const int sub = threadIdx.x & 31;
+  const int64_t row = (int64_t)blockIdx.x * kMergeRowsPerBlock + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
   if (row >= (int64_t)p.batch * nhq) return;
   const int b = (int)(row / nhq);
   int q0 = b * p.n, nb = p.n;
@@ -344,42 +350,52 @@ __global__ void __launch_bounds__(256) decode_merge_kernel(DecodeParams p) {
   const int f0 = p.full_prefix[b];
   const int nf = p.full_prefix[b + 1] - f0;
   const int tail_slot = p.hdr->total_full + p.tail_prefix[b];
+  auto partial_row = [&](int i) { return (int64_t)(i < nf ? f0 + i : tail_slot) * nhq + rem; };
 
-  float m = neg_inf, ssum = 0.0f;
-  float o[2][4] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};  // head_dim <= 256: two float4 per thread
-  for (int i = 0; i < cnt; ++i) {
-    const int sc = i < nf ? f0 + i : tail_slot;
-    const int64_t prow = (int64_t)sc * nhq + rem;
-    const float li = p.partial_lse[prow];
-    if (li == neg_inf) continue;
-    const float m_new = fmaxf(m, li);
-    const float a = __builtin_amdgcn_exp2f(m - m_new);
-    const float w = __builtin_amdgcn_exp2f(li - m_new);
-    ssum = ssum * a + w;
-    const float* po = p.partial_out + prow * D;
+  // 1. maximum and denominator over the chunks' log-sum-exps
+  float m = neg_inf;
+  for (int i = lane; i < cnt; i += 64) m = fmaxf(m, p.partial_lse[partial_row(i)]);
+  m = wave_max(m);
+  const float m_safe = m == neg_inf ? 0.0f : m;
+  float ssum = 0.0f;
+  for (int i = lane; i < cnt; i += 64) ssum += __builtin_amdgcn_exp2f(p.partial_lse[partial_row(i)] - m_safe);
+  ssum = wave_sum(ssum);
+
+  // 2. weighted sum of the partial rows: lane covers columns lane, lane + 64, ... (head_dim <= 256)
+  float o[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  // kUnroll chunks at a time: their loads are all issued before the first is used
+  auto add_chunks = [&](int i0, auto unroll) {
+    constexpr int kUnroll = decltype(unroll)::value;
+    float w[kUnroll], v[kUnroll][4];
 #pragma unroll
-    for (int q4 = 0; q4 < 2; ++q4) {
+    for (int u = 0; u < kUnroll; ++u) {
+      const int i = min(i0 + u, cnt - 1);
+      const int64_t prow = partial_row(i);
+      const float li = p.partial_lse[prow];
+      w[u] = (i0 + u < cnt && li != neg_inf) ? __builtin_amdgcn_exp2f(li - m_safe) : 0.0f;
+      const float* po = p.partial_out + prow * D;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int d = (sub + 32 * q4) * 4 + e;
-        if (d < D) o[q4][e] = o[q4][e] * a + w * po[d];
-      }
+      for (int k = 0; k < 4; ++k) v[u][k] = lane + 64 * k < D ? po[lane + 64 * k] : 0.0f;
     }
-    m = m_new;
-  }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) o[k] += w[u] != 0.0f ? w[u] * v[u][k] : 0.0f;  // an empty chunk's row may hold anything
+    }
+  };
+  int i0 = 0;
+  for (; i0 + 16 <= cnt; i0 += 16) add_chunks(i0, std::integral_constant<int, 16>{});
+  for (; i0 < cnt; i0 += 4) add_chunks(i0, std::integral_constant<int, 4>{});
   const float inv = ssum > 0.0f ? 1.0f / ssum : 0.0f;
   const int64_t tok = (int64_t)q0 + j;
-  if (p.lse != nullptr && sub == 0) {
+  if (p.lse != nullptr && lane == 0) {
     p.lse[tok * p.num_q_heads + head] = ssum > 0.0f ? m + __builtin_amdgcn_logf(ssum) : neg_inf;
   }
   const int64_t obase = tok * p.out_token_stride + (int64_t)head * D;
 #pragma unroll
-  for (int q4 = 0; q4 < 2; ++q4) {
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int d = (sub + 32 * q4) * 4 + e;
-      if (d < D) Elem<Q_DT>::store(p.out, obase + d, o[q4][e] * inv);
-    }
+  for (int k = 0; k < 4; ++k) {
+    const int d = lane + 64 * k;
+    if (d < D) Elem<Q_DT>::store(p.out, obase + d, o[k] * inv);
   }
 }
 
@@ -2017,16 +2033,16 @@ extern "C" int xllm_hip_paged_decode_run_timed(const xllm_hip_kv_cache* cache,
   if (p.implicit_plan) return XLLM_HIP_OK;  // nothing was split: the outputs are final
 
   const int64_t rows = (int64_t)p.batch * p.n * p.num_q_heads;
-  const unsigned mgrid = (unsigned)((rows + 7) / 8);
+  const unsigned mgrid = (unsigned)((rows + kMergeRowsPerBlock - 1) / kMergeRowsPerBlock);
   switch (args->q_dtype) {
     case XLLM_HIP_BF16:
-      decode_merge_kernel<XLLM_HIP_BF16><<<mgrid, 256, 0, st>>>(p);
+      decode_merge_kernel<XLLM_HIP_BF16><<<mgrid, 64 * kMergeRowsPerBlock, 0, st>>>(p);
       break;
     case XLLM_HIP_FP16:
-      decode_merge_kernel<XLLM_HIP_FP16><<<mgrid, 256, 0, st>>>(p);
+      decode_merge_kernel<XLLM_HIP_FP16><<<mgrid, 64 * kMergeRowsPerBlock, 0, st>>>(p);
       break;
     default:
-      decode_merge_kernel<XLLM_HIP_FP32><<<mgrid, 256, 0, st>>>(p);
+      decode_merge_kernel<XLLM_HIP_FP32><<<mgrid, 64 * kMergeRowsPerBlock, 0, st>>>(p);
       break;
   }
   return check_launch("decode_merge_kernel");

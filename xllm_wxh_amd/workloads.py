@@ -82,6 +82,15 @@ WORKLOADS = {
         name="aux_d256_int8_spec_verify", batch=32, num_q_heads=64, num_kv_heads=8, head_dim=256, block_size=128,
         q_per_seq=4, kv_dtype="int8", seq_len_kind="fixed", seq_len=16384,
         description="head_dim 256 speculative verify over an int8 cache: 64q/8kv, D=256, bs=128, B=32, L=16384, 4 draft tokens"),
+    # Small batches: the split-KV schedule (plan, attention over chunks, merge) is what is measured.
+    "aux_b1_ctx32k": DecodeWorkload(
+        name="aux_b1_ctx32k", batch=1, num_q_heads=32, num_kv_heads=8, head_dim=128, block_size=16,
+        seq_len_kind="fixed", seq_len=32768, value_std=0.5,
+        description="one sequence: bf16, 32q/8kv, D=128, bs=16, B=1, L=32768"),
+    "aux_b8_ctx8k": DecodeWorkload(
+        name="aux_b8_ctx8k", batch=8, num_q_heads=32, num_kv_heads=8, head_dim=128, block_size=16,
+        seq_len_kind="fixed", seq_len=8192, value_std=0.5,
+        description="small batch: bf16, 32q/8kv, D=128, bs=16, B=8, L=8192"),
 }
 
 
