@@ -29,14 +29,16 @@ def _run(c, q_counts, max_q, **kw):
 
 
 @pytest.mark.parametrize("kv", ["bf16", "fp8", "int8"])
-@pytest.mark.parametrize("Hq,Hkv", [(32, 8), (64, 8), (8, 8)])
-def test_mixed_step_matches_oracle(gpu, kv, Hq, Hkv):
+@pytest.mark.parametrize("Hq,Hkv,D,bs", [(32, 8, 128, 16), (64, 8, 128, 16), (8, 8, 128, 16), (32, 8, 256, 16),
+                                         (16, 8, 256, 64), (32, 8, 64, 32)])
+def test_mixed_step_matches_oracle(gpu, kv, Hq, Hkv, D, bs):
     """A mixed step: decode sequences (1 token), speculative verify (4) and prefill chunks (up to 70
     tokens, some reaching back to the start of the sequence) in one call."""
-    print("case mixed step", kv, Hq, Hkv, flush=True)
+    print("case mixed step", kv, Hq, Hkv, D, bs, flush=True)
     lens = [300, 70, 33, 1, 129, 4096, 64, 40]
     q_counts = [1, 70, 4, 1, 17, 64, 0, 40]   # 70 == len and 40 == len: the whole sequence is the chunk
-    c = Case(len(lens), Hq, Hkv, 128, 16, lens, kv=kv, seed=21)
+    c = Case(len(lens), Hq, Hkv, D, bs, lens, kv=kv, seed=21)
+    assert c.variant() == {64: "mfma_d64", 128: "mfma_d128", 256: "mfma_d256"}[D]
     out, lse, ref, ref_lse, q_indptr = _run(c, q_counts, max(q_counts))
     err = float(np.abs(out - ref).max())
     print("   err %.3e" % err, flush=True)
@@ -130,10 +132,11 @@ def test_many_row_kernel_split_sequences_and_window(gpu):
     assert float(np.abs(out.float().cpu().numpy() - ref).max()) <= 1.2e-2
 
 
-def test_garbage_past_the_sequence_end_does_not_reach_the_many_row_kernel(gpu):
-    print("case many rows garbage", flush=True)
+@pytest.mark.parametrize("D", [128, 256])
+def test_garbage_past_the_sequence_end_does_not_reach_the_many_row_kernel(gpu, D):
+    print("case many rows garbage", D, flush=True)
     lens = [45, 200]
-    c = Case(2, 32, 8, 128, 16, lens, n=24, seed=34)
+    c = Case(2, 32, 8, D, 16, lens, n=24, seed=34)
     ref, _ = c.oracle()
     # NaN in every slot past the end of each sequence's last block and in unused blocks
     nan = float("nan")

@@ -273,12 +273,13 @@ def test_block_table_permutation_invariance_is_bitwise(gpu):
     assert torch.equal(out, out2)
 
 
+@pytest.mark.parametrize("D", [128, 256])
 @pytest.mark.parametrize("kv", ["bf16", "fp8"])
-def test_garbage_outside_the_sequence_is_ignored(gpu, kv):
+def test_garbage_outside_the_sequence_is_ignored(gpu, kv, D):
     """Slots past seq_len, padded block-table entries and unused blocks may hold anything (NaN included)."""
-    print("case garbage", kv, flush=True)
+    print("case garbage", kv, D, flush=True)
     lens = [37, 16, 1000, 5]
-    case = Case(4, 32, 8, 128, 16, lens, kv=kv, seed=13)
+    case = Case(4, 32, 8, D, 16, lens, kv=kv, seed=13)
     ref_out, _ = case.run()
     used = np.zeros((case.nblocks, 16), bool)
     for b, L in enumerate(lens):
