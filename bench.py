@@ -38,6 +38,9 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default=DEFAULT_WORKLOAD)
     ap.add_argument("--pools", type=int, default=3, help="disjoint KV pools rotated between steps")
+    ap.add_argument("--kv-layout", choices=["HND", "NHD"], default="HND",
+                    help="HND [blocks, heads, slots, dim] is the path's native layout; NHD [blocks, slots, heads, dim] "
+                         "is what the reference's CUDA backend allocates")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget of the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -51,13 +54,14 @@ def parse_args():
     return ap.parse_args()
 
 
-def build_pools(w, torch, ops, num_blocks, npools, device):
-    """KV pools in the native HND layout.  Quantised pools are produced by the path's own quantising
+def build_pools(w, torch, ops, num_blocks, npools, device, layout="HND"):
+    """KV pools (HND is the native layout).  Quantised pools are produced by the path's own quantising
     KV write from N(0,1) bf16 values, as the workload defines them."""
     pools = []
     gen = torch.Generator(device=device)
     gen.manual_seed(1234)
-    shape = (num_blocks, w.num_kv_heads, w.block_size, w.head_dim)
+    shape = (num_blocks, w.num_kv_heads, w.block_size, w.head_dim) if layout == "HND" else \
+        (num_blocks, w.block_size, w.num_kv_heads, w.head_dim)
     for _ in range(npools):
         if w.kv_dtype in ("bf16", "fp32"):
             dt = torch.bfloat16 if w.kv_dtype == "bf16" else torch.float32
@@ -79,7 +83,7 @@ def build_pools(w, torch, ops, num_blocks, npools, device):
             slots = torch.arange(s0, s0 + t, device=device, dtype=torch.int32)
             ops.quant_to_paged_cache(ops.ReshapePagedCacheParams(
                 key=src_k, value=src_v, k_cache=k, v_cache=v, slot_mapping=slots, k_cache_scale=ks,
-                v_cache_scale=vs))
+                v_cache_scale=vs, kv_layout=layout))
         torch.cuda.synchronize()
         pools.append((k, v, ks, vs))
     return pools
@@ -119,7 +123,7 @@ def main():
     io_dtype = torch.float32 if w.kv_dtype == "fp32" else torch.bfloat16  # query, output, new K/V rows
     seq_lens = workloads.make_seq_lens(w, seed=0)
     table, num_blocks, lists = workloads.make_block_tables(w, seq_lens, seed=0)
-    pools = build_pools(w, torch, ops, num_blocks, args.pools, device)
+    pools = build_pools(w, torch, ops, num_blocks, args.pools, device, args.kv_layout)
     T = w.batch * w.q_per_seq
     gen = torch.Generator(device=device)
     gen.manual_seed(99)
@@ -135,10 +139,11 @@ def main():
         k, v, ks, vs = pools[i % len(pools)]
         ops.batch_decode(q, k, out, block_table, seq_lens_d, v, None, None, ks, vs, scale=w.sm_scale,
                          q_per_seq=w.q_per_seq, workspace=ws, kv_cache_quant_bit_size=quant_bits,
-                         max_seq_len=int(seq_lens.max()), total_kv_len=int(seq_lens.sum()), events=events)
+                         max_seq_len=int(seq_lens.max()), total_kv_len=int(seq_lens.sum()), events=events,
+                         kv_layout=args.kv_layout)
 
     variant = ops.decode_variant(q, pools[0][0], pools[0][1], block_table, seq_lens_d, pools[0][2], pools[0][3],
-                                 q_per_seq=w.q_per_seq)
+                                 q_per_seq=w.q_per_seq, kv_layout=args.kv_layout)
 
     # HIP events around the attention kernel of every timed step (recorded on the launch stream by
     # the library itself).  torch creates the handles; the first record materialises them.
@@ -182,7 +187,7 @@ def main():
     def kv_write(i):
         k, v, ks, vs = pools[i % len(pools)]
         p = ops.ReshapePagedCacheParams(key=new_k, value=new_v, k_cache=k, v_cache=v, slot_mapping=slots,
-                                        k_cache_scale=ks, v_cache_scale=vs)
+                                        k_cache_scale=ks, v_cache_scale=vs, kv_layout=args.kv_layout)
         if ks is not None:
             ops.quant_to_paged_cache(p)
         else:
@@ -234,7 +239,7 @@ def main():
             "kv_dtype": w.kv_dtype,
             "sum_seq_len": int(seq_lens.sum()),
             "max_seq_len": int(seq_lens.max()),
-            "kv_layout": "HND",
+            "kv_layout": args.kv_layout,
             "kv_pools_rotated": len(pools),
             "kernel_variant": variant,
         },
@@ -378,6 +383,10 @@ def cpu_baseline(w, torch, pool, q, block_table, seq_lens, out, step, args):
 
     cores = torch.get_num_threads()
     k, v, ks, vs = pool
+    if args.kv_layout == "NHD":  # the CPU path reads [blocks, heads, slots, dim] views
+        k, v = k.permute(0, 2, 1, 3), v.permute(0, 2, 1, 3)
+        if ks is not None:
+            ks, vs = ks.permute(0, 2, 1), vs.permute(0, 2, 1)
     total_tokens = int(seq_lens.sum())
     # sample: whole batch unless it is very large
     nseq = w.batch

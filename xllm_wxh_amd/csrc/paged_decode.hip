@@ -1839,12 +1839,18 @@ static int fill_params(const xllm_hip_kv_cache* c,
   // partial per chunk and row would be large, so nothing is split.
   if (never_split(a->q_per_seq, a->num_q_heads, c->num_kv_heads)) p.fixed_chunk = 1 << 30;
   p.implicit_plan = p.direct_single && p.fixed_chunk == (1 << 30) ? 1 : 0;
-  // XCD clusters: the row groups of a (chunk, kv head); and, for a quantised cache whose scale rows
-  // are shorter than a 128-byte line and contiguous over the heads, the heads that share a line.
+  // XCD clusters: the row groups of a (chunk, kv head); and the kv heads whose rows share 128-byte
+  // lines — scale rows shorter than a line (HND: block_size * 4 bytes per head; NHD: the heads of a
+  // slot are adjacent floats) or cache rows shorter than a line (NHD with 64 one-byte elements).
   int heads_per_line = 1;
-  if (quant && c->scale_stride_slot == 1 && c->scale_stride_head == c->block_size && c->block_size * 4 < 128) {
-    heads_per_line = 128 / (c->block_size * 4);
-    while (heads_per_line > 1 && c->num_kv_heads % heads_per_line != 0) heads_per_line >>= 1;
+  {
+    auto shared_by = [](int64_t head_stride_bytes) {
+      return head_stride_bytes > 0 && head_stride_bytes < 128 ? (int)(128 / head_stride_bytes) : 1;
+    };
+    heads_per_line = shared_by(c->stride_head * elem_bytes(c->dtype));
+    if (quant) heads_per_line = max(heads_per_line, shared_by(c->scale_stride_head * 4));
+    if (heads_per_line > c->num_kv_heads) heads_per_line = c->num_kv_heads;
+    while (heads_per_line > 1 && c->num_kv_heads % heads_per_line != 0) --heads_per_line;
   }
   p.cluster = p.row_groups * heads_per_line;
   p.q_dtype = a->q_dtype;
