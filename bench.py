@@ -41,6 +41,13 @@ def parse_args():
     ap.add_argument("--kv-layout", choices=["HND", "NHD"], default="HND",
                     help="HND [blocks, heads, slots, dim] is the path's native layout; NHD [blocks, slots, heads, dim] "
                          "is what the reference's CUDA backend allocates")
+    ap.add_argument("--set", action="append", default=[], metavar="FIELD=VALUE",
+                    help="replace a field of the workload (e.g. --set block_size=128 --set batch=16): a variation "
+                         "of the named workload, reported under the name <workload>+<field>=<value>")
+    ap.add_argument("--kv-skew-bytes", type=int, default=None,
+                    help="bytes (a multiple of 16) by which a V pool is displaced from a 2 MiB boundary behind its K "
+                         "pool; default: the library's allocation policy (ops.allocate_kv_cache, 4096).  -1 allocates "
+                         "K and V separately, as torch.empty per tensor does")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget of the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -54,9 +61,20 @@ def parse_args():
     return ap.parse_args()
 
 
-def build_pools(w, torch, ops, num_blocks, npools, device, layout="HND"):
-    """KV pools (HND is the native layout).  Quantised pools are produced by the path's own quantising
-    KV write from N(0,1) bf16 values, as the workload defines them."""
+def build_pools(w, torch, ops, num_blocks, npools, device, layout="HND", skew_bytes=None):
+    """KV pools (HND is the native layout), allocated by the library's policy (ops.allocate_kv_cache).
+    Quantised pools are produced by the path's own quantising KV write from N(0,1) bf16 values, as
+    the workload defines them."""
+    def allocate(dt, with_scales):
+        if skew_bytes is not None and skew_bytes < 0:  # separate allocations
+            k, v = torch.empty(shape, device=device, dtype=dt), torch.empty(shape, device=device, dtype=dt)
+            if not with_scales:
+                return k, v, None, None
+            return (k, v, torch.empty(shape[:3], device=device, dtype=torch.float32),
+                    torch.empty(shape[:3], device=device, dtype=torch.float32))
+        kw = {} if skew_bytes is None else {"skew_bytes": skew_bytes}
+        return ops.allocate_kv_cache(shape, dt, device, with_scales, **kw)
+
     pools = []
     gen = torch.Generator(device=device)
     gen.manual_seed(1234)
@@ -65,15 +83,16 @@ def build_pools(w, torch, ops, num_blocks, npools, device, layout="HND"):
     for _ in range(npools):
         if w.kv_dtype in ("bf16", "fp32"):
             dt = torch.bfloat16 if w.kv_dtype == "bf16" else torch.float32
-            k = torch.randn(shape, device=device, dtype=dt, generator=gen) * w.value_std
-            v = torch.randn(shape, device=device, dtype=dt, generator=gen) * w.value_std
+            k, v, _, _ = allocate(dt, False)
+            for t in (k, v):  # generated in slices: a whole-pool temporary would double the footprint
+                flat = t.view(-1)
+                for s0 in range(0, flat.numel(), 1 << 28):
+                    part = flat[s0:s0 + (1 << 28)]
+                    part.copy_(torch.randn(part.numel(), device=device, dtype=dt, generator=gen) * w.value_std)
             pools.append((k, v, None, None))
             continue
         cdt = torch.int8 if w.kv_dtype == "int8" else torch.float8_e4m3fn
-        k = torch.empty(shape, device=device, dtype=cdt)
-        v = torch.empty(shape, device=device, dtype=cdt)
-        ks = torch.empty(shape[:3], device=device, dtype=torch.float32)
-        vs = torch.empty(shape[:3], device=device, dtype=torch.float32)
+        k, v, ks, vs = allocate(cdt, True)
         total_slots = num_blocks * w.block_size
         chunk = 1 << 16
         for s0 in range(0, total_slots, chunk):
@@ -120,10 +139,19 @@ def main():
         print(json.dumps(aux_kernels(torch, ops, device)), flush=True)
         return
     w = workloads.WORKLOADS[args.workload]
+    if args.set:
+        import dataclasses
+
+        changes = {}
+        for item in args.set:
+            field, _, value = item.partition("=")
+            current = getattr(w, field)
+            changes[field] = type(current)(value) if not isinstance(current, str) else value
+        w = dataclasses.replace(w, name=w.name + "+" + ",".join(args.set), **changes)
     io_dtype = torch.float32 if w.kv_dtype == "fp32" else torch.bfloat16  # query, output, new K/V rows
     seq_lens = workloads.make_seq_lens(w, seed=0)
     table, num_blocks, lists = workloads.make_block_tables(w, seq_lens, seed=0)
-    pools = build_pools(w, torch, ops, num_blocks, args.pools, device, args.kv_layout)
+    pools = build_pools(w, torch, ops, num_blocks, args.pools, device, args.kv_layout, args.kv_skew_bytes)
     T = w.batch * w.q_per_seq
     gen = torch.Generator(device=device)
     gen.manual_seed(99)
@@ -240,6 +268,9 @@ def main():
             "sum_seq_len": int(seq_lens.sum()),
             "max_seq_len": int(seq_lens.max()),
             "kv_layout": args.kv_layout,
+            "kv_allocation": ("separate K and V allocations" if (args.kv_skew_bytes or 0) < 0 else
+                              "ops.allocate_kv_cache: one buffer, V %d bytes past a 2 MiB boundary behind K"
+                              % (ops.KV_SKEW_BYTES if args.kv_skew_bytes is None else args.kv_skew_bytes)),
             "kv_pools_rotated": len(pools),
             "kernel_variant": variant,
         },

@@ -1181,8 +1181,16 @@ __device__ inline int first_visible_tile(const DecodeParams& p, const Item& it) 
   return t0;
 }
 
+#ifndef XLLM_HIP_DEPTH16
+#define XLLM_HIP_DEPTH16 1
+#endif
+// Register stages of the 16-row kernel (tiles in flight while one is consumed) and the waves per SIMD
+// it is compiled for.
+constexpr int decode_depth(int kt, int tok) { return (!quant_of(kt) && tok != 0) ? XLLM_HIP_DEPTH16 : 1; }
+constexpr int decode_waves_per_simd(int kt, int tok) { return (tok == 0 || decode_depth(kt, tok) > 1) ? 1 : 2; }
+
 template <int KV_DT, int TOK>
-__global__ void __launch_bounds__(64 * kWaves, TOK == 0 ? 1 : 2) decode_mfma_d128_kernel(DecodeParams p) {
+__global__ void __launch_bounds__(64 * kWaves, decode_waves_per_simd(KV_DT, TOK)) decode_mfma_d128_kernel(DecodeParams p) {
   __shared__ __attribute__((aligned(16))) uint8_t lds_all[kWaves * kLdsTile];
   __shared__ float lds_ml[kWaves * 16 * 2];  // (running max, denominator) per wave and query row
 
@@ -1216,7 +1224,7 @@ __global__ void __launch_bounds__(64 * kWaves, TOK == 0 ? 1 : 2) decode_mfma_d12
   // head_dim 256, which run one wave per SIMD and so have few bytes in flight per CU, were slower:
   // 458 against 367 us on 64 x 8192 tokens of fp8 — the registers they take are paid for in copies
   // between the two register files.)
-  constexpr int kDepth = 1;
+  constexpr int kDepth = decode_depth(KV_DT, TOK);
   KvHalf<KV_DT> st[kDepth][2];  // per stage: the two halves (16 rows each) of a tile
   int blk[kDepth][2];           // block ids of the halves each stage loads next, fetched a round earlier
 
@@ -1261,6 +1269,12 @@ __global__ void __launch_bounds__(64 * kWaves, TOK == 0 ? 1 : 2) decode_mfma_d12
       step(st[0], blk[0], tb);
       if constexpr (kDepth > 1) {
         if (tb + kT < w_end) step(st[1], blk[1], tb + kT);
+      }
+      if constexpr (kDepth > 2) {
+        if (tb + 2 * kT < w_end) step(st[2], blk[2], tb + 2 * kT);
+      }
+      if constexpr (kDepth > 3) {
+        if (tb + 3 * kT < w_end) step(st[3], blk[3], tb + 3 * kT);
       }
     }
   }
@@ -1823,7 +1837,8 @@ static int fill_params(const xllm_hip_kv_cache* c,
   p.log2_bs = is_pow2(c->block_size) ? ilog2(c->block_size) : 0;
   p.max_blocks_per_seq = a->max_blocks_per_seq;
   p.window_left = a->window_left;
-  p.target_items = target_items(is_mfma(variant), p.rows, variant == kMfmaD256);
+  p.target_items = target_items(is_mfma(variant), p.rows,
+                                variant == kMfmaD256 || (p.rows <= 16 && decode_waves_per_simd(c->dtype, 1) == 1));
   // Only the MFMA kernel finishes single-chunk sequences itself.  When the caller's host-side
   // lengths (the reference keeps both in AttentionMetadata) show that the chunk the plan would
   // pick covers the longest sequence, no sequence is split: the plan is told never to split

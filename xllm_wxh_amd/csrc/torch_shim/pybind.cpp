@@ -65,6 +65,12 @@ PYBIND11_MODULE(_xllm_hip_torch, m) {
       .def(py::init<>())
       .def(py::init<torch::Tensor, torch::Tensor>())
       .def(py::init<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor>())
+      .def_static("allocate",
+                  [](const std::vector<int64_t>& shape, py::object dtype, const std::string& device, bool with_scales) {
+                    return KVCache::allocate(shape, torch::python::detail::py_object_to_dtype(dtype),
+                                             torch::Device(device), with_scales);
+                  },
+                  py::arg("shape"), py::arg("dtype"), py::arg("device"), py::arg("with_scales") = false)
       .def("get_k_cache", &KVCache::get_k_cache)
       .def("get_v_cache", &KVCache::get_v_cache)
       .def("get_k_cache_scale", &KVCache::get_k_cache_scale)
