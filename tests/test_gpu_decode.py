@@ -520,3 +520,21 @@ def test_large_batch_of_short_sequences(gpu):
         assert not torch.isnan(out.float()).any()
         assert max_abs_err(out, ref) <= REG_TOL
         assert float(out[::97].float().abs().max()) == 0.0  # empty sequences give zeros
+
+
+@pytest.mark.parametrize("kv,n", [("bf16", 1), ("int8", 4), ("bf16", 12)])
+def test_split_sequences_merge_in_the_attention_kernel_repeatably(gpu, kv, n):
+    """Split sequences are merged by the workgroup that finishes a row group's last chunk: whichever
+    that is, the result is the same bits on every run (the partials are summed in chunk order), the
+    finished-chunk counters are left at zero (a second run on the same plan works), and sequences
+    of one chunk beside split ones are untouched."""
+    print("case fused merge", kv, n, flush=True)
+    case = Case(5, 64, 8, 128, 16, [9000, 40, 5000, 1, 20000], n=n, kv=kv, seed=91)
+    ref, lse_ref = case.oracle()
+    first, lse_first = case.run()
+    assert max_abs_err(first, ref) <= (REG_TOL_QUANT if kv == "int8" else REG_TOL)
+    assert lse_err(lse_first, lse_ref) <= LSE_TOL
+    ws = ops.get_workspace(gpu, ops.decode_workspace_bytes(5, n, 64, 8, 128))
+    for i in range(40):
+        out, lse = case.run(workspace=ws, plan=(i == 0))  # one plan, many runs: the counters reset themselves
+        assert torch.equal(out, first) and torch.equal(lse, lse_first), i

@@ -76,6 +76,7 @@ struct WorkspaceLayout {
   size_t seq_chunks;    // SeqChunk [max_seq_chunks]
   size_t partial_lse;   // float [max_seq_chunks][n][Hq]
   size_t partial_out;   // float [max_seq_chunks][n][Hq][D]
+  size_t counters;      // int32 [B][Hkv][row groups]  chunks of a (sequence, kv head, row group) that have finished
   size_t total_bytes;
   int64_t max_seq_chunks;
 };
@@ -117,6 +118,8 @@ inline WorkspaceLayout workspace_layout(int batch, int q_per_seq, int num_q_head
   off = align_up(off + sizeof(float) * (size_t)w.max_seq_chunks * q_per_seq * num_q_heads, 256);
   w.partial_out = off;
   off = align_up(off + sizeof(float) * (size_t)w.max_seq_chunks * q_per_seq * num_q_heads * head_dim, 256);
+  w.counters = off;
+  off = align_up(off + sizeof(int32_t) * (size_t)batch * num_kv_heads * row_groups(q_per_seq, num_q_heads, num_kv_heads), 256);
   w.total_bytes = off;
   return w;
 }

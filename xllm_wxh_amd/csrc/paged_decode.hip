@@ -7,8 +7,9 @@
 //   decode_*_kernel      one workgroup per (sequence chunk, kv head, row group): its waves stream
 //                        the chunk's K and V once; a sequence that is a single chunk gets its
 //                        output rows written directly, otherwise a normalised partial +
-//                        log2-sum-exp is written
-//   decode_merge_kernel  combines the partials of the sequences that were split
+//                        log2-sum-exp is written, and (16-row MFMA kernel) the workgroup that finishes
+//                        the last chunk of a (sequence, kv head) combines its partials
+//   decode_merge_kernel  combines the partials of the sequences that were split (the other kernels)
 // When the host-side length hints show that no sequence needs splitting, only the middle one is
 // launched: a work item is then (sequence, kv head, row group) and needs no schedule.
 //
@@ -49,6 +50,7 @@ struct DecodeParams {
   SeqChunk* seq_chunks;
   float* partial_lse;
   float* partial_out;
+  int32_t* counters;  // per (sequence, kv head, row group): chunks finished so far (fused merge)
   int64_t q_token_stride;
   int64_t out_token_stride;
   int64_t stride_block;
@@ -81,6 +83,8 @@ struct DecodeParams {
   int32_t direct_single;  // the attention kernel writes the output rows of single-chunk sequences itself
   int32_t implicit_plan;  // nothing is split and nothing is merged: item = (sequence, kv head, row group),
                           // lengths come straight from the inputs and no plan kernel runs
+  int32_t fused_merge;    // the attention kernel merges a split sequence itself: the workgroup that finishes the
+                          // last chunk of a (sequence, kv head, row group) combines the partials
   int32_t q_dtype;
   float scale_log2;  // sm_scale * log2(e)
 };
@@ -108,6 +112,12 @@ __global__ void __launch_bounds__(64) decode_plan_kernel(DecodeParams p) {
   __shared__ int tail_fill[64];
   tail_hist[lane] = 0;
   tail_fill[lane] = 0;
+  // the finished-chunk counters of the fused merge start every step at zero (the attention kernel
+  // leaves them at zero again, so one plan serves every layer of the step)
+  if (p.fused_merge) {
+    const int ncounters = p.batch * p.num_kv_heads * p.row_groups;
+    for (int i = lane; i < ncounters; i += 64) p.counters[i] = 0;
+  }
 
   // 1. kv lengths, their sum and their maximum.
   long long total = 0;
@@ -327,24 +337,24 @@ __device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it)
 
 constexpr int kMergeRowsPerBlock = 4;
 
-template <int Q_DT>
-__global__ void __launch_bounds__(64 * kMergeRowsPerBlock) decode_merge_kernel(DecodeParams p) {
+// Partials that another workgroup of the same launch wrote are stored and loaded as device-scope
+// atomics (relaxed): such accesses go past the caches that are not coherent across the XCDs, so the
+// fused merge needs no cache write-back or invalidation, only the ordering its barrier and counter give.
+__device__ inline void store_coherent(float* ptr, float v) {
+  __hip_atomic_store(ptr, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <bool COHERENT>
+__device__ inline float load_partial(const float* ptr) {
+  if (COHERENT) return __hip_atomic_load(ptr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return *ptr;
+}
+
+// One wave merges the partials of output row (sequence b, query token j, head): all 64 lanes call.
+template <int Q_DT, bool COHERENT>
+__device__ inline void merge_row(const DecodeParams& p, int b, int j, int head, int q0, int lane) {
   const int nhq = p.n * p.num_q_heads;
-  const int64_t row = (int64_t)blockIdx.x * kMergeRowsPerBlock + (threadIdx.x >> 6);
-  const int lane = threadIdx.x & 63;
-  if (row >= (int64_t)p.batch * nhq) return;
-  const int b = (int)(row / nhq);
-  int q0 = b * p.n, nb = p.n;
-  if (p.q_indptr != nullptr) {
-    q0 = p.q_indptr[b];
-    nb = min(p.n, p.q_indptr[b + 1] - q0);
-  }
+  const int rem = j * p.num_q_heads + head;
   const int cnt = p.num_chunks[b];
-  if (p.direct_single && cnt == 1) return;  // already written by the attention kernel
-  const int rem = (int)(row - (int64_t)b * nhq);  // j * Hq + head
-  const int j = rem / p.num_q_heads;
-  if (j >= nb) return;
-  const int head = rem - j * p.num_q_heads;
   const int D = p.head_dim;
   const float neg_inf = -INFINITY;
   const int f0 = p.full_prefix[b];
@@ -354,11 +364,13 @@ __global__ void __launch_bounds__(64 * kMergeRowsPerBlock) decode_merge_kernel(D
 
   // 1. maximum and denominator over the chunks' log-sum-exps
   float m = neg_inf;
-  for (int i = lane; i < cnt; i += 64) m = fmaxf(m, p.partial_lse[partial_row(i)]);
+  for (int i = lane; i < cnt; i += 64) m = fmaxf(m, load_partial<COHERENT>(p.partial_lse + partial_row(i)));
   m = wave_max(m);
   const float m_safe = m == neg_inf ? 0.0f : m;
   float ssum = 0.0f;
-  for (int i = lane; i < cnt; i += 64) ssum += __builtin_amdgcn_exp2f(p.partial_lse[partial_row(i)] - m_safe);
+  for (int i = lane; i < cnt; i += 64) {
+    ssum += __builtin_amdgcn_exp2f(load_partial<COHERENT>(p.partial_lse + partial_row(i)) - m_safe);
+  }
   ssum = wave_sum(ssum);
 
   // 2. weighted sum of the partial rows: lane covers columns lane, lane + 64, ... (head_dim <= 256)
@@ -371,11 +383,11 @@ __global__ void __launch_bounds__(64 * kMergeRowsPerBlock) decode_merge_kernel(D
     for (int u = 0; u < kUnroll; ++u) {
       const int i = min(i0 + u, cnt - 1);
       const int64_t prow = partial_row(i);
-      const float li = p.partial_lse[prow];
+      const float li = load_partial<COHERENT>(p.partial_lse + prow);
       w[u] = (i0 + u < cnt && li != neg_inf) ? __builtin_amdgcn_exp2f(li - m_safe) : 0.0f;
       const float* po = p.partial_out + prow * D;
 #pragma unroll
-      for (int k = 0; k < 4; ++k) v[u][k] = lane + 64 * k < D ? po[lane + 64 * k] : 0.0f;
+      for (int k = 0; k < 4; ++k) v[u][k] = lane + 64 * k < D ? load_partial<COHERENT>(po + lane + 64 * k) : 0.0f;
     }
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
@@ -396,6 +408,58 @@ __global__ void __launch_bounds__(64 * kMergeRowsPerBlock) decode_merge_kernel(D
   for (int k = 0; k < 4; ++k) {
     const int d = lane + 64 * k;
     if (d < D) Elem<Q_DT>::store(p.out, obase + d, o[k] * inv);
+  }
+}
+
+template <int Q_DT>
+__global__ void __launch_bounds__(64 * kMergeRowsPerBlock) decode_merge_kernel(DecodeParams p) {
+  const int nhq = p.n * p.num_q_heads;
+  const int64_t row = (int64_t)blockIdx.x * kMergeRowsPerBlock + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= (int64_t)p.batch * nhq) return;
+  const int b = (int)(row / nhq);
+  int q0 = b * p.n, nb = p.n;
+  if (p.q_indptr != nullptr) {
+    q0 = p.q_indptr[b];
+    nb = min(p.n, p.q_indptr[b + 1] - q0);
+  }
+  if (p.direct_single && p.num_chunks[b] == 1) return;  // already written by the attention kernel
+  const int rem = (int)(row - (int64_t)b * nhq);  // j * Hq + head
+  const int j = rem / p.num_q_heads;
+  if (j >= nb) return;
+  merge_row<Q_DT, false>(p, b, j, rem - j * p.num_q_heads, q0, lane);
+}
+
+// Fused merge, called by every thread of a workgroup after it has written the partials of its item:
+// the workgroup that finishes the last chunk of a (sequence, kv head, row group) combines that row
+// group's partials, so no merge kernel follows.  Every wave waits until its partial stores (coherent,
+// see store_coherent) have completed, the workgroup meets, and one thread counts the chunk in with a
+// device-scope atomic; the workgroup that reads count - 1 knows that every other chunk's stores
+// completed before its increment, resets the counter for the next launch and reads the partials with
+// coherent loads.  (Device-scope fences instead — cache write-back and invalidation on every
+// workgroup — made an 8 x 8192-token step three times slower.)
+template <int Q_DT>
+__device__ inline void merge_if_last(const DecodeParams& p, const Item& it, int* lds_flag) {
+  if (!p.fused_merge || p.implicit_plan) return;
+  const int cnt = p.num_chunks[it.b];
+  if (p.direct_single && cnt == 1) return;  // written directly
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's stores have completed
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int32_t* c = p.counters + ((int64_t)it.b * p.num_kv_heads + it.hk) * p.row_groups + it.rg;
+    const int old = __hip_atomic_fetch_add(c, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const int last = old == cnt - 1;
+    if (last) __hip_atomic_store(c, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    *lds_flag = last;
+  }
+  __syncthreads();
+  if (!*lds_flag) return;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nwaves = blockDim.x >> 6;
+  const int first = it.rg * p.rows_per_item;
+  const int end = min(first + p.rows_per_item, it.n * p.group);
+  for (int r = first + wave; r < end; r += nwaves) {
+    const int j = r / p.group;
+    merge_row<Q_DT, true>(p, it.b, j, it.hk * p.group + (r - j * p.group), it.q0, lane);
   }
 }
 
@@ -1154,6 +1218,13 @@ __device__ inline void finish_item(const DecodeParams& p, const Item& it, RowTil
         ob[4 + e] = (decltype(ob[0] + ob[0]))o_hi[e];
       }
       *(decltype(ob)*)((uint16_t*)p.out + tok * p.out_token_stride + (int64_t)head * kD + d0) = ob;
+    } else if (p.fused_merge) {
+      float* po = p.partial_out + prow * kD + d0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        store_coherent(po + e, o_lo[e]);
+        store_coherent(po + 4 + e, o_hi[e]);
+      }
     } else {
       float* po = p.partial_out + prow * kD + d0;
       *(f32x4*)(po) = o_lo;
@@ -1163,6 +1234,8 @@ __device__ inline void finish_item(const DecodeParams& p, const Item& it, RowTil
   if (tw == 0 && kg == 0) {
     if (single) {
       if (p.lse != nullptr) p.lse[tok * p.num_q_heads + head] = lse2;
+    } else if (p.fused_merge) {
+      store_coherent(p.partial_lse + prow, lse2);
     } else {
       p.partial_lse[prow] = lse2;
     }
@@ -1193,6 +1266,7 @@ template <int KV_DT, int TOK>
 __global__ void __launch_bounds__(64 * kWaves, decode_waves_per_simd(KV_DT, TOK)) decode_mfma_d128_kernel(DecodeParams p) {
   __shared__ __attribute__((aligned(16))) uint8_t lds_all[kWaves * kLdsTile];
   __shared__ float lds_ml[kWaves * 16 * 2];  // (running max, denominator) per wave and query row
+  __shared__ int lds_last;
 
   constexpr int kT = tile_tokens_of(TOK);  // tokens per tile
   constexpr int kH = half_tokens_of(TOK);  // tokens from the tile's first half to its second
@@ -1279,6 +1353,7 @@ __global__ void __launch_bounds__(64 * kWaves, decode_waves_per_simd(KV_DT, TOK)
     }
   }
   finish_item<KV_DT, TOK, kWaves>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, 0, wave, lane, 0);
+  merge_if_last<qf16_of(KV_DT) ? XLLM_HIP_FP16 : XLLM_HIP_BF16>(p, it, &lds_last);
 }
 
 template <int KV_DT, int TOK>
@@ -1807,6 +1882,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
   p.seq_chunks = (SeqChunk*)(ws + w.seq_chunks);
   p.partial_lse = (float*)(ws + w.partial_lse);
   p.partial_out = (float*)(ws + w.partial_out);
+  p.counters = (int32_t*)(ws + w.counters);
   p.q_token_stride = a->q_token_stride;
   p.out_token_stride = a->out_token_stride;
   p.stride_block = c->stride_block;
@@ -1844,6 +1920,11 @@ static int fill_params(const xllm_hip_kv_cache* c,
   // pick covers the longest sequence, no sequence is split: the plan is told never to split
   // (which stays correct even if the hints were wrong) and the merge launch is dropped.
   p.direct_single = is_mfma(variant) ? 1 : 0;
+  // Up to 16 rows per kv head the attention kernel merges split sequences itself (no merge launch).
+  // With more rows the work of a merge is large enough to want the whole GPU: fused into the 32-row
+  // kernel it made the int8 verify workload 7 % slower (401 against 377 us), the tails of all row
+  // groups ending together.
+  p.fused_merge = is_mfma(variant) && p.rows <= 16 ? 1 : 0;
   p.fixed_chunk = 0;
   if (p.direct_single && a->max_seq_len > 0 && a->total_kv_len > 0 &&
       a->max_seq_len <= choose_chunk(a->total_kv_len, a->max_seq_len, p.batch, p.num_kv_heads, p.row_groups,
@@ -2051,7 +2132,7 @@ extern "C" int xllm_hip_paged_decode_run_timed(const xllm_hip_kv_cache* cache,
   if (ev_end != nullptr && hipEventRecord((hipEvent_t)ev_end, st) != hipSuccess) {
     return fail(XLLM_HIP_RUNTIME_ERROR, "hipEventRecord(ev_end) failed");
   }
-  if (p.implicit_plan) return XLLM_HIP_OK;  // nothing was split: the outputs are final
+  if (p.implicit_plan || p.fused_merge) return XLLM_HIP_OK;  // nothing was split, or the attention kernel merged
 
   const int64_t rows = (int64_t)p.batch * p.n * p.num_q_heads;
   const unsigned mgrid = (unsigned)((rows + kMergeRowsPerBlock - 1) / kMergeRowsPerBlock);
