@@ -340,6 +340,70 @@ def test_attention_impl_chunked_prefill_step(gpu, shim, kv):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["int8", "fp8"])
+def test_prefill_chunks_over_a_quantised_cache_take_the_dense_route(gpu, shim, kind):
+    """Large chunks over a 1-byte cache: AttentionImpl dequantises the cached ranges into a dense copy
+    and attends that (the reference's MLU order of operations); same result as attending the
+    quantised cache in place, and the oracle's."""
+    print("case shim dense prefill route", kind, flush=True)
+    Hq, Hkv, D, bs = 32, 8, 128, 16
+    lens = np.array([700, 300, 1031, 129], np.int32)      # kv lengths including this step's tokens
+    q_counts = np.array([300, 300, 131, 129], np.int32)   # rows per kv head: 4 * 215 on average
+    B, T = len(lens), int(q_counts.sum())
+    rng = np.random.default_rng(17)
+    need = (lens + bs - 1) // bs
+    nblocks = int(need.sum()) + 2
+    perm = rng.permutation(nblocks - 1) + 1
+    lists, o = [], 0
+    for b in range(B):
+        lists.append(perm[o:o + need[b]].astype(np.int32))
+        o += int(need[b])
+    table = orc.pad_block_tables(lists)
+    slots = np.concatenate([orc.kv_cache_slots(lists[b], bs, int(lens[b] - q_counts[b]), int(lens[b]))
+                            for b in range(B)]).astype(np.int32)
+    g = torch.Generator().manual_seed(18)
+    kf = torch.randn(nblocks, Hkv, bs, D, generator=g)
+    vf = torch.randn(nblocks, Hkv, bs, D, generator=g)
+    qkv = torch.randn(T, (Hq + 2 * Hkv) * D, generator=g).to(torch.bfloat16)
+    q = qkv[:, : Hq * D]
+    k_new = qkv[:, Hq * D:(Hq + Hkv) * D].float().numpy().reshape(T, Hkv, D)
+    v_new = qkv[:, (Hq + Hkv) * D:].float().numpy().reshape(T, Hkv, D)
+    qk, sk = orc.quantize_per_token_head(kf.numpy(), kind)
+    qv, sv = orc.quantize_per_token_head(vf.numpy(), kind)
+    tdt = torch.int8 if kind == "int8" else torch.float8_e4m3fn
+
+    def fresh_cache():
+        return shim.KVCache(torch.from_numpy(qk.view(np.uint8).copy()).view(tdt).to(gpu),
+                            torch.from_numpy(qv.view(np.uint8).copy()).view(tdt).to(gpu),
+                            torch.from_numpy(sk.copy()).to(gpu), torch.from_numpy(sv.copy()).to(gpu))
+
+    qk2, qv2, sk2, sv2 = qk.copy(), qv.copy(), sk.copy(), sv.copy()
+    orc.quant_to_paged_cache(slots, k_new, v_new, qk2, qv2, sk2, sv2, kind, "HND")
+    k_ref, v_ref = orc.dequantize(qk2, sk2, kind), orc.dequantize(qv2, sv2, kind)
+    q_indptr = np.concatenate([[0], np.cumsum(q_counts)]).astype(np.int32)
+    scale = 1.0 / float(np.sqrt(D))
+    ref, _ = orc.paged_decode_ragged(q.float().numpy().reshape(T, Hq, D), k_ref, v_ref, table, lens, q_indptr, scale)
+    i32 = lambda a: torch.tensor(np.asarray(a), dtype=torch.int32, device=gpu)
+    md = shim.build_decode_metadata(i32(q_indptr), i32(np.concatenate([[0], np.cumsum(lens)])), i32(slots), i32(table),
+                                    int(q_counts.max()), int(lens.max()), int(lens.sum()))
+    md.is_chunked_prefill = True
+    outs = []
+    for rows in (128, 0):  # dense route, then in place
+        attn = shim.AttentionImpl(Hq, D, scale, Hkv, -1)
+        attn.set_prefill_dequant_rows(rows)
+        qkv_d = qkv.to(gpu)
+        out, _ = attn.forward(md, qkv_d[:, : Hq * D], qkv_d[:, Hq * D:(Hq + Hkv) * D], qkv_d[:, (Hq + Hkv) * D:],
+                              fresh_cache())
+        torch.cuda.synchronize()
+        outs.append(out.float().cpu().numpy().reshape(T, Hq, D))
+        err = float(np.abs(outs[-1] - ref).max())
+        print("   dequant rows %d: err %.3e" % (rows, err), flush=True)
+        assert err <= 5e-2
+    # the dense copy is the dequantised cache rounded to bf16: the two routes differ by that rounding only
+    assert float(np.abs(outs[0] - outs[1]).max()) <= 2e-2
+
+
+@pytest.mark.gpu
 def test_forward_qkv_replays_under_hip_graph(gpu, shim):
     """AttentionImpl::forward_qkv (norm + rotation + KV write, then decode) captured in a HIP graph and
     replayed on changing persistent inputs; total_kv_len = 0 in the metadata keeps host-side lengths

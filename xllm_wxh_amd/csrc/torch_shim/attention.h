@@ -41,6 +41,13 @@ class AttentionImpl {
                                                                        double eps,
                                                                        KVCache& kv_cache);
 
+  // Prefill chunks over a quantised cache: from this many query rows per kv head on (averaged over
+  // the step's sequences) the cached ranges are first dequantised into a dense 16-bit copy, which the
+  // 128-row kernel then attends — the order of operations of the reference's MLU layer
+  // (xllm/core/layers/mlu/attention.cpp:179-228).  Below it the quantised cache is attended in place.
+  // 0 disables the dense route.
+  void set_prefill_dequant_rows(int64_t rows) { prefill_dequant_rows_ = rows; }
+
  private:
   void decoder_forward(const AttentionMetadata& attn_metadata,
                        torch::Tensor& query,
@@ -55,6 +62,7 @@ class AttentionImpl {
   float scale_;
   int64_t num_kv_heads_;
   int64_t sliding_window_;
+  int64_t prefill_dequant_rows_ = 128;
 };
 
 }  // namespace xllm::layer

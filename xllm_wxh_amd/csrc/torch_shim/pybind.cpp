@@ -140,6 +140,7 @@ PYBIND11_MODULE(_xllm_hip_torch, m) {
 
   py::class_<AttentionImpl>(m, "AttentionImpl")
       .def(py::init<int64_t, int64_t, float, int64_t, int64_t>())
+      .def("set_prefill_dequant_rows", &AttentionImpl::set_prefill_dequant_rows)
       .def("forward", [](AttentionImpl& self, const AttentionMetadata& md, torch::Tensor query, torch::Tensor key,
                          torch::Tensor value, KVCache& kv) { return self.forward(md, query, key, value, kv); })
       .def("forward_qkv", [](AttentionImpl& self, const AttentionMetadata& md, torch::Tensor positions,
