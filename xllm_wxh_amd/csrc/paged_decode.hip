@@ -362,42 +362,76 @@ __device__ inline void merge_row(const DecodeParams& p, int b, int j, int head, 
   const int tail_slot = p.hdr->total_full + p.tail_prefix[b];
   auto partial_row = [&](int i) { return (int64_t)(i < nf ? f0 + i : tail_slot) * nhq + rem; };
 
-  // 1. maximum and denominator over the chunks' log-sum-exps
-  float m = neg_inf;
-  for (int i = lane; i < cnt; i += 64) m = fmaxf(m, load_partial<COHERENT>(p.partial_lse + partial_row(i)));
-  m = wave_max(m);
-  const float m_safe = m == neg_inf ? 0.0f : m;
-  float ssum = 0.0f;
-  for (int i = lane; i < cnt; i += 64) {
-    ssum += __builtin_amdgcn_exp2f(load_partial<COHERENT>(p.partial_lse + partial_row(i)) - m_safe);
-  }
-  ssum = wave_sum(ssum);
-
-  // 2. weighted sum of the partial rows: lane covers columns lane, lane + 64, ... (head_dim <= 256)
+  // Columns lane, lane + 64, ... of the output row (head_dim <= 256), summed over the chunks kUnroll
+  // at a time: their loads are all issued before the first is used.  `weight(i)` is chunk i's factor.
   float o[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-  // kUnroll chunks at a time: their loads are all issued before the first is used
-  auto add_chunks = [&](int i0, auto unroll) {
-    constexpr int kUnroll = decltype(unroll)::value;
-    float w[kUnroll], v[kUnroll][4];
+  auto load_rows = [&](int i0, auto unroll, float (&v)[decltype(unroll)::value][4]) {
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-      const int i = min(i0 + u, cnt - 1);
-      const int64_t prow = partial_row(i);
-      const float li = load_partial<COHERENT>(p.partial_lse + prow);
-      w[u] = (i0 + u < cnt && li != neg_inf) ? __builtin_amdgcn_exp2f(li - m_safe) : 0.0f;
-      const float* po = p.partial_out + prow * D;
+    for (int u = 0; u < decltype(unroll)::value; ++u) {
+      const float* po = p.partial_out + partial_row(min(i0 + u, cnt - 1)) * D;
 #pragma unroll
       for (int k = 0; k < 4; ++k) v[u][k] = lane + 64 * k < D ? load_partial<COHERENT>(po + lane + 64 * k) : 0.0f;
     }
+  };
+  auto add_rows = [&](int i0, auto unroll, const float (&v)[decltype(unroll)::value][4], auto weight) {
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
+    for (int u = 0; u < decltype(unroll)::value; ++u) {
+      const float w = i0 + u < cnt ? weight(i0 + u) : 0.0f;
 #pragma unroll
-      for (int k = 0; k < 4; ++k) o[k] += w[u] != 0.0f ? w[u] * v[u][k] : 0.0f;  // an empty chunk's row may hold anything
+      for (int k = 0; k < 4; ++k) o[k] += w != 0.0f ? w * v[u][k] : 0.0f;  // an empty chunk's row may hold anything
     }
   };
-  int i0 = 0;
-  for (; i0 + 16 <= cnt; i0 += 16) add_chunks(i0, std::integral_constant<int, 16>{});
-  for (; i0 < cnt; i0 += 4) add_chunks(i0, std::integral_constant<int, 4>{});
+  typedef std::integral_constant<int, 8> Eight;
+  typedef std::integral_constant<int, 4> Four;
+  float m, ssum;
+  if (cnt <= 256) {
+    // The usual case.  Each lane keeps the log-sum-exps of chunks lane, lane + 64, ... in registers and
+    // the first rows are already on their way while the maximum and the denominator are reduced:
+    // two memory round trips for a row instead of four.
+    float l[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int i = lane + 64 * q;
+      l[q] = i < cnt ? load_partial<COHERENT>(p.partial_lse + partial_row(i)) : neg_inf;
+    }
+    float first[8][4];
+    load_rows(0, Eight{}, first);
+    m = wave_max(fmaxf(fmaxf(l[0], l[1]), fmaxf(l[2], l[3])));
+    const float m_safe = m == neg_inf ? 0.0f : m;
+    float e[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) e[q] = __builtin_amdgcn_exp2f(l[q] - m_safe);  // 2^-inf = 0: empty or absent chunk
+    ssum = wave_sum(e[0] + e[1] + e[2] + e[3]);
+    auto weight = [&](int i) {
+      const int q = i >> 6;
+      const float mine = q == 0 ? e[0] : q == 1 ? e[1] : q == 2 ? e[2] : e[3];
+      return __shfl(mine, i & 63);
+    };
+    add_rows(0, Eight{}, first, weight);
+    for (int i0 = 8; i0 < cnt; i0 += 8) {
+      float v[8][4];
+      load_rows(i0, Eight{}, v);
+      add_rows(i0, Eight{}, v, weight);
+    }
+  } else {
+    m = neg_inf;
+    for (int i = lane; i < cnt; i += 64) m = fmaxf(m, load_partial<COHERENT>(p.partial_lse + partial_row(i)));
+    m = wave_max(m);
+    const float m_safe = m == neg_inf ? 0.0f : m;
+    ssum = 0.0f;
+    for (int i = lane; i < cnt; i += 64) {
+      ssum += __builtin_amdgcn_exp2f(load_partial<COHERENT>(p.partial_lse + partial_row(i)) - m_safe);
+    }
+    ssum = wave_sum(ssum);
+    auto weight = [&](int i) {
+      return __builtin_amdgcn_exp2f(load_partial<COHERENT>(p.partial_lse + partial_row(i)) - m_safe);
+    };
+    for (int i0 = 0; i0 < cnt; i0 += 4) {
+      float v[4][4];
+      load_rows(i0, Four{}, v);
+      add_rows(i0, Four{}, v, weight);
+    }
+  }
   const float inv = ssum > 0.0f ? 1.0f / ssum : 0.0f;
   const int64_t tok = (int64_t)q0 + j;
   if (p.lse != nullptr && lane == 0) {
