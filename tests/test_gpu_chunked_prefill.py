@@ -151,3 +151,29 @@ def test_garbage_past_the_sequence_end_does_not_reach_the_many_row_kernel(gpu, D
     got = out.float().cpu().numpy()
     assert not np.isnan(got).any()
     assert float(np.abs(got - ref).max()) <= 1.2e-2
+
+
+@pytest.mark.parametrize("g,n,D,bs", [(8, 5, 128, 16), (8, 8, 128, 128), (4, 9, 128, 16), (16, 4, 64, 32), (11, 3, 128, 16)])
+@pytest.mark.parametrize("qdt", ["bf16", "fp16"])
+def test_thirty_three_to_sixty_four_rows(gpu, g, n, D, bs, qdt):
+    """33 to 64 query rows per kv head over a 16-bit cache (speculative verify of five to eight draft
+    tokens at eight heads per kv head): the many-row kernel with half of its rows absent.  Sequences
+    long enough to be split, shorter than the draft count plus one tile, a sliding window."""
+    print("case 33-64 rows", g, n, D, bs, qdt, flush=True)
+    assert 32 < g * n <= 64
+    kv = "bf16" if qdt == "bf16" else "fp16"
+    c = Case(4, 4 * g, 4, D, bs, [9000, n, 517, 40], n=n, kv=kv, qdt=qdt, seed=51)
+    ref, lse_ref = c.oracle()
+    out, lse = c.run()
+    assert not torch.isnan(out.float()).any()
+    assert float(np.abs(out.float().cpu().numpy() - ref).max()) <= 1.2e-2
+    fin = np.isfinite(lse_ref)
+    assert np.allclose(lse.cpu().numpy()[fin], lse_ref[fin], atol=2e-2)
+    ref_w, _ = c.oracle(301)
+    out_w, _ = c.run(301)
+    assert float(np.abs(out_w.float().cpu().numpy() - ref_w).max()) <= 1.2e-2
+    # different numbers of query tokens per sequence, at most n
+    counts = [n, 1, max(1, n - 2), 0]
+    out_r, _, ref_r, _, _ = _run(c, counts, n) if qdt == "bf16" else (None, None, None, None, None)
+    if out_r is not None:
+        assert float(np.abs(out_r - ref_r).max()) <= 1.2e-2
