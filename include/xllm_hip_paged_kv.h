@@ -228,7 +228,11 @@ int xllm_hip_paged_decode_plan(const xllm_hip_kv_cache* cache,
                                size_t workspace_bytes,
                                xllm_hip_stream_t stream);
 
-/* Attention proper; requires a schedule built by xllm_hip_paged_decode_plan in `workspace`. */
+/* Attention proper; requires a schedule built by xllm_hip_paged_decode_plan in `workspace`.
+ * Split sequences leave normalised partial results in the workspace; up to 16 query rows per kv
+ * head the attention kernel combines them itself (the workgroup that finishes a sequence's last
+ * chunk; it counts in counters that the plan zeroes and every run leaves at zero), otherwise a merge
+ * kernel follows.  Two runs must not share a workspace concurrently. */
 int xllm_hip_paged_decode_run(const xllm_hip_kv_cache* cache,
                               const xllm_hip_decode_args* args,
                               void* workspace,
@@ -238,7 +242,7 @@ int xllm_hip_paged_decode_run(const xllm_hip_kv_cache* cache,
 /*
  * xllm_hip_paged_decode_run that also records two caller-created hipEvent_t on `stream`: ev_begin
  * just before the attention kernel (the launch that streams the KV cache) and ev_end just after
- * it, before the merge.  A measurement hook for benchmarks; it has no counterpart in the
+ * it, before the merge kernel if one follows.  A measurement hook for benchmarks; it has no counterpart in the
  * reference.  Either event may be NULL.
  */
 int xllm_hip_paged_decode_run_timed(const xllm_hip_kv_cache* cache,
