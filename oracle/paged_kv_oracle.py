@@ -8,7 +8,8 @@ Every function restates one piece of the reference (paths relative to the xLLM
 tree); how each one is pinned is listed beside it:
 
   fnv1a64 / SplitMix64 / seeded_tensor   xllm/core/layers/common/tests/tests_utils.cpp:159-272
-      pinned by the published FNV-1a and SplitMix64 test vectors.
+      pinned by the published FNV-1a and SplitMix64 test vectors and by the reference's own statistics of
+      a seeded float32 tensor (layers/common/tests/deepseek_v2_decoder_layer_tests.cpp:1594-1599).
   kv_cache_slots                         xllm/core/framework/request/sequence_kv_state.cpp:120-134
   calc_slot_id / calc_kv_len             xllm/core/runtime/spec_input_builder.cpp:76-109
   build_paged_kv_csr / pad_block_tables  xllm/core/framework/batch/batch_input_builder.cpp:438-494,565-582

@@ -39,6 +39,16 @@ def test_seeded_tensor_matches_scalar_generator():
     np.testing.assert_array_equal(b, np.array([x & 1 for x in u], bool))
 
 
+def test_seeded_tensor_reference_statistics():
+    """The reference's own known answer for a seeded tensor: min / max / sum of a float32 one."""
+    g = GOLDEN["seeded_tensor_stats"]
+    t = orc.seeded_tensor(g["key"], tuple(g["shape"]), np.float32).astype(np.float64)
+    for got, want in ((t.min(), g["expected_min"]), (t.max(), g["expected_max"]), (t.sum(), g["expected_sum"])):
+        assert abs(got - want) <= g["atol"] + g["rtol"] * abs(want), (got, want)
+    # tighter than the reference asks: the golden values are the true ones rounded to 3-4 digits
+    assert abs(t.min() - g["expected_min"]) < 5e-7 and abs(t.sum() - g["expected_sum"]) < 0.1
+
+
 def test_batch_test_known_answers():
     g = GOLDEN["batch_test_basic"]
     bs = g["block_size"]
