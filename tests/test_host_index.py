@@ -61,6 +61,23 @@ def test_spec_rows_known_answers(shim, name):
         assert rows.block_tables[0] == rows.block_tables[2] == g["block_tables"][0]
 
 
+@pytest.mark.parametrize("name", ["spec_first_decode_rows", "spec_rows_with_offsets"])
+def test_spec_rows_with_their_own_offsets(shim, name):
+    g = GOLDEN[name]
+    cu = np.concatenate([[0], np.cumsum(g["kv_seq_lens"])]).tolist()
+    rows = shim.decode_rows(g["positions"], cu, g["block_tables"], g["block_size"], [tuple(r) for r in g["rows"]])
+    assert rows.positions == g["expected_positions"]
+    assert rows.new_cache_slots == g["expected_new_cache_slots"]
+    assert rows.kv_seq_lens == g["expected_kv_seq_lens"]
+    assert len(rows.block_tables) == len(g["rows"])
+    # and the oracle's restatement
+    for (seq, off), pos, slot, kv in zip(g["rows"], g["expected_positions"], g["expected_new_cache_slots"],
+                                         g["expected_kv_seq_lens"]):
+        assert g["positions"][seq] + off == pos
+        assert orc.calc_slot_id(pos, g["block_tables"][seq], g["block_size"]) == slot
+        assert orc.calc_kv_len(cu, seq, off) == kv
+
+
 def test_minimal_decode_metadata(shim):
     g = GOLDEN["minimal_decode_metadata"]
     batch = shim.DecodeBatchInputs(g["block_size"])

@@ -146,6 +146,23 @@ struct ExpandedDecodeRows {
   int32_t kv_max_seq_len = 0;
 };
 
+// One row of a speculative step (append_decode_row, xllm/core/runtime/spec_input_builder.cpp:112-147):
+// sequence seq_id at position positions[seq_id] + position_offset, appended to `out`.
+inline void append_decode_row(const std::vector<int32_t>& positions, const std::vector<int32_t>& kv_seq_lens_cumulative,
+                              const std::vector<std::vector<int32_t>>& block_tables, int32_t block_size, int32_t seq_id,
+                              int32_t position_offset, ExpandedDecodeRows& out) {
+  require(seq_id >= 0, "invalid seq_id");
+  if ((size_t)seq_id >= positions.size() || (size_t)seq_id >= block_tables.size()) throw std::out_of_range("seq_id out of range");
+  const int32_t pos = positions[seq_id] + position_offset;
+  require(pos >= 0, "invalid decode position");
+  out.positions.push_back(pos);
+  out.new_cache_slots.push_back(calc_slot_id(pos, block_tables[seq_id], block_size));
+  const int32_t kv_len = calc_kv_len(kv_seq_lens_cumulative, seq_id, position_offset);
+  out.kv_max_seq_len = std::max(out.kv_max_seq_len, kv_len);
+  out.kv_seq_lens.push_back(kv_len);
+  out.block_tables.push_back(block_tables[seq_id]);
+}
+
 inline ExpandedDecodeRows expand_decode_rows(const std::vector<int32_t>& positions,
                                              const std::vector<int32_t>& kv_seq_lens_cumulative,
                                              const std::vector<std::vector<int32_t>>& block_tables, int32_t block_size,
@@ -154,14 +171,7 @@ inline ExpandedDecodeRows expand_decode_rows(const std::vector<int32_t>& positio
   ExpandedDecodeRows out;
   for (size_t s = 0; s < positions.size(); ++s) {
     for (const int32_t off : position_offsets) {
-      const int32_t pos = positions[s] + off;
-      require(pos >= 0, "invalid decode position");
-      out.positions.push_back(pos);
-      out.new_cache_slots.push_back(calc_slot_id(pos, block_tables[s], block_size));
-      const int32_t kv_len = calc_kv_len(kv_seq_lens_cumulative, (int32_t)s, off);
-      out.kv_max_seq_len = std::max(out.kv_max_seq_len, kv_len);
-      out.kv_seq_lens.push_back(kv_len);
-      out.block_tables.push_back(block_tables[s]);
+      append_decode_row(positions, kv_seq_lens_cumulative, block_tables, block_size, (int32_t)s, off, out);
     }
   }
   return out;

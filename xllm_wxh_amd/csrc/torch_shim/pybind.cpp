@@ -137,6 +137,13 @@ PYBIND11_MODULE(_xllm_hip_torch, m) {
       .def_readonly("block_tables", &hi::ExpandedDecodeRows::block_tables)
       .def_readonly("kv_max_seq_len", &hi::ExpandedDecodeRows::kv_max_seq_len);
   m.def("expand_decode_rows", &hi::expand_decode_rows);
+  m.def("decode_rows", [](const std::vector<int32_t>& positions, const std::vector<int32_t>& kv_cu,
+                          const std::vector<std::vector<int32_t>>& block_tables, int32_t block_size,
+                          const std::vector<std::pair<int32_t, int32_t>>& rows) {
+    hi::ExpandedDecodeRows out;
+    for (const auto& r : rows) hi::append_decode_row(positions, kv_cu, block_tables, block_size, r.first, r.second, out);
+    return out;
+  });
 
   py::class_<AttentionImpl>(m, "AttentionImpl")
       .def(py::init<int64_t, int64_t, float, int64_t, int64_t>())
