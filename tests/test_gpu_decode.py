@@ -538,3 +538,25 @@ def test_split_sequences_merge_in_the_attention_kernel_repeatably(gpu, kv, n):
     for i in range(40):
         out, lse = case.run(workspace=ws, plan=(i == 0))  # one plan, many runs: the counters reset themselves
         assert torch.equal(out, first) and torch.equal(lse, lse_first), i
+
+
+@pytest.mark.parametrize("kv", ["bf16", "fp8"])
+@pytest.mark.parametrize("name,lens", [
+    ("equal lengths, a few chunks each", [6000] * 3),
+    ("equal lengths, one workgroup per (sequence, head) is enough", [1100] * 24),
+    ("one long sequence among short ones", [30000, 700, 900, 650, 100]),
+    ("lengths so close that a split would only shed short tails", [2500 + 16 * i for i in range(20)]),
+    ("ragged, as many items as the budget takes", [4000, 2500, 900, 3300, 1700, 2900]),
+])
+def test_small_batch_chunk_choices(gpu, kv, name, lens):
+    """Small batches are cut for one workgroup per CU rather than for every slot; each branch of that
+    choice (equal lengths, the item budget, the parallelism floor, the short-tail rule) against the
+    oracle, with and without the host's length hints."""
+    print("case small batch", kv, name, flush=True)
+    case = Case(len(lens), 32, 8, 128, 16, lens, kv=kv, seed=57)
+    ref, lse_ref = case.oracle()
+    out, lse = case.run()
+    assert max_abs_err(out, ref) <= (REG_TOL_QUANT if kv == "fp8" else REG_TOL)
+    assert lse_err(lse, lse_ref) <= LSE_TOL
+    out_h, _ = case.run(hints=True)
+    assert torch.equal(out, out_h)

@@ -35,19 +35,51 @@ constexpr int kPrefillMinRows = 32;
 #define XLLM_HIP_HD
 #endif
 
-// Chunk size for a batch whose kv lengths sum to `total` with maximum `max_len`: split so that
-// about `target` work items exist — a quarter more when the batch is ragged (longest sequence above
-// 1.5x the mean): the tail chunks then differ in size, and although they are dispatched longest
-// first a little slack helps the last ones pack.  (Measured on the ragged workload: 512 to 900
-// items are equally good, 2000 items cost 4 %.)  Shared by the device-side plan and by the host's
-// check that nothing is split.
+// Chunk size for a batch whose kv lengths sum to `total` with maximum `max_len`.  Shared by the
+// device-side plan and by the host's check that nothing is split, so it uses these aggregates only.
+//
+// `target` is the number of work items the GPU holds at once (workgroup slots).  A batch with at least
+// that many (sequence, kv head, row group) triples is cut so that about `target` items exist — a quarter
+// more when it is ragged (longest sequence above 1.5x the mean): the tail chunks then differ in size,
+// and although they are dispatched longest first a little slack helps the last ones pack.  (Measured on
+// the ragged workload: 320 to 900 items are equally good, 2000 items cost 4 %.)
+//
+// A smaller batch is cut against `target_small`, for the 16-row kernel one workgroup per CU: a split
+// launch is bound by HBM from about 150 equal items on, and what more items add is partials for the
+// merge and workgroups whose prologue and epilogue nothing overlaps.  Measured, one sequence of 32768
+// tokens x 8 kv heads: 192 to 256 items 33-34 us, 320 and more 40-43 us; 3 x 20000 tokens: 47 us at 192
+// items, 53-58 us at 264 to 504.
+//   equal lengths   the item count is exact: k = target_small / triples chunks per sequence (at least
+//                   one: 24 x 8192 tokens x 8 kv heads run unsplit as 192 items in 119 us, cut in three
+//                   for 512 slots — 576 items, a second round — 145 us);
+//   else            items <= triples + work / chunk, so chunk = work / (target_small - triples) keeps them
+//                   within target_small; but no coarser than work / (9/16 target_small) — below about 144
+//                   equal items the longest one, streaming alone at some 50 GB/s, would set the time
+//                   (one long sequence in a batch of short ones); and a sequence that would only shed a
+//                   tail under a quarter of a chunk is left whole.
 XLLM_HIP_HD inline int choose_chunk(long long total, long long max_len, int batch, int num_kv_heads,
-                                    int row_groups, int target, int min_chunk, int tile = kTileTokens) {
-  long long t = target;
-  if (max_len * batch * 2 > total * 3) t += t / 4;
-  if (t > kMaxTargetItems) t = kMaxTargetItems;
+                                    int row_groups, int target, int target_small, int min_chunk,
+                                    int tile = kTileTokens) {
+  const long long triples = (long long)batch * num_kv_heads * row_groups;
   const long long work = total * num_kv_heads * row_groups;
-  long long c = (work + t - 1) / t;
+  long long c;
+  if (max_len * batch == total) {
+    long long k = triples > 0 ? target_small / triples : 1;
+    if (k < 1) k = 1;
+    c = (max_len + k - 1) / k;
+  } else if (triples < target_small) {
+    const long long within = target_small - triples;
+    const long long enough = (long long)target_small * 9 / 16;
+    const long long c_within = (work + within - 1) / within;
+    const long long c_enough = (work + enough - 1) / enough;
+    c = c_within < c_enough ? c_within : c_enough;
+    if (max_len <= c + c / 4) c = max_len;
+  } else {
+    long long t = target;
+    if (max_len * batch * 2 > total * 3) t += t / 4;
+    if (t > kMaxTargetItems) t = kMaxTargetItems;
+    c = (work + t - 1) / t;
+  }
   c = (c + tile - 1) / tile * tile;
   if (c < min_chunk) c = min_chunk;
   if (c > (1 << 30)) c = 1 << 30;
@@ -63,8 +95,10 @@ struct PlanHeader {
 };
 
 struct SeqChunk {
-  int32_t seq;    // sequence index b
-  int32_t chunk;  // chunk index within the sequence (token range [chunk*C, min(L, (chunk+1)*C)))
+  int32_t seq;     // sequence index b
+  int32_t chunk;   // chunk index within the sequence (token range [chunk*C, min(L, (chunk+1)*C)))
+  int32_t len;     // kv length of the sequence
+  int32_t chunks;  // chunks of the sequence (full + tail): one record tells a work item all it needs
 };
 
 struct WorkspaceLayout {

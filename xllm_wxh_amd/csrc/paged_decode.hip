@@ -60,6 +60,7 @@ struct DecodeParams {
   int64_t sc_stride_head;
   int64_t sc_stride_slot;
   int64_t bt_stride;
+  int32_t max_seq_chunks;  // entries of seq_chunks
   int32_t batch;
   int32_t n;  // query tokens per sequence (the largest count when q_indptr is set)
   int32_t num_q_heads;
@@ -78,7 +79,8 @@ struct DecodeParams {
   int32_t log2_bs;
   int32_t max_blocks_per_seq;
   int32_t window_left;
-  int32_t target_items;
+  int32_t target_items;   // workgroup slots of the launch (see choose_chunk)
+  int32_t target_small;   // ... and the item budget of a batch with fewer (sequence, kv head, row group) triples
   int32_t fixed_chunk;    // > 0: chunk size chosen on the host (1 << 30 = never split)
   int32_t direct_single;  // the attention kernel writes the output rows of single-chunk sequences itself
   int32_t implicit_plan;  // nothing is split and nothing is merged: item = (sequence, kv head, row group),
@@ -145,8 +147,8 @@ __global__ void __launch_bounds__(64) decode_plan_kernel(DecodeParams p) {
   // 2. Chunk size.
   const int chunk = p.fixed_chunk > 0
                         ? p.fixed_chunk
-                        : choose_chunk(total, max_len, p.batch, p.num_kv_heads, p.row_groups, p.target_items, p.min_chunk,
-                                       p.tile_tokens);
+                        : choose_chunk(total, max_len, p.batch, p.num_kv_heads, p.row_groups, p.target_items,
+                                       p.target_small, p.min_chunk, p.tile_tokens);
 
   // 3. Prefix sums of the full-chunk and tail-chunk counts (lengths are re-derived rather than
   //    re-read so that no lane depends on another lane's global store).
@@ -220,12 +222,12 @@ __global__ void __launch_bounds__(64) decode_plan_kernel(DecodeParams p) {
     wave_scan2(sf, st, lane);
     if (b < p.batch) {
       const int f0 = run_full + sf - nf;
-      for (int ci = 0; ci < nf; ++ci) p.seq_chunks[f0 + ci] = SeqChunk{b, ci};
+      for (int ci = 0; ci < nf; ++ci) p.seq_chunks[f0 + ci] = SeqChunk{b, ci, len_b, nf + nt};
       if (nt) {
         const int cls = tail_class(len_b - nf * chunk);
         const int slot = tail_hist[cls] + atomicAdd(&tail_fill[cls], 1);
         p.tail_prefix[b] = slot;
-        p.seq_chunks[total_full + slot] = SeqChunk{b, nf};
+        p.seq_chunks[total_full + slot] = SeqChunk{b, nf, len_b, nf + nt};
       }
     }
     run_full += __shfl(sf, 63);
@@ -249,6 +251,7 @@ struct Item {
   int nblk;     // valid entries in ids (>= 1)
   int n;        // query tokens of the sequence
   int q0;       // index of its first query token
+  int chunks;   // chunks the sequence was cut into (1: this item writes the output rows itself)
   int64_t head_off;     // hk * stride_head (cache elements)
   int64_t sc_head_off;  // hk * sc_stride_head (scale elements)
 };
@@ -272,14 +275,19 @@ __device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it)
   it.hk = rest % p.num_kv_heads;
   it.sc = rest / p.num_kv_heads;
   int chunk = 0, chunk_tokens = 1 << 30;
+  it.chunks = 1;
   if (p.implicit_plan) {
     if (it.sc >= p.batch) return false;
     it.b = it.sc;
   } else {
+    // The header and the item's record are independent loads (the record's index is clamped to the
+    // table, whose last entries the plan may not have written: such a record is not used).
+    const SeqChunk s = p.seq_chunks[it.sc < p.max_seq_chunks ? it.sc : 0];
     const PlanHeader hdr = *p.hdr;
     if (rest * p.row_groups >= hdr.total_items) return false;
-    const SeqChunk s = p.seq_chunks[it.sc];
     it.b = s.seq;
+    it.len = s.len;
+    it.chunks = s.chunks;
     chunk = s.chunk;
     chunk_tokens = hdr.chunk_tokens;
   }
@@ -301,8 +309,6 @@ __device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it)
       len = p.seq_lens[it.b];
     }
     it.len = len > 0 ? len : 0;
-  } else {
-    it.len = p.kv_len[it.b];
   }
   it.t_begin = chunk * chunk_tokens;
   const long long end = (long long)it.t_begin + chunk_tokens;
@@ -350,8 +356,9 @@ __device__ inline float load_partial(const float* ptr) {
 }
 
 // One wave merges the partials of output row (sequence b, query token j, head): all 64 lanes call.
-template <int Q_DT, bool COHERENT>
-__device__ inline void merge_row(const DecodeParams& p, int b, int j, int head, int q0, int lane) {
+// COLS: columns per lane (2 covers head_dim <= 128, 4 head_dim <= 256).
+template <int Q_DT, bool COHERENT, int COLS, int MAXB = 32>
+__device__ inline void merge_row_cols(const DecodeParams& p, int b, int j, int head, int q0, int lane) {
   const int nhq = p.n * p.num_q_heads;
   const int rem = j * p.num_q_heads + head;
   const int cnt = p.num_chunks[b];
@@ -362,56 +369,76 @@ __device__ inline void merge_row(const DecodeParams& p, int b, int j, int head, 
   const int tail_slot = p.hdr->total_full + p.tail_prefix[b];
   auto partial_row = [&](int i) { return (int64_t)(i < nf ? f0 + i : tail_slot) * nhq + rem; };
 
-  // Columns lane, lane + 64, ... of the output row (head_dim <= 256), summed over the chunks kUnroll
-  // at a time: their loads are all issued before the first is used.  `weight(i)` is chunk i's factor.
-  float o[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-  auto load_rows = [&](int i0, auto unroll, float (&v)[decltype(unroll)::value][4]) {
+  // Columns lane, lane + 64, ... of the output row, summed over the chunks a batch at a time: the
+  // loads of a batch are all issued before the first is used.  `weight(i)` is chunk i's factor.
+  float o[COLS];
+#pragma unroll
+  for (int k = 0; k < COLS; ++k) o[k] = 0.0f;
+  auto load_rows = [&](int i0, auto unroll, float (&v)[decltype(unroll)::value][COLS]) {
 #pragma unroll
     for (int u = 0; u < decltype(unroll)::value; ++u) {
-      const float* po = p.partial_out + partial_row(min(i0 + u, cnt - 1)) * D;
+      if (u == 0 || i0 + u < cnt) {  // (uniform over the wave)
+        const float* po = p.partial_out + partial_row(i0 + u) * D;
 #pragma unroll
-      for (int k = 0; k < 4; ++k) v[u][k] = lane + 64 * k < D ? load_partial<COHERENT>(po + lane + 64 * k) : 0.0f;
+        for (int k = 0; k < COLS; ++k) v[u][k] = lane + 64 * k < D ? load_partial<COHERENT>(po + lane + 64 * k) : 0.0f;
+      } else {
+#pragma unroll
+        for (int k = 0; k < COLS; ++k) v[u][k] = 0.0f;
+      }
     }
   };
-  auto add_rows = [&](int i0, auto unroll, const float (&v)[decltype(unroll)::value][4], auto weight) {
+  auto add_rows = [&](int i0, auto unroll, const float (&v)[decltype(unroll)::value][COLS], auto weight) {
 #pragma unroll
     for (int u = 0; u < decltype(unroll)::value; ++u) {
       const float w = i0 + u < cnt ? weight(i0 + u) : 0.0f;
 #pragma unroll
-      for (int k = 0; k < 4; ++k) o[k] += w != 0.0f ? w * v[u][k] : 0.0f;  // an empty chunk's row may hold anything
+      for (int k = 0; k < COLS; ++k) o[k] += w != 0.0f ? w * v[u][k] : 0.0f;  // an empty chunk's row may hold anything
     }
   };
-  typedef std::integral_constant<int, 8> Eight;
-  typedef std::integral_constant<int, 4> Four;
   float m, ssum;
   if (cnt <= 256) {
-    // The usual case.  Each lane keeps the log-sum-exps of chunks lane, lane + 64, ... in registers and
-    // the first rows are already on their way while the maximum and the denominator are reduced:
-    // two memory round trips for a row instead of four.
+    // The usual case.  Each lane keeps the log-sum-exps of chunks lane, lane + 64, ... in registers, and
+    // the partial rows (all of them up to 64 registers' worth, then further batches) are on their way
+    // while the maximum and the denominator are reduced: one memory round trip for a row of up to
+    // 128 / COLS chunks — these loads go to memory past the caches when the merge is fused, at
+    // more than a microsecond each way.
     float l[4];
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int i = lane + 64 * q;
       l[q] = i < cnt ? load_partial<COHERENT>(p.partial_lse + partial_row(i)) : neg_inf;
     }
-    float first[8][4];
-    load_rows(0, Eight{}, first);
-    m = wave_max(fmaxf(fmaxf(l[0], l[1]), fmaxf(l[2], l[3])));
-    const float m_safe = m == neg_inf ? 0.0f : m;
-    float e[4];
+    auto reduce_lse = [&](float (&e)[4]) {
+      m = wave_max(fmaxf(fmaxf(l[0], l[1]), fmaxf(l[2], l[3])));
+      const float m_safe = m == neg_inf ? 0.0f : m;
 #pragma unroll
-    for (int q = 0; q < 4; ++q) e[q] = __builtin_amdgcn_exp2f(l[q] - m_safe);  // 2^-inf = 0: empty or absent chunk
-    ssum = wave_sum(e[0] + e[1] + e[2] + e[3]);
-    auto weight = [&](int i) {
-      const int q = i >> 6;
-      const float mine = q == 0 ? e[0] : q == 1 ? e[1] : q == 2 ? e[2] : e[3];
-      return __shfl(mine, i & 63);
+      for (int q = 0; q < 4; ++q) e[q] = __builtin_amdgcn_exp2f(l[q] - m_safe);  // 2^-inf = 0: empty or absent chunk
+      ssum = wave_sum(e[0] + e[1] + e[2] + e[3]);
     };
-    add_rows(0, Eight{}, first, weight);
-    for (int i0 = 8; i0 < cnt; i0 += 8) {
-      float v[8][4];
-      load_rows(i0, Eight{}, v);
-      add_rows(i0, Eight{}, v, weight);
+    auto run = [&](auto batch) {
+      constexpr int kB = decltype(batch)::value;
+      float first[kB][COLS];
+      load_rows(0, batch, first);
+      float e[4];
+      reduce_lse(e);
+      auto weight = [&](int i) {
+        const int q = i >> 6;
+        const float mine = q == 0 ? e[0] : q == 1 ? e[1] : q == 2 ? e[2] : e[3];
+        return __shfl(mine, i & 63);
+      };
+      add_rows(0, batch, first, weight);
+      for (int i0 = kB; i0 < cnt; i0 += kB) {
+        float v[kB][COLS];
+        load_rows(i0, batch, v);
+        add_rows(i0, batch, v, weight);
+      }
+    };
+    if (cnt <= 8 || COLS > 2) {
+      run(std::integral_constant<int, 8>{});
+    } else if (cnt <= 16 || MAXB <= 16) {
+      run(std::integral_constant<int, 16>{});
+    } else {
+      run(std::integral_constant<int, 32>{});
     }
   } else {
     m = neg_inf;
@@ -426,8 +453,9 @@ __device__ inline void merge_row(const DecodeParams& p, int b, int j, int head, 
     auto weight = [&](int i) {
       return __builtin_amdgcn_exp2f(load_partial<COHERENT>(p.partial_lse + partial_row(i)) - m_safe);
     };
+    typedef std::integral_constant<int, 4> Four;
     for (int i0 = 0; i0 < cnt; i0 += 4) {
-      float v[4][4];
+      float v[4][COLS];
       load_rows(i0, Four{}, v);
       add_rows(i0, Four{}, v, weight);
     }
@@ -439,9 +467,18 @@ __device__ inline void merge_row(const DecodeParams& p, int b, int j, int head, 
   }
   const int64_t obase = tok * p.out_token_stride + (int64_t)head * D;
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
+  for (int k = 0; k < COLS; ++k) {
     const int d = lane + 64 * k;
     if (d < D) Elem<Q_DT>::store(p.out, obase + d, o[k] * inv);
+  }
+}
+
+template <int Q_DT, bool COHERENT>
+__device__ inline void merge_row(const DecodeParams& p, int b, int j, int head, int q0, int lane) {
+  if (p.head_dim <= 128) {
+    merge_row_cols<Q_DT, COHERENT, 2>(p, b, j, head, q0, lane);
+  } else {
+    merge_row_cols<Q_DT, COHERENT, 4>(p, b, j, head, q0, lane);
   }
 }
 
@@ -472,10 +509,10 @@ __global__ void __launch_bounds__(64 * kMergeRowsPerBlock) decode_merge_kernel(D
 // completed before its increment, resets the counter for the next launch and reads the partials with
 // coherent loads.  (Device-scope fences instead — cache write-back and invalidation on every
 // workgroup — made an 8 x 8192-token step three times slower.)
-template <int Q_DT>
+template <int Q_DT, int COLS, int MAXB>
 __device__ inline void merge_if_last(const DecodeParams& p, const Item& it, int* lds_flag) {
   if (!p.fused_merge || p.implicit_plan) return;
-  const int cnt = p.num_chunks[it.b];
+  const int cnt = it.chunks;
   if (p.direct_single && cnt == 1) return;  // written directly
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's stores have completed
   __syncthreads();
@@ -493,7 +530,7 @@ __device__ inline void merge_if_last(const DecodeParams& p, const Item& it, int*
   const int end = min(first + p.rows_per_item, it.n * p.group);
   for (int r = first + wave; r < end; r += nwaves) {
     const int j = r / p.group;
-    merge_row<Q_DT, true>(p, it.b, j, it.hk * p.group + (r - j * p.group), it.q0, lane);
+    merge_row_cols<Q_DT, true, COLS, MAXB>(p, it.b, j, it.hk * p.group + (r - j * p.group), it.q0, lane);
   }
 }
 
@@ -1193,7 +1230,7 @@ __device__ inline void finish_item(const DecodeParams& p, const Item& it, RowTil
   const float neg_inf = -INFINITY;
   const int mi = lane & 15, kg = lane >> 4;
   const int nhq = p.n * p.num_q_heads;
-  const bool single = p.implicit_plan != 0 || (p.direct_single != 0 && p.num_chunks[it.b] == 1);
+  const bool single = p.implicit_plan != 0 || (p.direct_single != 0 && it.chunks == 1);
   const float l = kg_sum(rt.l_run);
   uint8_t* mine = xch_base + wave * xch_stride;
 #pragma unroll
@@ -1387,7 +1424,8 @@ __global__ void __launch_bounds__(64 * kWaves, decode_waves_per_simd(KV_DT, TOK)
     }
   }
   finish_item<KV_DT, TOK, kWaves>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, 0, wave, lane, 0);
-  merge_if_last<qf16_of(KV_DT) ? XLLM_HIP_FP16 : XLLM_HIP_BF16>(p, it, &lds_last);
+  // (32 rows in flight make the int8 head_dim-64 instantiation spill)
+  merge_if_last<qf16_of(KV_DT) ? XLLM_HIP_FP16 : XLLM_HIP_BF16, TOK == 0 ? 4 : 2, (TOK == 2 && quant_of(KV_DT)) ? 16 : 32>(p, it, &lds_last);
 }
 
 template <int KV_DT, int TOK>
@@ -1914,6 +1952,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
   p.tail_prefix = (int32_t*)(ws + w.tail_prefix);
   p.num_chunks = (int32_t*)(ws + w.num_chunks);
   p.seq_chunks = (SeqChunk*)(ws + w.seq_chunks);
+  p.max_seq_chunks = (int32_t)w.max_seq_chunks;
   p.partial_lse = (float*)(ws + w.partial_lse);
   p.partial_out = (float*)(ws + w.partial_out);
   p.counters = (int32_t*)(ws + w.counters);
@@ -1947,8 +1986,11 @@ static int fill_params(const xllm_hip_kv_cache* c,
   p.log2_bs = is_pow2(c->block_size) ? ilog2(c->block_size) : 0;
   p.max_blocks_per_seq = a->max_blocks_per_seq;
   p.window_left = a->window_left;
-  p.target_items = target_items(is_mfma(variant), p.rows,
-                                variant == kMfmaD256 || (p.rows <= 16 && decode_waves_per_simd(c->dtype, 1) == 1));
+  const bool one_wave_per_simd = variant == kMfmaD256 || (p.rows <= 16 && decode_waves_per_simd(c->dtype, 1) == 1);
+  p.target_items = target_items(is_mfma(variant), p.rows, one_wave_per_simd);
+  // A small batch on the 16-row kernel: one of the two workgroups a CU holds (the 32-row kernel wants
+  // all its slots filled: 4 x 32768 tokens of int8 with 4 draft tokens, 65 us at 1024 items, 84 at 512).
+  p.target_small = is_mfma(variant) && p.rows <= 16 && !one_wave_per_simd ? p.target_items / 2 : p.target_items;
   // Only the MFMA kernel finishes single-chunk sequences itself.  When the caller's host-side
   // lengths (the reference keeps both in AttentionMetadata) show that the chunk the plan would
   // pick covers the longest sequence, no sequence is split: the plan is told never to split
@@ -1962,7 +2004,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
   p.fixed_chunk = 0;
   if (p.direct_single && a->max_seq_len > 0 && a->total_kv_len > 0 &&
       a->max_seq_len <= choose_chunk(a->total_kv_len, a->max_seq_len, p.batch, p.num_kv_heads, p.row_groups,
-                                     p.target_items, p.min_chunk, p.tile_tokens)) {
+                                     p.target_items, p.target_small, p.min_chunk, p.tile_tokens)) {
     p.fixed_chunk = 1 << 30;
   }
   // Many query rows per kv head (chunked prefill): the row groups supply the parallelism, and one
