@@ -61,7 +61,7 @@ def test_spec_rows_known_answers(shim, name):
         assert rows.block_tables[0] == rows.block_tables[2] == g["block_tables"][0]
 
 
-@pytest.mark.parametrize("name", ["spec_first_decode_rows", "spec_rows_with_offsets"])
+@pytest.mark.parametrize("name", ["spec_first_decode_rows", "spec_rows_with_offsets", "spec_rows_from_last_step"])
 def test_spec_rows_with_their_own_offsets(shim, name):
     g = GOLDEN[name]
     cu = np.concatenate([[0], np.cumsum(g["kv_seq_lens"])]).tolist()
