@@ -1,0 +1,104 @@
+// What a workgroup of an attention kernel works on, decoded from its index.
+#pragma once
+
+#include "decode_params.h"
+
+namespace xllm_hip {
+
+// ---------------------------------------------------------------------------------
+// Work-item decoding shared by the attention kernels.
+// ---------------------------------------------------------------------------------
+
+struct Item {
+  int sc;       // sequence-chunk slot (indexes the partial arrays)
+  int b;        // sequence
+  int hk;       // kv head
+  int rg;       // row group
+  int len;      // kv length of the sequence
+  int t_begin;  // first token of the chunk (multiple of kTileTokens)
+  int t_end;    // one past the last token of the chunk (<= len)
+  const int32_t* ids;  // block list of the sequence
+  int nblk;     // valid entries in ids (>= 1)
+  int n;        // query tokens of the sequence
+  int q0;       // index of its first query token
+  int chunks;   // chunks the sequence was cut into (1: this item writes the output rows itself)
+  int64_t head_off;     // hk * stride_head (cache elements)
+  int64_t sc_head_off;  // hk * sc_stride_head (scale elements)
+};
+
+constexpr int kXcds = 8;  // workgroup x runs on XCD x % 8, each with its own L2
+
+__device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it) {
+  // Work items in their natural order are (sequence chunk, kv head, row group), row group fastest.
+  // Some neighbours in that order read the same memory: the row groups of one (chunk, kv head) stream
+  // the same K/V, and with small blocks the scale rows of neighbouring kv heads share cache lines.
+  // Consecutive workgroup ids land on different XCDs, so a cluster of `p.cluster` neighbours is
+  // given ids that are congruent mod 8 and consecutive on that XCD: its members then run there at
+  // about the same time, and all but the first find the shared lines in that XCD's L2.
+  int linear = item_id;
+  if (p.cluster > 1) {
+    const int on_xcd = item_id / kXcds;
+    linear = ((on_xcd / p.cluster) * kXcds + item_id % kXcds) * p.cluster + on_xcd % p.cluster;
+  }
+  it.rg = linear % p.row_groups;
+  const int rest = linear / p.row_groups;
+  it.hk = rest % p.num_kv_heads;
+  it.sc = rest / p.num_kv_heads;
+  int chunk = 0, chunk_tokens = 1 << 30;
+  it.chunks = 1;
+  if (p.implicit_plan) {
+    if (it.sc >= p.batch) return false;
+    it.b = it.sc;
+  } else {
+    // The header and the item's record are independent loads (the record's index is clamped to the
+    // table, whose last entries the plan may not have written: such a record is not used).
+    const SeqChunk s = p.seq_chunks[it.sc < p.max_seq_chunks ? it.sc : 0];
+    const PlanHeader hdr = *p.hdr;
+    if (rest * p.row_groups >= hdr.total_items) return false;
+    it.b = s.seq;
+    it.len = s.len;
+    it.chunks = s.chunks;
+    chunk = s.chunk;
+    chunk_tokens = hdr.chunk_tokens;
+  }
+  if (p.q_indptr != nullptr) {
+    it.q0 = p.q_indptr[it.b];
+    const int cnt = p.q_indptr[it.b + 1] - it.q0;
+    it.n = cnt < 0 ? 0 : (cnt > p.n ? p.n : cnt);  // never beyond what the launch and the workspace were sized for
+  } else {
+    it.q0 = it.b * p.n;
+    it.n = p.n;
+  }
+  if (it.rg * p.rows_per_item >= it.n * p.group) return false;  // this sequence has no rows in the group
+  if (p.implicit_plan) {
+    int len;
+    if (p.kv_indptr != nullptr) {
+      const int nb = p.kv_indptr[it.b + 1] - p.kv_indptr[it.b];
+      len = nb > 0 ? (nb - 1) * p.block_size + p.kv_last_page_len[it.b] : 0;
+    } else {
+      len = p.seq_lens[it.b];
+    }
+    it.len = len > 0 ? len : 0;
+  }
+  it.t_begin = chunk * chunk_tokens;
+  const long long end = (long long)it.t_begin + chunk_tokens;
+  it.t_end = end < it.len ? (int)end : it.len;
+  {  // no row of the item sees beyond the causal limit of its last row
+    const int rows = it.n * p.group;
+    const int last = min((it.rg + 1) * p.rows_per_item, rows) - 1;
+    const int lim = it.len - (it.n - 1 - last / p.group);
+    it.t_end = it.t_end < lim ? it.t_end : lim;
+  }
+  if (p.kv_indptr != nullptr) {
+    it.ids = p.block_ids + p.kv_indptr[it.b];
+  } else {
+    it.ids = p.block_ids + (int64_t)it.b * p.bt_stride;
+  }
+  it.nblk = (it.len + p.block_size - 1) >> p.log2_bs;
+  if (it.nblk < 1) it.nblk = 1;
+  it.head_off = (int64_t)it.hk * p.stride_head;
+  it.sc_head_off = (int64_t)it.hk * p.sc_stride_head;
+  return true;
+}
+
+}  // namespace xllm_hip

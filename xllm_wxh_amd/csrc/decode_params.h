@@ -1,0 +1,72 @@
+// Arguments of the decode kernels: one struct, passed by value, filled by fill_params on the host.
+#pragma once
+
+#include "decode_plan.h"
+
+#include <stdint.h>
+
+namespace xllm_hip {
+
+struct DecodeParams {
+  const void* q;
+  void* out;
+  float* lse;
+  const uint8_t* k_cache;
+  const uint8_t* v_cache;
+  const float* k_scale;
+  const float* v_scale;
+  const int32_t* block_ids;  // block_table, or kv_indices in CSR form
+  const int32_t* kv_indptr;  // non-NULL selects the CSR form
+  const int32_t* seq_lens;
+  const int32_t* kv_last_page_len;
+  const int32_t* q_indptr;  // [batch+1] first query token of each sequence; NULL: n tokens each
+  PlanHeader* hdr;
+  int32_t* kv_len;
+  int32_t* full_prefix;
+  int32_t* tail_prefix;
+  int32_t* num_chunks;
+  SeqChunk* seq_chunks;
+  float* partial_lse;
+  float* partial_out;
+  int32_t* counters;  // per (sequence, kv head, row group): chunks finished so far (fused merge)
+  int64_t q_token_stride;
+  int64_t out_token_stride;
+  int64_t stride_block;
+  int64_t stride_head;
+  int64_t stride_slot;
+  int64_t sc_stride_block;
+  int64_t sc_stride_head;
+  int64_t sc_stride_slot;
+  int64_t bt_stride;
+  int32_t max_seq_chunks;  // entries of seq_chunks
+  int32_t batch;
+  int32_t n;  // query tokens per sequence (the largest count when q_indptr is set)
+  int32_t num_q_heads;
+  int32_t num_kv_heads;
+  int32_t group;  // q heads per kv head
+  int32_t rows;   // group * n
+  int32_t row_groups;
+  int32_t cluster;        // neighbouring work items kept on one XCD (see decode_item)
+  int32_t rows_per_item;  // query rows one work item handles (32 or 128 MFMA, 1 generic)
+  int32_t min_chunk;      // smallest chunk the plan may choose
+  int32_t head_dim;
+  int32_t tok;          // tokens per 256-byte LDS row of the MFMA kernels: 1 (head_dim 128), 2 (head_dim 64),
+                        // 0 (head_dim 256: a token is two rows, one in each half of the tile)
+  int32_t tile_tokens;  // tokens per tile: 32 * tok (16 at head_dim 256); chunk sizes are multiples of it
+  int32_t block_size;
+  int32_t log2_bs;
+  int32_t max_blocks_per_seq;
+  int32_t window_left;
+  int32_t target_items;   // workgroup slots of the launch (see choose_chunk)
+  int32_t target_small;   // ... and the item budget of a batch with fewer (sequence, kv head, row group) triples
+  int32_t fixed_chunk;    // > 0: chunk size chosen on the host (1 << 30 = never split)
+  int32_t direct_single;  // the attention kernel writes the output rows of single-chunk sequences itself
+  int32_t implicit_plan;  // nothing is split and nothing is merged: item = (sequence, kv head, row group),
+                          // lengths come straight from the inputs and no plan kernel runs
+  int32_t fused_merge;    // the attention kernel merges a split sequence itself: the workgroup that finishes the
+                          // last chunk of a (sequence, kv head, row group) combines the partials
+  int32_t q_dtype;
+  float scale_log2;  // sm_scale * log2(e)
+};
+
+}  // namespace xllm_hip
