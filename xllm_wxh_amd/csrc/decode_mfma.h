@@ -801,16 +801,11 @@ __device__ inline int first_visible_tile(const DecodeParams& p, const Item& it) 
   return t0;
 }
 
-#ifndef XLLM_HIP_DEPTH16
-#define XLLM_HIP_DEPTH16 1
-#endif
-// Register stages of the 16-row kernel (tiles in flight while one is consumed) and the waves per SIMD
-// it is compiled for.
-constexpr int decode_depth(int kt, int tok) { return (!quant_of(kt) && tok != 0) ? XLLM_HIP_DEPTH16 : 1; }
-constexpr int decode_waves_per_simd(int kt, int tok) { return (tok == 0 || decode_depth(kt, tok) > 1) ? 1 : 2; }
+// Waves per SIMD the 16-row kernel is compiled for: head_dim 256 needs the registers of one.
+constexpr int decode_waves_per_simd(int tok) { return tok == 0 ? 1 : 2; }
 
 template <int KV_DT, int TOK>
-__global__ void __launch_bounds__(64 * kWaves, decode_waves_per_simd(KV_DT, TOK)) decode_mfma_d128_kernel(DecodeParams p) {
+__global__ void __launch_bounds__(64 * kWaves, decode_waves_per_simd(TOK)) decode_mfma_d128_kernel(DecodeParams p) {
   __shared__ __attribute__((aligned(16))) uint8_t lds_all[kWaves * kLdsTile];
   __shared__ float lds_ml[kWaves * 16 * 2];  // (running max, denominator) per wave and query row
   __shared__ int lds_last;
@@ -841,34 +836,34 @@ __global__ void __launch_bounds__(64 * kWaves, decode_waves_per_simd(KV_DT, TOK)
 
   typename KvHalf<KV_DT>::Geom geom;
   geom.init(p, lane);
-  // Register stages: the tiles in flight while one is consumed.  (Two stages for the 1-byte caches of
-  // head_dim 256, which run one wave per SIMD and so have few bytes in flight per CU, were slower:
-  // 458 against 367 us on 64 x 8192 tokens of fp8 — the registers they take are paid for in copies
-  // between the two register files.)
-  constexpr int kDepth = decode_depth(KV_DT, TOK);
-  KvHalf<KV_DT> st[kDepth][2];  // per stage: the two halves (16 rows each) of a tile
-  int blk[kDepth][2];           // block ids of the halves each stage loads next, fetched a round earlier
+  // One register stage: the loads of tile i+1 are in flight while tile i is consumed.  (More stages were
+  // slower wherever they were tried: two for the 1-byte caches of head_dim 256, which run one wave per
+  // SIMD and so have few bytes in flight per CU, 458 against 367 us on 64 x 8192 tokens of fp8 — the
+  // registers they take are paid for in copies between the two register files; two for 16-bit caches
+  // at one wave per SIMD no better than one at two.)
+  KvHalf<KV_DT> st[2];  // the two halves (16 rows each) of the tile in flight
+  int blk[2];           // block ids of the halves loaded next, fetched a round earlier
 
-  // Tile at tb: park it from its stage, put the tile kDepth further in flight into the same stage,
-  // attend.  The scalar loads of the ids go out before the tile is parked: they share a counter with
-  // the LDS traffic, so the next wait on LDS also waits for them.
-  auto step = [&](KvHalf<KV_DT> (&s)[2], int (&b)[2], int tb) {
+  // Tile at tb: park it, put the next tile in flight, attend.  The scalar loads of the ids go out
+  // before the tile is parked: they share a counter with the LDS traffic, so the next wait on LDS
+  // also waits for them.
+  auto step = [&](int tb) {
     const bool masked = (tb + kT > mask_hi_from) || (tb < mask_lo_until);
-    const int nblk0 = block_of(p, it, tb + 2 * kDepth * kT);
-    const int nblk1 = block_of(p, it, tb + 2 * kDepth * kT + kH);
+    const int nblk0 = block_of(p, it, tb + 2 * kT);
+    const int nblk1 = block_of(p, it, tb + 2 * kT + kH);
     if (masked) {
-      s[0].template park<true>(tile, 0, tb, it.len, p.scale_log2, geom);
-      s[1].template park<true>(tile, 1, tb + kH, it.len, p.scale_log2, geom);
+      st[0].template park<true>(tile, 0, tb, it.len, p.scale_log2, geom);
+      st[1].template park<true>(tile, 1, tb + kH, it.len, p.scale_log2, geom);
     } else {
-      s[0].template park<false>(tile, 0, tb, it.len, p.scale_log2, geom);
-      s[1].template park<false>(tile, 1, tb + kH, it.len, p.scale_log2, geom);
+      st[0].template park<false>(tile, 0, tb, it.len, p.scale_log2, geom);
+      st[1].template park<false>(tile, 1, tb + kH, it.len, p.scale_log2, geom);
     }
-    if (tb + kDepth * kT < w_end) {
-      s[0].issue(p, it, tb + kDepth * kT, b[0], geom);
-      s[1].issue(p, it, tb + kDepth * kT + kH, b[1], geom, kP1);
+    if (tb + kT < w_end) {
+      st[0].issue(p, it, tb + kT, blk[0], geom);
+      st[1].issue(p, it, tb + kT + kH, blk[1], geom, kP1);
     }
-    b[0] = nblk0;
-    b[1] = nblk1;
+    blk[0] = nblk0;
+    blk[1] = nblk1;
     if (masked) {
       rt.template attend<true>(tile, tb, p.scale_log2);
     } else {
@@ -876,28 +871,11 @@ __global__ void __launch_bounds__(64 * kWaves, decode_waves_per_simd(KV_DT, TOK)
     }
   };
   if (w_begin < w_end) {
-#pragma unroll
-    for (int d = 0; d < kDepth; ++d) {
-      const int tb = w_begin + d * kT;
-      if (tb < w_end) {
-        st[d][0].issue(p, it, tb, block_of(p, it, tb), geom);
-        st[d][1].issue(p, it, tb + kH, block_of(p, it, tb + kH), geom, kP1);
-      }
-      blk[d][0] = block_of(p, it, tb + kDepth * kT);
-      blk[d][1] = block_of(p, it, tb + kDepth * kT + kH);
-    }
-    for (int tb = w_begin; tb < w_end; tb += kDepth * kT) {
-      step(st[0], blk[0], tb);
-      if constexpr (kDepth > 1) {
-        if (tb + kT < w_end) step(st[1], blk[1], tb + kT);
-      }
-      if constexpr (kDepth > 2) {
-        if (tb + 2 * kT < w_end) step(st[2], blk[2], tb + 2 * kT);
-      }
-      if constexpr (kDepth > 3) {
-        if (tb + 3 * kT < w_end) step(st[3], blk[3], tb + 3 * kT);
-      }
-    }
+    st[0].issue(p, it, w_begin, block_of(p, it, w_begin), geom);
+    st[1].issue(p, it, w_begin + kH, block_of(p, it, w_begin + kH), geom, kP1);
+    blk[0] = block_of(p, it, w_begin + kT);
+    blk[1] = block_of(p, it, w_begin + kT + kH);
+    for (int tb = w_begin; tb < w_end; tb += kT) step(tb);
   }
   finish_item<KV_DT, TOK, kWaves>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, 0, wave, lane, 0);
   // (32 rows in flight make the int8 head_dim-64 instantiation spill)

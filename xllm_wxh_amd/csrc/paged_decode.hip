@@ -192,7 +192,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
   p.log2_bs = is_pow2(c->block_size) ? ilog2(c->block_size) : 0;
   p.max_blocks_per_seq = a->max_blocks_per_seq;
   p.window_left = a->window_left;
-  const bool one_wave_per_simd = variant == kMfmaD256 || (p.rows <= 16 && decode_waves_per_simd(c->dtype, 1) == 1);
+  const bool one_wave_per_simd = variant == kMfmaD256;
   p.target_items = target_items(is_mfma(variant), p.rows, one_wave_per_simd);
   // A small batch on the 16-row kernel: one of the two workgroups a CU holds (the 32-row kernel wants
   // all its slots filled: 4 x 32768 tokens of int8 with 4 draft tokens, 65 us at 1024 items, 84 at 512).
