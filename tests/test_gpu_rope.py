@@ -126,6 +126,43 @@ def test_rope_kv_write_equals_the_two_steps(gpu, cache_kind, layout, norm):
         assert np.array_equal(_bits(row), _bits(b[t, hq * D:(hq + hk) * D].view(hk, D)))
 
 
+@pytest.mark.parametrize("cache_kind", ["bf16", "int8"])
+def test_prefill_sized_launch(gpu, cache_kind):
+    """A prefill-sized launch (3001 tokens x 48 heads, a ragged last workgroup): the rotation bit-exact
+    against the oracle, and the cache rows and scales equal to those of the separate KV write."""
+    print("case rope many tokens", cache_kind, flush=True)
+    T, hq, hk, D, bs = 3001, 32, 8, 128, 16
+    nb = (T + bs - 1) // bs + 2
+    qkv, _, _, cos_sin, pos = _inputs(T, hq, hk, hk, D, D, 4096, "bf16", seed=5, cache_kind="bf16", scale=1.0)
+    want = orc.fused_qk_norm_rope(qkv.float().numpy(), hq, hk, hk, D, 0.0, None, None, cos_sin.float().numpy(),
+                                  False, pos.numpy(), "bf16", round_each_op=True)
+    slots = torch.from_numpy(np.random.default_rng(4).permutation(nb * bs)[:T].astype(np.int32)).to(gpu)
+    shape = (nb, hk, bs, D)
+    if cache_kind == "bf16":
+        kc, vc = torch.zeros(shape, dtype=torch.bfloat16, device=gpu), torch.zeros(shape, dtype=torch.bfloat16, device=gpu)
+        ks = vs = None
+    else:
+        kc, vc = torch.zeros(shape, dtype=torch.int8, device=gpu), torch.zeros(shape, dtype=torch.int8, device=gpu)
+        ks, vs = torch.zeros(shape[:3], device=gpu), torch.zeros(shape[:3], device=gpu)
+    d = qkv.to(gpu)
+    ops.rope_kv_write(d, hq, hk, D, cos_sin.to(gpu), pos.to(gpu), kc, vc, slots, round_each_op=True,
+                      k_cache_scale=ks, v_cache_scale=vs)
+    torch.cuda.synchronize()
+    assert np.array_equal(_bits(d), _bits(torch.from_numpy(want).to(torch.bfloat16)))
+    # the separate write of the rotated keys and the values
+    k2, v2 = torch.zeros_like(kc), torch.zeros_like(vc)
+    ks2 = vs2 = None
+    if ks is not None:
+        ks2, vs2 = torch.zeros_like(ks), torch.zeros_like(vs)
+    params = ops.ReshapePagedCacheParams(key=d[:, hq * D:(hq + hk) * D].view(T, hk, D), value=d[:, (hq + hk) * D:].view(T, hk, D),
+                                         k_cache=k2, v_cache=v2, slot_mapping=slots, k_cache_scale=ks2, v_cache_scale=vs2)
+    (ops.reshape_paged_cache if cache_kind == "bf16" else ops.quant_to_paged_cache)(params)
+    torch.cuda.synchronize()
+    assert np.array_equal(_bits(kc), _bits(k2)) and np.array_equal(_bits(vc), _bits(v2))
+    if ks is not None:
+        assert np.array_equal(_bits(ks), _bits(ks2)) and np.array_equal(_bits(vs), _bits(vs2))
+
+
 def test_rope_edge_cases_and_errors(gpu):
     print("case rope edges", flush=True)
     qkv, qw, kw, cos_sin, pos = _inputs(4, 2, 1, 1, 128, 128, 16, "bf16", seed=1)

@@ -42,12 +42,11 @@ __device__ inline float bf16_bits_to_float(uint16_t b) {
   return __uint_as_float(((uint32_t)b) << 16);
 }
 
-// Round-to-nearest-even float -> bf16 bits (NaN stays NaN).
+// Round-to-nearest-even float -> bf16 bits (NaN stays NaN): gfx950 converts in hardware
+// (v_cvt_pk_bf16_f32), an eighth of the instructions of the integer form.
 __device__ inline uint16_t float_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
+  const __bf16 h = (__bf16)f;
+  return __builtin_bit_cast(uint16_t, h);
 }
 
 __device__ inline float fp8_e4m3_to_float(uint8_t b) {
