@@ -154,15 +154,17 @@ __device__ inline void merge_row_cols(const DecodeParams& p, int b, int j, int h
 
 template <int Q_DT, bool COHERENT>
 __device__ inline void merge_row(const DecodeParams& p, int b, int j, int head, int q0, int lane) {
+  // (the merge kernel's form: up to 16 rows in flight and so few enough registers for six waves per SIMD —
+  // its loads are ordinary cached ones, and a row per wave wants many waves resident)
   if (p.head_dim <= 128) {
-    merge_row_cols<Q_DT, COHERENT, 2>(p, b, j, head, q0, lane);
+    merge_row_cols<Q_DT, COHERENT, 2, 16>(p, b, j, head, q0, lane);
   } else {
     merge_row_cols<Q_DT, COHERENT, 4>(p, b, j, head, q0, lane);
   }
 }
 
 template <int Q_DT>
-__global__ void __launch_bounds__(64 * kMergeRowsPerBlock) decode_merge_kernel(DecodeParams p) {
+__global__ void __launch_bounds__(64 * kMergeRowsPerBlock, 6) decode_merge_kernel(DecodeParams p) {
   const int nhq = p.n * p.num_q_heads;
   const int64_t row = (int64_t)blockIdx.x * kMergeRowsPerBlock + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
