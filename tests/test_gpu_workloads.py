@@ -177,6 +177,8 @@ SMALL = {
     "aux_d256_bf16_b64_ctx4k": dict(batch=5, seq_len=4096),
     "aux_d256_fp8_b64_ctx8k": dict(batch=3, seq_len=2048),
     "aux_d256_int8_spec_verify": dict(batch=2, seq_len=4096),
+    "aux_d64_bf16_b512_ctx4k": dict(batch=6, seq_len=3000),
+    "aux_d64_int8_b512_ctx8k": dict(batch=4, seq_len=5000),
     "aux_b1_ctx32k": dict(),
     "aux_b8_ctx8k": dict(batch=3),
 }

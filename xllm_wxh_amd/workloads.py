@@ -82,6 +82,16 @@ WORKLOADS = {
         name="aux_d256_int8_spec_verify", batch=32, num_q_heads=64, num_kv_heads=8, head_dim=256, block_size=128,
         q_per_seq=4, kv_dtype="int8", seq_len_kind="fixed", seq_len=16384,
         description="head_dim 256 speculative verify over an int8 cache: 64q/8kv, D=256, bs=128, B=32, L=16384, 4 draft tokens"),
+    # head_dim 64 (the head size of the reference's own CPU-sized test shape, Qwen2-0.5B: 14q/2kv) at a
+    # size that fills the GPU.
+    "aux_d64_bf16_b512_ctx4k": DecodeWorkload(
+        name="aux_d64_bf16_b512_ctx4k", batch=512, num_q_heads=14, num_kv_heads=2, head_dim=64, block_size=32,
+        seq_len_kind="fixed", seq_len=4096, value_std=0.5,
+        description="head_dim 64 decode: bf16, 14q/2kv, D=64, bs=32, B=512, L=4096"),
+    "aux_d64_int8_b512_ctx8k": DecodeWorkload(
+        name="aux_d64_int8_b512_ctx8k", batch=512, num_q_heads=14, num_kv_heads=2, head_dim=64, block_size=32,
+        kv_dtype="int8", seq_len_kind="fixed", seq_len=8192,
+        description="head_dim 64 decode over an int8 cache: 14q/2kv, D=64, bs=32, B=512, L=8192"),
     # Small batches: the split-KV schedule (plan, attention over chunks, merge) is what is measured.
     "aux_b1_ctx32k": DecodeWorkload(
         name="aux_b1_ctx32k", batch=1, num_q_heads=32, num_kv_heads=8, head_dim=128, block_size=16,
