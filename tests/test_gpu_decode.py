@@ -560,3 +560,38 @@ def test_small_batch_chunk_choices(gpu, kv, name, lens):
     assert lse_err(lse, lse_ref) <= LSE_TOL
     out_h, _ = case.run(hints=True)
     assert torch.equal(out, out_h)
+
+
+@pytest.mark.parametrize("kv,qdt,tol", [("bf16", "bf16", 2e-2), ("fp16", "fp16", 2e-3), ("int8", "bf16", 2e-2)])
+def test_two_stage_decode_merged_by_lse_equals_one_stage(gpu, kv, qdt, tol):
+    """The returned log-sum-exps are base 2 and merge as the reference merges two partial attentions
+    (xllm/core/kernels/cuda/xattention/lse_combine.cu:61-73): attention over a prefix and over the rest
+    of each sequence, two calls, combined by that formula, against the one call over the whole — the
+    reference's own check of its two-stage decode, with its tolerances
+    (xllm/core/layers/cuda/xattention_test.cpp:224-273: fp16 2e-3, bf16 2e-2)."""
+    print("case two-stage", kv, qdt, flush=True)
+    bs = 16
+    lens = [700, 33, 2500, 160, 6000]
+    cut = [320, 16, 1024, 96, 4096]  # block-aligned prefix lengths, all inside the sequences
+    case = Case(len(lens), 32, 8, 128, bs, lens, kv=kv, qdt=qdt, seed=77)
+    whole, lse_whole = case.run()
+
+    def part(table, part_lens):
+        saved = case.block_table, case.seq_lens
+        case.block_table = torch.from_numpy(np.ascontiguousarray(table)).to(gpu)
+        case.seq_lens = torch.tensor(part_lens, dtype=torch.int32, device=gpu)
+        try:
+            return case.run()
+        finally:
+            case.block_table, case.seq_lens = saved
+
+    out_a, lse_a = part(case.table, cut)
+    width = case.table.shape[1]
+    rest = np.zeros_like(case.table)
+    for b, c in enumerate(cut):
+        rest[b, : width - c // bs] = case.table[b, c // bs:]
+    out_b, lse_b = part(rest, [l - c for l, c in zip(lens, cut)])
+    merged, lse_m = orc.lse_combine(out_a.float().cpu().numpy(), lse_a.cpu().numpy(),
+                                    out_b.float().cpu().numpy(), lse_b.cpu().numpy())
+    assert max_abs_err(whole, merged.astype(np.float64)) <= tol
+    assert lse_err(lse_whole, lse_m.astype(np.float64)) <= 1e-4
