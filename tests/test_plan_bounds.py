@@ -1,0 +1,98 @@
+"""The split-KV plan on the host: whatever the lengths, the chunk size `choose_chunk` picks yields no
+more sequence chunks than the workspace holds records and partial rows for (the plan kernel writes one
+record per chunk, the attention kernels one partial per chunk and row), and the choices it is meant to
+make for small batches.  The header the kernels are built from is compiled with g++ into a small
+library; no GPU is involved."""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+REPO = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC = os.path.join(REPO, "xllm_wxh_amd", "csrc")
+
+
+@pytest.fixture(scope="module")
+def plan(tmp_path_factory):
+    out = str(tmp_path_factory.mktemp("plan") / "libplan_harness.so")
+    subprocess.run(["g++", "-O1", "-std=c++17", "-shared", "-fPIC", "-I", CSRC,
+                    os.path.join(REPO, "tests", "plan_bounds_harness.cpp"), "-o", out], check=True)
+    lib = ctypes.CDLL(out)
+    lib.harness_choose_chunk.argtypes = [ctypes.c_longlong, ctypes.c_longlong] + [ctypes.c_int] * 7
+    lib.harness_max_seq_chunks.restype = ctypes.c_longlong
+    return lib
+
+
+def _chunks(lens, c):
+    lens = np.asarray(lens, np.int64)
+    return int(np.maximum(1, -(-lens // c)).sum())  # an empty sequence keeps one (empty) chunk
+
+
+# (workgroup slots, budget of a small batch, rows per item, smallest chunk, tile): the 16-row kernel, the
+# 32-row kernel, head_dim 256, head_dim 64, the generic kernel, and the largest target a caller can force
+KERNELS = [(512, 256, 32, 512, 32), (1024, 1024, 32, 512, 32), (256, 256, 32, 512, 16), (512, 256, 32, 512, 64),
+           (2048, 2048, 1, 64, 32), (4096, 2048, 32, 512, 32), (64, 32, 32, 512, 32), (1, 0, 32, 512, 32)]
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_chunk_count_never_exceeds_the_workspace(plan, seed):
+    rng = np.random.default_rng(seed)
+    for _ in range(3000):
+        target, small, rows_per_item, min_chunk, tile = KERNELS[int(rng.integers(len(KERNELS)))]
+        hkv = int(rng.choice([1, 2, 4, 8, 16]))
+        g = int(rng.choice([1, 2, 4, 7, 8, 16]))
+        n = int(rng.choice([1, 1, 2, 4, 8]))
+        rg = plan.harness_row_groups(n, hkv * g, hkv, rows_per_item)
+        if rows_per_item > 1 and rg > 4:
+            continue  # never split
+        batch = int(rng.choice([1, 2, 3, 7, 24, 64, 200, 1000]))
+        kind = rng.random()
+        if kind < 0.25:
+            lens = np.full(batch, int(rng.integers(1, 200000)))
+        elif kind < 0.5:
+            lens = rng.integers(0, 40000, size=batch)
+        elif kind < 0.75:
+            lens = rng.integers(1, 300, size=batch)
+            lens[int(rng.integers(batch))] = int(rng.integers(1000, 1000000))  # one long among short
+        else:
+            lens = np.clip(np.round(rng.lognormal(np.log(2048), 0.8, size=batch)), 16, 32768).astype(np.int64)
+        total, max_len = int(lens.sum()), int(lens.max())
+        c = plan.harness_choose_chunk(total, max_len, batch, hkv, rg, target, small, min_chunk, tile)
+        assert c >= min_chunk and c % tile == 0
+        bound = plan.harness_max_seq_chunks(batch, n, hkv * g, hkv, 128)
+        assert _chunks(lens, c) <= bound, (target, small, hkv, rg, batch, total, max_len, c)
+
+
+def test_small_batch_choices(plan):
+    def chunk(lens, hkv=8, rg=1, target=512, small=256):
+        lens = np.asarray(lens, np.int64)
+        return plan.harness_choose_chunk(int(lens.sum()), int(lens.max()), len(lens), hkv, rg, target, small, 512, 32)
+
+    # equal lengths: 256 / (batch * kv heads) chunks per sequence, each a whole number of tiles
+    assert chunk([32768]) == 1024                       # 32 chunks x 8 heads = 256 items
+    assert chunk([8192] * 8) == 2048                    # 4 chunks each
+    assert chunk([8192] * 16) == 4096                   # 2 chunks each
+    assert chunk([8192] * 24) >= 8192                   # 192 (sequence, head) pairs: unsplit
+    assert chunk([4096] * 48) >= 4096                   # more pairs than the budget: unsplit
+    assert chunk([4096] * 64) >= 4096                   # the Llama-3-8B shape: one item per pair
+    assert chunk([20000] * 3) == 2016                   # 10 chunks each, 240 items
+    # ragged small batch: the item count stays within the budget ...
+    lens = [4000, 2500, 900, 3300, 1700, 2900]
+    c = chunk(lens)
+    assert _chunks(lens, c) * 8 <= 256
+    # ... except that one long sequence among short ones is still cut finely enough to fill the GPU
+    lens = [100000] + [1000] * 30
+    c = chunk(lens)
+    assert 100 <= _chunks(lens, c) * 8 and c <= 100000 // 12
+    # lengths so close that a split would only shed short tails: left whole
+    lens = [2500 + 16 * i for i in range(20)]
+    assert chunk(lens) >= max(lens)
+    # the 32-row kernel keeps all its slots as the budget
+    assert chunk([32768] * 32, target=1024, small=1024) == 8192
+    # a large ragged batch: about 640 items' worth of work per chunk
+    rng = np.random.default_rng(0)
+    lens = np.clip(np.round(rng.lognormal(np.log(2048), 0.8, size=256)), 16, 32768).astype(np.int64)
+    c = chunk(lens)
+    assert abs(c - int(lens.sum()) * 8 / 640) <= 32
