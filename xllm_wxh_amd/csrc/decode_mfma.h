@@ -918,7 +918,7 @@ __global__ void __launch_bounds__(128, TOK == 0 ? 1 : 2) decode_mfma_d128_rows32
   // i is consumed (a wave fetches only half a tile, so one stage would leave too few bytes in flight
   // per CU to cover the HBM latency; four stages for head_dim 256, which runs one wave per SIMD,
   // were slower than two).  Both waves run the same iterations.
-  constexpr int kDepth = 2;
+  constexpr int kDepth = 2;  // (the loop below is written out for two)
   KvHalf<KV_DT> mine[kDepth];  // the 16 rows this wave fetches: rows 16*rs .. of the tile
   int blk[kDepth];             // block id of the half each stage loads next, fetched a round earlier
 
@@ -955,10 +955,6 @@ __global__ void __launch_bounds__(128, TOK == 0 ? 1 : 2) decode_mfma_d128_rows32
   for (int i = 0; i < iters; i += kDepth) {
     step(mine[0], blk[0], i);
     if (i + 1 < iters) step(mine[1], blk[1], i + 1);
-    if constexpr (kDepth > 2) {
-      if (i + 2 < iters) step(mine[2], blk[2], i + 2);
-      if (i + 3 < iters) step(mine[3], blk[3], i + 3);
-    }
   }
   __syncthreads();  // all tiles consumed before the buffers are reused for the exchange
   finish_item<KV_DT, TOK, 1>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, rs, 0, lane, rs);
