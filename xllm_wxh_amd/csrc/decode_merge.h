@@ -77,10 +77,10 @@ __device__ inline void merge_row_cols(const DecodeParams& p, int b, int j, int h
   float m, ssum;
   if (cnt <= 256) {
     // The usual case.  Each lane keeps the log-sum-exps of chunks lane, lane + 64, ... in registers, and
-    // the partial rows (all of them up to 64 registers' worth, then further batches) are on their way
+    // the partial rows (up to MAXB of them — 8 at head_dim 256 —, then further batches) are on their way
     // while the maximum and the denominator are reduced: one memory round trip for a row of up to
-    // 128 / COLS chunks — these loads go to memory past the caches when the merge is fused, at
-    // more than a microsecond each way.
+    // that many chunks — these loads go to memory past the caches when the merge is fused, at more
+    // than a microsecond each way.
     float l[4];
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
