@@ -595,3 +595,83 @@ def test_two_stage_decode_merged_by_lse_equals_one_stage(gpu, kv, qdt, tol):
                                     out_b.float().cpu().numpy(), lse_b.cpu().numpy())
     assert max_abs_err(whole, merged.astype(np.float64)) <= tol
     assert lse_err(lse_whole, lse_m.astype(np.float64)) <= 1e-4
+
+
+def test_int8_verify_step_replays_under_hip_graph(gpu):
+    """The speculative-verify form of the step under a HIP graph: quantising write of 4 draft tokens per
+    sequence, plan, the 32-row kernel over an int8 cache and the merge kernel, captured once and
+    replayed while lengths and slots change; every replay equals the eager result."""
+    print("case hip graph int8 verify", flush=True)
+    B, n, Hq, Hkv, D, bs, max_blocks = 3, 4, 64, 8, 128, 32, 200
+    nblocks = B * max_blocks + 1
+    g = torch.Generator().manual_seed(52)
+    k_cache = torch.zeros(nblocks, Hkv, bs, D, dtype=torch.int8, device=gpu)
+    v_cache = torch.zeros_like(k_cache)
+    k_scale = torch.zeros(nblocks, Hkv, bs, device=gpu)
+    v_scale = torch.zeros_like(k_scale)
+    # a cache full of quantised random rows, written through the operator itself
+    fill = torch.arange(1 * bs, nblocks * bs, dtype=torch.int32, device=gpu)
+    for s in range(0, fill.numel(), 4096):
+        sl = fill[s:s + 4096]
+        kk = torch.randn(sl.numel(), Hkv, D, generator=g).to(torch.bfloat16).to(gpu)
+        vv = torch.randn(sl.numel(), Hkv, D, generator=g).to(torch.bfloat16).to(gpu)
+        ops.quant_to_paged_cache(ops.ReshapePagedCacheParams(key=kk, value=vv, k_cache=k_cache, v_cache=v_cache,
+                                                             slot_mapping=sl, k_cache_scale=k_scale, v_cache_scale=v_scale))
+    perm = (torch.randperm(nblocks - 1, generator=g) + 1).to(torch.int32)
+    table_full = perm[: B * max_blocks].view(B, max_blocks)
+    q = torch.zeros(B * n, Hq, D, dtype=torch.bfloat16, device=gpu)
+    new_k = torch.zeros(B * n, Hkv, D, dtype=torch.bfloat16, device=gpu)
+    new_v = torch.zeros(B * n, Hkv, D, dtype=torch.bfloat16, device=gpu)
+    slots = torch.zeros(B * n, dtype=torch.int32, device=gpu)
+    block_table = table_full.to(gpu).contiguous()
+    seq_lens = torch.full((B,), n, dtype=torch.int32, device=gpu)
+    out = torch.zeros_like(q)
+    ws = torch.empty(ops.decode_workspace_bytes(B, n, Hq, Hkv, D), dtype=torch.uint8, device=gpu)
+    scale = 1.0 / float(np.sqrt(D))
+
+    def step(o):
+        ops.quant_to_paged_cache(ops.ReshapePagedCacheParams(key=new_k, value=new_v, k_cache=k_cache, v_cache=v_cache,
+                                                             slot_mapping=slots, k_cache_scale=k_scale,
+                                                             v_cache_scale=v_scale))
+        ops.batch_decode(q, k_cache, o, block_table, seq_lens, v_cache, None, None, k_scale, v_scale, scale=scale,
+                         q_per_seq=n, workspace=ws, kv_cache_quant_bit_size=8)
+
+    def load_inputs(lens, seed):
+        gg = torch.Generator().manual_seed(seed)
+        q.copy_(torch.randn(B * n, Hq, D, generator=gg).to(torch.bfloat16))
+        new_k.copy_(torch.randn(B * n, Hkv, D, generator=gg).to(torch.bfloat16))
+        new_v.copy_(torch.randn(B * n, Hkv, D, generator=gg).to(torch.bfloat16))
+        sl = []
+        for b, L in enumerate(lens):  # the draft tokens are the last n positions of the sequence
+            for j in range(n):
+                pos = L - n + j
+                sl.append(int(table_full[b, pos // bs]) * bs + pos % bs)
+        slots.copy_(torch.tensor(sl, dtype=torch.int32))
+        seq_lens.copy_(torch.tensor(lens, dtype=torch.int32))
+
+    load_inputs([3000, 40, 6000], 0)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step(out)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step(out)
+    for it, lens in enumerate(([3000, 40, 6000], [6399, 4, 17], [9, 9, 9], [1000, 5003, 2004])):
+        load_inputs(lens, 20 + it)
+        saved = [t.clone() for t in (k_cache, v_cache, k_scale, v_scale)]
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        after = [t.clone() for t in (k_cache, v_cache, k_scale, v_scale)]
+        for t, s in zip((k_cache, v_cache, k_scale, v_scale), saved):
+            t.copy_(s)
+        eager = torch.zeros_like(out)
+        step(eager)
+        torch.cuda.synchronize()
+        assert torch.equal(got, eager), "replay %d differs from eager" % it
+        for t, a in zip((k_cache, v_cache, k_scale, v_scale), after):
+            assert torch.equal(t.view(torch.uint8) if t.dtype == torch.int8 else t, a.view(torch.uint8) if a.dtype == torch.int8 else a)
+        _ = (k_scale[:8] * 2).sum().item()  # unrelated eager work between replays
