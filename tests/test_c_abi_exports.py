@@ -119,3 +119,47 @@ def test_variant_selection_is_host_only(lib):
     assert lib.xllm_hip_paged_decode_variant(ctypes.byref(desc), ctypes.byref(args)) == b"generic"
     desc.head_dim = 512
     assert lib.xllm_hip_paged_decode_variant(ctypes.byref(desc), ctypes.byref(args)) == b""
+
+
+def _header_struct_fields(name):
+    """Field names of `typedef struct <name> { ... } <name>;` in declaration order."""
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"//[^\n]*", "", text)
+    body = re.search(r"typedef struct %s \{(.*?)\} %s;" % (name, name), text, flags=re.S).group(1)
+    return [re.search(r"([A-Za-z0-9_]+)\s*$", d.strip()).group(1) for d in body.split(";") if d.strip()]
+
+
+def test_header_is_plain_c_and_its_layouts_are_those_of_the_ctypes_binding(tmp_path):
+    """The boundary is a C ABI: the header compiles as C99 without a HIP toolchain in sight, and
+    every field of its three structs sits where the ctypes binding (what the tests, bench.py and
+    any Python caller go through) puts it — offsets taken from the C compiler, not retyped."""
+    import shutil
+    import subprocess
+
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    structs = {"xllm_hip_kv_cache": _lib.KvCacheDesc, "xllm_hip_decode_args": _lib.DecodeArgs,
+               "xllm_hip_rope_args": _lib.RopeArgs}
+    lines = ['#include <stddef.h>', '#include <stdio.h>', '#include "xllm_hip_paged_kv.h"', "int main(void) {"]
+    for cname in structs:
+        lines.append('  printf("%s . %%zu\\n", sizeof(%s));' % (cname, cname))
+        for f in _header_struct_fields(cname):
+            lines.append('  printf("%s %s %%zu\\n", offsetof(%s, %s));' % (cname, f, cname, f))
+    lines += ["  return 0;", "}"]
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines) + "\n")
+    exe = tmp_path / "layout"
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.dirname(HEADER),
+                    str(src), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout
+    seen = {}
+    for line in out.splitlines():
+        cname, field, value = line.split()
+        seen.setdefault(cname, {})[field] = int(value)
+    for cname, cls in structs.items():
+        assert seen[cname].pop(".") == ctypes.sizeof(cls), cname
+        assert list(seen[cname]) == [f[0] for f in cls._fields_], cname  # same fields, same order
+        for field, offset in seen[cname].items():
+            assert getattr(cls, field).offset == offset, (cname, field)
