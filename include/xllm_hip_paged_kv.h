@@ -156,10 +156,12 @@ int xllm_hip_quant_to_paged_cache(const xllm_hip_kv_cache* cache,
  * The block list of sequence b is given in one of two forms:
  *   block_table form (mlu_ops_api.h:130-131): block_table != NULL, row b starts at
  *       block_table + b*block_table_stride, padded with any valid block id;
- *       seq_lens[b] is the kv length.
+ *       seq_lens[b] is the kv length (an entry above max_blocks_per_seq*block_size, which the row
+ *       cannot hold, is cut to that: no block id is read from outside the row).
  *   CSR form (cuda_ops_api.h:129-131): block_table == NULL; the list is
  *       kv_indices[kv_indptr[b] .. kv_indptr[b+1]) and the kv length is
- *       (kv_indptr[b+1]-kv_indptr[b]-1)*block_size + kv_last_page_len[b].
+ *       (kv_indptr[b+1]-kv_indptr[b]-1)*block_size + kv_last_page_len[b]
+ *       (kv_last_page_len is taken within 0 .. block_size).
  *
  * q/out are [batch*n, num_q_heads, head_dim] of q_dtype (BF16, FP16 or FP32),
  * head_dim contiguous, head stride = head_dim, token strides free.

@@ -332,6 +332,26 @@ def test_zero_length_and_empty_batch(gpu):
 
 
 @pytest.mark.parametrize("force_generic", [False, True])
+def test_lengths_beyond_the_block_list_are_cut_to_it(gpu, force_generic, monkeypatch):
+    """A seq_lens entry above what a block_table row holds is cut to the row's capacity, so that no
+    block id is read from the next row (or from past the table): the result is that of the cut
+    length, bit for bit.  The rows after the long one hold valid ids, so nothing here reads outside
+    the cache either way."""
+    print("case length beyond the block list generic=%s" % force_generic, flush=True)
+    if force_generic:
+        monkeypatch.setenv("XLLM_HIP_DECODE_FORCE_GENERIC", "1")
+    case = Case(3, 32, 8, 128, 16, [64, 40, 64], seed=23)
+    assert case.block_table.shape[1] == 4
+    out = torch.empty_like(case.q)
+    ops.batch_decode(case.q, case.k_cache, out, case.block_table, case.seq_lens, case.v_cache, scale=case.scale)
+    longer = torch.tensor([100, 40, 64], dtype=torch.int32, device=gpu)
+    out2 = torch.empty_like(case.q)
+    ops.batch_decode(case.q, case.k_cache, out2, case.block_table, longer, case.v_cache, scale=case.scale)
+    torch.cuda.synchronize()
+    assert torch.equal(out, out2)
+
+
+@pytest.mark.parametrize("force_generic", [False, True])
 def test_sliding_window(gpu, force_generic, monkeypatch):
     print("case window", force_generic, flush=True)
     if force_generic:

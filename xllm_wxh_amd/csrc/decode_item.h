@@ -70,16 +70,7 @@ __device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it)
     it.n = p.n;
   }
   if (it.rg * p.rows_per_item >= it.n * p.group) return false;  // this sequence has no rows in the group
-  if (p.implicit_plan) {
-    int len;
-    if (p.kv_indptr != nullptr) {
-      const int nb = p.kv_indptr[it.b + 1] - p.kv_indptr[it.b];
-      len = nb > 0 ? (nb - 1) * p.block_size + p.kv_last_page_len[it.b] : 0;
-    } else {
-      len = p.seq_lens[it.b];
-    }
-    it.len = len > 0 ? len : 0;
-  }
+  if (p.implicit_plan) it.len = kv_length(p, it.b);
   it.t_begin = chunk * chunk_tokens;
   const long long end = (long long)it.t_begin + chunk_tokens;
   it.t_end = end < it.len ? (int)end : it.len;

@@ -56,6 +56,7 @@ struct DecodeParams {
   int32_t block_size;
   int32_t log2_bs;
   int32_t max_blocks_per_seq;
+  int32_t len_cap;  // block_table form: tokens a table row can hold (a longer seq_lens entry is cut to it)
   int32_t window_left;
   int32_t target_items;   // workgroup slots of the launch (see choose_chunk)
   int32_t target_small;   // ... and the item budget of a batch with fewer (sequence, kv head, row group) triples
@@ -68,5 +69,21 @@ struct DecodeParams {
   int32_t q_dtype;
   float scale_log2;  // sm_scale * log2(e)
 };
+
+// kv length of sequence b as every kernel uses it: never negative and never beyond what the
+// sequence's block list holds, so that no block id is read from outside the list.
+__device__ inline int kv_length(const DecodeParams& p, int b) {
+  int len;
+  if (p.kv_indptr != nullptr) {
+    const int nb = p.kv_indptr[b + 1] - p.kv_indptr[b];
+    int last = p.kv_last_page_len[b];
+    last = last < p.block_size ? last : p.block_size;
+    len = nb > 0 ? (nb - 1) * p.block_size + (last > 0 ? last : 0) : 0;
+  } else {
+    len = p.seq_lens[b];
+    len = len < p.len_cap ? len : p.len_cap;
+  }
+  return len > 0 ? len : 0;
+}
 
 }  // namespace xllm_hip

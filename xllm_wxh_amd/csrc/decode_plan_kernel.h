@@ -40,14 +40,7 @@ __global__ void __launch_bounds__(64) decode_plan_kernel(DecodeParams p) {
   long long total = 0;
   int max_len = 0;
   for (int b = lane; b < p.batch; b += 64) {
-    int len;
-    if (p.kv_indptr != nullptr) {
-      const int nb = p.kv_indptr[b + 1] - p.kv_indptr[b];
-      len = nb > 0 ? (nb - 1) * p.block_size + p.kv_last_page_len[b] : 0;
-    } else {
-      len = p.seq_lens[b];
-    }
-    len = len > 0 ? len : 0;
+    const int len = kv_length(p, b);
     p.kv_len[b] = len;
     total += len;
     max_len = len > max_len ? len : max_len;
@@ -67,16 +60,7 @@ __global__ void __launch_bounds__(64) decode_plan_kernel(DecodeParams p) {
 
   // 3. Prefix sums of the full-chunk and tail-chunk counts (lengths are re-derived rather than
   //    re-read so that no lane depends on another lane's global store).
-  auto length_of = [&](int b) {
-    int len;
-    if (p.kv_indptr != nullptr) {
-      const int nb = p.kv_indptr[b + 1] - p.kv_indptr[b];
-      len = nb > 0 ? (nb - 1) * p.block_size + p.kv_last_page_len[b] : 0;
-    } else {
-      len = p.seq_lens[b];
-    }
-    return len > 0 ? len : 0;
-  };
+  auto length_of = [&](int b) { return kv_length(p, b); };
   // The tail chunks differ in size.  They are dispatched after the (equal) full chunks, longest
   // first — in 64 size classes — so that the launch ends with the shortest work items.
   auto tail_class = [&](int tail_len) { return (int)(((long long)tail_len * 64) / chunk); };  // tail_len < chunk

@@ -191,6 +191,10 @@ static int fill_params(const xllm_hip_kv_cache* c,
   p.block_size = c->block_size;
   p.log2_bs = is_pow2(c->block_size) ? ilog2(c->block_size) : 0;
   p.max_blocks_per_seq = a->max_blocks_per_seq;
+  {
+    const int64_t cap = (int64_t)a->max_blocks_per_seq * c->block_size;
+    p.len_cap = a->block_table != nullptr && cap < INT32_MAX ? (int32_t)cap : INT32_MAX;
+  }
   p.window_left = a->window_left;
   const bool one_wave_per_simd = variant == kMfmaD256;
   p.target_items = target_items(is_mfma(variant), p.rows, one_wave_per_simd);
