@@ -163,6 +163,9 @@ int xllm_hip_quant_to_paged_cache(const xllm_hip_kv_cache* cache,
  *       (kv_indptr[b+1]-kv_indptr[b]-1)*block_size + kv_last_page_len[b]
  *       (kv_last_page_len is taken within 0 .. block_size).
  *
+ * Block ids are expected within 0 .. num_blocks-1; one outside is taken as the nearest valid block
+ * (the result for that sequence is then meaningless, but nothing outside the cache is read).
+ *
  * q/out are [batch*n, num_q_heads, head_dim] of q_dtype (BF16, FP16 or FP32),
  * head_dim contiguous, head stride = head_dim, token strides free.
  * lse, if not NULL, receives the base-2 log-sum-exp of the scaled scores,

@@ -332,6 +332,29 @@ def test_zero_length_and_empty_batch(gpu):
 
 
 @pytest.mark.parametrize("force_generic", [False, True])
+def test_block_ids_are_taken_within_the_cache(gpu, force_generic, monkeypatch):
+    """A block id outside 0 .. num_blocks-1 in a used table entry is a caller's mistake; the kernels
+    take it within the cache (the nearest valid block) rather than read outside it, so the result is
+    that of the table with those ids, bit for bit."""
+    print("case block ids within the cache generic=%s" % force_generic, flush=True)
+    if force_generic:
+        monkeypatch.setenv("XLLM_HIP_DECODE_FORCE_GENERIC", "1")
+    case = Case(2, 32, 8, 128, 16, [64, 40], seed=29)
+    last = case.nblocks - 1
+    wrong = case.block_table.clone()
+    wrong[0, 1] = case.nblocks + 5
+    wrong[1, 0] = -3
+    right = case.block_table.clone()
+    right[0, 1] = last
+    right[1, 0] = 0
+    out, out2 = torch.empty_like(case.q), torch.empty_like(case.q)
+    ops.batch_decode(case.q, case.k_cache, out, right, case.seq_lens, case.v_cache, scale=case.scale)
+    ops.batch_decode(case.q, case.k_cache, out2, wrong, case.seq_lens, case.v_cache, scale=case.scale)
+    torch.cuda.synchronize()
+    assert torch.equal(out, out2)
+
+
+@pytest.mark.parametrize("force_generic", [False, True])
 def test_lengths_beyond_the_block_list_are_cut_to_it(gpu, force_generic, monkeypatch):
     """A seq_lens entry above what a block_table row holds is cut to the row's capacity, so that no
     block id is read from the next row (or from past the table): the result is that of the cut

@@ -84,7 +84,7 @@ __global__ void __launch_bounds__(64) decode_generic_kernel(DecodeParams p) {
       int64_t vrow = 0;  // invisible tokens point at the start of the cache and carry weight 0
       if (vis) {
         int bi = tok >> p.log2_bs;
-        const int64_t blk = it.ids[bi];
+        const int64_t blk = block_in_cache(p, it.ids[bi]);
         const int slot = tok & (p.block_size - 1);
         const int64_t row = blk * p.stride_block + (int64_t)it.hk * p.stride_head + (int64_t)slot * p.stride_slot;
         float dot = dot_row<KV_DT>(p.k_cache, row, qs, D, vec_ok);

@@ -61,7 +61,7 @@ __device__ inline uint32_t swz_v(int row, int piece) {
 __device__ inline int block_of(const DecodeParams& p, const Item& it, int tok) {
   int bi = tok >> p.log2_bs;
   bi = bi < it.nblk ? bi : it.nblk - 1;
-  return __builtin_amdgcn_readfirstlane(it.ids[bi]);
+  return block_in_cache(p, __builtin_amdgcn_readfirstlane(it.ids[bi]));
 }
 
 // The same through the constant address space, which makes the load a scalar one whatever else the
@@ -71,7 +71,7 @@ __device__ inline int block_of(const DecodeParams& p, const Item& it, int tok) {
 __device__ inline int block_of_const(const DecodeParams& p, const Item& it, int tok) {
   int bi = tok >> p.log2_bs;
   bi = bi < it.nblk ? bi : it.nblk - 1;
-  return ((const __attribute__((address_space(4))) int32_t*)it.ids)[bi];
+  return block_in_cache(p, ((const __attribute__((address_space(4))) int32_t*)it.ids)[bi]);
 }
 
 // Uniform (scalar-register) part of the addresses of 16 consecutive tokens starting at `tok`

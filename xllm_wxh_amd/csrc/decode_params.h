@@ -56,6 +56,7 @@ struct DecodeParams {
   int32_t block_size;
   int32_t log2_bs;
   int32_t max_blocks_per_seq;
+  int32_t last_block;  // num_blocks - 1: block ids are taken within 0 .. last_block
   int32_t len_cap;  // block_table form: tokens a table row can hold (a longer seq_lens entry is cut to it)
   int32_t window_left;
   int32_t target_items;   // workgroup slots of the launch (see choose_chunk)
@@ -84,6 +85,12 @@ __device__ inline int kv_length(const DecodeParams& p, int b) {
     len = len < p.len_cap ? len : p.len_cap;
   }
   return len > 0 ? len : 0;
+}
+
+// A block id as the kernels use it: within the cache, whatever the table holds.
+__device__ inline int block_in_cache(const DecodeParams& p, int id) {
+  id = id > 0 ? id : 0;
+  return id < p.last_block ? id : p.last_block;
 }
 
 }  // namespace xllm_hip

@@ -191,6 +191,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
   p.block_size = c->block_size;
   p.log2_bs = is_pow2(c->block_size) ? ilog2(c->block_size) : 0;
   p.max_blocks_per_seq = a->max_blocks_per_seq;
+  p.last_block = c->num_blocks - 1 < INT32_MAX ? (int32_t)(c->num_blocks - 1) : INT32_MAX;
   {
     const int64_t cap = (int64_t)a->max_blocks_per_seq * c->block_size;
     p.len_cap = a->block_table != nullptr && cap < INT32_MAX ? (int32_t)cap : INT32_MAX;
