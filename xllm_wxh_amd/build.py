@@ -1,6 +1,6 @@
 """Build recipe of the gfx950 shared library behind the C ABI.
 
-`build_library()` runs one explicit hipcc line over the HIP sources in `csrc/`
+`build_library()` compiles the HIP sources in `csrc/` with explicit hipcc lines
 and leaves `libxllm_hip_paged_kv.so` beside this file, where the loader in
 `_lib.py` looks for it.  Intermediate files go to `<repo>/build/`.
 """
@@ -36,24 +36,36 @@ def hipcc_path():
     raise RuntimeError("hipcc not found (looked on PATH and in /opt/rocm/bin)")
 
 
-def build_library(verbose=True, save_temps=False):
-    """Compile every HIP source for gfx950 into LIB_PATH; raises on failure."""
-    build_dir = os.path.join(REPO_DIR, "build")
-    os.makedirs(build_dir, exist_ok=True)
-    tmp_out = os.path.join(build_dir, LIB_NAME)
-    cmd = [hipcc_path()] + HIPCC_FLAGS
-    if save_temps:
-        cmd.append("-save-temps=obj")
-    cmd += [os.path.join(CSRC_DIR, s) for s in HIP_SOURCES] + ["-o", tmp_out]
+def _run(cmd, verbose):
     if verbose:
         print("[build]", " ".join(cmd), flush=True)
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     # hipcc's host pass warns that it does not know the packed-fp32 feature; that is expected.
     lines = [l for l in proc.stdout.splitlines() if "packed-fp32-ops" not in l]
     if proc.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + "\n".join(lines))
+        raise RuntimeError("%s failed:\n%s" % (cmd[0], "\n".join(lines)))
     if verbose and lines:
         print("\n".join(lines))
+
+
+def build_library(verbose=True, save_temps=False, extra_flags=()):
+    """Compile every HIP source for gfx950 (one hipcc process per source, side by side) and link
+    them into LIB_PATH; raises on failure."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    build_dir = os.path.join(REPO_DIR, "build")
+    os.makedirs(build_dir, exist_ok=True)
+    tmp_out = os.path.join(build_dir, LIB_NAME)
+    compile_flags = [f for f in HIPCC_FLAGS if f != "-shared"] + list(extra_flags)
+    if save_temps:
+        compile_flags.append("-save-temps=obj")
+    objects = [os.path.join(build_dir, os.path.splitext(s)[0] + ".o") for s in HIP_SOURCES]
+    jobs = [[hipcc_path()] + compile_flags + ["-c", os.path.join(CSRC_DIR, s), "-o", o]
+            for s, o in zip(HIP_SOURCES, objects)]
+    with ThreadPoolExecutor(max_workers=min(len(jobs), os.cpu_count() or 1)) as pool:
+        for fut in [pool.submit(_run, cmd, verbose) for cmd in jobs]:
+            fut.result()
+    _run([hipcc_path(), "--offload-arch=gfx950", "-shared", "-fPIC"] + objects + ["-o", tmp_out], verbose)
     os.replace(tmp_out, LIB_PATH)
     return LIB_PATH
 
