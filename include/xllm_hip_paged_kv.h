@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define XLLM_HIP_ABI_VERSION 2
+#define XLLM_HIP_ABI_VERSION 3
 
 /* A hipStream_t, passed as an opaque pointer so that C callers need no HIP headers. */
 typedef void* xllm_hip_stream_t;
@@ -264,6 +264,28 @@ int xllm_hip_paged_decode(const xllm_hip_kv_cache* cache,
                           void* workspace,
                           size_t workspace_bytes,
                           xllm_hip_stream_t stream);
+
+/*
+ * xllm_hip_paged_decode without a workspace argument, for callers that cannot allocate device memory
+ * (code under HIP graph capture, serving loops and harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  The schedule, the split partials and the merge counters live in an
+ * array of XLLM_HIP_STATIC_WORKSPACE_BYTES bytes that is part of the library's device code: each GPU
+ * the library runs on holds its own copy from the first launch until the process ends, and this
+ * call neither allocates nor frees anything.  Sizes for which xllm_hip_paged_decode_workspace_bytes
+ * exceeds that constant are refused with XLLM_HIP_WORKSPACE_TOO_SMALL and a message (the need is
+ * about 4096 * q_per_seq * (num_q_heads / num_kv_heads) * head_dim * 4 bytes plus a few KiB per
+ * sequence: plain decode up to 16 query heads per kv head at head_dim 128 fits).
+ * Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two streams, two
+ * threads) race; calls ordered on a stream, or by events, do not.  Nothing needs clearing between
+ * calls: each call rebuilds the schedule and zeroes the counters it uses with a kernel, not a memset.
+ * The device current at the call must be the one `stream` belongs to.  The array's address is looked
+ * up on the first call per device (hipGetSymbolAddress): make one call on each device before
+ * capturing a graph that contains this entry point.
+ */
+#define XLLM_HIP_STATIC_WORKSPACE_BYTES (48u << 20)
+int xllm_hip_paged_decode_static(const xllm_hip_kv_cache* cache,
+                                 const xllm_hip_decode_args* args,
+                                 xllm_hip_stream_t stream);
 
 /*
  * Index-only conversion between the two block-list forms

@@ -10,7 +10,8 @@ import os
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG_DIR, "libxllm_hip_paged_kv.so")
 
-ABI_VERSION = 2
+ABI_VERSION = 3
+STATIC_WORKSPACE_BYTES = 48 << 20
 
 # xllm_hip_dtype
 BF16, FP16, FP32, FP8_E4M3, INT8 = 0, 1, 2, 3, 4
@@ -33,6 +34,7 @@ EXPORTED_SYMBOLS = (
     "xllm_hip_paged_decode_run",
     "xllm_hip_paged_decode_run_timed",
     "xllm_hip_paged_decode",
+    "xllm_hip_paged_decode_static",
     "xllm_hip_csr_to_block_table",
     "xllm_hip_rope_kv_write",
     "xllm_hip_swap_blocks_staging_bytes",
@@ -158,6 +160,8 @@ def load():
         fn.restype = ctypes.c_int
     lib.xllm_hip_paged_decode_run_timed.argtypes = [P(KvCacheDesc), P(DecodeArgs), vp, ctypes.c_size_t, vp, vp, vp]
     lib.xllm_hip_paged_decode_run_timed.restype = ctypes.c_int
+    lib.xllm_hip_paged_decode_static.argtypes = [P(KvCacheDesc), P(DecodeArgs), vp]
+    lib.xllm_hip_paged_decode_static.restype = ctypes.c_int
     lib.xllm_hip_csr_to_block_table.argtypes = [vp, vp, vp, i32, i32, vp, i64, i32, vp, vp]
     lib.xllm_hip_csr_to_block_table.restype = ctypes.c_int
     lib.xllm_hip_rope_kv_write.argtypes = [P(RopeArgs), P(KvCacheDesc), vp, vp]

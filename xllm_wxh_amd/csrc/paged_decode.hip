@@ -32,7 +32,13 @@
 #include <math.h>
 #include <stdlib.h>
 
+#include <mutex>
 #include <type_traits>
+
+// Workspace of xllm_hip_paged_decode_static: one array per GPU, part of the loaded code object (it is
+// never allocated or freed).  In host code the name is only a handle for hipGetSymbolAddress; kernels
+// get the address that call returns, like any caller-owned workspace.
+static __device__ __align__(256) unsigned char scratch[XLLM_HIP_STATIC_WORKSPACE_BYTES];
 
 namespace xllm_hip {
 
@@ -444,6 +450,49 @@ extern "C" int xllm_hip_paged_decode(const xllm_hip_kv_cache* cache,
                                      xllm_hip_stream_t stream) {
   if (int s = xllm_hip_paged_decode_plan(cache, args, workspace, workspace_bytes, stream)) return s;
   return xllm_hip_paged_decode_run(cache, args, workspace, workspace_bytes, stream);
+}
+
+// Device address of `scratch` on the current device, looked up once per device.
+static int static_workspace(void** out) {
+  constexpr int kMaxDevices = 64;
+  static std::mutex mu;
+  static void* ptrs[kMaxDevices] = {nullptr};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    return fail(XLLM_HIP_RUNTIME_ERROR, "hipGetDevice failed or device index beyond %d", kMaxDevices - 1);
+  }
+  std::lock_guard<std::mutex> lock(mu);
+  if (ptrs[dev] == nullptr) {
+    void* ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr) {
+      return fail(XLLM_HIP_RUNTIME_ERROR, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+    }
+    ptrs[dev] = ptr;
+  }
+  *out = ptrs[dev];
+  return XLLM_HIP_OK;
+}
+
+extern "C" int xllm_hip_paged_decode_static(const xllm_hip_kv_cache* cache,
+                                            const xllm_hip_decode_args* args,
+                                            xllm_hip_stream_t stream) {
+  XLLM_HIP_REQUIRE(cache != nullptr && args != nullptr, "cache or args is NULL");
+  XLLM_HIP_REQUIRE(args->batch >= 0 && args->q_per_seq >= 1 && args->num_q_heads >= 1 && cache->num_kv_heads >= 1 &&
+                       cache->head_dim >= 1,
+                   "bad batch/q_per_seq/num_q_heads/num_kv_heads/head_dim");
+  const size_t need =
+      workspace_layout(args->batch, args->q_per_seq, args->num_q_heads, cache->num_kv_heads, cache->head_dim)
+          .total_bytes;
+  if (need > (size_t)XLLM_HIP_STATIC_WORKSPACE_BYTES) {
+    return fail(XLLM_HIP_WORKSPACE_TOO_SMALL,
+                "these sizes need %zu bytes of workspace, the built-in one holds %zu: call xllm_hip_paged_decode "
+                "with a caller-owned workspace",
+                need, (size_t)XLLM_HIP_STATIC_WORKSPACE_BYTES);
+  }
+  void* ws = nullptr;
+  if (int s = static_workspace(&ws)) return s;
+  return xllm_hip_paged_decode(cache, args, ws, (size_t)XLLM_HIP_STATIC_WORKSPACE_BYTES, stream);
 }
 
 extern "C" int xllm_hip_csr_to_block_table(const int32_t* kv_indptr,
