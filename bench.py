@@ -63,8 +63,8 @@ def parse_args():
 
 def build_pools(w, torch, ops, num_blocks, npools, device, layout="HND", skew_bytes=None):
     """KV pools (HND is the native layout), allocated by the library's policy (ops.allocate_kv_cache).
-    Quantised pools are produced by the path's own quantising KV write from N(0,1) bf16 values, as
-    the workload defines them."""
+    Quantised pools are produced by the path's own quantising KV write from N(0,1) fp32 values, as
+    the workloads define them (generated in fp32, then quantised per token and head)."""
     def allocate(dt, with_scales):
         if skew_bytes is not None and skew_bytes < 0:  # separate allocations
             k, v = torch.empty(shape, device=device, dtype=dt), torch.empty(shape, device=device, dtype=dt)
@@ -97,8 +97,11 @@ def build_pools(w, torch, ops, num_blocks, npools, device, layout="HND", skew_by
         chunk = 1 << 16
         for s0 in range(0, total_slots, chunk):
             t = min(chunk, total_slots - s0)
-            src_k = torch.randn(t, w.num_kv_heads, w.head_dim, device=device, dtype=torch.bfloat16, generator=gen)
-            src_v = torch.randn(t, w.num_kv_heads, w.head_dim, device=device, dtype=torch.bfloat16, generator=gen)
+            src_k = torch.randn(t, w.num_kv_heads, w.head_dim, device=device, dtype=torch.float32, generator=gen)
+            src_v = torch.randn(t, w.num_kv_heads, w.head_dim, device=device, dtype=torch.float32, generator=gen)
+            if w.value_std != 1.0:
+                src_k *= w.value_std
+                src_v *= w.value_std
             slots = torch.arange(s0, s0 + t, device=device, dtype=torch.int32)
             ops.quant_to_paged_cache(ops.ReshapePagedCacheParams(
                 key=src_k, value=src_v, k_cache=k, v_cache=v, slot_mapping=slots, k_cache_scale=ks,
@@ -155,7 +158,7 @@ def main():
     T = w.batch * w.q_per_seq
     gen = torch.Generator(device=device)
     gen.manual_seed(99)
-    q = torch.randn(T, w.num_q_heads, w.head_dim, device=device, dtype=io_dtype, generator=gen)
+    q = (torch.randn(T, w.num_q_heads, w.head_dim, device=device, dtype=torch.float32, generator=gen) * w.q_std).to(io_dtype)
     out = torch.empty_like(q)
     block_table = torch.from_numpy(table).to(device)
     seq_lens_d = torch.from_numpy(seq_lens).to(device)

@@ -114,11 +114,13 @@ int xllm_hip_reshape_paged_cache(const xllm_hip_kv_cache* cache,
  * xllm::kernel::quant_to_paged_cache (xllm/core/kernels/ops_api.cpp:196-210,
  * xllm/core/kernels/mlu/mlu_ops_api.h:66-77).  src_dtype is BF16, FP16 or FP32;
  * cache->dtype is INT8 (qmax 127) or FP8_E4M3 (qmax 448).
- *   absmax = max_d |x_d|
+ *   absmax = max_d |x_d|                     (fmaxf: a NaN element does not take part)
  *   scale  = max(absmax / qmax, min_scale)   min_scale = FLT_EPSILON (int8), 1/(448*512) (fp8)
  *            (xllm/core/kernels/cuda/fp8_quant_utils.cuh:38-53)
  *   q_d    = int8: clamp(rint(x_d / scale), -127, 127)   (round half to even)
  *            fp8 : e4m3fn_rne(clamp(x_d / scale, -448, 448))  (fp8_quant_utils.cuh:112-131)
+ *   clamp(y, -m, m) = fmaxf(-m, fminf(y, m)) as in fp8_quant_utils.cuh:121-122, so a NaN quotient (a NaN
+ *   element, or an infinite one: inf / inf) becomes +m; an all-zero row gets scale = min_scale and zeros.
  */
 int xllm_hip_quant_to_paged_cache(const xllm_hip_kv_cache* cache,
                                   const void* key,
@@ -237,7 +239,14 @@ int xllm_hip_paged_decode_plan(const xllm_hip_kv_cache* cache,
  * Split sequences leave normalised partial results in the workspace; up to 16 query rows per kv
  * head the attention kernel combines them itself (the workgroup that finishes a sequence's last
  * chunk; it counts in counters that the plan zeroes and every run leaves at zero), otherwise a merge
- * kernel follows.  Two runs must not share a workspace concurrently. */
+ * kernel follows.  Two runs must not share a workspace concurrently.
+ * The in-kernel combine rests on how gfx950 treats device-scope atomic accesses, not on the HIP
+ * memory model alone: partials are stored and loaded as relaxed device-scope atomics (which go to
+ * memory past the caches that are private to an XCD), a wave waits for its stores to complete
+ * (s_waitcnt vmcnt(0)) before the workgroup's thread 0 increments the counter, and the workgroup that
+ * reads the final count reads the partials.  No release/acquire fence pair is issued (it was
+ * measured three times slower).  XLLM_HIP_OPTION_DECODE_SEPARATE_MERGE selects the separate merge
+ * kernel, which depends on stream order alone, for every shape. */
 int xllm_hip_paged_decode_run(const xllm_hip_kv_cache* cache,
                               const xllm_hip_decode_args* args,
                               void* workspace,
@@ -273,8 +282,9 @@ int xllm_hip_paged_decode(const xllm_hip_kv_cache* cache,
  * the library runs on holds its own copy from the first launch until the process ends, and this
  * call neither allocates nor frees anything.  Sizes for which xllm_hip_paged_decode_workspace_bytes
  * exceeds that constant are refused with XLLM_HIP_WORKSPACE_TOO_SMALL and a message (the need is
- * about 4096 * q_per_seq * (num_q_heads / num_kv_heads) * head_dim * 4 bytes plus a few KiB per
- * sequence: plain decode up to 16 query heads per kv head at head_dim 128 fits).
+ * at most 1280 * r * head_dim * 4 bytes, r = min(q_per_seq * num_q_heads / num_kv_heads, 128), plus
+ * r * num_kv_heads * head_dim * 4 bytes per sequence: 20 MiB + 128 KiB per sequence for 32 query rows
+ * per kv head at head_dim 128 and 8 kv heads).
  * Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two streams, two
  * threads) race; calls ordered on a stream, or by events, do not.  Nothing needs clearing between
  * calls: each call rebuilds the schedule and zeroes the counters it uses with a kernel, not a memset.
@@ -344,9 +354,11 @@ typedef struct xllm_hip_rope_args {
   int32_t cos_sin_dtype;     /* BF16 / FP16 / FP32 */
   const void* cos_sin_cache; /* [max_position, rotary_dim] */
   int64_t max_position;
-  const int64_t* positions;  /* [num_tokens] */
+  const void* positions;     /* [num_tokens], int64 (or int32, see positions_int32) */
   int32_t interleave;        /* 0: NeoX pairs (j, j + rotary_dim/2); 1: GPT-J pairs (2j, 2j+1) */
   int32_t round_each_op;
+  int32_t positions_int32;   /* nonzero: positions is const int32_t* (the type the reference's attention
+                              * modules pass, xllm/core/layers/common/tests/qwen2_attention_tests.cpp:226) */
 } xllm_hip_rope_args;
 
 int xllm_hip_rope_kv_write(const xllm_hip_rope_args* args,
@@ -393,6 +405,22 @@ int xllm_hip_copy_blocks(const xllm_hip_kv_cache* cache,
                          int32_t num_groups,
                          int32_t num_dst,
                          xllm_hip_stream_t stream);
+
+/*
+ * Process-wide diagnostic switches; none is needed in service and none has a counterpart in the
+ * reference.  Each starts at the integer value of the environment variable of the same name with
+ * the prefix XLLM_HIP_ (XLLM_HIP_DECODE_FORCE_GENERIC, ...), read once when the first decode call or
+ * option call is made, or 0.  Safe to call from any thread; a change applies to calls made after it.
+ */
+enum xllm_hip_option {
+  XLLM_HIP_OPTION_DECODE_FORCE_GENERIC = 0,  /* != 0: every decode call takes the generic kernel */
+  XLLM_HIP_OPTION_DECODE_TARGET_ITEMS = 1,   /* > 0: work items a split decode step is cut for, if that is fewer
+                                              * than the kernel's own target (256 to 2048) */
+  XLLM_HIP_OPTION_DECODE_SEPARATE_MERGE = 2, /* != 0: split sequences are always combined by the merge kernel */
+  XLLM_HIP_OPTION_COUNT = 3
+};
+int xllm_hip_set_option(int32_t which, int64_t value);
+int64_t xllm_hip_get_option(int32_t which); /* -1 for an unknown option */
 
 /* Message of the last non-OK status returned on this host thread ("" if none). */
 const char* xllm_hip_last_error(void);

@@ -452,19 +452,25 @@ def float_to_e4m3fn(x):
 def quantize_per_token_head(x, kind):
     """x: float32 [..., head_dim] -> (q, scale) with one scale per leading index.
     kind 'int8': q int8 = clamp(rint(x/scale), -127, 127), scale = max(absmax/127, FLT_EPSILON)
-    kind 'fp8' : q uint8 (e4m3fn bits) = rne(clamp(x/scale, -448, 448)), scale = max(absmax/448, 1/(448*512))."""
+    kind 'fp8' : q uint8 (e4m3fn bits) = rne(clamp(x/scale, -448, 448)), scale = max(absmax/448, 1/(448*512)).
+    Non-finite inputs follow C's fmaxf/fminf, which return the other operand for a NaN: absmax skips NaN
+    elements, and clamp(y, -m, m) = fmaxf(-m, fminf(y, m)) — the order of
+    xllm/core/kernels/cuda/fp8_quant_utils.cuh:121-122 — turns a NaN quotient (a NaN element, or an
+    infinite one: inf / inf) into +m.  (The int8 quantiser of the reference is closed source; the same
+    order is used for it.)"""
     x = np.asarray(x, np.float32)
-    amax = np.max(np.abs(x), axis=-1, keepdims=True).astype(np.float32)
-    if kind == "int8":
-        scale = np.maximum(amax / np.float32(INT8_MAX), MIN_SCALE_INT8).astype(np.float32)
-        y = (x / scale).astype(np.float32)
-        q = np.clip(np.rint(y), -127, 127).astype(np.int8)
-    elif kind == "fp8":
-        scale = np.maximum(amax / np.float32(FP8_E4M3_MAX), MIN_SCALE_FP8).astype(np.float32)
-        y = np.clip((x / scale).astype(np.float32), -FP8_E4M3_MAX, FP8_E4M3_MAX)
-        q = float_to_e4m3fn(y)
-    else:
-        raise ValueError(kind)
+    amax = np.fmax.reduce(np.abs(x), axis=-1, keepdims=True, initial=np.float32(0)).astype(np.float32)
+    with np.errstate(invalid="ignore", divide="ignore", over="ignore"):
+        if kind == "int8":
+            scale = np.maximum(amax / np.float32(INT8_MAX), MIN_SCALE_INT8).astype(np.float32)
+            y = (x / scale).astype(np.float32)
+            q = np.fmax(np.float32(-127), np.fmin(np.rint(y), np.float32(127))).astype(np.int8)
+        elif kind == "fp8":
+            scale = np.maximum(amax / np.float32(FP8_E4M3_MAX), MIN_SCALE_FP8).astype(np.float32)
+            y = np.fmax(np.float32(-FP8_E4M3_MAX), np.fmin((x / scale).astype(np.float32), np.float32(FP8_E4M3_MAX)))
+            q = float_to_e4m3fn(y)
+        else:
+            raise ValueError(kind)
     return q, scale[..., 0]
 
 

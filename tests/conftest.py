@@ -19,3 +19,21 @@ def gpu():
     if not torch.cuda.is_available():
         pytest.skip("no GPU visible")
     return torch.device("cuda:0")
+
+
+@pytest.fixture
+def lib_option():
+    """Sets process-wide diagnostic switches of the library for one test and restores them after it:
+    lib_option("force_generic"), lib_option("target_items", 64), lib_option("separate_merge")."""
+    from xllm_wxh_amd import ops
+
+    active = []
+
+    def set_option(name, value=1):
+        ctx = ops.option(name, value)
+        ctx.__enter__()
+        active.append(ctx)
+
+    yield set_option
+    for ctx in reversed(active):
+        ctx.__exit__(None, None, None)

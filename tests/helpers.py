@@ -100,6 +100,21 @@ def max_abs_err(out, ref):
     return float(np.abs(out.float().cpu().numpy().astype(np.float64) - ref).max())
 
 
+def max_rel_err_per_seq(out, ref, q_per_seq=1):
+    """Largest, over the sequences, of (max-abs error of the sequence's output rows) / (RMS of its
+    reference rows).  Long sequences of zero-mean values have outputs of a few hundredths, where an
+    absolute bound alone would let a wrong V scale or a dropped chunk through."""
+    got = out.float().cpu().numpy().astype(np.float64)
+    got = got.reshape(-1, q_per_seq, *got.shape[1:])
+    want = np.asarray(ref, np.float64).reshape(got.shape)
+    worst = 0.0
+    for b in range(got.shape[0]):
+        rms = float(np.sqrt(np.mean(want[b] ** 2)))
+        if rms > 0.0:
+            worst = max(worst, float(np.abs(got[b] - want[b]).max()) / rms)
+    return worst
+
+
 def lse_err(lse, ref):
     got = lse.cpu().numpy().astype(np.float64)
     fin = np.isfinite(ref)

@@ -51,9 +51,10 @@ def test_struct_sizes_match_the_header_layout():
     assert _lib.DecodeArgs.max_seq_len.offset == 120
     assert _lib.DecodeArgs.q_indptr.offset == 136
     assert ctypes.sizeof(_lib.DecodeArgs) == 144
-    # xllm_hip_rope_args: ptr, 2 i64, 6 i32, 2 ptr, f32 + i32, ptr, i64, ptr, 2 i32
+    # xllm_hip_rope_args: ptr, 2 i64, 6 i32, 2 ptr, f32 + i32, ptr, i64, ptr, 3 i32 (+ 4 bytes of padding)
     assert _lib.RopeArgs.q_weight.offset == 48 and _lib.RopeArgs.cos_sin_cache.offset == 72
-    assert ctypes.sizeof(_lib.RopeArgs) == 104
+    assert _lib.RopeArgs.positions_int32.offset == 104
+    assert ctypes.sizeof(_lib.RopeArgs) == 112
 
 
 def test_workspace_bytes_is_a_pure_size_function(lib):
@@ -62,8 +63,9 @@ def test_workspace_bytes_is_a_pure_size_function(lib):
     assert 0 < a < b
     assert a % 256 == 0
     assert lib.xllm_hip_paged_decode_workspace_bytes(64, 0, 32, 8, 128) == 0
-    # partial outputs dominate: (4096/Hkv + B + 1) sequence chunks x n x Hq x D fp32
-    assert a >= (4096 // 8 + 64 + 1) * 32 * 128 * 4
+    # partial outputs dominate: (640/Hkv + B + 1) sequence chunks x n x Hq x D fp32 (four rows per kv head:
+    # the 16-row kernel's 512 work items and a quarter more)
+    assert a >= (640 // 8 + 64 + 1) * 32 * 128 * 4
 
 
 def test_argument_errors_are_reported_not_launched(lib):

@@ -163,3 +163,67 @@ def test_quant_to_paged_cache_bit_exact(gpu, layout, kind, src):
     else:
         np.testing.assert_array_equal(got_k, kc_ref)
         np.testing.assert_array_equal(got_v, vc_ref)
+
+
+@pytest.mark.parametrize("kind", ["int8", "fp8"])
+@pytest.mark.parametrize("fused", [False, True])
+def test_quantisers_on_nan_inf_and_zero_rows(gpu, kind, fused):
+    """Rows holding NaN, +-Inf or only zeros through both quantisers (quant_to_paged_cache and the
+    write fused behind the rotary embedding, here with an identity rotation), bit-exact against the
+    oracle: absmax skips NaN, and the clamp — in the reference's order,
+    xllm/core/kernels/cuda/fp8_quant_utils.cuh:121-122 — turns a NaN quotient into +max."""
+    print("case quant non-finite", kind, fused, flush=True)
+    nb, bs, H, D, T = 4, 16, 2, 128, 6
+    g = torch.Generator().manual_seed(8)
+    key = torch.randn(T, H, D, generator=g)
+    val = torch.randn(T, H, D, generator=g)
+    key[0, 0, 5] = float("nan")
+    key[1, 1, 0] = float("inf")
+    key[1, 1, 9] = float("-inf")
+    key[2, 0] = 0.0
+    val[3, 1, 100] = float("nan")
+    val[3, 1, 101] = float("-inf")
+    val[4, 0] = float("nan")  # nothing finite in the row
+    val[5, 1] = 0.0
+    key, val = key.to(torch.bfloat16), val.to(torch.bfloat16)
+    slots = np.array([3, 17, 40, 5, 63, 22], np.int32)
+    cdt = torch.int8 if kind == "int8" else torch.float8_e4m3fn
+    cshape, sshape = (nb, H, bs, D), (nb, H, bs)
+    kc = torch.zeros(cshape, dtype=torch.int8).view(cdt).to(gpu)
+    vc = torch.zeros(cshape, dtype=torch.int8).view(cdt).to(gpu)
+    ks = torch.full(sshape, -1.0, device=gpu)
+    vs = torch.full(sshape, -1.0, device=gpu)
+    sm = torch.from_numpy(slots).to(gpu)
+    if fused:
+        # one query head of zeros in front, cos = 1 and sin = 0: the rotation leaves K as it is
+        qkv = torch.cat([torch.zeros(T, D, dtype=torch.bfloat16), key.reshape(T, -1), val.reshape(T, -1)], 1).to(gpu)
+        cos_sin = torch.cat([torch.ones(4, D // 2), torch.zeros(4, D // 2)], 1).to(torch.bfloat16).to(gpu)
+        pos = torch.zeros(T, dtype=torch.int32, device=gpu)
+        ops.rope_kv_write(qkv, 1, H, D, cos_sin, pos, kc, vc, sm, k_cache_scale=ks, v_cache_scale=vs)
+    else:
+        ops.quant_to_paged_cache(ops.ReshapePagedCacheParams(key=key.to(gpu), value=val.to(gpu), k_cache=kc, v_cache=vc,
+                                                             slot_mapping=sm, k_cache_scale=ks, v_cache_scale=vs))
+    torch.cuda.synchronize()
+    np_dt = np.int8 if kind == "int8" else np.uint8
+    kc_ref, vc_ref = np.zeros(cshape, np_dt), np.zeros(cshape, np_dt)
+    ks_ref, vs_ref = np.full(sshape, -1.0, np.float32), np.full(sshape, -1.0, np.float32)
+    kf, vf = key.float().numpy(), val.float().numpy()
+    if fused:
+        # NaN * 0 of the rotation's sine term: a row's NaN reaches its rotation partner too
+        half = D // 2
+        part = np.concatenate([kf[..., half:], kf[..., :half]], -1)
+        kf = np.where(np.isnan(part) | np.isinf(part), np.float32("nan"), kf)
+    orc.quant_to_paged_cache(slots, kf, vf, kc_ref, vc_ref, ks_ref, vs_ref, kind, "HND")
+    np.testing.assert_array_equal(ks.cpu().numpy(), ks_ref)
+    np.testing.assert_array_equal(vs.cpu().numpy(), vs_ref)
+    for got, ref in ((_bits(kc).view(np_dt), kc_ref), (_bits(vc).view(np_dt), vc_ref)):
+        if kind == "fp8":  # +0 and -0 are the same value
+            same = (got == ref) | (((got & 0x7F) == 0) & ((ref & 0x7F) == 0))
+            assert same.all(), int((~same).sum())
+        else:
+            np.testing.assert_array_equal(got, ref)
+    # the saturated codes are where the oracle's docstring says they are
+    top = 127 if kind == "int8" else 0x7E
+    assert int(_bits(kc).view(np_dt)[0, 0, 3, 5]) == top      # NaN element
+    assert int(_bits(kc).view(np_dt)[1, 1, 1, 9]) == top      # -inf / inf = NaN -> +max
+    assert (_bits(vc).view(np_dt)[3, 0, 15, :] == top).all()  # a row of NaN

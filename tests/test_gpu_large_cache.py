@@ -2,7 +2,6 @@
 deployment passes 2^31 elements and 2^32 bytes): every kernel of the path on blocks that straddle
 those offsets and on the last blocks of the pool, against the oracle run on a compact copy of the
 same blocks.  The big tensors are allocated uninitialised; only the blocks in use are written."""
-import os
 
 import numpy as np
 import pytest
@@ -148,15 +147,11 @@ def test_decode_reads_high_blocks(big, n, generic):
     kf, vf = big.float_caches()
     ref, _ = orc.paged_decode(q.float().numpy(), kf, vf, big.table, lens, 1.0 / np.sqrt(D), q_per_seq=n)
     out = torch.full((B * n, HQ, D), float("nan"), dtype=torch.bfloat16, device=big.gpu)
-    if generic:
-        os.environ["XLLM_HIP_DECODE_FORCE_GENERIC"] = "1"
-    try:
+    with ops.option("force_generic", int(bool(generic))):
         ops.batch_decode(q.to(big.gpu), big.big_k, out, big.dev(big.big_table), big.dev(lens), big.big_v,
                          k_cache_quant_scale=big.big_ks, v_cache_quant_scale=big.big_vs, scale=1.0 / float(np.sqrt(D)),
                          q_per_seq=n, kv_cache_quant_bit_size=8 if big.kind == "int8" else -1)
         torch.cuda.synchronize()
-    finally:
-        os.environ.pop("XLLM_HIP_DECODE_FORCE_GENERIC", None)
     err = float(np.abs(out.float().cpu().numpy() - ref).max())
     assert err <= (5e-2 if big.kind == "int8" else 2e-2), err
 

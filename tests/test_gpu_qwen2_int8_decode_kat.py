@@ -59,14 +59,11 @@ def test_hip_operators_reproduce_the_reference_known_answer(gpu, fixed):
     assert np.all(np.abs(got - want) <= 2.0 ** -7 * np.abs(want))
     check(out, fixed["w"], fixed["ref_out"])
     # the generic kernel, on the same inputs
-    os.environ["XLLM_HIP_DECODE_FORCE_GENERIC"] = "1"
-    try:
+    with ops.option("force_generic"):
         out2 = torch.empty_like(out)
         ops.batch_decode(q, k, out2, dev(table), dev(lens), v, k_cache_quant_scale=ks, v_cache_quant_scale=vs,
                          scale=float(np.sqrt(1.0 / case.HEAD_DIM)), kv_cache_quant_bit_size=8)
         torch.cuda.synchronize()
-    finally:
-        del os.environ["XLLM_HIP_DECODE_FORCE_GENERIC"]
     check(out2, fixed["w"], fixed["ref_out"])
 
 

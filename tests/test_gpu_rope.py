@@ -181,3 +181,19 @@ def test_rope_edge_cases_and_errors(gpu):
                                False, pos.to(gpu))
     with pytest.raises(_lib.XllmHipError):  # more heads than the row holds
         ops.fused_qk_norm_rope(e, 4, 1, 1, 128, 1e-6, qw.to(gpu), kw.to(gpu), cos_sin.to(gpu), False, pos.to(gpu))
+
+
+@pytest.mark.parametrize("D,kind", [(128, "bf16"), (192, "fp16")])  # the 16-lanes-per-head kernel and the general one
+def test_int32_positions_are_read_as_they_are(gpu, D, kind):
+    """The reference's attention modules hand int32 positions over
+    (xllm/core/layers/common/tests/qwen2_attention_tests.cpp:226,549): same bits as with int64."""
+    print("case rope int32 positions", D, kind, flush=True)
+    T, hq, hk = 13, 4, 2
+    qkv, qw, kw, cos_sin, pos = _inputs(T, hq, hk, hk, D, D, 700, kind, seed=31)
+    a, b = qkv.to(gpu), qkv.to(gpu)
+    ops.fused_qk_norm_rope(a, hq, hk, hk, D, 1e-6, qw.to(gpu), kw.to(gpu), cos_sin.to(gpu), False, pos.to(gpu))
+    ops.fused_qk_norm_rope(b, hq, hk, hk, D, 1e-6, qw.to(gpu), kw.to(gpu), cos_sin.to(gpu), False,
+                           pos.to(torch.int32).to(gpu))
+    torch.cuda.synchronize()
+    assert not np.array_equal(_bits(a), _bits(qkv))
+    assert np.array_equal(_bits(a), _bits(b))

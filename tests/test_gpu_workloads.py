@@ -22,7 +22,7 @@ TDT = {"bf16": torch.bfloat16, "fp32": torch.float32, "fp8": torch.float8_e4m3fn
 
 def build(w, gpu, seed=0):
     """Device tensors of a workload.  KV values come from N(0, value_std); quantised pools are
-    written by quant_to_paged_cache from bf16 sources that are kept for the bit-exact check."""
+    written by quant_to_paged_cache from fp32 sources that are kept for the bit-exact check."""
     seq_lens = workloads.make_seq_lens(w, seed)
     table, num_blocks, lists = workloads.make_block_tables(w, seq_lens, seed)
     gen = torch.Generator(device=gpu).manual_seed(100 + seed)
@@ -44,8 +44,9 @@ def build(w, gpu, seed=0):
         for s0 in range(0, total, chunk):
             t = min(chunk, total - s0)
             g2 = torch.Generator(device=gpu).manual_seed(7919 * (s0 // chunk) + seed)
-            src_k = torch.randn(t, w.num_kv_heads, w.head_dim, device=gpu, dtype=torch.bfloat16, generator=g2)
-            src_v = torch.randn(t, w.num_kv_heads, w.head_dim, device=gpu, dtype=torch.bfloat16, generator=g2)
+            # generated in fp32, then quantised per token and head (as the fp8 workload is defined)
+            src_k = torch.randn(t, w.num_kv_heads, w.head_dim, device=gpu, dtype=torch.float32, generator=g2)
+            src_v = torch.randn(t, w.num_kv_heads, w.head_dim, device=gpu, dtype=torch.float32, generator=g2)
             ops.quant_to_paged_cache(ops.ReshapePagedCacheParams(
                 key=src_k, value=src_v, k_cache=d["k"], v_cache=d["v"],
                 slot_mapping=torch.arange(s0, s0 + t, device=gpu, dtype=torch.int32),
@@ -53,7 +54,7 @@ def build(w, gpu, seed=0):
             if s0 == 0:  # keep the first chunk's sources for the bit-exact sample check
                 d["src_k0"], d["src_v0"] = src_k[:2048].cpu(), src_v[:2048].cpu()
     T = w.batch * w.q_per_seq
-    d["q"] = torch.randn(T, w.num_q_heads, w.head_dim, device=gpu, dtype=torch.float32, generator=gen).to(qdt)
+    d["q"] = (torch.randn(T, w.num_q_heads, w.head_dim, device=gpu, dtype=torch.float32, generator=gen) * w.q_std).to(qdt)
     d["block_table"] = torch.from_numpy(table).to(gpu)
     d["seq_lens_d"] = torch.from_numpy(seq_lens).to(gpu)
     return d

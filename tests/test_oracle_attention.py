@@ -324,3 +324,48 @@ def test_torch_cpu_path_quantised_and_write():
     tcp.reshape_paged_cache(torch.from_numpy(slots), torch.from_numpy(keys), torch.from_numpy(keys * 2), kc2, vc2)
     np.testing.assert_array_equal(kc2.numpy(), kc1)
     np.testing.assert_array_equal(vc2.numpy(), vc1)
+
+
+def test_quantisers_on_non_finite_rows_follow_c_fmaxf_fminf(tmp_path):
+    """NaN, +-Inf and all-zero rows: the oracle's quantiser against the clamp of
+    xllm/core/kernels/cuda/fp8_quant_utils.cuh:121-122 compiled as C (fmaxf / fminf return the other
+    operand for a NaN, so a NaN quotient saturates to +max and absmax skips NaN elements), with the
+    e4m3 encoding of the clamped value taken from torch."""
+    import ctypes
+    import os
+    import subprocess
+
+    src = os.path.join(os.path.dirname(os.path.abspath(__file__)), "quant_clamp_ref.c")
+    so = str(tmp_path / "libquant_clamp_ref.so")
+    subprocess.run(["gcc", "-O1", "-shared", "-fPIC", src, "-lm", "-o", so], check=True)
+    lib = ctypes.CDLL(so)
+    lib.ref_absmax.restype = ctypes.c_float
+    lib.ref_absmax.argtypes = [ctypes.c_void_p, ctypes.c_int]
+    lib.ref_scaled_clamp.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_float, ctypes.c_int,
+                                     ctypes.c_void_p]
+    rng = np.random.default_rng(5)
+    rows = rng.standard_normal((6, 64)).astype(np.float32)
+    rows[0, 3] = np.nan
+    rows[1, 0], rows[1, 9] = np.inf, -np.inf
+    rows[2] = 0.0
+    rows[3] = np.nan
+    rows[4, 5], rows[4, 6] = np.nan, -np.inf
+    for kind, qmax, min_scale in (("int8", 127.0, np.finfo(np.float32).eps), ("fp8", 448.0, 1.0 / (448.0 * 512.0))):
+        q, s = orc.quantize_per_token_head(rows, kind)
+        for r in range(rows.shape[0]):
+            row = np.ascontiguousarray(rows[r])
+            amax = lib.ref_absmax(row.ctypes.data, row.size)
+            scale = np.float32(max(np.float32(amax) / np.float32(qmax), np.float32(min_scale)))
+            assert s[r] == scale or (np.isinf(s[r]) and np.isinf(scale))
+            y = np.empty_like(row)
+            lib.ref_scaled_clamp(row.ctypes.data, row.size, ctypes.c_float(float(scale)), ctypes.c_float(qmax),
+                                 int(kind == "int8"), y.ctypes.data)
+            assert not np.isnan(y).any()
+            if kind == "int8":
+                np.testing.assert_array_equal(q[r], y.astype(np.int8))
+            else:
+                want = torch.from_numpy(y).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+                same = (q[r] == want) | (((q[r] & 0x7F) == 0) & ((want & 0x7F) == 0))
+                assert same.all()
+        top = 127 if kind == "int8" else 0x7E
+        assert q[0, 3] == top and q[1, 0] == top and q[1, 9] == top and (q[3] == top).all() and (q[2] == 0).all()

@@ -30,22 +30,33 @@ def _chunks(lens, c):
     return int(np.maximum(1, -(-lens // c)).sum())  # an empty sequence keeps one (empty) chunk
 
 
-# (workgroup slots, budget of a small batch, rows per item, smallest chunk, tile): the 16-row kernel, the
-# 32-row kernel, head_dim 256, head_dim 64, the generic kernel, and the largest target a caller can force
-KERNELS = [(512, 256, 32, 512, 32), (1024, 1024, 32, 512, 32), (256, 256, 32, 512, 16), (512, 256, 32, 512, 64),
-           (2048, 2048, 1, 64, 32), (4096, 2048, 32, 512, 32), (64, 32, 32, 512, 32), (1, 0, 32, 512, 32)]
+def kernels_for(rows, rng):
+    """(workgroup slots, budget of a small batch, rows per item, smallest chunk, tile) of the kernels
+    that can serve `rows` query rows per kv head: the generic kernel, the MFMA kernel for that row
+    count at head_dim 128 / 64 / 256, and a target lowered by the diagnostic option."""
+    out = [(2048, 2048, 1, 64, 32)]
+    if rows <= 16:
+        out += [(512, 256, 32, 512, 32), (512, 256, 32, 512, 64), (256, 256, 32, 512, 16)]
+    elif rows <= 32:
+        out += [(1024, 1024, 32, 512, 32), (1024, 1024, 32, 512, 64), (512, 512, 32, 512, 16)]
+    else:
+        out += [(512, 512, 128, 512, 32), (512, 512, 32, 512, 32), (256, 256, 32, 512, 16)]
+    lowered = int(rng.choice([1, 64, 200]))
+    out += [(lowered, lowered // 2, 32, 512, 32)]
+    return out
 
 
 @pytest.mark.parametrize("seed", range(6))
 def test_chunk_count_never_exceeds_the_workspace(plan, seed):
     rng = np.random.default_rng(seed)
     for _ in range(3000):
-        target, small, rows_per_item, min_chunk, tile = KERNELS[int(rng.integers(len(KERNELS)))]
         hkv = int(rng.choice([1, 2, 4, 8, 16]))
         g = int(rng.choice([1, 2, 4, 7, 8, 16]))
         n = int(rng.choice([1, 1, 2, 4, 8]))
+        choices = kernels_for(g * n, rng)
+        target, small, rows_per_item, min_chunk, tile = choices[int(rng.integers(len(choices)))]
         rg = plan.harness_row_groups(n, hkv * g, hkv, rows_per_item)
-        if rows_per_item > 1 and rg > 4:
+        if plan.harness_row_groups(n, hkv * g, hkv, 32) > 4:
             continue  # never split
         batch = int(rng.choice([1, 2, 3, 7, 24, 64, 200, 1000]))
         kind = rng.random()
@@ -63,6 +74,18 @@ def test_chunk_count_never_exceeds_the_workspace(plan, seed):
         assert c >= min_chunk and c % tile == 0
         bound = plan.harness_max_seq_chunks(batch, n, hkv * g, hkv, 128)
         assert _chunks(lens, c) <= bound, (target, small, hkv, rg, batch, total, max_len, c)
+
+
+def test_workspace_stays_within_the_shared_buffer_of_the_reference():
+    """The reference reserves 128 MiB for split-KV partials (FLAGS_flashinfer_workspace_buffer_size,
+    xllm/core/common/global_flags.cpp:564-567): every shape up to 128 query rows per kv head and
+    head_dim 256 fits a buffer of that size at batch 64."""
+    from xllm_wxh_amd import _lib
+
+    lib = _lib.load()
+    for rows, hkv, d in ((1, 8, 128), (4, 8, 128), (16, 8, 128), (32, 8, 128), (96, 8, 256), (128, 4, 256)):
+        need = lib.xllm_hip_paged_decode_workspace_bytes(64, rows, hkv, hkv, d)
+        assert 0 < need <= 128 << 20, (rows, hkv, d, need)
 
 
 def test_small_batch_choices(plan):

@@ -469,3 +469,62 @@ def test_forward_qkv_replays_under_hip_graph(gpu, shim):
         assert torch.equal(got, eager), "replay %d differs from eager" % it
         assert torch.equal(k_after, k_cache)
         _ = (k_cache[:8].float() @ torch.ones(D, 4, device=gpu)).sum().item()
+
+
+@pytest.mark.gpu
+def test_graphs_of_ascending_batch_sizes_keep_their_workspace(gpu, shim):
+    """Two decode graphs captured one after the other, the second for a larger batch (one graph per
+    batch-size bucket, xllm/core/runtime/cuda_graph_executor_impl.cpp:548-601): the workspace of a
+    stream is allocated once at a fixed capacity and never moved, so the first graph still replays
+    correctly after the second was captured and run — split sequences, i.e. plan, partials and counters
+    all live in that workspace.  A step that needs more than the capacity is refused, not grown."""
+    print("case shim graph buckets", flush=True)
+    from tests.helpers import Case
+
+    cap = shim.decode_workspace_capacity()
+    assert cap == 128 << 20
+    small = Case(2, 32, 8, 128, 16, [9000, 5000], seed=71)
+    large = Case(24, 32, 8, 128, 16, [3000 + 100 * i for i in range(24)], seed=72)
+
+    def run(case, out):
+        shim.batch_decode(case.q.view(case.B, 1, case.Hq, case.D), case.k_cache, out.view(case.B, 1, case.Hq, case.D),
+                          case.block_table, case.seq_lens, case.v_cache, None, None, None, 0, -1, case.scale, False, -1)
+
+    side = torch.cuda.Stream()
+    outs, graphs, eager = {}, {}, {}
+    for name, case in (("small", small), ("large", large)):
+        eager[name] = torch.empty_like(case.q)
+        run(case, eager[name])
+        torch.cuda.synchronize()
+        outs[name] = torch.zeros_like(case.q)
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            run(case, outs[name])  # first decode on the capture stream: its workspace is created here, before capture
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        ptr = shim.decode_workspace_ptr("cuda:0", side.cuda_stream)
+        graphs[name] = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graphs[name], stream=side):
+            run(case, outs[name])
+        assert shim.decode_workspace_ptr("cuda:0", side.cuda_stream) == ptr  # not moved by a capture
+        assert ptr != shim.decode_workspace_ptr("cuda:0", torch.cuda.current_stream().cuda_stream)  # one per stream
+    for round_ in range(3):
+        for name in ("large", "small", "small", "large"):
+            outs[name].zero_()
+            graphs[name].replay()
+            torch.cuda.synchronize()
+            assert torch.equal(outs[name], eager[name]), (round_, name)
+        # eager work of the program's own between the replays
+        _ = (small.k_cache[:8].float() @ torch.ones(128, 4, device=gpu)).sum().item()
+    # a step beyond the capacity of its stream's buffer is refused, not grown: a fresh stream gets a
+    # 1 MiB buffer here, too small for the partials of any split
+    shim.set_decode_workspace_bytes(1 << 20)
+    try:
+        tiny = torch.cuda.Stream()
+        tiny.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(tiny):
+            with pytest.raises(RuntimeError, match="set_decode_workspace_bytes"):
+                run(small, torch.empty_like(small.q))
+    finally:
+        shim.set_decode_workspace_bytes(cap)
+    torch.cuda.synchronize()

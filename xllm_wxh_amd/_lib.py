@@ -18,6 +18,9 @@ BF16, FP16, FP32, FP8_E4M3, INT8 = 0, 1, 2, 3, 4
 # xllm_hip_status
 OK, INVALID_ARGUMENT, UNSUPPORTED, WORKSPACE_TOO_SMALL, RUNTIME_ERROR = 0, 1, 2, 3, 4
 
+# xllm_hip_option
+OPTION_DECODE_FORCE_GENERIC, OPTION_DECODE_TARGET_ITEMS, OPTION_DECODE_SEPARATE_MERGE = 0, 1, 2
+
 STATUS_NAMES = {
     OK: "OK",
     INVALID_ARGUMENT: "INVALID_ARGUMENT",
@@ -41,6 +44,8 @@ EXPORTED_SYMBOLS = (
     "xllm_hip_swap_blocks",
     "xllm_hip_copy_blocks",
     "xllm_hip_gather_from_cache",
+    "xllm_hip_set_option",
+    "xllm_hip_get_option",
     "xllm_hip_last_error",
     "xllm_hip_abi_version",
     "xllm_hip_paged_decode_variant",
@@ -119,6 +124,7 @@ class RopeArgs(ctypes.Structure):
         ("positions", ctypes.c_void_p),
         ("interleave", ctypes.c_int32),
         ("round_each_op", ctypes.c_int32),
+        ("positions_int32", ctypes.c_int32),
     ]
 
 
@@ -175,6 +181,10 @@ def load():
     lib.xllm_hip_gather_from_cache.argtypes = [P(KvCacheDesc), vp, vp, i32, i64, i64, vp, vp, vp, vp, i64, i32, i32,
                                                i32, i32, vp]
     lib.xllm_hip_gather_from_cache.restype = ctypes.c_int
+    lib.xllm_hip_set_option.argtypes = [i32, i64]
+    lib.xllm_hip_set_option.restype = ctypes.c_int
+    lib.xllm_hip_get_option.argtypes = [i32]
+    lib.xllm_hip_get_option.restype = ctypes.c_int64
     lib.xllm_hip_last_error.argtypes = []
     lib.xllm_hip_last_error.restype = ctypes.c_char_p
     lib.xllm_hip_abi_version.argtypes = []

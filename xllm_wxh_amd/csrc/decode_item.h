@@ -54,7 +54,7 @@ __device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it)
     // table, whose last entries the plan may not have written: such a record is not used).
     const SeqChunk s = p.seq_chunks[it.sc < p.max_seq_chunks ? it.sc : 0];
     const PlanHeader hdr = *p.hdr;
-    if (rest * p.row_groups >= hdr.total_items) return false;
+    if (rest * p.row_groups >= hdr.total_items || it.sc >= p.max_seq_chunks) return false;
     it.b = s.seq;
     it.len = s.len;
     it.chunks = s.chunks;

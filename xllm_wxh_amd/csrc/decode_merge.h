@@ -71,7 +71,9 @@ __device__ inline void merge_row_cols(const DecodeParams& p, int b, int j, int h
     for (int u = 0; u < decltype(unroll)::value; ++u) {
       const float w = i0 + u < cnt ? weight(i0 + u) : 0.0f;
 #pragma unroll
-      for (int k = 0; k < COLS; ++k) o[k] += w != 0.0f ? w * v[u][k] : 0.0f;  // an empty chunk's row may hold anything
+      // (an empty chunk's row may hold anything; the fused multiply-add is spelled out so that every
+      // instantiation of this function rounds alike and the two merges give the same bits)
+      for (int k = 0; k < COLS; ++k) o[k] = w != 0.0f ? __builtin_fmaf(w, v[u][k], o[k]) : o[k];
     }
   };
   float m, ssum;

@@ -947,10 +947,12 @@ __global__ void __launch_bounds__(128, TOK == 0 ? 1 : 2) decode_mfma_d128_rows32
       rt.template attend<false>(tile, tb, p.scale_log2);
     }
   };
+  if (iters > 0) {  // (an item without visible tokens reads no block id: its list may be empty)
 #pragma unroll
-  for (int d = 0; d < kDepth; ++d) {
-    issue(mine[d], block_of(p, it, w_begin + d * kT + kH * rs), w_begin + d * kT);
-    blk[d] = block_of(p, it, w_begin + (kDepth + d) * kT + kH * rs);
+    for (int d = 0; d < kDepth; ++d) {
+      issue(mine[d], block_of(p, it, w_begin + d * kT + kH * rs), w_begin + d * kT);
+      blk[d] = block_of(p, it, w_begin + (kDepth + d) * kT + kH * rs);
+    }
   }
   for (int i = 0; i < iters; i += kDepth) {
     step(mine[0], blk[0], i);

@@ -24,7 +24,7 @@ namespace xllm_hip {
 constexpr int kTileTokens = 32;       // rows per MFMA tile (one token each, two at head_dim 64); chunk sizes are multiples of a tile
 constexpr int kMinChunkTokens = 512;  // smallest split worth a partial round trip (128 tokens per wave)
 constexpr int kMinChunkTokensGeneric = 64;  // the one-wave kernel: one 64-token step
-constexpr int kMaxTargetItems = 4096; // upper bound of the split target (sizes the workspace)
+constexpr int kMaxTargetItems = 2048; // largest split target of any kernel: eight one-wave items of the generic kernel per CU
 constexpr int kMaxRowsPerItem = 32;   // query rows (g * n) one work item of the MFMA decode kernels handles
 constexpr int kPrefillRowsPerItem = 128;  // ... and of the many-row (prefill) kernel, used above kPrefillMinRows rows
 constexpr int kPrefillMinRows = 32;
@@ -129,11 +129,35 @@ inline bool never_split(int q_per_seq, int num_q_heads, int num_kv_heads) {
   return row_groups(q_per_seq, num_q_heads, num_kv_heads) > kMaxRowGroupsForSplit;
 }
 
-// Sum_b ceil(L_b / C) <= sum(L)/C + B and C >= sum(L)*Hkv*RG/target, hence the bound below
-// for every target <= kMaxTargetItems.
+// Split target of each kernel: about this many work items (workgroups) per launch.  A workgroup of the
+// 16-row and the 128-row MFMA kernels is four waves, one per SIMD of a CU, and two fit on a CU (256
+// VGPRs, < 80 KiB of LDS); four two-wave workgroups of the 32-row kernel do; the generic kernel runs
+// one wave per item, eight per CU.  head_dim 256 runs one wave per SIMD: half as many workgroups.
+constexpr int kNumCUs = 256;
+inline int natural_target_items(bool mfma, int rows, bool one_wave_per_simd) {
+  int v = !mfma ? 8 * kNumCUs : (rows > 16 && rows <= kPrefillMinRows) ? 4 * kNumCUs : 2 * kNumCUs;
+  if (one_wave_per_simd) v /= 2;
+  return v;
+}
+
+// Sequence chunks any lengths can produce, for any kernel that may serve the shape (the workspace is
+// sized before the kernel is chosen).  Sum_b ceil(L_b / C) <= sum(L)/C + B, and choose_chunk keeps
+// C >= sum(L) * Hkv * RG / t with t at most the kernel's target plus a quarter, so a kernel with
+// target T and RG row groups yields at most 1.25 T / (Hkv * RG) + B chunks:
+//   generic kernel   T = 2048, one row per item: RG = rows
+//   MFMA kernels     up to 16 rows T = 512, 17..32 rows T = 1024 (RG = 1); more rows T = 512 with 128
+//                    (16-bit cache) or 32 (1-byte cache) rows per item: RG >= ceil(rows / 128)
+inline int64_t max_seq_chunks_for(int batch, int rows, int num_kv_heads) {
+  auto bound = [&](int64_t target, int64_t rg) { return (target + target / 4 + num_kv_heads * rg - 1) / (num_kv_heads * rg); };
+  const int64_t generic = bound(natural_target_items(false, rows, false), rows);
+  const int64_t mfma = bound(natural_target_items(true, rows, false),
+                             rows <= kPrefillMinRows ? 1 : (rows + kPrefillRowsPerItem - 1) / kPrefillRowsPerItem);
+  return (generic > mfma ? generic : mfma) + batch + 1;
+}
+
 inline WorkspaceLayout workspace_layout(int batch, int q_per_seq, int num_q_heads, int num_kv_heads, int head_dim) {
   WorkspaceLayout w;
-  w.max_seq_chunks = (int64_t)kMaxTargetItems / num_kv_heads + batch + 1;
+  w.max_seq_chunks = max_seq_chunks_for(batch, q_per_seq * (num_q_heads / num_kv_heads), num_kv_heads);
   if (never_split(q_per_seq, num_q_heads, num_kv_heads)) w.max_seq_chunks = batch + 1;
   size_t off = 0;
   w.header = off;

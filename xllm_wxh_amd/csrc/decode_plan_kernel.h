@@ -121,12 +121,16 @@ __global__ void __launch_bounds__(64) decode_plan_kernel(DecodeParams p) {
     wave_scan2(sf, st, lane);
     if (b < p.batch) {
       const int f0 = run_full + sf - nf;
-      for (int ci = 0; ci < nf; ++ci) p.seq_chunks[f0 + ci] = SeqChunk{b, ci, len_b, nf + nt};
+      // (the table holds every chunk any lengths can produce — see workspace_layout —; the bound is
+      // checked here all the same, so that nothing is ever written outside it)
+      for (int ci = 0; ci < nf; ++ci) {
+        if (f0 + ci < p.max_seq_chunks) p.seq_chunks[f0 + ci] = SeqChunk{b, ci, len_b, nf + nt};
+      }
       if (nt) {
         const int cls = tail_class(len_b - nf * chunk);
         const int slot = tail_hist[cls] + atomicAdd(&tail_fill[cls], 1);
         p.tail_prefix[b] = slot;
-        p.seq_chunks[total_full + slot] = SeqChunk{b, nf, len_b, nf + nt};
+        if (total_full + slot < p.max_seq_chunks) p.seq_chunks[total_full + slot] = SeqChunk{b, nf, len_b, nf + nt};
       }
     }
     run_full += __shfl(sf, 63);

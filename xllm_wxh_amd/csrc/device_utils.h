@@ -98,6 +98,25 @@ struct Elem<XLLM_HIP_INT8> {
   }
 };
 
+// ---- saturating quantisers of the KV writes ------------------------------------------------------
+// clamp(y, -m, m) = fmaxf(-m, fminf(y, m)), the order of xllm/core/kernels/cuda/fp8_quant_utils.cuh:121-122:
+// fminf / fmaxf return their other operand for a NaN, so a NaN (a NaN element, or inf / inf in a row
+// that holds an infinity) becomes +m.  The NaN case is spelled out because the compiler may fuse the
+// two operations into one median instruction, which answers a NaN with the smallest operand.
+
+// Round half to even, saturate to +-127.
+__device__ inline uint8_t quantise_int8(float y) {
+  const float r = y != y ? 127.0f : fmaxf(-127.0f, fminf(rintf(y), 127.0f));
+  return (uint8_t)(int8_t)(int)r;
+}
+
+// Saturating round-to-nearest-even float -> OCP e4m3fn byte.
+__device__ inline uint8_t quantise_fp8_e4m3(float y) {
+  y = y != y ? 448.0f : fmaxf(-448.0f, fminf(y, 448.0f));
+  const int packed = __builtin_amdgcn_cvt_pk_fp8_f32(y, y, 0, false);
+  return (uint8_t)(packed & 0xff);
+}
+
 // ---- wave-level reductions ------------------------------------------------------
 
 __device__ inline float wave_max(float v) {

@@ -59,13 +59,6 @@ __global__ void __launch_bounds__(256) reshape_paged_cache_kernel(KvWriteParams 
   }
 }
 
-// Saturating round-to-nearest-even float -> OCP e4m3fn byte.
-__device__ inline uint8_t float_to_fp8_e4m3(float x) {
-  x = fminf(fmaxf(x, -448.0f), 448.0f);  // NaN passes through fmin/fmax as the other operand -> guard below
-  const int packed = __builtin_amdgcn_cvt_pk_fp8_f32(x, x, 0, false);
-  return (uint8_t)(packed & 0xff);
-}
-
 // One wave per (token, head, K|V): absmax over head_dim, scale, quantise, scatter.
 template <int SRC_DT, int DST_DT>
 __global__ void __launch_bounds__(256) quant_to_paged_cache_kernel(KvWriteParams p) {
@@ -105,14 +98,7 @@ __global__ void __launch_bounds__(256) quant_to_paged_cache_kernel(KvWriteParams
     const int d = lane + i * 64;
     if (d < p.head_dim) {
       const float y = x[i] / scale;
-      uint8_t q;
-      if (DST_DT == XLLM_HIP_INT8) {
-        const float r = fminf(fmaxf(rintf(y), -127.0f), 127.0f);
-        q = (uint8_t)(int8_t)(int)r;
-      } else {
-        q = float_to_fp8_e4m3(y);
-      }
-      dst[d] = q;
+      dst[d] = DST_DT == XLLM_HIP_INT8 ? quantise_int8(y) : quantise_fp8_e4m3(y);
     }
   }
   if (lane == 0) {
@@ -251,12 +237,7 @@ __global__ void __launch_bounds__(256) quant_to_paged_cache_d128_kernel(KvWriteP
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
     const float y = x[e] / scale;
-    uint32_t q;
-    if (DST_DT == XLLM_HIP_INT8) {
-      q = (uint8_t)(int8_t)(int)fminf(fmaxf(rintf(y), -127.0f), 127.0f);
-    } else {
-      q = float_to_fp8_e4m3(y);
-    }
+    const uint32_t q = DST_DT == XLLM_HIP_INT8 ? quantise_int8(y) : quantise_fp8_e4m3(y);
     q2[e >> 2] |= q << (8 * (e & 3));
   }
   uint8_t* dst = (is_v ? p.v_cache : p.k_cache) + block * p.stride_block + (int64_t)h * p.stride_head +

@@ -32,6 +32,7 @@
 #include <math.h>
 #include <stdlib.h>
 
+#include <atomic>
 #include <mutex>
 #include <type_traits>
 
@@ -49,21 +50,31 @@ namespace xllm_hip {
 enum Variant { kNone = 0, kMfmaD128 = 1, kGeneric = 2, kMfmaD64 = 3, kMfmaD256 = 4 };
 static bool is_mfma(Variant v) { return v == kMfmaD128 || v == kMfmaD64 || v == kMfmaD256; }
 
-// Split target: about this many work items (workgroups) per launch.  A workgroup of the MFMA kernel
-// is four waves, one per SIMD of a CU, and two workgroups fit on a CU (256 VGPRs, < 80 KiB of LDS).
-// The generic kernel runs one wave per item.
-constexpr int kNumCUs = 256;
-
-// Work items to aim for: two 4-wave workgroups per CU for the 16-row and the 128-row MFMA kernels,
-// four 2-wave workgroups for the 32-row one, eight single waves for the generic kernel.
-static int target_items(int variant_is_mfma, int rows, bool one_wave_per_simd) {
-  int v = !variant_is_mfma ? 8 * kNumCUs : (rows > 16 && rows <= kPrefillMinRows) ? 4 * kNumCUs : 2 * kNumCUs;
-  if (one_wave_per_simd) v /= 2;  // head_dim 256: half as many workgroups fit a CU
-  if (const char* e = getenv("XLLM_HIP_DECODE_TARGET_ITEMS")) {
-    const int t = atoi(e);
-    if (t > 0) v = t;
+// Process-wide diagnostic switches (xllm_hip_set_option).  Their initial values come from the
+// environment, read once, when the first of them is used.
+struct Options {
+  std::atomic<int64_t> v[XLLM_HIP_OPTION_COUNT];
+  Options() {
+    static const char* const names[XLLM_HIP_OPTION_COUNT] = {
+        "XLLM_HIP_DECODE_FORCE_GENERIC", "XLLM_HIP_DECODE_TARGET_ITEMS", "XLLM_HIP_DECODE_SEPARATE_MERGE"};
+    for (int i = 0; i < XLLM_HIP_OPTION_COUNT; ++i) {
+      const char* e = getenv(names[i]);
+      v[i].store(e != nullptr ? atoll(e) : 0, std::memory_order_relaxed);
+    }
   }
-  return v > kMaxTargetItems ? kMaxTargetItems : v;
+};
+static Options& options() {
+  static Options o;  // (initialisation of a function-local static is thread-safe)
+  return o;
+}
+static int64_t option(int which) { return options().v[which].load(std::memory_order_relaxed); }
+
+// Work items to aim for (natural_target_items), or fewer when the diagnostic option says so: the
+// workspace is sized for the natural targets, so the option can only lower them.
+static int target_items(int variant_is_mfma, int rows, bool one_wave_per_simd) {
+  const int v = natural_target_items(variant_is_mfma != 0, rows, one_wave_per_simd);
+  const int64_t t = option(XLLM_HIP_OPTION_DECODE_TARGET_ITEMS);
+  return t > 0 && t < v ? (int)t : v;
 }
 
 static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
@@ -73,7 +84,7 @@ static Variant pick_variant(const xllm_hip_kv_cache* c, const xllm_hip_decode_ar
   // 16-bit queries; a 16-bit cache must have the queries' type
   const bool q16 = a->q_dtype == XLLM_HIP_BF16 || a->q_dtype == XLLM_HIP_FP16;
   const bool kv_ok = q16 && (c->dtype == a->q_dtype || c->dtype == XLLM_HIP_FP8_E4M3 || c->dtype == XLLM_HIP_INT8);
-  const bool force_generic = getenv("XLLM_HIP_DECODE_FORCE_GENERIC") != nullptr;
+  const bool force_generic = option(XLLM_HIP_OPTION_DECODE_FORCE_GENERIC) != 0;
   // head_dim 64 rides on the head_dim-128 kernels with two tokens per tile row: half a tile
   // (32 tokens) must then lie in one block.
   // head_dim 256 rides on them with two tile rows per token: a tile is 16 tokens.
@@ -83,8 +94,9 @@ static Variant pick_variant(const xllm_hip_kv_cache* c, const xllm_hip_decode_ar
   if (!force_generic && (d128 || d64 || d256) && kv_ok && is_pow2(c->block_size) && a->sm_scale >= 0.0f) {
     const int vec = 16 / eb;  // elements per 16-byte load
     const bool strides_ok = c->stride_block % vec == 0 && c->stride_head % vec == 0 && c->stride_slot % vec == 0 &&
-                            a->q_token_stride % 8 == 0;
-    const bool ptrs_ok = aligned16(c->k_cache) && aligned16(c->v_cache) && aligned16(a->q);
+                            a->q_token_stride % 8 == 0 && a->out_token_stride % 8 == 0;
+    // (the output rows are written as 16-byte vectors, like the query rows are read)
+    const bool ptrs_ok = aligned16(c->k_cache) && aligned16(c->v_cache) && aligned16(a->q) && aligned16(a->out);
     const int64_t lim32 = (int64_t)1 << 31;  // the kernels form block and slot offsets from 32-bit factors
     bool scales_ok = true;
     if (eb == 1) {
@@ -217,7 +229,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
   // With more rows the work of a merge is large enough to want the whole GPU: fused into the 32-row
   // kernel it made the int8 verify workload 7 % slower (401 against 377 us), the tails of all row
   // groups ending together.
-  p.fused_merge = is_mfma(variant) && p.rows <= 16 ? 1 : 0;
+  p.fused_merge = is_mfma(variant) && p.rows <= 16 && option(XLLM_HIP_OPTION_DECODE_SEPARATE_MERGE) == 0 ? 1 : 0;
   p.fixed_chunk = 0;
   if (p.direct_single && a->max_seq_len > 0 && a->total_kv_len > 0 &&
       a->max_seq_len <= choose_chunk(a->total_kv_len, a->max_seq_len, p.batch, p.num_kv_heads, p.row_groups,
@@ -321,6 +333,16 @@ extern "C" size_t xllm_hip_paged_decode_workspace_bytes(int32_t batch,
                                                         int32_t head_dim) {
   if (batch < 0 || q_per_seq < 1 || num_q_heads < 1 || num_kv_heads < 1 || head_dim < 1) return 0;
   return workspace_layout(batch, q_per_seq, num_q_heads, num_kv_heads, head_dim).total_bytes;
+}
+
+extern "C" int xllm_hip_set_option(int32_t which, int64_t value) {
+  XLLM_HIP_REQUIRE(which >= 0 && which < XLLM_HIP_OPTION_COUNT, "unknown option %d", which);
+  options().v[which].store(value, std::memory_order_relaxed);
+  return XLLM_HIP_OK;
+}
+
+extern "C" int64_t xllm_hip_get_option(int32_t which) {
+  return which >= 0 && which < XLLM_HIP_OPTION_COUNT ? option(which) : -1;
 }
 
 extern "C" const char* xllm_hip_paged_decode_variant(const xllm_hip_kv_cache* cache,

@@ -24,7 +24,8 @@ struct RopeParams {
   const void* q_weight;
   const void* k_weight;
   const void* cos_sin;  // [max_position, rotary_dim]: cos of the rotary_dim/2 frequencies, then sin
-  const int64_t* positions;
+  const void* positions;
+  int32_t positions_int32;  // nonzero: positions holds int32 entries, else int64
   const int32_t* slots;  // NULL: no cache write
   uint8_t* k_cache;
   uint8_t* v_cache;
@@ -72,13 +73,6 @@ __device__ inline float rounded(float x) {
 }
 
 enum { kNoCache = 0, kVerbatim = 1, kInt8 = 2, kFp8 = 3 };
-
-// Saturating round-to-nearest-even float -> OCP e4m3fn byte (same conversion as the quantising write).
-__device__ inline uint8_t to_fp8_e4m3(float x) {
-  x = fminf(fmaxf(x, -448.0f), 448.0f);
-  const int packed = __builtin_amdgcn_cvt_pk_fp8_f32(x, x, 0, false);
-  return (uint8_t)(packed & 0xff);
-}
 
 template <int DT, int CACHE>
 __global__ void __launch_bounds__(256) rope_kv_write_kernel(RopeParams p) {
@@ -129,7 +123,7 @@ __global__ void __launch_bounds__(256) rope_kv_write_kernel(RopeParams p) {
       if (d < D) mine[d] = x[i];
     }
     __builtin_amdgcn_wave_barrier();
-    int64_t pos = p.positions[t];
+    int64_t pos = p.positions_int32 ? (int64_t)((const int32_t*)p.positions)[t] : ((const int64_t*)p.positions)[t];
     pos = pos < 0 ? 0 : (pos >= p.max_position ? p.max_position - 1 : pos);  // never read outside the table
     const int half = R >> 1;
 #pragma unroll
@@ -201,9 +195,9 @@ __global__ void __launch_bounds__(256) rope_kv_write_kernel(RopeParams p) {
       const float y = x[i] / scale;
       uint8_t q;
       if (CACHE == kInt8) {
-        q = (uint8_t)(int8_t)(int)fminf(fmaxf(rintf(y), -127.0f), 127.0f);
+        q = quantise_int8(y);
       } else {
-        q = to_fp8_e4m3(y);
+        q = quantise_fp8_e4m3(y);
       }
       cache[row + d] = q;
     }
@@ -323,7 +317,7 @@ __global__ void __launch_bounds__(256) rope_kv_write_d128_kernel(RopeParams p, i
         if (p.per_op) x[e] = rounded<DT>(x[e]);
       }
     }
-    int64_t pos = p.positions[t];
+    int64_t pos = p.positions_int32 ? (int64_t)((const int32_t*)p.positions)[t] : ((const int64_t*)p.positions)[t];
     pos = pos < 0 ? 0 : (pos >= p.max_position ? p.max_position - 1 : pos);
     const int half = R >> 1;
     const int hl = R >> 4;  // lanes per half of the rotated range
@@ -408,9 +402,9 @@ __global__ void __launch_bounds__(256) rope_kv_write_d128_kernel(RopeParams p, i
     const float yv = x[e] / scale;
     uint32_t q;
     if (CACHE == kInt8) {
-      q = (uint8_t)(int8_t)(int)fminf(fmaxf(rintf(yv), -127.0f), 127.0f);
+      q = quantise_int8(yv);
     } else {
-      q = to_fp8_e4m3(yv);
+      q = quantise_fp8_e4m3(yv);
     }
     q2[e >> 2] |= q << (8 * (e & 3));
   }
@@ -497,6 +491,7 @@ extern "C" int xllm_hip_rope_kv_write(const xllm_hip_rope_args* a,
   p.k_weight = a->k_weight;
   p.cos_sin = a->cos_sin_cache;
   p.positions = a->positions;
+  p.positions_int32 = a->positions_int32;
   p.token_stride = a->token_stride;
   p.num_tokens = a->num_tokens;
   p.max_position = a->max_position;

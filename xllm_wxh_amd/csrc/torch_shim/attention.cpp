@@ -64,7 +64,10 @@ std::tuple<torch::Tensor, std::optional<torch::Tensor>> AttentionImpl::forward_q
   // the fused CUDA kernel serves 1-D positions with the norm weights; without them the reference
   // rotates with rope.cu, whose arithmetic rounds every operation
   const bool with_norm = q_norm_weight.has_value() && q_norm_weight->defined();
-  torch::Tensor pos = positions.to(torch::kLong).contiguous();
+  // int32 positions (what the reference's modules pass) and int64 ones are both read as they are
+  torch::Tensor pos = positions.scalar_type() == torch::kInt || positions.scalar_type() == torch::kLong
+                          ? positions.contiguous()
+                          : positions.to(torch::kLong).contiguous();
   xllm::kernel::hip::rope_kv_write(qkv, num_heads_, num_kv_heads_, head_size_, q_norm_weight, k_norm_weight, eps,
                                    cos_sin_cache, interleaved, /*round_each_op=*/!with_norm, pos, k_cache, v_cache,
                                    k_cache_scale, v_cache_scale, attn_metadata.slot_mapping);

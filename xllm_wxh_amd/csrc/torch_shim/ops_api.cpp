@@ -2,8 +2,9 @@
 
 #include <c10/hip/HIPStream.h>
 
+#include <map>
 #include <mutex>
-#include <unordered_map>
+#include <utility>
 
 #include "../../../include/xllm_hip_paged_kv.h"
 
@@ -201,13 +202,27 @@ void dequant_from_paged_cache(ReshapeFromCacheParams& params) { gather_from_cach
 
 namespace hip {
 
-torch::Tensor decode_workspace(const torch::Device& device, size_t bytes) {
-  static std::mutex mu;
-  static std::unordered_map<int, torch::Tensor> per_device;
-  std::lock_guard<std::mutex> lock(mu);
-  torch::Tensor& ws = per_device[device.index()];
-  if (!ws.defined() || (size_t)ws.numel() < bytes) {
-    ws = torch::empty({(int64_t)bytes}, torch::TensorOptions().dtype(torch::kUInt8).device(device));
+namespace {
+std::mutex workspace_mu;
+size_t workspace_capacity = 128u << 20;  // FLAGS_flashinfer_workspace_buffer_size's default
+std::map<std::pair<int, void*>, torch::Tensor> workspaces;  // (device, stream) -> buffer
+}  // namespace
+
+void set_decode_workspace_bytes(size_t bytes) {
+  std::lock_guard<std::mutex> lock(workspace_mu);
+  workspace_capacity = bytes;
+}
+
+size_t decode_workspace_capacity() {
+  std::lock_guard<std::mutex> lock(workspace_mu);
+  return workspace_capacity;
+}
+
+torch::Tensor decode_workspace(const torch::Device& device, xllm_hip_stream_t stream) {
+  std::lock_guard<std::mutex> lock(workspace_mu);
+  torch::Tensor& ws = workspaces[{(int)device.index(), stream}];
+  if (!ws.defined()) {
+    ws = torch::empty({(int64_t)workspace_capacity}, torch::TensorOptions().dtype(torch::kUInt8).device(device));
   }
   return ws;
 }
@@ -217,8 +232,13 @@ namespace {
 void run_decode(const xllm_hip_kv_cache& cache, xllm_hip_decode_args& a, const torch::Tensor& q3) {
   const size_t need =
       xllm_hip_paged_decode_workspace_bytes(a.batch, a.q_per_seq, a.num_q_heads, cache.num_kv_heads, cache.head_dim);
-  torch::Tensor ws = decode_workspace(q3.device(), need);
-  check_status(xllm_hip_paged_decode(&cache, &a, ws.data_ptr(), (size_t)ws.numel(), current_stream(q3)));
+  const xllm_hip_stream_t stream = current_stream(q3);
+  torch::Tensor ws = decode_workspace(q3.device(), stream);
+  // Never grown: a captured graph keeps the buffer's address, and a step under capture must not allocate.
+  TORCH_CHECK(need <= (size_t)ws.numel(), "this decode step needs ", need, " bytes of workspace; the buffer of this ",
+              "stream holds ", ws.numel(), " (raise it with set_decode_workspace_bytes before the first decode call ",
+              "on a stream)");
+  check_status(xllm_hip_paged_decode(&cache, &a, ws.data_ptr(), (size_t)ws.numel(), stream));
 }
 
 void fill_q_out(xllm_hip_decode_args& a, const torch::Tensor& q3, torch::Tensor& o3, int64_t q_per_seq) {
@@ -385,9 +405,9 @@ void rope_call(torch::Tensor& qkv, int64_t hq, int64_t hk, int64_t hv, int64_t h
                const torch::Tensor& cos_sin_cache, bool interleaved, bool round_each_op,
                const torch::Tensor& position_ids, const xllm_hip_kv_cache* cache, const torch::Tensor* slot_mapping) {
   TORCH_CHECK(qkv.is_cuda() && qkv.dim() == 2 && qkv.stride(1) == 1, "qkv must be a 2-D GPU tensor, rows contiguous");
-  TORCH_CHECK(position_ids.scalar_type() == torch::kLong && position_ids.dim() == 1 && position_ids.is_contiguous() &&
-                  position_ids.numel() == qkv.size(0),
-              "position_ids must be contiguous int64 [num_tokens]");
+  TORCH_CHECK((position_ids.scalar_type() == torch::kLong || position_ids.scalar_type() == torch::kInt) &&
+                  position_ids.dim() == 1 && position_ids.is_contiguous() && position_ids.numel() == qkv.size(0),
+              "position_ids must be contiguous int64 or int32 [num_tokens]");
   TORCH_CHECK(cos_sin_cache.dim() == 2 && cos_sin_cache.is_contiguous(),
               "cos_sin_cache must be contiguous [max_position, rotary_dim]");
   xllm_hip_rope_args a{};
@@ -414,7 +434,8 @@ void rope_call(torch::Tensor& qkv, int64_t hq, int64_t hk, int64_t hv, int64_t h
   a.cos_sin_dtype = dtype_code(cos_sin_cache);
   a.cos_sin_cache = cos_sin_cache.data_ptr();
   a.max_position = cos_sin_cache.size(0);
-  a.positions = position_ids.data_ptr<int64_t>();
+  a.positions = position_ids.data_ptr();
+  a.positions_int32 = position_ids.scalar_type() == torch::kInt ? 1 : 0;
   a.interleave = interleaved ? 1 : 0;
   a.round_each_op = round_each_op ? 1 : 0;
   const int32_t* slots = nullptr;

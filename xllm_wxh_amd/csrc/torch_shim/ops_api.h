@@ -156,9 +156,16 @@ void copy_blocks(const torch::Tensor& k_cache,
                  const torch::Tensor& dst_block_indices,
                  const torch::Tensor& cum_sum);
 
-// Scratch of the decode kernels for this device, grown on demand — the role of the reference's
-// FlashinferWorkspace singleton (xllm/core/layers/cuda/flashinfer_workspace.cpp:24-38).
-torch::Tensor decode_workspace(const torch::Device& device, size_t bytes);
+// Scratch of the decode kernels — the role of the reference's FlashinferWorkspace singleton
+// (xllm/core/layers/cuda/flashinfer_workspace.cpp:24-38, sized by FLAGS_flashinfer_workspace_buffer_size,
+// default 128 MiB: xllm/core/common/global_flags.cpp:564-567).  One buffer per (device, stream),
+// allocated at the capacity in force when that stream first decodes and never reallocated: a captured
+// HIP graph keeps the buffer's address, so a later, larger step must not move it, and steps on two
+// streams must not share the plan, counters and partials.  A step that needs more than the buffer
+// holds fails (TORCH_CHECK) instead of growing it.  `stream` is the hipStream_t the step runs on.
+void set_decode_workspace_bytes(size_t bytes);  // capacity of buffers created from now on
+size_t decode_workspace_capacity();
+torch::Tensor decode_workspace(const torch::Device& device, void* stream);
 
 }  // namespace hip
 }  // namespace xllm::kernel

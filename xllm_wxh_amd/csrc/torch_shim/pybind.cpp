@@ -156,6 +156,11 @@ PYBIND11_MODULE(_xllm_hip_torch, m) {
                              double eps, KVCache& kv) {
         return self.forward_qkv(md, positions, qkv, cos_sin_cache, interleaved, q_norm_weight, k_norm_weight, eps, kv);
       });
+  m.def("set_decode_workspace_bytes", [](int64_t bytes) { xllm::kernel::hip::set_decode_workspace_bytes((size_t)bytes); });
+  m.def("decode_workspace_capacity", []() { return (int64_t)xllm::kernel::hip::decode_workspace_capacity(); });
+  m.def("decode_workspace_ptr", [](const std::string& device, int64_t stream) {
+    return (int64_t)(intptr_t)xllm::kernel::hip::decode_workspace(torch::Device(device), (void*)(intptr_t)stream).data_ptr();
+  });
   m.def("fused_qk_norm_rope", [](torch::Tensor qkv, int64_t hq, int64_t hk, int64_t hv, int64_t head_dim, double eps,
                                  torch::Tensor q_weight, torch::Tensor k_weight, torch::Tensor cos_sin_cache,
                                  bool interleaved, torch::Tensor position_ids) {

@@ -57,6 +57,27 @@ def _require(cond, msg):
         raise _lib.XllmHipError(_lib.INVALID_ARGUMENT, msg)
 
 
+class option:
+    """Context manager: a process-wide diagnostic switch of the library (xllm_hip_set_option) set for
+    the duration of a block.  Names: "force_generic", "target_items", "separate_merge"."""
+
+    _IDS = {"force_generic": _lib.OPTION_DECODE_FORCE_GENERIC, "target_items": _lib.OPTION_DECODE_TARGET_ITEMS,
+            "separate_merge": _lib.OPTION_DECODE_SEPARATE_MERGE}
+
+    def __init__(self, name, value=1):
+        self.which, self.value = self._IDS[name], int(value)
+
+    def __enter__(self):
+        lib = _lib.load()
+        self.old = lib.xllm_hip_get_option(self.which)
+        _lib.check(lib.xllm_hip_set_option(self.which, self.value))
+        return self
+
+    def __exit__(self, *exc):
+        _lib.check(_lib.load().xllm_hip_set_option(self.which, self.old))
+        return False
+
+
 def _as_hnd(cache, kv_layout):
     if cache is None:
         return None
@@ -199,6 +220,7 @@ def allocate_kv_cache(shape, dtype, device, with_scales=False, skew_bytes=KV_SKE
 # ---------------------------------------------------------------------------------------
 
 _workspaces = {}
+WORKSPACE_BYTES = 128 << 20
 
 
 def decode_workspace_bytes(batch, q_per_seq, num_q_heads, num_kv_heads, head_dim):
@@ -206,13 +228,18 @@ def decode_workspace_bytes(batch, q_per_seq, num_q_heads, num_kv_heads, head_dim
 
 
 def get_workspace(device, nbytes):
-    """Process-wide scratch per device, grown on demand — the role of the reference's
-    FlashinferWorkspace singleton (xllm/core/layers/cuda/flashinfer_workspace.cpp:24-38).
-    Callers that must not allocate pass their own `workspace=` tensor instead."""
-    ws = _workspaces.get(device)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(int(nbytes), dtype=torch.uint8, device=device)
-        _workspaces[device] = ws
+    """Process-wide scratch per (device, stream) of WORKSPACE_BYTES bytes — the role of the reference's
+    FlashinferWorkspace singleton (xllm/core/layers/cuda/flashinfer_workspace.cpp:24-38; 128 MiB is the
+    default of its FLAGS_flashinfer_workspace_buffer_size).  Allocated when a stream first decodes and
+    never reallocated, so that a captured graph's workspace address stays valid; a step that needs more
+    raises.  Callers with other needs pass their own `workspace=` tensor instead."""
+    _require(nbytes <= WORKSPACE_BYTES, "this decode step needs %d bytes of workspace, the shared buffer holds %d: "
+             "pass workspace= or raise ops.WORKSPACE_BYTES before the first call on a stream" % (nbytes, WORKSPACE_BYTES))
+    key = (torch.device(device), torch.cuda.current_stream(device).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None:
+        ws = torch.empty(WORKSPACE_BYTES, dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
     return ws
 
 
@@ -476,8 +503,8 @@ def _rope_call(qkv, num_q, num_k, num_v, head_dim, eps, q_weight, k_weight, cos_
                round_each_op, cache_desc=None, slot_mapping=None):
     lib = _lib.load()
     _require(qkv.is_cuda and qkv.dim() == 2 and qkv.stride(1) == 1, "qkv must be a 2-D GPU tensor, rows contiguous")
-    _require(positions.dtype == torch.int64 and positions.dim() == 1 and positions.is_contiguous(),
-             "position_ids must be a contiguous 1-D int64 tensor")
+    _require(positions.dtype in (torch.int64, torch.int32) and positions.dim() == 1 and positions.is_contiguous(),
+             "position_ids must be a contiguous 1-D int64 or int32 tensor")
     _require(positions.numel() == qkv.size(0), "one position per token")
     _require(cos_sin_cache.dim() == 2 and cos_sin_cache.is_contiguous(), "cos_sin_cache must be [max_position, rotary_dim]")
     a = _lib.RopeArgs()
@@ -494,6 +521,7 @@ def _rope_call(qkv, num_q, num_k, num_v, head_dim, eps, q_weight, k_weight, cos_
     a.cos_sin_dtype, a.cos_sin_cache, a.max_position = _dtype_code(cos_sin_cache), cos_sin_cache.data_ptr(), \
         cos_sin_cache.size(0)
     a.positions = positions.data_ptr()
+    a.positions_int32 = int(positions.dtype == torch.int32)
     a.interleave, a.round_each_op = int(bool(interleaved)), int(bool(round_each_op))
     _lib.check(lib.xllm_hip_rope_kv_write(ctypes.byref(a), ctypes.byref(cache_desc) if cache_desc is not None else None,
                                           _ptr(slot_mapping), _stream()))

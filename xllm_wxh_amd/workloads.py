@@ -26,7 +26,8 @@ class DecodeWorkload:
     seq_len_sigma: float = 0.0
     seq_len_min: int = 1
     seq_len_max: int = 0
-    value_std: float = 1.0
+    value_std: float = 1.0       # K and V values ~ N(0, 1) * value_std
+    q_std: float = 1.0           # queries ~ N(0, 1) * q_std
     pool_blocks: int = 0         # 0: exactly the blocks the sequences need
     description: str = ""
 
@@ -54,8 +55,8 @@ WORKLOADS = {
         description="fp32, 14q/2kv, D=64, bs=16, B=4, L~U{1..512}, 256-block pool, +4-token KV write"),
     "cfg2_llama3_8b_b64_ctx4k": DecodeWorkload(
         name="cfg2_llama3_8b_b64_ctx4k", batch=64, num_q_heads=32, num_kv_heads=8, head_dim=128, block_size=16,
-        seq_len_kind="fixed", seq_len=4096, value_std=0.5,
-        description="Llama-3-8B decode: bf16, 32q/8kv, D=128, bs=16, B=64, L=4096"),
+        seq_len_kind="fixed", seq_len=4096, value_std=0.5, q_std=0.5,
+        description="Llama-3-8B decode: bf16, 32q/8kv, D=128, bs=16, B=64, L=4096, q/k/v ~ N(0,1)*0.5"),
     "cfg3_ragged_b256": DecodeWorkload(
         name="cfg3_ragged_b256", batch=256, num_q_heads=32, num_kv_heads=8, head_dim=128, block_size=128,
         seq_len_kind="lognormal", seq_len=2048, seq_len_sigma=0.8, seq_len_min=16, seq_len_max=32768,
