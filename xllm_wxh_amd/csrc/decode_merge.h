@@ -36,8 +36,10 @@ __device__ inline float load_partial(const float* ptr) {
 
 // One wave merges the partials of output row (sequence b, query token j, head): all 64 lanes call.
 // COLS: columns per lane (2 covers head_dim <= 128, 4 head_dim <= 256).
-template <int Q_DT, bool COHERENT, int COLS, int MAXB = 32>
-__device__ inline void merge_row_cols(const DecodeParams& p, int b, int j, int head, int q0, int lane) {
+// (P: DecodeParams, or DecodeParams qualified with the constant address space when the caller reads
+// its arguments straight from the kernel-argument segment.)
+template <int Q_DT, bool COHERENT, int COLS, int MAXB = 32, class P>
+__device__ inline void merge_row_cols(const P& p, int b, int j, int head, int q0, int lane) {
   const int nhq = p.n * p.num_q_heads;
   const int rem = j * p.num_q_heads + head;
   const int cnt = p.num_chunks[b];
@@ -192,8 +194,8 @@ __global__ void __launch_bounds__(64 * kMergeRowsPerBlock, 6) decode_merge_kerne
 // completed before its increment, resets the counter for the next launch and reads the partials with
 // coherent loads.  (Device-scope fences instead — cache write-back and invalidation on every
 // workgroup — made an 8 x 8192-token step three times slower.)
-template <int Q_DT, int COLS, int MAXB>
-__device__ inline void merge_if_last(const DecodeParams& p, const Item& it, int* lds_flag) {
+template <int Q_DT, int COLS, int MAXB, class P>
+__device__ inline void merge_if_last(const P& p, const Item& it, int* lds_flag) {
   if (!p.fused_merge || p.implicit_plan) return;
   const int cnt = it.chunks;
   if (p.direct_single && cnt == 1) return;  // written directly

@@ -692,6 +692,10 @@ __device__ __forceinline__ void attend_pair(RowTile<KV_DT, TOK> (&rt)[2], const 
   }
 }
 
+// The lane's index within its wave, counted afresh (after the token loop: threadIdx.x would otherwise
+// hold a register through it).
+__device__ inline int lane_id() { return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); }
+
 // End of an item: the TW waves that share a set of 16 query rows exchange (m, l, acc) through LDS
 // (each wave's own region `xch_base + wave * xch_stride` of 16 rows of head_dim floats + 16 bytes), then each finishes head_dim/TW columns:
 // a sequence that is a single chunk gets its bf16 output rows (and LSE) written directly, a split
@@ -877,9 +881,19 @@ __global__ void __launch_bounds__(64 * kWaves, decode_waves_per_simd(TOK)) decod
     blk[1] = block_of(p, it, w_begin + kT + kH);
     for (int tb = w_begin; tb < w_end; tb += kT) step(tb);
   }
-  finish_item<KV_DT, TOK, kWaves>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, 0, wave, lane, 0);
+  // The merge reads its arguments afresh from the kernel-argument segment (DecodeParams is the kernel's
+  // only argument: it sits at the start of that segment), through a pointer the compiler cannot see
+  // through: handed `p` itself, it loads every field the merge uses at the kernel's entry and keeps
+  // them in scalar registers across the token loop, which then runs out of them (scalars get parked in
+  // vector-register lanes and are fetched back with one vector operation each: 32 per tile in the
+  // 1-byte kernels).  The pointer is formed here, ahead of the end-of-item exchange, so that the
+  // loads are under way while the waves exchange their results.
+  const __attribute__((address_space(4))) DecodeParams* pm =
+      (const __attribute__((address_space(4))) DecodeParams*)__builtin_amdgcn_kernarg_segment_ptr();
+  asm volatile("" : "+s"(pm));
+  finish_item<KV_DT, TOK, kWaves>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, 0, wave, lane_id(), 0);
   // (32 rows in flight make the int8 head_dim-64 instantiation spill)
-  merge_if_last<qf16_of(KV_DT) ? XLLM_HIP_FP16 : XLLM_HIP_BF16, TOK == 0 ? 4 : 2, (TOK == 2 && quant_of(KV_DT)) ? 16 : 32>(p, it, &lds_last);
+  merge_if_last<qf16_of(KV_DT) ? XLLM_HIP_FP16 : XLLM_HIP_BF16, TOK == 0 ? 4 : 2, (TOK == 2 && quant_of(KV_DT)) ? 16 : 32>(*pm, it, &lds_last);
 }
 
 template <int KV_DT, int TOK>
@@ -959,7 +973,7 @@ __global__ void __launch_bounds__(128, TOK == 0 ? 1 : 2) decode_mfma_d128_rows32
     if (i + 1 < iters) step(mine[1], blk[1], i + 1);
   }
   __syncthreads();  // all tiles consumed before the buffers are reused for the exchange
-  finish_item<KV_DT, TOK, 1>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, rs, 0, lane, rs);
+  finish_item<KV_DT, TOK, 1>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, rs, 0, lane_id(), rs);
 }
 
 // Many query rows per kv head (prefill chunks, long verify steps) over a 16-bit cache: a workgroup is
