@@ -99,6 +99,20 @@ constexpr int kQF16 = 64;
 constexpr int kv_of(int kt) { return kt & (kQF16 - 1); }
 constexpr bool qf16_of(int kt) { return (kt & kQF16) != 0 || kv_of(kt) == XLLM_HIP_FP16; }
 constexpr bool quant_of(int kt) { return kv_of(kt) == XLLM_HIP_FP8_E4M3 || kv_of(kt) == XLLM_HIP_INT8; }
+// An int8 cache at head_dim 128: the K rows stay bytes in LDS and meet the queries in the int8 MFMA
+// (v_mfma_i32_16x16x64_i8); see RowTile.  V is still converted to fp16 for the second MFMA.
+#ifndef XLLM_HIP_RAW_K
+#define XLLM_HIP_RAW_K 1
+#endif
+constexpr bool raw_k_of(int kt, int tok) { return XLLM_HIP_RAW_K && kv_of(kt) == XLLM_HIP_INT8 && tok == 1; }
+// LDS placement of raw K rows: 128 bytes each, the eight 16-byte pieces of a row permuted by an XOR
+// whose key takes all eight values over rows r .. r+7 (the MFMA operand read: 8 lanes, same piece,
+// consecutive rows) and differs in bit 2 between rows r and r+1 (the park: 8 lanes write four
+// neighbouring pieces of two neighbouring rows).
+__device__ inline uint32_t swz_kraw(int row, int piece) {
+  return (uint32_t)(row * 128 + ((piece ^ (((row & 1) << 2) | ((row >> 1) & 3))) << 4));
+}
+typedef __attribute__((ext_vector_type(4))) int i32x4;
 
 // KvHalf<KV>: the registers that hold 16 tokens (half a tile) of K and V in flight, the per-lane
 // geometry of their loads, and how they are parked in rows 16*h .. 16*h+15 of an LDS tile.
@@ -152,7 +166,7 @@ struct KvHalf16 {
   }
   // V rows at or beyond `len` may hold anything (unwritten slots); zero them so that 0 * x stays 0.
   // (K rows need no such care: their scores are replaced by -inf.)
-  template <bool MASKED>
+  template <bool MASKED, bool RAWK = false>
   __device__ inline void park(uint8_t* tile, int h, int tok, int len, float, const Geom& g) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -262,6 +276,7 @@ struct KvHalfQuant {
     int sc_tok;       // token (of the 16 * tok) whose scale this lane carries
     bool sc_on;       // lanes 0 .. 32 * tok - 1 carry a scale: first the K scales, then the V scales
     bool sc_is_v;
+    uint32_t wkraw;   // LDS offset of raw K row krow, this lane's 16-byte piece (int8 cache, head_dim 128)
     __device__ inline void init(const DecodeParams& p, int lane) {
       const int chunk = 4 * ((lane >> 3) & 1) + (lane & 3);
       const int pair = (lane >> 2) & 1;
@@ -273,6 +288,7 @@ struct KvHalfQuant {
       gk_off = (uint32_t)((krow * tok + second) * p.stride_slot + in_tok);
       gv_off = (uint32_t)((vrow * tok + second) * p.stride_slot + in_tok);
       wk = kLdsK + swz_k(krow, 2 * chunk);
+      wkraw = kLdsK + swz_kraw(krow, chunk);
       wv = kLdsV + swz_v(vrow, 2 * chunk);
       const int per_half = 16 * tok;  // tokens per half tile
       sc_tok = lane % per_half;
@@ -311,16 +327,21 @@ struct KvHalfQuant {
     if (g.sc_on) sc = *(const float*)((const uint8_t*)sb + g.sc_g);
   }
 
-  template <bool MASKED>
+  // RAWK: the K rows are parked as they are (rows krow + 8j at 128 bytes each).
+  template <bool MASKED, bool RAWK = false>
   __device__ inline void park(uint8_t* tile, int h, int tok, int len, float scale_log2, const Geom& g) {
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       u32x4 klo, khi, vlo, vhi;
-      dequant16<KV_DT>(k[j], klo, khi);
+      if constexpr (RAWK) {
+        *(u32x4*)(tile + g.wkraw + j * 1024 + h * 2048) = k[j];
+      } else {
+        dequant16<KV_DT>(k[j], klo, khi);
+        *(u32x4*)(tile + g.k_row(j, 0, h)) = klo;
+        *(u32x4*)(tile + g.k_row(j, 1, h)) = khi;
+      }
       dequant16<KV_DT>(v[j], vlo, vhi);
       if (MASKED && tok + g.tok * (g.vrow + 4 * j) + g.second >= len) vlo = vhi = u32x4{0, 0, 0, 0};
-      *(u32x4*)(tile + g.k_row(j, 0, h)) = klo;
-      *(u32x4*)(tile + g.k_row(j, 1, h)) = khi;
       *(u32x4*)(tile + g.v_row(j, 0, h)) = vlo;
       *(u32x4*)(tile + g.v_row(j, 1, h)) = vhi;
     }
@@ -401,6 +422,12 @@ struct RowTile {
   //                                                       operand is all ones (wacc)
   // Rows zeroed because they lie past the sequence end carry weight 0 in both sums.
   static constexpr bool kOffset = kv_of(KV_DT) == XLLM_HIP_INT8;
+  // Raw K: the K rows are bytes in LDS and the scores come from the int8 MFMA.  The queries are held as
+  // two int8 parts on one scale for the whole workgroup, q = q_scale * (256 hi + lo) with
+  // q_scale = absmax / (127 * 256), |hi|, |lo| <= 127 — 16 bits against the rows' largest element —
+  // so a score is q_scale * k_scale * (256 S_hi + S_lo) with both sums exact in 32-bit integers
+  // (|S| <= 128 * 127 * 127).  q_scale rides in the per-token factor the park prepares.
+  static constexpr bool kRawK = raw_k_of(KV_DT, TOK);
   static constexpr int kD = head_dim_of(TOK);
   static constexpr int kQC = kD / 32;    // 32-element chunks of a query row
   static constexpr int kDT = TOK == 0 ? 16 : 8;  // O^T accumulator tiles
@@ -414,13 +441,51 @@ struct RowTile {
   float m_run;     // reference point of the exponents: follows the running maximum of the log2-scaled scores (of score + log2 v_scale if quantised) lazily, see softmax
   float l_run;     // this lane's share of the softmax denominator
   float s_init;    // initial value of the score accumulators: -1152 * sum_d q[r][d] (int8), else 0
+  float q_scale;   // raw K: see above; else 1
   int lim;         // tokens >= lim are invisible to the row (causal among draft tokens)
   int lo;          // tokens < lo are outside the sliding window
   uint32_t k_off0; // LDS offset of K row mi, piece kg        (piece 4c + kg: XOR c << 6)
   uint32_t v_off0; // LDS offset of the transpose read, tile 0 (tile dt: XOR dt << 5)
   int kg;
 
-  __device__ inline void init(const DecodeParams& p, const Item& it, int row_in_item, int lane) {
+  // 16 query elements (two 16-byte loads) as floats.
+  __device__ static inline void q_floats(const uint16_t* src, bool valid, float (&f)[16]) {
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      u32x4 raw = {0, 0, 0, 0};
+      if (valid) raw = *(const u32x4*)(src + 8 * half);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        if constexpr (qf16_of(KV_DT)) {
+          f[8 * half + e] = (float)__builtin_bit_cast(f16x8, raw)[e];
+        } else {
+          f[8 * half + e] = (float)__builtin_bit_cast(bf16x8, raw)[e];
+        }
+      }
+    }
+  }
+  // Raw K: largest magnitude among the wave's 16 query rows (every lane gets the wave's value).
+  __device__ inline float q_absmax(const DecodeParams& p, const Item& it, int row_in_item, int lane) const {
+    const int mi = lane & 15, kgl = lane >> 4;
+    const int row = it.rg * p.rows_per_item + row_in_item + mi;
+    const bool valid = row < it.n * p.group;
+    const int j = valid ? row / p.group : 0;
+    const int gq = valid ? row - j * p.group : 0;
+    const uint16_t* qrow = (const uint16_t*)p.q + (int64_t)(it.q0 + j) * p.q_token_stride +
+                           (int64_t)(it.hk * p.group + gq) * kD;
+    float m = 0.0f;
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      float f[16];
+      q_floats(qrow + 64 * c + 16 * kgl, valid, f);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) m = fmaxf(m, fabsf(f[e]));
+    }
+    return wave_max(m);
+  }
+
+  // `absmax`: raw K only, the largest query magnitude of the workgroup's rows (q_absmax of its waves).
+  __device__ inline void init(const DecodeParams& p, const Item& it, int row_in_item, int lane, float absmax = 0.0f) {
     const int mi = lane & 15;  // MFMA row of A / column of B and D
     kg = lane >> 4;            // k-group of the operands; row block of D
     const int row = it.rg * p.rows_per_item + row_in_item + mi;
@@ -432,8 +497,32 @@ struct RowTile {
     const uint16_t* qrow = (const uint16_t*)p.q + (int64_t)(it.q0 + j) * p.q_token_stride +
                            (int64_t)(it.hk * p.group + gq) * kD;
     float sq = 0.0f;
+    q_scale = 1.0f;
+    if constexpr (kRawK) {
+      // qf[0], qf[1]: the high parts of elements 64c + 16kg .. + 15 (c = 0, 1), sixteen bytes in the
+      // order the K bytes lie in memory; qf[2], qf[3]: the low parts.
+      const float top = fmaxf(absmax, 1e-30f);
+      const float inv = 127.0f / top;
+      q_scale = top * (1.0f / (127.0f * 256.0f));
 #pragma unroll
-    for (int c = 0; c < kQC; ++c) {
+      for (int c = 0; c < 2; ++c) {
+        float f[16];
+        q_floats(qrow + 64 * c + 16 * kg, valid, f);
+        uint32_t hi4[4] = {0, 0, 0, 0}, lo4[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const float qn = f[e] * inv;
+          const float h = fmaxf(-127.0f, fminf(rintf(qn), 127.0f));
+          const float l = fmaxf(-127.0f, fminf(rintf((qn - h) * 256.0f), 127.0f));
+          hi4[e >> 2] |= ((uint32_t)(int)h & 0xffu) << (8 * (e & 3));
+          lo4[e >> 2] |= ((uint32_t)(int)l & 0xffu) << (8 * (e & 3));
+        }
+        qf[c] = __builtin_bit_cast(Op, u32x4{hi4[0], hi4[1], hi4[2], hi4[3]});
+        qf[2 + c] = __builtin_bit_cast(Op, u32x4{lo4[0], lo4[1], lo4[2], lo4[3]});
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < (kRawK ? 0 : kQC); ++c) {
       u32x4 raw = {0, 0, 0, 0};
       if (valid) raw = *(const u32x4*)(qrow + c * 32 + kg * 8);
       if constexpr (qf16_of(KV_DT) || !f16_ops(KV_DT)) {
@@ -449,13 +538,13 @@ struct RowTile {
         for (int e = 0; e < 8; ++e) sq += (float)qf[c][e];
       }
     }
-    s_init = kOffset ? -kInt8Offset * kg_sum(sq) : 0.0f;
+    s_init = kOffset && !kRawK ? -kInt8Offset * kg_sum(sq) : 0.0f;
     m_run = -INFINITY;
     l_run = 0.0f;
     wacc = f32x4{0, 0, 0, 0};
 #pragma unroll
     for (int dt = 0; dt < kDT; ++dt) acc[dt] = f32x4{0, 0, 0, 0};
-    k_off0 = kLdsK + swz_k(mi, kg);
+    k_off0 = kLdsK + (kRawK ? swz_kraw(mi, kg) : swz_k(mi, kg));
     const int tau = 4 * kg + (mi >> 2);  // row (within 16) this lane points the transpose read at
     v_off0 = kLdsV + swz_v(tau, (mi & 3) >> 1) + (mi & 1) * 8;
   }
@@ -463,7 +552,9 @@ struct RowTile {
   static constexpr int kN = 4 * kU * kHalves;  // scores per lane and tile
   // (per-token factors of a quantised tile travel as three arrays in score order: as one struct
   // they cost registers to the point of spilling)
-  typedef f32x4 Scores[kU][2];  // head_dim 256: the two halves' shares of one score tile
+  // head_dim 256: the two halves' shares of one score tile.  Raw K: [part][half], the integer sums
+  // S_hi and S_lo as bits.
+  typedef f32x4 Scores[kRawK ? 2 : kU][2];
 
   __device__ __forceinline__ void load_factors(const uint8_t* tile, float (&kscl)[kN], float (&lv)[kN], float (&rvs)[kN]) const {
     if (!kQuant) return;
@@ -491,9 +582,21 @@ struct RowTile {
 
   // ---- S^T = K Q^T: chunk c of the rows' 128 elements, K fragments of the tile's two halves ----
   __device__ __forceinline__ void scores_init(Scores& s) const {
+    if constexpr (kRawK) {
+      s[0][0] = s[0][1] = s[1][0] = s[1][1] = f32x4{0, 0, 0, 0};  // (integer zeros)
+      return;
+    }
 #pragma unroll
     for (int u = 0; u < kU; ++u) s[u][0] = s[u][1] = f32x4{s_init, s_init, s_init, s_init};
     if (TOK == 0) s[0][1] = f32x4{0, 0, 0, 0};  // the halves are added: the offset term enters once
+  }
+  // Raw K: chunk c (0, 1) of the rows' 128 bytes against the queries' high and low parts.
+  __device__ __forceinline__ void scores_step_raw(int c, const i32x4& kf0, const i32x4& kf1, Scores& s) const {
+    const i32x4 qh = __builtin_bit_cast(i32x4, qf[c]), ql = __builtin_bit_cast(i32x4, qf[2 + c]);
+    s[0][0] = __builtin_bit_cast(f32x4, __builtin_amdgcn_mfma_i32_16x16x64_i8(kf0, qh, __builtin_bit_cast(i32x4, s[0][0]), 0, 0, 0));
+    s[0][1] = __builtin_bit_cast(f32x4, __builtin_amdgcn_mfma_i32_16x16x64_i8(kf1, qh, __builtin_bit_cast(i32x4, s[0][1]), 0, 0, 0));
+    s[1][0] = __builtin_bit_cast(f32x4, __builtin_amdgcn_mfma_i32_16x16x64_i8(kf0, ql, __builtin_bit_cast(i32x4, s[1][0]), 0, 0, 0));
+    s[1][1] = __builtin_bit_cast(f32x4, __builtin_amdgcn_mfma_i32_16x16x64_i8(kf1, ql, __builtin_bit_cast(i32x4, s[1][1]), 0, 0, 0));
   }
   __device__ __forceinline__ void scores_step(int c, const Op& kf0, const Op& kf1, Scores& s) const {
     if constexpr (TOK == 0) {
@@ -526,7 +629,14 @@ struct RowTile {
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) {
           const int i = (u * kHalves + h) * 4 + rr;
-          const float raw = TOK == 0 ? s[0][0][rr] + s[0][1][rr] : s[u][h][rr];
+          float raw;
+          if constexpr (kRawK) {
+            // (whole vectors are reinterpreted: a bit cast of one element of a vector reads element 0)
+            const i32x4 both = (__builtin_bit_cast(i32x4, s[0][h]) << 8) + __builtin_bit_cast(i32x4, s[1][h]);
+            raw = (float)both[rr];
+          } else {
+            raw = TOK == 0 ? s[0][0][rr] + s[0][1][rr] : s[u][h][rr];
+          }
           float v = kFold ? raw : kQuant ? __builtin_fmaf(raw, kscl[i], lv[i]) : raw * scale_log2;
           if (MASKED) {
             const int tok = tb + kU * (16 * h + 4 * kg + rr) + u;
@@ -627,10 +737,18 @@ struct RowTile {
     load_factors(tile, kscl, lv, rvs);
     Scores s;
     scores_init(s);
+    if constexpr (kRawK) {
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const uint32_t ko = k_off0 ^ (uint32_t)(c << 6);
-      scores_step(c, *(const Op*)(tile + ko), *(const Op*)(tile + ko + 4096), s);
+      for (int c = 0; c < 2; ++c) {
+        const uint32_t ko = k_off0 ^ (uint32_t)(c << 6);
+        scores_step_raw(c, *(const i32x4*)(tile + ko), *(const i32x4*)(tile + ko + 2048), s);
+      }
+    } else {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const uint32_t ko = k_off0 ^ (uint32_t)(c << 6);
+        scores_step(c, *(const Op*)(tile + ko), *(const Op*)(tile + ko + 4096), s);
+      }
     }
     Op pf[kU];
     float alpha;
@@ -827,7 +945,9 @@ __global__ void __launch_bounds__(64 * kWaves, decode_waves_per_simd(TOK)) decod
   uint8_t* tile = lds_all + wave * kLdsTile;  // this wave's private K/V tile
 
   RowTile<KV_DT, TOK> rt;
-  rt.init(p, it, 0, lane);
+  constexpr bool kRawK = raw_k_of(KV_DT, TOK);
+  rt.init(p, it, 0, lane, kRawK ? rt.q_absmax(p, it, 0, lane) : 0.0f);  // (the four waves hold the same rows)
+  const float park_scale = p.scale_log2 * rt.q_scale;
 
   // This wave's share of the item's tokens.
   const int t0 = first_visible_tile(p, it);
@@ -856,11 +976,11 @@ __global__ void __launch_bounds__(64 * kWaves, decode_waves_per_simd(TOK)) decod
     const int nblk0 = block_of(p, it, tb + 2 * kT);
     const int nblk1 = block_of(p, it, tb + 2 * kT + kH);
     if (masked) {
-      st[0].template park<true>(tile, 0, tb, it.len, p.scale_log2, geom);
-      st[1].template park<true>(tile, 1, tb + kH, it.len, p.scale_log2, geom);
+      st[0].template park<true, kRawK>(tile, 0, tb, it.len, park_scale, geom);
+      st[1].template park<true, kRawK>(tile, 1, tb + kH, it.len, park_scale, geom);
     } else {
-      st[0].template park<false>(tile, 0, tb, it.len, p.scale_log2, geom);
-      st[1].template park<false>(tile, 1, tb + kH, it.len, p.scale_log2, geom);
+      st[0].template park<false, kRawK>(tile, 0, tb, it.len, park_scale, geom);
+      st[1].template park<false, kRawK>(tile, 1, tb + kH, it.len, park_scale, geom);
     }
     if (tb + kT < w_end) {
       st[0].issue(p, it, tb + kT, blk[0], geom);
@@ -918,7 +1038,16 @@ __global__ void __launch_bounds__(128, TOK == 0 ? 1 : 2) decode_mfma_d128_rows32
   uint8_t* tiles = lds_all;
 
   RowTile<KV_DT, TOK> rt;
-  rt.init(p, it, 16 * rs, lane);
+  constexpr bool kRawK = raw_k_of(KV_DT, TOK);
+  float absmax = 0.0f;
+  if constexpr (kRawK) {  // one scale for the queries of both waves: they share the parked per-token factors
+    lds_ml[wave] = rt.q_absmax(p, it, 16 * rs, lane);
+    __syncthreads();
+    absmax = fmaxf(lds_ml[0], lds_ml[1]);
+    __syncthreads();
+  }
+  rt.init(p, it, 16 * rs, lane, absmax);
+  const float park_scale = p.scale_log2 * rt.q_scale;
 
   const int w_begin = first_visible_tile(p, it);
   const int w_end = it.t_end;
@@ -948,9 +1077,9 @@ __global__ void __launch_bounds__(128, TOK == 0 ? 1 : 2) decode_mfma_d128_rows32
     uint8_t* tile = tiles + (i & 1) * kLdsTile;
     const bool masked = (tb + kT > mask_hi_from) || (tb < mask_lo_until);
     if (masked) {
-      m.template park<true>(tile, rs, tb + kH * rs, it.len, p.scale_log2, geom);
+      m.template park<true, kRawK>(tile, rs, tb + kH * rs, it.len, park_scale, geom);
     } else {
-      m.template park<false>(tile, rs, tb + kH * rs, it.len, p.scale_log2, geom);
+      m.template park<false, kRawK>(tile, rs, tb + kH * rs, it.len, park_scale, geom);
     }
     issue(m, b, tb + kDepth * kT);
     b = nblk;
