@@ -177,3 +177,64 @@ def test_thirty_three_to_sixty_four_rows(gpu, g, n, D, bs, qdt):
     out_r, _, ref_r, _, _ = _run(c, counts, n) if qdt == "bf16" else (None, None, None, None, None)
     if out_r is not None:
         assert float(np.abs(out_r - ref_r).max()) <= 1.2e-2
+
+
+@pytest.mark.parametrize("kv", ["fp8", "int8"])
+@pytest.mark.parametrize("bs", [16, 128])
+@pytest.mark.parametrize("qdt", ["bf16", "fp16"])
+def test_many_row_kernel_over_one_byte_caches(gpu, kv, bs, qdt):
+    """1-byte caches at head_dim 128 with more than 32 query rows per kv head take the 128-row kernel
+    that brings raw bytes and scales to LDS and converts each tile once per row group: lengths around
+    its tile (32 tokens) and its four raw buffers, chunks that are the whole sequence, chunks shorter
+    than one row group, sequences without query tokens; then a sliding window."""
+    print("case many rows, 1-byte cache", kv, bs, qdt, flush=True)
+    lens = [1, 31, 32, 33, 95, 96, 97, 127, 128, 129, 160, 1000, 2500]
+    q_counts = [1, 31, 32, 33, 95, 9, 97, 100, 128, 129, 0, 300, 257]
+    c = Case(len(lens), 32, 8, 128, bs, lens, kv=kv, qdt=qdt, seed=61)
+    q_indptr = np.concatenate([[0], np.cumsum(q_counts)]).astype(np.int32)
+    T = int(q_indptr[-1])
+    dt = torch.bfloat16 if qdt == "bf16" else torch.float16
+    q = torch.randn(T, c.Hq, c.D, generator=torch.Generator().manual_seed(79)).to(dt)
+    qd = q.to(c.q.device)
+    for window in (-1, 75):
+        out = torch.full_like(qd, 7.0)
+        lse = torch.full((T, c.Hq), 3.0, dtype=torch.float32, device=qd.device)
+        ops.batch_decode(qd, c.k_cache, out, c.block_table, c.seq_lens, c.v_cache, lse, None, c.k_scale, c.v_scale,
+                         scale=c.scale, return_lse=True, q_per_seq=max(q_counts), kv_cache_quant_bit_size=8,
+                         q_indptr=torch.from_numpy(q_indptr).to(qd.device), window_size_left=window)
+        torch.cuda.synchronize()
+        ref, ref_lse = orc.paged_decode_ragged(q.float().numpy(), c.k_ref, c.v_ref, c.table, c.lens, q_indptr, c.scale,
+                                               window_left=window)
+        got = out.float().cpu().numpy()
+        assert not np.isnan(got).any()
+        err = float(np.abs(got - ref).max())
+        print("   window %d err %.3e" % (window, err), flush=True)
+        assert err <= 1.2e-2
+        fin = np.isfinite(ref_lse)
+        assert np.allclose(lse.cpu().numpy()[fin], ref_lse[fin], atol=2e-2)
+
+
+@pytest.mark.parametrize("kv", ["fp8", "int8"])
+def test_many_row_kernel_over_one_byte_caches_split_and_garbage(gpu, kv):
+    """33 to 128 rows per kv head over a 1-byte cache (one row group, long sequences split into chunks
+    and merged), with bytes that decode to NaN / huge values and NaN scales in every slot that no
+    sequence owns: none of it may reach the output."""
+    print("case many rows, 1-byte cache, split + garbage", kv, flush=True)
+    lens = [9000, 45, 700, 12]
+    c = Case(4, 64, 8, 128, 16, lens, n=12, kv=kv, seed=62)  # 96 rows per kv head
+    ref, lse_ref = c.oracle()
+    used = torch.zeros(c.k_cache.size(0), 16, dtype=torch.bool)
+    for b, L in enumerate(lens):
+        for t in range(L):
+            used[c.table[b, t // 16], t % 16] = True
+    mask = (~used).to(c.k_cache.device)
+    for cache in (c.k_cache, c.v_cache):
+        cache.view(torch.uint8).permute(0, 2, 1, 3)[mask] = 0x7F  # NaN in e4m3fn, 127 in int8
+    for sc in (c.k_scale, c.v_scale):
+        sc.permute(0, 2, 1)[mask] = float("nan")
+    out, lse = c.run()
+    got = out.float().cpu().numpy()
+    assert not np.isnan(got).any()
+    assert float(np.abs(got - ref).max()) <= 1.2e-2
+    fin = np.isfinite(lse_ref)
+    assert np.allclose(lse.cpu().numpy()[fin], lse_ref[fin], atol=2e-2)

@@ -413,7 +413,10 @@ constexpr int half_tokens_of(int tok) { return 16 * tok; }  // tokens between th
 constexpr int head_dim_of(int tok) { return tok == 0 ? 256 : 128 / tok; }
 constexpr int xch_row_bytes(int tok) { return head_dim_of(tok) * 4 + 16; }  // a query row in the end-of-item exchange
 
-template <int KV_DT, int TOK>
+// RAWK: see kRawK.  OFFSET / OFFSET_K: int8 V / K rows sit in LDS with the offset 1152 (see kOffset); a
+// caller that parks them as exact fp16 numbers passes false.
+template <int KV_DT, int TOK, bool RAWK = raw_k_of(KV_DT, TOK), bool OFFSET = kv_of(KV_DT) == XLLM_HIP_INT8,
+          bool OFFSET_K = OFFSET && !RAWK>
 struct RowTile {
   static constexpr bool kQuant = quant_of(KV_DT);
   // int8 rows sit in LDS as x + 1152.  With K' = K + 1152 and V' = V + 1152:
@@ -421,13 +424,14 @@ struct RowTile {
   //   sum_t w_t V_t = sum_t w_t V'_t - 1152 * sum_t w_t   sum_t w_t comes from one more MFMA whose A
   //                                                       operand is all ones (wacc)
   // Rows zeroed because they lie past the sequence end carry weight 0 in both sums.
-  static constexpr bool kOffset = kv_of(KV_DT) == XLLM_HIP_INT8;
+  static constexpr bool kOffset = OFFSET;     // V rows (costs an MFMA per tile and its accumulator, wacc)
+  static constexpr bool kOffsetK = OFFSET_K;  // K rows (costs nothing per tile: the MFMA's initial C operand)
   // Raw K: the K rows are bytes in LDS and the scores come from the int8 MFMA.  The queries are held as
   // two int8 parts on one scale for the whole workgroup, q = q_scale * (256 hi + lo) with
   // q_scale = absmax / (127 * 256), |hi|, |lo| <= 127 — 16 bits against the rows' largest element —
   // so a score is q_scale * k_scale * (256 S_hi + S_lo) with both sums exact in 32-bit integers
   // (|S| <= 128 * 127 * 127).  q_scale rides in the per-token factor the park prepares.
-  static constexpr bool kRawK = raw_k_of(KV_DT, TOK);
+  static constexpr bool kRawK = RAWK;
   static constexpr int kD = head_dim_of(TOK);
   static constexpr int kQC = kD / 32;    // 32-element chunks of a query row
   static constexpr int kDT = TOK == 0 ? 16 : 8;  // O^T accumulator tiles
@@ -533,12 +537,12 @@ struct RowTile {
 #pragma unroll
         for (int e = 0; e < 8; ++e) qf[c][e] = (_Float16)(float)qb[e];
       }
-      if constexpr (kOffset) {
+      if constexpr (kOffsetK) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) sq += (float)qf[c][e];
       }
     }
-    s_init = kOffset && !kRawK ? -kInt8Offset * kg_sum(sq) : 0.0f;
+    s_init = kOffsetK ? -kInt8Offset * kg_sum(sq) : 0.0f;
     m_run = -INFINITY;
     l_run = 0.0f;
     wacc = f32x4{0, 0, 0, 0};
@@ -580,6 +584,24 @@ struct RowTile {
     }
   }
 
+  // One of the three factor arrays (0: kscl, 1: lv, 2: rvs) alone.
+  __device__ __forceinline__ void load_factor(const uint8_t* tile, int which, float (&f)[kN]) const {
+    constexpr int kArr = 32 * kU * 4;
+#pragma unroll
+    for (int h = 0; h < kHalves; ++h) {
+      const int first = kU * (16 * h + 4 * kg) * 4;
+#pragma unroll
+      for (int v4 = 0; v4 < kU; ++v4) {
+        const f32x4 a = *(const f32x4*)(tile + kLdsSc + which * kArr + first + 16 * v4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int t = 4 * v4 + e;
+          f[((t % kU) * kHalves + h) * 4 + t / kU] = a[e];
+        }
+      }
+    }
+  }
+
   // ---- S^T = K Q^T: chunk c of the rows' 128 elements, K fragments of the tile's two halves ----
   __device__ __forceinline__ void scores_init(Scores& s) const {
     if constexpr (kRawK) {
@@ -612,16 +634,14 @@ struct RowTile {
   // Score / weight index i = (u * kHalves + h) * 4 + rr: token kU * (16h + 4kg + rr) + u of the tile.
   // Leaves the weights as B operand of the second MFMA (k-slot e = 4h + rr) in pf and the factor
   // the accumulators are to be scaled by in alpha; returns whether any row's maximum moved.
+  // First half: the scaled (and masked) scores x of the tile.  A plain tile of a 16-bit cache keeps the raw
+  // scores here (the scale is not negative: the host sends other scales to the generic kernel) and the
+  // scale rides in the FMA that forms the exponent, one operation per score less.
   template <bool MASKED>
-  __device__ __forceinline__ bool softmax(const Scores& s, const float (&kscl)[kN], const float (&lv)[kN], const float (&rvs)[kN], int tb, float scale_log2, Op (&pf)[kU],
-                                 float& alpha) {
+  __device__ __forceinline__ void scaled_scores(const Scores& s, const float (&kscl)[kN], const float (&lv)[kN], int tb,
+                                                float scale_log2, float (&x)[kN]) const {
     const float neg_inf = -INFINITY;
-    // A plain tile of a 16-bit cache: the maximum is taken over the raw scores (the scale is
-    // not negative: the host sends other scales to the generic kernel) and the scale rides in the FMA
-    // that forms the exponent, one operation per score less.
     constexpr bool kFold = !kQuant && !MASKED;
-    float x[kN];
-    float mt = neg_inf;
 #pragma unroll
     for (int u = 0; u < kU; ++u) {
 #pragma unroll
@@ -643,10 +663,20 @@ struct RowTile {
             v = (tok < lim && tok >= lo) ? v : neg_inf;
           }
           x[i] = v;
-          mt = fmaxf(mt, v);
         }
       }
     }
+  }
+
+  // Second half: running maximum, weights, denominator.
+  template <bool MASKED>
+  __device__ __forceinline__ bool weights(const float (&x)[kN], const float (&rvs)[kN], float scale_log2, Op (&pf)[kU],
+                                          float& alpha) {
+    const float neg_inf = -INFINITY;
+    constexpr bool kFold = !kQuant && !MASKED;
+    float mt = neg_inf;
+#pragma unroll
+    for (int i = 0; i < kN; ++i) mt = fmaxf(mt, x[i]);
     mt = kg_max(mt);
     if (kFold) mt *= scale_log2;
     // The reference point of the exponents follows the running maximum lazily: it moves (for every
@@ -682,6 +712,14 @@ struct RowTile {
       }
     }
     return moved;
+  }
+
+  template <bool MASKED>
+  __device__ __forceinline__ bool softmax(const Scores& s, const float (&kscl)[kN], const float (&lv)[kN], const float (&rvs)[kN], int tb, float scale_log2, Op (&pf)[kU],
+                                 float& alpha) {
+    float x[kN];
+    scaled_scores<MASKED>(s, kscl, lv, tb, scale_log2, x);
+    return weights<MASKED>(x, rvs, scale_log2, pf, alpha);
   }
 
   // ---- O^T = O^T * alpha + V^T P^T, tile dt of the rows' 128 elements ----
@@ -767,12 +805,12 @@ struct RowTile {
 
 // The same for two row tiles held by one wave (32 query rows): every K and V fragment read from
 // LDS feeds two MFMAs, which is what keeps a prefill-sized step from being bound by LDS bandwidth.
-template <bool MASKED, int KV_DT, int TOK>
-__device__ __forceinline__ void attend_pair(RowTile<KV_DT, TOK> (&rt)[2], const uint8_t* tile, int tb, float scale_log2) {
-  typedef RowTile<KV_DT, TOK> RT;
+template <bool MASKED, class RT>
+__device__ __forceinline__ void attend_pair(RT (&rt)[2], const uint8_t* tile, int tb, float scale_log2) {
+  static_assert(!RT::kRawK, "two row tiles per wave read converted K rows");
   typedef typename RT::Op Op;
   float kscl[RT::kN], lv[RT::kN], rvs[RT::kN];
-  rt[0].load_factors(tile, kscl, lv, rvs);
+  if constexpr (!RT::kQuant) rt[0].load_factors(tile, kscl, lv, rvs);  // (nothing to load)
   typename RT::Scores s0, s1;
   rt[0].scores_init(s0);
   rt[1].scores_init(s1);
@@ -783,12 +821,30 @@ __device__ __forceinline__ void attend_pair(RowTile<KV_DT, TOK> (&rt)[2], const 
     const Op kf1 = *(const Op*)(tile + ko + 4096);
     rt[0].scores_step(c, kf0, kf1, s0);
     rt[1].scores_step(c, kf0, kf1, s1);
+    if (RT::kQuant && c < 3) __builtin_amdgcn_sched_barrier(0);  // (the fragments are read as they are needed: no register to spare)
   }
   Op pf0[RT::kU], pf1[RT::kU];
   float alpha0, alpha1;
-  const bool moved0 = rt[0].template softmax<MASKED>(s0, kscl, lv, rvs, tb, scale_log2, pf0, alpha0);
-  __builtin_amdgcn_sched_barrier(0);  // one softmax at a time: interleaving the two costs registers
-  const bool moved1 = rt[1].template softmax<MASKED>(s1, kscl, lv, rvs, tb, scale_log2, pf1, alpha1);
+  bool moved0, moved1;
+  if constexpr (RT::kQuant) {
+    // The per-token factors live as briefly as they can (the kernel has no register to spare): the two
+    // that turn scores into exponents are loaded, used for both row tiles and dropped; the third is
+    // loaded for the sums.
+    float x0[RT::kN], x1[RT::kN];
+    rt[0].load_factor(tile, 0, kscl);
+    rt[0].load_factor(tile, 1, lv);
+    rt[0].template scaled_scores<MASKED>(s0, kscl, lv, tb, scale_log2, x0);
+    rt[1].template scaled_scores<MASKED>(s1, kscl, lv, tb, scale_log2, x1);
+    __builtin_amdgcn_sched_barrier(0);
+    rt[0].load_factor(tile, 2, rvs);
+    moved0 = rt[0].template weights<MASKED>(x0, rvs, scale_log2, pf0, alpha0);
+    __builtin_amdgcn_sched_barrier(0);
+    moved1 = rt[1].template weights<MASKED>(x1, rvs, scale_log2, pf1, alpha1);
+  } else {
+    moved0 = rt[0].template softmax<MASKED>(s0, kscl, lv, rvs, tb, scale_log2, pf0, alpha0);
+    __builtin_amdgcn_sched_barrier(0);  // one softmax at a time: interleaving the two costs registers
+    moved1 = rt[1].template softmax<MASKED>(s1, kscl, lv, rvs, tb, scale_log2, pf1, alpha1);
+  }
   if (moved0 || moved1) {  // the factor of a tile whose maxima stayed is exactly 1
 #pragma unroll
     for (int dt = 0; dt < 8; ++dt) {
@@ -819,10 +875,10 @@ __device__ inline int lane_id() { return (int)__builtin_amdgcn_mbcnt_hi(~0u, __b
 // a sequence that is a single chunk gets its bf16 output rows (and LSE) written directly, a split
 // sequence a normalised fp32 partial and its log2-sum-exp.  `row_set` says which 16 rows of the item
 // these are.  All waves of the workgroup must call it.
-template <int KV_DT, int TOK, int TW>
-__device__ inline void finish_item(const DecodeParams& p, const Item& it, RowTile<KV_DT, TOK>& rt, uint8_t* xch_base,
+template <int KV_DT, int TOK, int TW, class RT>
+__device__ inline void finish_item(const DecodeParams& p, const Item& it, RT& rt, uint8_t* xch_base,
                                    int xch_stride, float* lds_ml, int wave, int rs, int tw, int lane, int row_set) {
-  constexpr bool kOffset = kv_of(KV_DT) == XLLM_HIP_INT8;
+  constexpr bool kOffset = RT::kOffset;
   constexpr int kD = head_dim_of(TOK);
   constexpr int kXchRow = xch_row_bytes(TOK);
   const float neg_inf = -INFINITY;
@@ -1264,6 +1320,178 @@ __global__ void __launch_bounds__(256, 2) prefill_mfma_d128_kernel(DecodeParams 
   finish_item<KV_DT, TOK, 1>(p, it, rt[0], xch, 0, lds_ml, wave, wave, 0, lane, 2 * wave);
   __syncthreads();
   finish_item<KV_DT, TOK, 1>(p, it, rt[1], xch, 0, lds_ml, wave, wave, 0, lane, 2 * wave + 1);
+}
+
+// Many query rows per kv head over a 1-byte cache (head_dim 128): the structure of prefill_mfma_d128_kernel
+// with a conversion stage.  A tile's bytes go from global memory straight into a raw LDS buffer (16 bytes
+// per lane, each wave the eight rows of K and of V it owns, plus their fp32 scales), four raw buffers
+// rotate (tiles i+1 .. i+3 in flight); a wave then converts its own rows — it reads back exactly the bytes
+// it fetched — into one of two converted tiles in the layout the MFMA operand reads expect, with the
+// per-token factors of the softmax, the waves meet, and all four attend the converted tile with two
+// row tiles each.  The conversion is paid once per 128 query rows instead of once per 32.
+constexpr int kQuantRawTile = 8192 + 1024;  // K and V bytes of 32 tokens, 4 x 256 bytes of scale loads
+
+#define XLLM_HIP_GLOBAL_TO_LDS_4(gptr, lptr)                                                    \
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gptr),       \
+                                   (__attribute__((address_space(3))) void*)(lptr), 4, 0, 0)
+
+template <int KV_DT>
+struct QuantPrefillLoader {
+  int wave, lane;
+
+  // Row (of the wave's eight) and 16-byte chunk of the row this lane fetches and converts: lanes in
+  // quads, so that the eight lanes of an LDS write group hold pieces of two neighbouring rows (the K
+  // swizzle then spreads them over all banks).  Recomputed at every use rather than held in registers.
+  __device__ inline void row_chunk(int& row8, int& chunk) const {
+    int l = lane;
+    asm volatile("" : "+v"(l));
+    chunk = 4 * ((l >> 3) & 1) + (l & 3);
+    row8 = 2 * (l >> 4) + ((l >> 2) & 1);
+  }
+
+  // Loads of the wave's rows of the tile starting at token tb into `raw` (in flight on return): three
+  // instructions, K bytes, V bytes, scales (lanes 0-7 the K scales of the eight tokens, 8-15 the V scales).
+  __device__ inline void issue(const DecodeParams& p, const Item& it, int tb, int blk, uint8_t* raw) const {
+    const HalfBase b = half_base(p, it, tb + 8 * wave, blk);
+    int row8, chunk;
+    row_chunk(row8, chunk);
+    const uint32_t off = (uint32_t)(row8 * p.stride_slot + chunk * 16);
+    XLLM_HIP_GLOBAL_TO_LDS_16(p.k_cache + b.elem + off, raw + 1024 * wave);
+    XLLM_HIP_GLOBAL_TO_LDS_16(p.v_cache + b.elem + off, raw + 4096 + 1024 * wave);
+    int l = lane;
+    asm volatile("" : "+v"(l));
+    const float* sp = ((l & 8) ? p.v_scale : p.k_scale) + b.scale + (int64_t)((l & 7) * p.sc_stride_slot);
+    XLLM_HIP_GLOBAL_TO_LDS_4(sp, raw + 8192 + 256 * wave);
+  }
+
+  // The wave's rows of the tile at tb: raw -> converted (K, V, per-token factors); see KvHalfQuant::park.
+  template <bool MASKED>
+  __device__ inline void convert(const uint8_t* raw, uint8_t* conv, int tb, int len, float scale_log2) const {
+    int row8, chunk;
+    row_chunk(row8, chunk);
+    const int row = 8 * wave + row8;
+    const u32x4 kraw = *(const u32x4*)(raw + 1024 * wave + lane * 16);
+    const u32x4 vraw = *(const u32x4*)(raw + 4096 + 1024 * wave + lane * 16);
+    u32x4 klo, khi, vlo, vhi;
+    dequant16<KV_DT>(kraw, klo, khi);
+    dequant16<KV_DT>(vraw, vlo, vhi);
+    if constexpr (kv_of(KV_DT) == XLLM_HIP_INT8) {
+      // 1152 + x -> x, exact in fp16 (paid once per 128 query rows here, it saves every row tile the
+      // bookkeeping of the offset: an MFMA per tile and its accumulator)
+      // (V only: the offset of the K rows leaves the scores through the MFMA's initial C operand)
+      auto exact = [](u32x4& v) { v = __builtin_bit_cast(u32x4, __builtin_bit_cast(f16x8, v) - (_Float16)kInt8Offset); };
+      exact(vlo);
+      exact(vhi);
+    }
+    if (MASKED && tb + row >= len) vlo = vhi = u32x4{0, 0, 0, 0};
+    const uint32_t ko = kLdsK + swz_k(row, 2 * chunk), vo = kLdsV + swz_v(row, 2 * chunk);
+    *(u32x4*)(conv + ko) = klo;
+    *(u32x4*)(conv + (ko ^ 16)) = khi;
+    *(u32x4*)(conv + vo) = vlo;
+    *(u32x4*)(conv + (vo ^ 16)) = vhi;
+    if (lane < 16) {
+      const float sc = *(const float*)(raw + 8192 + 256 * wave + lane * 4);
+      const int t = 8 * wave + (lane & 7);  // token of the tile
+      const bool is_v = lane >= 8;
+      const float vs = fmaxf(sc, 0x1p-100f);
+      float a = is_v ? __builtin_amdgcn_logf(vs) : sc * scale_log2;
+      float r = __builtin_amdgcn_rcpf(vs);
+      if (MASKED && tb + t >= len) a = r = 0.0f;
+      *(float*)(conv + kLdsSc + (is_v ? 128 : 0) + t * 4) = a;
+      if (is_v) *(float*)(conv + kLdsSc + 256 + t * 4) = r;
+    }
+  }
+};
+
+template <int KV_DT>
+__global__ void __launch_bounds__(256, 2) prefill_quant_d128_kernel(DecodeParams p) {
+  static_assert(quant_of(KV_DT), "16-bit caches need no conversion: prefill_mfma_d128_kernel");
+  __shared__ __attribute__((aligned(16))) uint8_t raw0[kQuantRawTile];
+  __shared__ __attribute__((aligned(16))) uint8_t raw1[kQuantRawTile];
+  __shared__ __attribute__((aligned(16))) uint8_t raw2[kQuantRawTile];
+  __shared__ __attribute__((aligned(16))) uint8_t raw3[kQuantRawTile];
+  __shared__ __attribute__((aligned(16))) uint8_t conv0[kLdsTile];
+  __shared__ __attribute__((aligned(16))) uint8_t conv1[kLdsTile];
+  __shared__ float lds_ml[4 * 16 * 2];
+  constexpr int kT = 32;
+  static_assert(2 * 16 * xch_row_bytes(1) <= kLdsTile, "two waves' end-of-item exchanges must fit a converted tile");
+
+  Item it;
+  if (!decode_item(p, blockIdx.x, it)) return;
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+
+  typedef RowTile<KV_DT, 1, false, false, kv_of(KV_DT) == XLLM_HIP_INT8> RT;
+  RT rt[2];
+  rt[0].init(p, it, 32 * wave, lane);
+  rt[1].init(p, it, 32 * wave + 16, lane);
+
+  const int rows = it.n * p.group;
+  const int r_first = it.rg * p.rows_per_item + 32 * wave;
+  const bool has_rows = r_first < rows;
+  const int r_last = min(r_first + 31, rows - 1);
+  const int lim_first = it.len - (it.n - 1 - r_first / p.group);
+  const int lim_last = has_rows ? it.len - (it.n - 1 - r_last / p.group) : 0;
+  const int lo_first = p.window_left >= 0 ? lim_first - 1 - p.window_left : 0;
+  const int lo_last = p.window_left >= 0 ? lim_last - 1 - p.window_left : 0;
+
+  const int w_begin = first_visible_tile(p, it);
+  const int w_end = it.t_end;
+  const int iters = w_end > w_begin ? (w_end - w_begin + kT - 1) / kT : 0;
+
+  QuantPrefillLoader<KV_DT> ld;
+  ld.wave = wave;
+  ld.lane = lane;
+  const int mine = 8 * wave;  // first of the tokens this wave fetches, within a tile
+
+  // Tile i: wait for this wave's three loads of it (tiles i+1 and i+2 stay in flight), convert its rows
+  // from `raw` into `conv`, meet the other waves — their rows are converted too, and everyone is done
+  // with the converted tile of step i-1 —, put tile i+3 in flight into `next` (which only this wave's
+  // conversion of step i-1 read) and attend.  Every step issues its loads, also past the item's end.
+  auto step = [&](int i, uint8_t* raw, uint8_t* next, uint8_t* conv, int& blk) {
+    const int tb = w_begin + i * kT;
+    const int nblk = block_of_const(p, it, tb + 4 * kT + mine);
+    __builtin_amdgcn_s_waitcnt(0x0f76);  // vmcnt(6)
+    if (tb + kT > it.len) {
+      ld.template convert<true>(raw, conv, tb, it.len, p.scale_log2);
+    } else {
+      ld.template convert<false>(raw, conv, tb, it.len, p.scale_log2);
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    ld.issue(p, it, tb + 3 * kT, blk, next);
+    blk = nblk;
+    if (!(tb >= lim_last || tb + kT <= lo_first)) {
+      if (tb + kT > lim_first || tb < lo_last) {
+        attend_pair<true>(rt, conv, tb, p.scale_log2);
+      } else {
+        attend_pair<false>(rt, conv, tb, p.scale_log2);
+      }
+    }
+  };
+  if (iters > 0) {
+    ld.issue(p, it, w_begin, block_of_const(p, it, w_begin + mine), raw0);
+    ld.issue(p, it, w_begin + kT, block_of_const(p, it, w_begin + kT + mine), raw1);
+    ld.issue(p, it, w_begin + 2 * kT, block_of_const(p, it, w_begin + 2 * kT + mine), raw2);
+    int blk = block_of_const(p, it, w_begin + 3 * kT + mine);
+    int i = 0;
+    for (; i + 4 <= iters; i += 4) {
+      step(i, raw0, raw3, conv0, blk);
+      step(i + 1, raw1, raw0, conv1, blk);
+      step(i + 2, raw2, raw1, conv0, blk);
+      step(i + 3, raw3, raw2, conv1, blk);
+    }
+    if (i < iters) step(i, raw0, raw3, conv0, blk);
+    if (i + 1 < iters) step(i + 1, raw1, raw0, conv1, blk);
+    if (i + 2 < iters) step(i + 2, raw2, raw1, conv0, blk);
+  }
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): nothing lands in LDS any more
+  __syncthreads();  // all tiles consumed before the buffers are reused for the exchange
+  uint8_t* xch = (wave < 2 ? conv0 : conv1) + (wave & 1) * (16 * xch_row_bytes(1));
+  finish_item<KV_DT, 1, 1>(p, it, rt[0], xch, 0, lds_ml, wave, wave, 0, lane, 2 * wave);
+  __syncthreads();
+  finish_item<KV_DT, 1, 1>(p, it, rt[1], xch, 0, lds_ml, wave, wave, 0, lane, 2 * wave + 1);
 }
 
 }  // namespace xllm_hip

@@ -198,9 +198,11 @@ static int fill_params(const xllm_hip_kv_cache* c,
   const Variant variant = pick_variant(c, a);
   // the many-row kernel moves tiles from global memory to LDS as they are: 16-bit caches only
   // (nor does head_dim 256: two row tiles of 256 elements per wave do not fit the registers)
+  // (a 1-byte cache at head_dim 128 has a many-row kernel of its own, which converts the tiles in LDS)
   p.rows_per_item = !is_mfma(variant) ? 1
-                    : (p.rows > kPrefillMinRows && !quant && variant != kMfmaD256) ? kPrefillRowsPerItem
-                                                                                   : kMaxRowsPerItem;
+                    : (p.rows > kPrefillMinRows && variant != kMfmaD256 && (!quant || variant == kMfmaD128))
+                        ? kPrefillRowsPerItem
+                        : kMaxRowsPerItem;
   p.min_chunk = is_mfma(variant) ? kMinChunkTokens : kMinChunkTokensGeneric;
   p.tok = variant == kMfmaD64 ? 2 : variant == kMfmaD256 ? 0 : 1;
   p.tile_tokens = variant == kMfmaD256 ? kTileTokens / 2 : kTileTokens * p.tok;
@@ -280,6 +282,7 @@ template <int KV_DT, int TOK>
 static void launch_mfma_tok(const DecodeParams& p, unsigned grid, hipStream_t st) {
   if (p.rows_per_item == kPrefillRowsPerItem) {
     if constexpr (!quant_of(KV_DT) && TOK != 0) prefill_mfma_d128_kernel<KV_DT, TOK><<<grid, 256, 0, st>>>(p);
+    if constexpr (quant_of(KV_DT) && TOK == 1) prefill_quant_d128_kernel<KV_DT><<<grid, 256, 0, st>>>(p);
   } else if (p.rows <= 16) {
     decode_mfma_d128_kernel<KV_DT, TOK><<<grid, 64 * kWaves, 0, st>>>(p);
   } else {

@@ -94,11 +94,11 @@ void AttentionImpl::decoder_forward(const AttentionMetadata& attn_metadata, torc
     const int64_t rows_avg = batch > 0 ? q3.size(0) * (num_heads_ / num_kv_heads_) / batch : 0;
     if (k_cache_scale.has_value() && prefill_dequant_rows_ > 0 && rows_avg >= prefill_dequant_rows_ &&
         attn_metadata.total_kv_len > 0) {
-      // Many query rows per kv head over a 1-byte cache.  Attended in place, every 32 rows stream and
-      // convert a sequence's K/V again; instead the cached ranges are dequantised once into a dense
-      // copy in the queries' type (sequence b at a block-aligned row offset, found on the device:
-      // no length is read back) and the 128-row kernel runs over that copy through a block table
-      // of consecutive blocks.  4 x 512 tokens on a 3584-token prefix, int8: 315 us in place.
+      // Very many query rows per kv head over a 1-byte cache.  Attended in place, every 128 rows stream
+      // and convert a sequence's K/V again; instead the cached ranges are dequantised once into a dense
+      // copy in the queries' type (sequence b at a block-aligned row offset, found on the device: no
+      // length is read back) and the 16-bit many-row kernel runs over that copy through a block table
+      // of consecutive blocks.
       const int64_t bs = k_cache.size(2);
       const int64_t total_blocks = (attn_metadata.total_kv_len + batch * (bs - 1)) / bs + 1;
       const auto i32 = torch::TensorOptions().dtype(torch::kInt32).device(query.device());
