@@ -51,6 +51,8 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-engine-step", action="store_true",
                     help="skip the write_plus_attend_us leg (the step through the C++ AttentionImpl under a HIP graph)")
+    ap.add_argument("--engine-layers", type=int, default=32,
+                    help="attention layers per captured model forward in the write_plus_attend_us leg")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget of the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain 1 GiB device-to-device copy a few times and exit: the known-size "
@@ -113,14 +115,17 @@ def build_pools(w, torch, ops, num_blocks, npools, device, layout="HND", skew_by
     return pools
 
 
-def engine_step_us(torch, w, pools, table, seq_lens, lists, layout, steps, device, hints):
+def engine_step_us(torch, w, pools, table, seq_lens, lists, layout, steps, device, hints, layers):
     """The step as the engine runs it, per layer: xllm::layer::AttentionImpl::forward_qkv of the C++
     libtorch shim (rotary embedding + KV write of the step's new tokens in one launch, then the decode
     attention), captured once in a HIP graph and replayed — graph mode of the reference,
-    xllm/core/runtime/cuda_graph_executor_impl.cpp:129-180,548-601.  One graph holds one step per KV pool;
-    returns microseconds per step over `steps` replayed steps.  `hints`: the metadata carries the host-side
-    max_seq_len / total_kv_len of the step (the engine knows them when it captures a batch-size bucket);
-    without them the kernel choice is independent of host values and a plan launch is part of the step."""
+    xllm/core/runtime/cuda_graph_executor_impl.cpp:129-180,548-601.  One graph holds one model forward:
+    `layers` attention layers (layer i on KV pool i mod pools) that share one AttentionMetadata, the
+    layer loop setting plan_info.layer_id (xllm/models/llm/llm_model_base.h:115) so that the split-KV
+    schedule is built at layer 0 only, as the reference plans (flashinfer_planinfo.cpp:252-253).
+    Returns microseconds per layer over at least `steps` replayed layers.  `hints`: the metadata carries
+    the host-side max_seq_len / total_kv_len of the step (the engine knows them when it captures a
+    batch-size bucket); without them the kernel choice is independent of host values."""
     import numpy as np
 
     from xllm_wxh_amd import _xllm_hip_torch as shim
@@ -142,6 +147,7 @@ def engine_step_us(torch, w, pools, table, seq_lens, lists, layout, steps, devic
     kv_cu = i32(np.concatenate([[0], np.cumsum(seq_lens.astype(np.int64))]))
     md = shim.build_decode_metadata(q_cu, kv_cu, slots, i32(table), w.q_per_seq, int(seq_lens.max()),
                                     int(seq_lens.sum()) if hints else 0)
+    md.plan_info.layer_id = 0
     if not hints:
         md.max_seq_len = max_pos  # non-zero (zero means an empty step) but not a tight bound
     hnd = (lambda t: t) if layout == "HND" else (lambda t: t.permute(0, 2, 1, 3))
@@ -151,8 +157,9 @@ def engine_step_us(torch, w, pools, table, seq_lens, lists, layout, steps, devic
     attn = shim.AttentionImpl(Hq, D, w.sm_scale, Hkv, -1)
 
     def run_all():
-        for cache in caches:
-            attn.forward_qkv(md, positions, qkv, cos_sin, False, None, None, 0.0, cache)
+        for layer in range(layers):
+            md.plan_info.layer_id = layer
+            attn.forward_qkv(md, positions, qkv, cos_sin, False, None, None, 0.0, caches[layer % len(caches)])
 
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -163,7 +170,7 @@ def engine_step_us(torch, w, pools, table, seq_lens, lists, layout, steps, devic
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph, stream=side):
         run_all()
-    replays = max(1, steps // len(caches))
+    replays = max(3, (steps + layers - 1) // layers)
     for _ in range(max(2, replays // 5)):
         graph.replay()
     torch.cuda.synchronize()
@@ -171,7 +178,7 @@ def engine_step_us(torch, w, pools, table, seq_lens, lists, layout, steps, devic
     for _ in range(replays):
         graph.replay()
     torch.cuda.synchronize()
-    return (time.perf_counter() - t0) * 1e6 / (replays * len(caches))
+    return (time.perf_counter() - t0) * 1e6 / (replays * layers)
 
 
 def main():
@@ -296,11 +303,55 @@ def main():
     torch.cuda.synchronize()
     kv_write_us = (time.perf_counter() - t2) * 1e6 / args.steps
 
+    # the schedule (plan) and the attention proper (run) on their own: an engine builds the schedule once per
+    # step, at layer 0, and every layer runs on it
+    def plan_or_run(i, plan):
+        k, v, ks, vs = pools[i % len(pools)]
+        ops.batch_decode(q, k, out, block_table, seq_lens_d, v, None, None, ks, vs, scale=w.sm_scale,
+                         q_per_seq=w.q_per_seq, workspace=ws, kv_cache_quant_bit_size=quant_bits,
+                         max_seq_len=int(seq_lens.max()), total_kv_len=int(seq_lens.sum()), kv_layout=args.kv_layout,
+                         plan=plan, run=not plan)
+
+    def run_loop_us():
+        for i in range(max(3, args.warmup // 2)):
+            plan_or_run(i, False)
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for i in range(args.steps):
+            plan_or_run(i, False)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t) * 1e6 / args.steps
+
+    def plan_graph_us(reps=50):
+        # a plan is a few microseconds of GPU time, less than the binding's launch cost: 50 of them in a graph
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        anchor = torch.zeros(64, device=device)
+        with torch.cuda.graph(graph, stream=side):
+            anchor.add_(1.0)  # (a plan may launch nothing: the graph is never empty)
+            for i in range(reps):
+                plan_or_run(i, True)
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(10):
+            graph.replay()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t) * 1e6 / (10 * reps)
+
+    plan_or_run(0, True)
+    run_us = run_loop_us()
+    plan_us = plan_graph_us()
+    plan_or_run(0, True)
+
     engine_us = engine_no_hints_us = None
     if io_dtype == torch.bfloat16 and not args.no_engine_step:
-        engine_us = engine_step_us(torch, w, pools, table, seq_lens, lists, args.kv_layout, args.steps, device, True)
+        engine_us = engine_step_us(torch, w, pools, table, seq_lens, lists, args.kv_layout, args.steps, device, True,
+                                   args.engine_layers)
         engine_no_hints_us = engine_step_us(torch, w, pools, table, seq_lens, lists, args.kv_layout, args.steps, device,
-                                            False)
+                                            False, args.engine_layers)
 
     alg_bytes = workloads.algorithmic_bytes(w, seq_lens)
     achieved_gbps = alg_bytes / us_per_step / 1e3
@@ -356,12 +407,21 @@ def main():
         "kv_write_us": round(kv_write_us, 2),
         "kv_write_us_note": "KV write of the step's new tokens issued through the Python (ctypes) binding, one call per "
                             "step: dominated by the binding's launch cost, not by the kernel (a few microseconds)",
+        "plan_us": round(plan_us, 2),
+        "run_us": round(run_us, 2),
+        "run_pct_of_hbm_peak": round(100.0 * alg_bytes / run_us / 1e3 / HBM_PEAK_GBPS, 2),
+        "plan_run_note": "value = plan + run of every step (xllm_hip_paged_decode); plan_us: the schedule alone "
+                         "(xllm_hip_paged_decode_plan; no launch at all when the host-side lengths show that nothing "
+                         "is split), run_us: attention (+ merge) on an existing schedule (xllm_hip_paged_decode_run), "
+                         "what every layer after layer 0 costs an engine that plans once per step",
+        "engine_layers": args.engine_layers,
         "write_plus_attend_us": None if engine_us is None else round(engine_us, 2),
         "write_plus_attend_no_hints_us": None if engine_no_hints_us is None else round(engine_no_hints_us, 2),
         "write_plus_attend_note": "per layer, as the engine runs the step: C++ AttentionImpl::forward_qkv (rotary "
-                                  "embedding + KV write in one launch, then decode attention) captured once in a HIP "
-                                  "graph and replayed over the rotated pools; no_hints: metadata without the host-side "
-                                  "total_kv_len, so a plan launch is part of every step",
+                                  "embedding + KV write in one launch, then decode attention) of engine_layers "
+                                  "layers sharing one AttentionMetadata, captured once in a HIP graph and replayed "
+                                  "(layer i on pool i mod pools; the schedule is built at layer 0 only); no_hints: "
+                                  "metadata without the host-side total_kv_len",
         "roofline": {
             "bound": "hbm",
             "kernel": kernel_name,

@@ -417,7 +417,10 @@ enum xllm_hip_option {
   XLLM_HIP_OPTION_DECODE_TARGET_ITEMS = 1,   /* > 0: work items a split decode step is cut for, if that is fewer
                                               * than the kernel's own target (256 to 2048) */
   XLLM_HIP_OPTION_DECODE_SEPARATE_MERGE = 2, /* != 0: split sequences are always combined by the merge kernel */
-  XLLM_HIP_OPTION_COUNT = 3
+  XLLM_HIP_OPTION_DECODE_STORED_SCHEDULE = 3, /* != 0: a split step always stores its schedule in the workspace
+                                               * (the plan kernel), also when the host-side lengths would let
+                                               * every work item derive its chunk by itself */
+  XLLM_HIP_OPTION_COUNT = 4
 };
 int xllm_hip_set_option(int32_t which, int64_t value);
 int64_t xllm_hip_get_option(int32_t which); /* -1 for an unknown option */

@@ -789,3 +789,45 @@ def test_int8_verify_step_replays_under_hip_graph(gpu):
         for t, a in zip((k_cache, v_cache, k_scale, v_scale), after):
             assert torch.equal(t.view(torch.uint8) if t.dtype == torch.int8 else t, a.view(torch.uint8) if a.dtype == torch.int8 else a)
         _ = (k_scale[:8] * 2).sum().item()  # unrelated eager work between replays
+
+
+@pytest.mark.parametrize("kv,n,qdt", [("bf16", 1, "bf16"), ("int8", 4, "bf16"), ("fp8", 8, "bf16"), ("fp16", 2, "fp16"),
+                                      ("fp32", 1, "fp32")])
+@pytest.mark.parametrize("name,lens", [
+    ("one long sequence", [32768]),
+    ("equal lengths", [8192] * 6),
+    ("nearly equal lengths, one of them empty", [8192, 7000, 0, 8192, 8100, 7777, 8192, 8000]),
+])
+def test_split_step_without_a_stored_schedule(gpu, kv, n, qdt, name, lens):
+    """A split step whose host-side lengths (max_seq_len, total_kv_len) are nearly equal stores no
+    schedule: every work item derives its chunk from its index and the sequence's length, and no plan
+    kernel runs.  Against the oracle, bit for bit against the same step with the stored schedule
+    (which cuts the same chunks), and with host-side lengths that are wrong: a max_seq_len below the
+    longest sequence (the last chunk then takes the rest) and a total that is too small."""
+    print("case no stored schedule", kv, n, qdt, name, flush=True)
+    Hq, Hkv = (32, 8) if kv != "fp32" else (14, 2)
+    D, bs = (128, 16) if kv != "fp32" else (64, 16)
+    case = Case(len(lens), Hq, Hkv, D, bs, lens, n=n, kv=kv, qdt=qdt, seed=91)
+    ref, lse_ref = case.oracle()
+    nbytes = ops.decode_workspace_bytes(case.B, n, Hq, Hkv, D)
+    ws = torch.full((nbytes,), 0xA5, dtype=torch.uint8, device=gpu)
+    out, lse = case.run(workspace=ws, hints=True)
+    # the schedule's header (first 64 bytes of the workspace) was never written
+    assert bool((ws[:64] == 0xA5).all()), "a schedule was stored"
+    tol = {"bf16": REG_TOL, "fp16": 2e-3, "fp32": 1e-4}.get(kv, REG_TOL_QUANT)
+    assert max_abs_err(out, ref) <= tol
+    assert lse_err(lse, lse_ref) <= (LSE_TOL_INT8 if kv == "int8" else LSE_TOL)
+    with ops.option("stored_schedule"):
+        out_s, lse_s = case.run(workspace=ws, hints=True)
+    assert not bool((ws[:64] == 0xA5).all())
+    assert torch.equal(out, out_s) and torch.equal(lse, lse_s)
+    # wrong host-side lengths
+    ws.fill_(0xA5)
+    longest, total = int(max(lens)), int(sum(lens))
+    out_w, lse_w = case.run(workspace=ws, max_seq_len=max(1, longest * 3 // 4), total_kv_len=max(1, total * 3 // 4))
+    assert max_abs_err(out_w, ref) <= tol
+    assert lse_err(lse_w, lse_ref) <= (LSE_TOL_INT8 if kv == "int8" else LSE_TOL)
+    # ... and a second step on the same workspace without a plan call in between (the counters of the
+    # fused merge reset themselves)
+    out2, _ = case.run(workspace=ws, hints=True, plan=False)
+    assert torch.equal(out2, out)

@@ -80,6 +80,7 @@ def test_attention_impl_reproduces_the_reference_known_answer(gpu, fixed):
     kv_len = case.SEQ_LEN + 1
     md = shim.build_decode_metadata(i32(np.arange(case.BATCH + 1)), i32(np.arange(case.BATCH + 1) * kv_len),
                                     i32(slots), i32(table), 1, kv_len, case.BATCH * kv_len)
+    md.plan_info.layer_id = 0
     attn = shim.AttentionImpl(case.N_HEADS, case.HEAD_DIM, float(np.sqrt(1.0 / case.HEAD_DIM)), case.N_KV_HEADS, -1)
     cache = shim.KVCache(k, v, ks, vs)
     qkv = fixed["qkv"].to(gpu).clone()

@@ -41,6 +41,7 @@ def test_batch_test_known_answers(shim):
     # blocks from the first written position on: seq1 all, seq2 block 1 of 4.. , seq3 block 3.., seq4 block 1..
     assert batch.write_block_ids == {1, 2, 3, 5, 6, 7, 11, 12, 14, 15}
     md = shim.build_decode_metadata(batch, "cpu")
+    md.plan_info.layer_id = 0
     assert md.kv_seq_lens.tolist() == g["expected_kv_seq_lens_npu_layout"]
     assert md.block_table.tolist() == g["expected_block_tables"]
     assert md.slot_mapping.tolist() == g["expected_new_cache_slots"]
@@ -163,6 +164,7 @@ def test_builder_feeds_a_write_then_attend_step(gpu, shim):
         batch.add_sequence(perm[o:o + nb], l - 1, l)
         o += nb
     md = shim.build_decode_metadata(batch, "cuda:0")
+    md.plan_info.layer_id = 0
     g = torch.Generator().manual_seed(8)
     kc = torch.randn(nblocks, Hkv, bs, D, generator=g).to(torch.bfloat16)
     vc = torch.randn(nblocks, Hkv, bs, D, generator=g).to(torch.bfloat16)

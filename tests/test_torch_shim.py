@@ -25,10 +25,12 @@ def test_metadata_builder_matches_reference_known_answers(shim):
     md = shim.build_decode_metadata(i32([0, 9, 10, 11, 15]), i32([0, 9, 17, 33, 41]), i32([4, 23, 47, 56]),
                                     i32([[1, 2, 3, 0, 0], [4, 5, 6, 7, 0], [8, 9, 10, 11, 12], [13, 14, 15, 0, 0]]),
                                     9, 16, 41)
+    md.plan_info.layer_id = 0
     assert md.kv_seq_lens.tolist() == [9, 8, 16, 8]
     assert md.q_seq_lens.tolist() == [9, 1, 1, 4]
     assert md.max_seq_len == 16 and md.max_query_len == 9 and not md.is_dummy
     dummy = shim.build_decode_metadata(i32([0, 0]), i32([0, 0]), i32([0]), i32([[0]]), 0, 0, 0)
+    dummy.plan_info.layer_id = 0
     assert dummy.is_dummy and dummy.slot_mapping.tolist() == [1]
 
 
@@ -107,6 +109,7 @@ def test_attention_impl_write_then_attend(gpu, shim, kv):
     cu_kv = np.concatenate([[0], np.cumsum(lens)])
     md = shim.build_decode_metadata(i32(np.arange(B + 1)), i32(cu_kv), i32(slots), i32(table), 1, int(lens.max()),
                                     int(lens.sum()))
+    md.plan_info.layer_id = 0
     attn = shim.AttentionImpl(Hq, D, scale, Hkv, -1)
     qkv_d = qkv.to(gpu)
     out, lse = attn.forward(md, qkv_d[:, : Hq * D], qkv_d[:, Hq * D:(Hq + Hkv) * D], qkv_d[:, (Hq + Hkv) * D:], cache)
@@ -257,6 +260,7 @@ def test_attention_impl_forward_qkv_equals_separate_steps(gpu, shim, norm):
     cu_kv = np.concatenate([[0], np.cumsum(lens)])
     md = shim.build_decode_metadata(i32(np.arange(B + 1)), i32(cu_kv), i32(slots), i32(table), 1, int(lens.max()),
                                     int(lens.sum()))
+    md.plan_info.layer_id = 0
     attn = shim.AttentionImpl(Hq, D, 1.0 / float(np.sqrt(D)), Hkv, -1)
 
     a = qkv.to(gpu)
@@ -329,6 +333,7 @@ def test_attention_impl_chunked_prefill_step(gpu, shim, kv):
     i32 = lambda a: torch.tensor(np.asarray(a), dtype=torch.int32, device=gpu)
     md = shim.build_decode_metadata(i32(q_indptr), i32(np.concatenate([[0], np.cumsum(lens)])), i32(slots), i32(table),
                                     int(q_counts.max()), int(lens.max()), int(lens.sum()))
+    md.plan_info.layer_id = 0
     md.is_chunked_prefill = True
     attn = shim.AttentionImpl(Hq, D, scale, Hkv, -1)
     qkv_d = qkv.to(gpu)
@@ -386,6 +391,7 @@ def test_prefill_chunks_over_a_quantised_cache_take_the_dense_route(gpu, shim, k
     i32 = lambda a: torch.tensor(np.asarray(a), dtype=torch.int32, device=gpu)
     md = shim.build_decode_metadata(i32(q_indptr), i32(np.concatenate([[0], np.cumsum(lens)])), i32(slots), i32(table),
                                     int(q_counts.max()), int(lens.max()), int(lens.sum()))
+    md.plan_info.layer_id = 0
     md.is_chunked_prefill = True
     outs = []
     for rows in (128, 0):  # dense route, then in place
@@ -427,6 +433,7 @@ def test_forward_qkv_replays_under_hip_graph(gpu, shim):
     q_cu = torch.arange(B + 1, dtype=torch.int32, device=gpu)
     block_table = table_full.to(gpu).contiguous()
     md = shim.build_decode_metadata(q_cu, kv_cu, slots, block_table, 1, max_blocks * bs, 0)
+    md.plan_info.layer_id = 0
     kv_seq_lens = torch.ones(B, dtype=torch.int32, device=gpu)
     md.kv_seq_lens = kv_seq_lens  # persistent, refreshed in place before every replay
     attn = shim.AttentionImpl(Hq, D, 1.0 / float(np.sqrt(D)), Hkv, -1)
@@ -528,3 +535,50 @@ def test_graphs_of_ascending_batch_sizes_keep_their_workspace(gpu, shim):
     finally:
         shim.set_decode_workspace_bytes(cap)
     torch.cuda.synchronize()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kv,n", [("bf16", 1), ("int8", 4), ("fp8", 8)])
+def test_schedule_built_at_layer_zero_serves_every_layer(gpu, shim, kv, n):
+    """The layer loop of a model (xllm/models/llm/llm_model_base.h:115) sets plan_info.layer_id before
+    each layer; layer 0 builds the step's split-KV schedule and the later layers run on it
+    (xllm/core/layers/cuda/flashinfer_planinfo.cpp:252-253).  Four layers with their own caches, a batch
+    small enough to be split: every layer's output equals the one a call that plans for itself gives,
+    bit for bit; an unset layer_id and a later layer with other inputs are refused."""
+    from tests.helpers import Case
+
+    print("case shim plan once per step", kv, n, flush=True)
+    Hq, Hkv, D, bs = 32, 8, 128, 16
+    lens = [9000, 700, 4100]
+    layers = [Case(3, Hq, Hkv, D, bs, lens, n=n, kv=kv, seed=70, value_seed=70 + i) for i in range(4)]
+    c0 = layers[0]
+    q_cu = torch.arange(0, 3 * n + 1, n, dtype=torch.int32, device=gpu)
+    kv_cu = torch.tensor(np.concatenate([[0], np.cumsum(lens)]), dtype=torch.int32, device=gpu)
+    slots = torch.zeros(3 * n, dtype=torch.int32, device=gpu)
+    md = shim.build_decode_metadata(q_cu, kv_cu, slots, c0.block_table, n, max(lens), 0)
+
+    def attend(c, layer_id):
+        md.plan_info.layer_id = layer_id
+        q4 = c.q.view(3, n, Hq, D)
+        out = torch.full_like(q4, float("nan"))
+        shim.batch_decode(q4, c.k_cache, out, md.block_table, md.kv_seq_lens, c.v_cache, None, c.k_scale, c.v_scale,
+                          0, -1, c.scale, False, 8 if c.k_scale is not None else -1, plan_info=md.plan_info)
+        torch.cuda.synchronize()
+        return out
+
+    with pytest.raises(RuntimeError, match="layer_id"):
+        attend(c0, -1)
+    shared = [attend(c, i) for i, c in enumerate(layers)]
+    alone = [attend(c, 0) for c in layers]
+    for i, (a, b, c) in enumerate(zip(shared, alone, layers)):
+        assert not torch.isnan(a.float()).any()
+        assert torch.equal(a, b), "layer %d differs from a call that plans for itself" % i
+        ref, _ = c.oracle()
+        assert float(np.abs(a.float().cpu().numpy().reshape(ref.shape) - ref).max()) <= c.tol
+    # a later layer that presents another block table than layer 0's
+    attend(c0, 0)
+    other = md.block_table
+    md.block_table = other.clone()
+    with pytest.raises(RuntimeError, match="layer 0"):
+        attend(c0, 1)
+    md.block_table = other

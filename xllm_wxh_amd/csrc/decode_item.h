@@ -46,9 +46,23 @@ __device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it)
   it.sc = rest / p.num_kv_heads;
   int chunk = 0, chunk_tokens = 1 << 30;
   it.chunks = 1;
+  bool to_the_end = false;  // the chunk runs to the end of the sequence whatever its length
   if (p.implicit_plan) {
     if (it.sc >= p.batch) return false;
     it.b = it.sc;
+  } else if (p.arith_chunks > 0) {
+    // No stored schedule: slot = sequence * arith_chunks + chunk.  The block list, the queries and the
+    // length are then independent loads.  A sequence longer than its slots hold (a host-side
+    // max_seq_len that was too small) gives the rest to its last chunk.
+    it.b = it.sc / p.arith_chunks;
+    chunk = it.sc - it.b * p.arith_chunks;
+    if (it.b >= p.batch) return false;
+    it.len = kv_length(p, it.b);
+    const int cnt = chunks_of_length(it.len, p.fixed_chunk);
+    it.chunks = cnt < p.arith_chunks ? cnt : p.arith_chunks;
+    if (chunk >= it.chunks) return false;
+    chunk_tokens = p.fixed_chunk;
+    to_the_end = chunk == p.arith_chunks - 1;
   } else {
     // The header and the item's record are independent loads (the record's index is clamped to the
     // table, whose last entries the plan may not have written: such a record is not used).
@@ -73,7 +87,7 @@ __device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it)
   if (p.implicit_plan) it.len = kv_length(p, it.b);
   it.t_begin = chunk * chunk_tokens;
   const long long end = (long long)it.t_begin + chunk_tokens;
-  it.t_end = end < it.len ? (int)end : it.len;
+  it.t_end = end < it.len && !to_the_end ? (int)end : it.len;
   {  // no row of the item sees beyond the causal limit of its last row
     const int rows = it.n * p.group;
     const int last = min((it.rg + 1) * p.rows_per_item, rows) - 1;

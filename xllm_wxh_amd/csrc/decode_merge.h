@@ -42,12 +42,15 @@ template <int Q_DT, bool COHERENT, int COLS, int MAXB = 32, class P>
 __device__ inline void merge_row_cols(const P& p, int b, int j, int head, int q0, int lane) {
   const int nhq = p.n * p.num_q_heads;
   const int rem = j * p.num_q_heads + head;
-  const int cnt = p.num_chunks[b];
+  const int cnt = chunks_of_sequence(p, b);
   const int D = p.head_dim;
   const float neg_inf = -INFINITY;
-  const int f0 = p.full_prefix[b];
-  const int nf = p.full_prefix[b + 1] - f0;
-  const int tail_slot = p.hdr->total_full + p.tail_prefix[b];
+  // slot of the sequence's chunk i: its full chunks are consecutive, its tail lies among the tails; or
+  // (no stored schedule) the sequence owns arith_chunks consecutive slots
+  const bool arith = p.arith_chunks > 0;
+  const int f0 = arith ? b * p.arith_chunks : p.full_prefix[b];
+  const int nf = arith ? cnt : p.full_prefix[b + 1] - f0;
+  const int tail_slot = arith ? 0 : p.hdr->total_full + p.tail_prefix[b];
   auto partial_row = [&](int i) { return (int64_t)(i < nf ? f0 + i : tail_slot) * nhq + rem; };
 
   // Columns lane, lane + 64, ... of the output row, summed over the chunks a batch at a time: the
@@ -179,14 +182,16 @@ __global__ void __launch_bounds__(64 * kMergeRowsPerBlock, 6) decode_merge_kerne
     q0 = p.q_indptr[b];
     nb = min(p.n, p.q_indptr[b + 1] - q0);
   }
-  if (p.direct_single && p.num_chunks[b] == 1) return;  // already written by the attention kernel
+  if (p.direct_single && chunks_of_sequence(p, b) == 1) return;  // already written by the attention kernel
   const int rem = (int)(row - (int64_t)b * nhq);  // j * Hq + head
   const int j = rem / p.num_q_heads;
   if (j >= nb) return;
   merge_row<Q_DT, false>(p, b, j, rem - j * p.num_q_heads, q0, lane);
 }
 
-// Fused merge, called by every thread of a workgroup after it has written the partials of its item:
+// Fused merge, called by every thread of a workgroup (wave `wave`, lane `lane` of it: passed in, so
+// that the caller need not keep its thread index in a register through its token loop) after it has
+// written the partials of its item:
 // the workgroup that finishes the last chunk of a (sequence, kv head, row group) combines that row
 // group's partials, so no merge kernel follows.  Every wave waits until its partial stores (coherent,
 // see store_coherent) have completed, the workgroup meets, and one thread counts the chunk in with a
@@ -195,13 +200,13 @@ __global__ void __launch_bounds__(64 * kMergeRowsPerBlock, 6) decode_merge_kerne
 // coherent loads.  (Device-scope fences instead — cache write-back and invalidation on every
 // workgroup — made an 8 x 8192-token step three times slower.)
 template <int Q_DT, int COLS, int MAXB, class P>
-__device__ inline void merge_if_last(const P& p, const Item& it, int* lds_flag) {
+__device__ inline void merge_if_last(const P& p, const Item& it, int* lds_flag, int wave, int lane) {
   if (!p.fused_merge || p.implicit_plan) return;
   const int cnt = it.chunks;
   if (p.direct_single && cnt == 1) return;  // written directly
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's stores have completed
   __syncthreads();
-  if (threadIdx.x == 0) {
+  if (wave == 0 && lane == 0) {
     int32_t* c = p.counters + ((int64_t)it.b * p.num_kv_heads + it.hk) * p.row_groups + it.rg;
     const int old = __hip_atomic_fetch_add(c, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const int last = old == cnt - 1;
@@ -210,7 +215,7 @@ __device__ inline void merge_if_last(const P& p, const Item& it, int* lds_flag) 
   }
   __syncthreads();
   if (!*lds_flag) return;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nwaves = blockDim.x >> 6;
+  const int nwaves = blockDim.x >> 6;
   const int first = it.rg * p.rows_per_item;
   const int end = min(first + p.rows_per_item, it.n * p.group);
   for (int r = first + wave; r < end; r += nwaves) {

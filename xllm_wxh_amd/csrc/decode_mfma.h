@@ -1069,7 +1069,7 @@ __global__ void __launch_bounds__(64 * kWaves, decode_waves_per_simd(TOK)) decod
   asm volatile("" : "+s"(pm));
   finish_item<KV_DT, TOK, kWaves>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, 0, wave, lane_id(), 0);
   // (32 rows in flight make the int8 head_dim-64 instantiation spill)
-  merge_if_last<qf16_of(KV_DT) ? XLLM_HIP_FP16 : XLLM_HIP_BF16, TOK == 0 ? 4 : 2, (TOK == 2 && quant_of(KV_DT)) ? 16 : 32>(*pm, it, &lds_last);
+  merge_if_last<qf16_of(KV_DT) ? XLLM_HIP_FP16 : XLLM_HIP_BF16, TOK == 0 ? 4 : 2, (TOK == 2 && quant_of(KV_DT)) ? 16 : 32>(*pm, it, &lds_last, wave, lane_id());
 }
 
 template <int KV_DT, int TOK>

@@ -62,6 +62,9 @@ struct DecodeParams {
   int32_t target_items;   // workgroup slots of the launch (see choose_chunk)
   int32_t target_small;   // ... and the item budget of a batch with fewer (sequence, kv head, row group) triples
   int32_t fixed_chunk;    // > 0: chunk size chosen on the host (1 << 30 = never split)
+  int32_t arith_chunks;   // > 0: no schedule is stored.  Every sequence owns this many chunk slots of fixed_chunk
+                          // tokens (slot = sequence * arith_chunks + chunk); a work item derives its chunk, and a
+                          // merge the row's partials, from the sequence's length alone
   int32_t direct_single;  // the attention kernel writes the output rows of single-chunk sequences itself
   int32_t implicit_plan;  // nothing is split and nothing is merged: item = (sequence, kv head, row group),
                           // lengths come straight from the inputs and no plan kernel runs
@@ -73,7 +76,9 @@ struct DecodeParams {
 
 // kv length of sequence b as every kernel uses it: never negative and never beyond what the
 // sequence's block list holds, so that no block id is read from outside the list.
-__device__ inline int kv_length(const DecodeParams& p, int b) {
+// (P: DecodeParams, possibly qualified with the constant address space)
+template <class P>
+__device__ inline int kv_length(const P& p, int b) {
   int len;
   if (p.kv_indptr != nullptr) {
     const int nb = p.kv_indptr[b + 1] - p.kv_indptr[b];
@@ -85,6 +90,24 @@ __device__ inline int kv_length(const DecodeParams& p, int b) {
     len = len < p.len_cap ? len : p.len_cap;
   }
   return len > 0 ? len : 0;
+}
+
+// Chunks of a sequence of `len` tokens cut every `chunk` tokens: the full ones and a tail; an empty
+// sequence keeps one (empty) chunk, which writes zeros.
+__device__ inline int chunks_of_length(int len, int chunk) {
+  const int full = len / chunk;
+  return full + ((len - full * chunk) > 0 || len == 0 ? 1 : 0);
+}
+
+// Chunks sequence b was cut into.  Without a stored schedule: never more than the slots a sequence
+// owns (the last slot's chunk then runs to the end of the sequence, see decode_item).
+template <class P>
+__device__ inline int chunks_of_sequence(const P& p, int b) {
+  if (p.arith_chunks > 0) {
+    const int cnt = chunks_of_length(kv_length(p, b), p.fixed_chunk);
+    return cnt < p.arith_chunks ? cnt : p.arith_chunks;
+  }
+  return p.num_chunks[b];
 }
 
 // A block id as the kernels use it: within the cache, whatever the table holds.

@@ -22,6 +22,12 @@ __device__ inline void wave_scan2(int& a, int& b, int lane) {
   }
 }
 
+// The finished-chunk counters of the fused merge at the start of a step that stores no schedule.
+__global__ void __launch_bounds__(256) decode_zero_counters_kernel(int32_t* counters, int n) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) counters[i] = 0;
+}
+
 __global__ void __launch_bounds__(64) decode_plan_kernel(DecodeParams p) {
   const int lane = threadIdx.x;
   // tails by size class: how many there are, then how many have been placed

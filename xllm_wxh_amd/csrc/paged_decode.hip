@@ -56,7 +56,8 @@ struct Options {
   std::atomic<int64_t> v[XLLM_HIP_OPTION_COUNT];
   Options() {
     static const char* const names[XLLM_HIP_OPTION_COUNT] = {
-        "XLLM_HIP_DECODE_FORCE_GENERIC", "XLLM_HIP_DECODE_TARGET_ITEMS", "XLLM_HIP_DECODE_SEPARATE_MERGE"};
+        "XLLM_HIP_DECODE_FORCE_GENERIC", "XLLM_HIP_DECODE_TARGET_ITEMS", "XLLM_HIP_DECODE_SEPARATE_MERGE",
+        "XLLM_HIP_DECODE_STORED_SCHEDULE"};
     for (int i = 0; i < XLLM_HIP_OPTION_COUNT; ++i) {
       const char* e = getenv(names[i]);
       v[i].store(e != nullptr ? atoll(e) : 0, std::memory_order_relaxed);
@@ -242,6 +243,24 @@ static int fill_params(const xllm_hip_kv_cache* c,
   // partial per chunk and row would be large, so nothing is split.
   if (never_split(a->q_per_seq, a->num_q_heads, c->num_kv_heads)) p.fixed_chunk = 1 << 30;
   p.implicit_plan = p.direct_single && p.fixed_chunk == (1 << 30) ? 1 : 0;
+  // A split step whose host-side lengths are (nearly) equal needs no stored schedule: with the chunk
+  // size the device-side plan would choose from the same aggregates, every sequence owns
+  // ceil(max_seq_len / chunk) chunk slots and a work item finds its chunk from its index and the
+  // sequence's length.  No plan kernel runs, and the item's block list, queries and length are
+  // independent loads.  Not for ragged batches: the slots of the shorter sequences would be empty
+  // workgroups (at most a quarter of them may be), and the tails would not be ordered by size.
+  p.arith_chunks = 0;
+  if (p.fixed_chunk == 0 && a->max_seq_len > 0 && a->total_kv_len > 0 &&
+      option(XLLM_HIP_OPTION_DECODE_STORED_SCHEDULE) == 0) {
+    const int c = choose_chunk(a->total_kv_len, a->max_seq_len, p.batch, p.num_kv_heads, p.row_groups, p.target_items,
+                               p.target_small, p.min_chunk, p.tile_tokens);
+    const int64_t per_seq = ((int64_t)a->max_seq_len + c - 1) / c;
+    if (per_seq * p.batch <= w.max_seq_chunks && per_seq * p.batch <= INT32_MAX &&
+        (int64_t)a->max_seq_len * p.batch * 4 <= a->total_kv_len * 5) {
+      p.fixed_chunk = c;
+      p.arith_chunks = (int32_t)per_seq;
+    }
+  }
   // XCD clusters: the row groups of a (chunk, kv head); and the kv heads whose rows share 128-byte
   // lines — scale rows shorter than a line (HND: block_size * 4 bytes per head; NHD: the heads of a
   // slot are adjacent floats) or cache rows shorter than a line (NHD with 64 one-byte elements).
@@ -265,7 +284,9 @@ static int fill_params(const xllm_hip_kv_cache* c,
 static int64_t max_items(const DecodeParams& p) {
   const int64_t per = (int64_t)p.num_kv_heads * p.row_groups;
   int64_t seq_chunks = p.batch;
-  if (p.fixed_chunk != (1 << 30)) {
+  if (p.arith_chunks > 0) {
+    seq_chunks = (int64_t)p.batch * p.arith_chunks;
+  } else if (p.fixed_chunk != (1 << 30)) {
     int64_t t = 2 * (int64_t)p.target_items;  // choose_chunk may raise the target (by a quarter)
     if (t > kMaxTargetItems) t = kMaxTargetItems;
     seq_chunks = t / per + p.batch + 1;
@@ -373,6 +394,15 @@ extern "C" int xllm_hip_paged_decode_plan(const xllm_hip_kv_cache* cache,
   DecodeParams p;
   if (int s = fill_params(cache, args, workspace, workspace_bytes, p)) return s;
   if (p.batch == 0 || p.implicit_plan) return XLLM_HIP_OK;  // an unsplit step needs no schedule
+  if (p.arith_chunks > 0) {
+    // nor does one whose work items find their chunks themselves; the counters of the fused merge
+    // still start the step at zero
+    if (!p.fused_merge) return XLLM_HIP_OK;
+    const int ncounters = p.batch * p.num_kv_heads * p.row_groups;
+    decode_zero_counters_kernel<<<(unsigned)((ncounters + 255) / 256), 256, 0, (hipStream_t)stream>>>(p.counters,
+                                                                                                   ncounters);
+    return check_launch("decode_zero_counters_kernel");
+  }
   decode_plan_kernel<<<1, 64, 0, (hipStream_t)stream>>>(p);
   return check_launch("decode_plan_kernel");
 }

@@ -135,7 +135,7 @@ void AttentionImpl::decoder_forward(const AttentionMetadata& attn_metadata, torc
                                            attn_metadata.kv_seq_lens, k_cache_scale, v_cache_scale,
                                            attn_metadata.block_table, attn_metadata.max_query_len,
                                            attn_metadata.max_seq_len, scale_, sliding_window_, false,
-                                           attn_metadata.total_kv_len);
+                                           attn_metadata.total_kv_len, attn_metadata.plan_info.get());
     return;
   }
   // One decode row per query token by default (speculative verify arrives expanded into rows,
@@ -153,7 +153,7 @@ void AttentionImpl::decoder_forward(const AttentionMetadata& attn_metadata, torc
                                     output_lse, std::nullopt, k_cache_scale, v_cache_scale, std::nullopt,
                                     std::nullopt, std::nullopt, "float", attn_metadata.max_seq_len, sliding_window_,
                                     -1, scale_, false, k_cache_scale.has_value() ? 8 : -1,
-                                    attn_metadata.total_kv_len);
+                                    attn_metadata.total_kv_len, attn_metadata.plan_info.get());
   } else {
     TORCH_CHECK(attn_metadata.paged_kv_indptr.defined(), "neither block_table nor the CSR arrays are set");
     TORCH_CHECK(!k_cache_scale.has_value(), "the CSR form serves unquantised caches");
@@ -162,7 +162,8 @@ void AttentionImpl::decoder_forward(const AttentionMetadata& attn_metadata, torc
     // the CSR entry point takes the CUDA backend's NHD shape: hand it the NHD view of our HND cache
     xllm::kernel::hip::batch_decode_csr(q3, k_cache.permute({0, 2, 1, 3}), v_cache.permute({0, 2, 1, 3}),
                                         attn_metadata.paged_kv_indptr, attn_metadata.paged_kv_indices,
-                                        attn_metadata.paged_kv_last_page_len, sliding_window_, scale_, o3, output_lse);
+                                        attn_metadata.paged_kv_last_page_len, sliding_window_, scale_, o3, output_lse,
+                                        attn_metadata.plan_info.get());
   }
 }
 

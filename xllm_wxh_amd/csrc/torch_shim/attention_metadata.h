@@ -6,9 +6,14 @@
 
 #include <torch/torch.h>
 
+#include <memory>
+
 #include "host_index.h"
+#include "ops_api.h"
 
 namespace xllm::layer {
+
+using PlanInfo = xllm::kernel::hip::PlanInfo;
 
 struct AttentionMetadata {
   torch::Tensor q_cu_seq_lens;
@@ -24,6 +29,9 @@ struct AttentionMetadata {
   bool is_chunked_prefill = false;
   bool is_dummy = false;
   bool is_causal = false;
+  // Split-KV schedule of the step, built at layer 0 and shared by every layer
+  // (attention_metadata.h:112-117).  Null: every call builds its own.
+  std::shared_ptr<PlanInfo> plan_info;
   // CSR form of the block lists (the CUDA backend's inputs).
   torch::Tensor paged_kv_indptr;
   torch::Tensor paged_kv_indices;
@@ -41,6 +49,7 @@ inline AttentionMetadata build_decode_metadata(const torch::Tensor& q_cu_seq_len
                                                int64_t kv_max_seq_len,
                                                int64_t total_kv_len) {
   AttentionMetadata m;
+  m.plan_info = std::make_shared<PlanInfo>();  // layer_id -1 until the layer loop sets it (attention_metadata_builder.cpp:60)
   m.q_cu_seq_lens = q_cu_seq_lens;
   m.kv_cu_seq_lens = kv_cu_seq_lens;
   m.max_query_len = q_max_seq_len;

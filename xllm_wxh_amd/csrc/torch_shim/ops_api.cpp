@@ -229,7 +229,40 @@ torch::Tensor decode_workspace(const torch::Device& device, xllm_hip_stream_t st
 
 namespace {
 
-void run_decode(const xllm_hip_kv_cache& cache, xllm_hip_decode_args& a, const torch::Tensor& q3) {
+// What a schedule depends on (FNV-1a over the fields): a later layer must present the same.
+uint64_t plan_key(const xllm_hip_kv_cache& c, const xllm_hip_decode_args& a) {
+  const uint64_t fields[] = {(uint64_t)a.batch,
+                             (uint64_t)a.q_per_seq,
+                             (uint64_t)a.num_q_heads,
+                             (uint64_t)a.q_dtype,
+                             (uint64_t)(uintptr_t)a.block_table,
+                             (uint64_t)a.block_table_stride,
+                             (uint64_t)a.max_blocks_per_seq,
+                             (uint64_t)(uintptr_t)a.seq_lens,
+                             (uint64_t)(uintptr_t)a.kv_indptr,
+                             (uint64_t)(uintptr_t)a.kv_indices,
+                             (uint64_t)(uintptr_t)a.kv_last_page_len,
+                             (uint64_t)(uintptr_t)a.q_indptr,
+                             (uint64_t)a.max_seq_len,
+                             (uint64_t)a.total_kv_len,
+                             (uint64_t)c.dtype,
+                             (uint64_t)c.num_kv_heads,
+                             (uint64_t)c.head_dim,
+                             (uint64_t)c.block_size,
+                             (uint64_t)c.num_blocks,
+                             // the kernel family chosen (it also depends on strides and alignments)
+                             (uint64_t)(uintptr_t)xllm_hip_paged_decode_variant(&c, &a)};
+  uint64_t h = 1469598103934665603ull;
+  for (uint64_t f : fields) {
+    for (int i = 0; i < 8; ++i) {
+      h ^= (f >> (8 * i)) & 0xff;
+      h *= 1099511628211ull;
+    }
+  }
+  return h;
+}
+
+void run_decode(const xllm_hip_kv_cache& cache, xllm_hip_decode_args& a, const torch::Tensor& q3, PlanInfo* plan) {
   const size_t need =
       xllm_hip_paged_decode_workspace_bytes(a.batch, a.q_per_seq, a.num_q_heads, cache.num_kv_heads, cache.head_dim);
   const xllm_hip_stream_t stream = current_stream(q3);
@@ -238,7 +271,22 @@ void run_decode(const xllm_hip_kv_cache& cache, xllm_hip_decode_args& a, const t
   TORCH_CHECK(need <= (size_t)ws.numel(), "this decode step needs ", need, " bytes of workspace; the buffer of this ",
               "stream holds ", ws.numel(), " (raise it with set_decode_workspace_bytes before the first decode call ",
               "on a stream)");
-  check_status(xllm_hip_paged_decode(&cache, &a, ws.data_ptr(), (size_t)ws.numel(), stream));
+  if (plan == nullptr) {
+    check_status(xllm_hip_paged_decode(&cache, &a, ws.data_ptr(), (size_t)ws.numel(), stream));
+    return;
+  }
+  TORCH_CHECK(plan->layer_id != -1, "Need to set layer_id to PlanInfo.");
+  const uint64_t key = plan_key(cache, a);
+  if (plan->layer_id == 0) {
+    check_status(xllm_hip_paged_decode_plan(&cache, &a, ws.data_ptr(), (size_t)ws.numel(), stream));
+    plan->workspace = ws.data_ptr();
+    plan->key = key;
+  } else {
+    TORCH_CHECK(plan->workspace == ws.data_ptr() && plan->key == key,
+                "layer ", plan->layer_id, " presents other lengths, block lists, sizes or another stream than the ",
+                "ones the step's schedule was built for at layer 0");
+  }
+  check_status(xllm_hip_paged_decode_run(&cache, &a, ws.data_ptr(), (size_t)ws.numel(), stream));
 }
 
 void fill_q_out(xllm_hip_decode_args& a, const torch::Tensor& q3, torch::Tensor& o3, int64_t q_per_seq) {
@@ -279,7 +327,8 @@ void batch_decode(const torch::Tensor& query,
                   float scale,
                   bool return_lse,
                   int64_t kv_cache_quant_bit_size,
-                  int64_t total_kv_len) {
+                  int64_t total_kv_len,
+                  PlanInfo* plan_info) {
   TORCH_CHECK(v_cache.has_value(), "v_cache is required (single-cache MLA decode is outside this path)");
   TORCH_CHECK(!q_quant_scale.has_value() && !out_quant_scale.has_value() && !alibi_slope.has_value() &&
                   !mask.has_value(),
@@ -319,7 +368,7 @@ void batch_decode(const torch::Tensor& query,
                 "output_lse must be contiguous float32 [tokens, heads]");
     a.lse = output_lse->data_ptr<float>();
   }
-  run_decode(cache, a, q3);
+  run_decode(cache, a, q3, plan_info);
 }
 
 void batch_prefill_paged(const torch::Tensor& query, const torch::Tensor& k_cache, const torch::Tensor& v_cache,
@@ -328,7 +377,7 @@ void batch_prefill_paged(const torch::Tensor& query, const torch::Tensor& k_cach
                          const std::optional<torch::Tensor>& k_cache_quant_scale,
                          const std::optional<torch::Tensor>& v_cache_quant_scale, const torch::Tensor& block_tables,
                          int64_t max_query_len, int64_t max_seq_len, float scale, int64_t window_size_left,
-                         bool return_lse, int64_t total_kv_len) {
+                         bool return_lse, int64_t total_kv_len, PlanInfo* plan_info) {
   TORCH_CHECK(query.dim() == 3 && output.dim() == 3, "query/output must be [tokens, heads, head_dim]");
   TORCH_CHECK(max_query_len >= 1, "max_query_len must be at least 1");
   const bool quant = k_cache_quant_scale.has_value();
@@ -366,7 +415,7 @@ void batch_prefill_paged(const torch::Tensor& query, const torch::Tensor& k_cach
                 "output_lse must be contiguous float32 [tokens, heads]");
     a.lse = output_lse->data_ptr<float>();
   }
-  run_decode(cache, a, query);
+  run_decode(cache, a, query, plan_info);
 }
 
 void batch_decode_csr(torch::Tensor query,
@@ -378,7 +427,8 @@ void batch_decode_csr(torch::Tensor query,
                       int64_t window_left,
                       double sm_scale,
                       torch::Tensor output,
-                      std::optional<torch::Tensor>& output_lse) {
+                      std::optional<torch::Tensor>& output_lse,
+                      PlanInfo* plan_info) {
   // NHD [blocks, block_size, Hkv, D] -> logical [blocks, Hkv, block_size, D] view
   const xllm_hip_kv_cache cache =
       make_cache(k_cache.permute({0, 2, 1, 3}), v_cache.permute({0, 2, 1, 3}), std::nullopt, std::nullopt);
@@ -395,7 +445,7 @@ void batch_decode_csr(torch::Tensor query,
   a.kv_indices = paged_kv_indices.data_ptr<int32_t>();
   a.kv_last_page_len = paged_kv_last_page_len.data_ptr<int32_t>();
   if (output_lse.has_value() && output_lse->defined()) a.lse = output_lse->data_ptr<float>();
-  run_decode(cache, a, query);
+  run_decode(cache, a, query, plan_info);
 }
 
 namespace {

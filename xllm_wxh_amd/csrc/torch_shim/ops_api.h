@@ -31,6 +31,19 @@ void dequant_from_paged_cache(ReshapeFromCacheParams& params);
 
 namespace hip {
 
+// The role of xllm::layer::PlanInfo (xllm/core/layers/common/attention_metadata.h:31-35): one per step,
+// shared by every layer.  The model's layer loop sets layer_id before each layer
+// (xllm/models/llm/llm_model_base.h:115); layer 0 builds the split-KV schedule of the step in the
+// stream's workspace and the later layers reuse it (the reference plans at layer 0 only,
+// xllm/core/layers/cuda/flashinfer_planinfo.cpp:252-253).  The schedule depends on the lengths, the
+// block lists' addresses and the sizes, not on q, out or the cache's contents; `key` records what
+// it was built for, and a later layer whose inputs differ is refused.
+struct PlanInfo {
+  int32_t layer_id = -1;
+  const void* workspace = nullptr;  // where layer 0 left the schedule
+  uint64_t key = 0;
+};
+
 // Argument list of xllm::kernel::mlu::batch_decode (xllm/core/kernels/mlu/mlu_ops_api.h:126-145).
 // query/output: [batch, q_len, Hq, D]; q_len > 1 = speculative verify, causal among the q_len tokens.
 void batch_decode(const torch::Tensor& query,
@@ -53,7 +66,8 @@ void batch_decode(const torch::Tensor& query,
                   float scale,
                   bool return_lse,
                   int64_t kv_cache_quant_bit_size,
-                  int64_t total_kv_len = 0);
+                  int64_t total_kv_len = 0,
+                  PlanInfo* plan_info = nullptr);
 
 // Chunked prefill / mixed steps over the paged cache: the block_tables form of
 // xllm::kernel::mlu::batch_prefill (xllm/core/kernels/mlu/mlu_ops_api.h:103-124, called with the caches
@@ -76,7 +90,8 @@ void batch_prefill_paged(const torch::Tensor& query,
                          float scale,
                          int64_t window_size_left,
                          bool return_lse,
-                         int64_t total_kv_len = 0);
+                         int64_t total_kv_len = 0,
+                         PlanInfo* plan_info = nullptr);
 
 // Tensor arguments of xllm::kernel::cuda::batch_decode (xllm/core/kernels/cuda/cuda_ops_api.h:120-136)
 // without the FlashInfer uri / plan / workspaces, which have no counterpart here.
@@ -90,7 +105,8 @@ void batch_decode_csr(torch::Tensor query,
                       int64_t window_left,
                       double sm_scale,
                       torch::Tensor output,
-                      std::optional<torch::Tensor>& output_lse);
+                      std::optional<torch::Tensor>& output_lse,
+                      PlanInfo* plan_info = nullptr);
 
 // xllm::kernel::cuda::fused_qk_norm_rope (xllm/core/kernels/cuda/cuda_ops_api.h:227-241): per-head RMSNorm
 // and rotary embedding of the q and k heads of the fused buffer, in place.

@@ -42,17 +42,24 @@ PYBIND11_MODULE(_xllm_hip_torch, m) {
   m.def("dequant_from_paged_cache", &xllm::kernel::dequant_from_paged_cache);
   m.def("reshape_paged_cache", &xllm::kernel::reshape_paged_cache);
   m.def("quant_to_paged_cache", &xllm::kernel::quant_to_paged_cache);
+  py::class_<xllm::layer::PlanInfo, std::shared_ptr<xllm::layer::PlanInfo>>(m, "PlanInfo")
+      .def(py::init<>())
+      .def_readwrite("layer_id", &xllm::layer::PlanInfo::layer_id);
   m.def("batch_decode",
         [](const torch::Tensor& query, const torch::Tensor& k_cache, torch::Tensor output,
            const torch::Tensor& block_table, const torch::Tensor& seq_lens, const std::optional<torch::Tensor>& v_cache,
            std::optional<torch::Tensor> output_lse, const std::optional<torch::Tensor>& k_scale,
            const std::optional<torch::Tensor>& v_scale, int64_t max_seq_len, int64_t window_size_left, float scale,
-           bool return_lse, int64_t kv_cache_quant_bit_size) {
+           bool return_lse, int64_t kv_cache_quant_bit_size, std::shared_ptr<xllm::layer::PlanInfo> plan_info) {
           xllm::kernel::hip::batch_decode(query, k_cache, output, block_table, seq_lens, v_cache, output_lse,
                                           std::nullopt, k_scale, v_scale, std::nullopt, std::nullopt, std::nullopt,
                                           "float", max_seq_len, window_size_left, -1, scale, return_lse,
-                                          kv_cache_quant_bit_size);
-        });
+                                          kv_cache_quant_bit_size, 0, plan_info.get());
+        },
+        py::arg("query"), py::arg("k_cache"), py::arg("output"), py::arg("block_table"), py::arg("seq_lens"),
+        py::arg("v_cache"), py::arg("output_lse"), py::arg("k_scale"), py::arg("v_scale"), py::arg("max_seq_len"),
+        py::arg("window_size_left"), py::arg("scale"), py::arg("return_lse"), py::arg("kv_cache_quant_bit_size"),
+        py::arg("plan_info") = nullptr);
   m.def("batch_decode_csr",
         [](torch::Tensor query, torch::Tensor k_cache, torch::Tensor v_cache, torch::Tensor indptr, torch::Tensor indices,
            torch::Tensor last_page_len, int64_t window_left, double sm_scale, torch::Tensor output) {
@@ -81,6 +88,7 @@ PYBIND11_MODULE(_xllm_hip_torch, m) {
 
   py::class_<AttentionMetadata>(m, "AttentionMetadata")
       .def(py::init<>())
+      .def_readwrite("plan_info", &AttentionMetadata::plan_info)
       .def_readwrite("kv_seq_lens", &AttentionMetadata::kv_seq_lens)
       .def_readwrite("q_seq_lens", &AttentionMetadata::q_seq_lens)
       .def_readwrite("block_table", &AttentionMetadata::block_table)
