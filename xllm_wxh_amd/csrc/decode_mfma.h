@@ -415,8 +415,10 @@ constexpr int xch_row_bytes(int tok) { return head_dim_of(tok) * 4 + 16; }  // a
 
 // RAWK: see kRawK.  OFFSET / OFFSET_K: int8 V / K rows sit in LDS with the offset 1152 (see kOffset); a
 // caller that parks them as exact fp16 numbers passes false.
+// FENCED: fragments and per-token factors are read where they are used and the LDS offsets of the
+// fragments are formed every tile anew (scheduling fences; see kFenced), for a kernel with no register to spare.
 template <int KV_DT, int TOK, bool RAWK = raw_k_of(KV_DT, TOK), bool OFFSET = kv_of(KV_DT) == XLLM_HIP_INT8,
-          bool OFFSET_K = OFFSET && !RAWK>
+          bool OFFSET_K = OFFSET && !RAWK, bool FENCED = false>
 struct RowTile {
   static constexpr bool kQuant = quant_of(KV_DT);
   // int8 rows sit in LDS as x + 1152.  With K' = K + 1152 and V' = V + 1152:
@@ -437,6 +439,10 @@ struct RowTile {
   static constexpr int kDT = TOK == 0 ? 16 : 8;  // O^T accumulator tiles
   static constexpr int kU = TOK == 2 ? 2 : 1;    // tokens per row
   static constexpr int kHalves = TOK == 0 ? 1 : 2;  // halves of the tile that hold different tokens
+  // head_dim 256 over a 1-byte cache fits two waves per SIMD (256 registers) only if fragments are read
+  // as they are needed: without the fences the compiler hoists the reads of a tile's 8 K and 16 V
+  // fragments and keeps the 12 XORed LDS offsets in registers through the loop (50 registers spilled).
+  static constexpr bool kFenced = FENCED;
   typedef typename Mma<KV_DT>::Op Op;
 
   Op qf[kQC];      // Q^T fragments (B operand) of the lane's query row
@@ -723,8 +729,15 @@ struct RowTile {
   }
 
   // ---- O^T = O^T * alpha + V^T P^T, tile dt of the rows' 128 elements ----
-  __device__ __forceinline__ Op v_fragment(const uint8_t* tile, int dt) const {
-    const uint32_t vo = v_off0 ^ (uint32_t)((dt & 7) << 5);
+  __device__ __forceinline__ Op v_fragment(const uint8_t* tile, int dt) const { return v_fragment(tile, dt, v_off0); }
+  // The offset of tile 0 made opaque: the XORs that give the other tiles' offsets are then computed where they
+  // are used, every tile anew, instead of being held in registers through the token loop.
+  __device__ __forceinline__ static uint32_t opaque(uint32_t v) {
+    asm volatile("" : "+v"(v));
+    return v;
+  }
+  __device__ __forceinline__ Op v_fragment(const uint8_t* tile, int dt, uint32_t v0) const {
+    const uint32_t vo = v0 ^ (uint32_t)((dt & 7) << 5);
     if constexpr (TOK == 0) {  // tile dt of the 16 tokens: from the first half (dt < 8) or the second
       const s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
           (__attribute__((address_space(3))) s16x4*)(tile + vo + (dt >> 3) * 4096));
@@ -763,8 +776,12 @@ struct RowTile {
   }
   template <bool RESCALE>
   __device__ __forceinline__ void accumulate(const uint8_t* tile, const Op (&pf)[kU], float alpha) {
+    const uint32_t v0 = kFenced ? opaque(v_off0) : v_off0;
 #pragma unroll
-    for (int dt = 0; dt < kDT; ++dt) accumulate_step<RESCALE>(dt, v_fragment(tile, dt), pf, alpha);
+    for (int dt = 0; dt < kDT; ++dt) {
+      accumulate_step<RESCALE>(dt, v_fragment(tile, dt, v0), pf, alpha);
+      if (kFenced && (dt & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+    }
     accumulate_weights<RESCALE>(pf, alpha);
   }
 
@@ -772,7 +789,7 @@ struct RowTile {
   template <bool MASKED>
   __device__ __forceinline__ void attend(const uint8_t* tile, int tb, float scale_log2) {
     float kscl[kN], lv[kN], rvs[kN];
-    load_factors(tile, kscl, lv, rvs);
+    if (!kFenced) load_factors(tile, kscl, lv, rvs);
     Scores s;
     scores_init(s);
     if constexpr (kRawK) {
@@ -782,15 +799,32 @@ struct RowTile {
         scores_step_raw(c, *(const i32x4*)(tile + ko), *(const i32x4*)(tile + ko + 2048), s);
       }
     } else {
+      const uint32_t k0 = kFenced ? opaque(k_off0) : k_off0;
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
-        const uint32_t ko = k_off0 ^ (uint32_t)(c << 6);
+        const uint32_t ko = k0 ^ (uint32_t)(c << 6);
         scores_step(c, *(const Op*)(tile + ko), *(const Op*)(tile + ko + 4096), s);
+        if (kFenced && c < 3) __builtin_amdgcn_sched_barrier(0);
       }
     }
     Op pf[kU];
     float alpha;
-    const bool moved = softmax<MASKED>(s, kscl, lv, rvs, tb, scale_log2, pf, alpha);
+    bool moved;
+    if constexpr (kFenced && kQuant) {
+      // the per-token factors are loaded when they are used: two for the exponents, then the third
+      float x[kN];
+      __builtin_amdgcn_sched_barrier(0);
+      load_factor(tile, 0, kscl);
+      load_factor(tile, 1, lv);
+      scaled_scores<MASKED>(s, kscl, lv, tb, scale_log2, x);
+      __builtin_amdgcn_sched_barrier(0);
+      load_factor(tile, 2, rvs);
+      moved = weights<MASKED>(x, rvs, scale_log2, pf, alpha);
+      __builtin_amdgcn_sched_barrier(0);
+    } else {
+      if (kFenced) load_factors(tile, kscl, lv, rvs);
+      moved = softmax<MASKED>(s, kscl, lv, rvs, tb, scale_log2, pf, alpha);
+    }
     // The accumulators need rescaling only when some row's maximum moved, which becomes rare a few
     // tiles into a sequence.  Both variants of the product are written out, so that each path ends
     // in the MFMAs that define the accumulators (a branch around the multiplies alone makes the
@@ -1072,8 +1106,11 @@ __global__ void __launch_bounds__(64 * kWaves, decode_waves_per_simd(TOK)) decod
   merge_if_last<qf16_of(KV_DT) ? XLLM_HIP_FP16 : XLLM_HIP_BF16, TOK == 0 ? 4 : 2, (TOK == 2 && quant_of(KV_DT)) ? 16 : 32>(*pm, it, &lds_last, wave, lane_id());
 }
 
+// head_dim 256 over a 16-bit cache: one wave per SIMD (its two tile stages alone are 64 registers).
+constexpr int rows32_waves_per_simd(int kv_dt, int tok) { return tok == 0 && !quant_of(kv_dt) ? 1 : 2; }
+
 template <int KV_DT, int TOK>
-__global__ void __launch_bounds__(128, TOK == 0 ? 1 : 2) decode_mfma_d128_rows32_kernel(DecodeParams p) {
+__global__ void __launch_bounds__(128, rows32_waves_per_simd(KV_DT, TOK)) decode_mfma_d128_rows32_kernel(DecodeParams p) {
   // A workgroup is one pair of waves: wave w owns query rows 16w .. 16w+15 and fetches rows 16w ..
   // of every tile.  A tile is parked while both waves still read the previous one from the other
   // buffer, so one barrier (of two waves) per tile suffices.  Four such workgroups share a CU.
@@ -1093,8 +1130,9 @@ __global__ void __launch_bounds__(128, TOK == 0 ? 1 : 2) decode_mfma_d128_rows32
   const int lane = threadIdx.x & 63;
   uint8_t* tiles = lds_all;
 
-  RowTile<KV_DT, TOK> rt;
   constexpr bool kRawK = raw_k_of(KV_DT, TOK);
+  constexpr bool kInt8 = kv_of(KV_DT) == XLLM_HIP_INT8;
+  RowTile<KV_DT, TOK, kRawK, kInt8, kInt8 && !kRawK, rows32_waves_per_simd(KV_DT, TOK) == 2 && TOK == 0> rt;
   float absmax = 0.0f;
   if constexpr (kRawK) {  // one scale for the queries of both waves: they share the parked per-token factors
     lds_ml[wave] = rt.q_absmax(p, it, 16 * rs, lane);

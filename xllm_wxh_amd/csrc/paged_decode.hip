@@ -218,7 +218,9 @@ static int fill_params(const xllm_hip_kv_cache* c,
     p.len_cap = a->block_table != nullptr && cap < INT32_MAX ? (int32_t)cap : INT32_MAX;
   }
   p.window_left = a->window_left;
-  const bool one_wave_per_simd = variant == kMfmaD256;
+  // head_dim 256 runs one wave per SIMD (registers), so half as many workgroups are resident — except the
+  // 32-row kernel over a 1-byte cache, which fits two
+  const bool one_wave_per_simd = variant == kMfmaD256 && !(p.rows > 16 && quant);
   p.target_items = target_items(is_mfma(variant), p.rows, one_wave_per_simd);
   // A small batch on the 16-row kernel: one of the two workgroups a CU holds (the 32-row kernel wants
   // all its slots filled: 4 x 32768 tokens of int8 with 4 draft tokens, 65 us at 1024 items, 84 at 512).
