@@ -99,12 +99,12 @@ constexpr int kQF16 = 64;
 constexpr int kv_of(int kt) { return kt & (kQF16 - 1); }
 constexpr bool qf16_of(int kt) { return (kt & kQF16) != 0 || kv_of(kt) == XLLM_HIP_FP16; }
 constexpr bool quant_of(int kt) { return kv_of(kt) == XLLM_HIP_FP8_E4M3 || kv_of(kt) == XLLM_HIP_INT8; }
-// An int8 cache at head_dim 128: the K rows stay bytes in LDS and meet the queries in the int8 MFMA
+// An int8 cache at head_dim 128 or 256: the K rows stay bytes in LDS and meet the queries in the int8 MFMA
 // (v_mfma_i32_16x16x64_i8); see RowTile.  V is still converted to fp16 for the second MFMA.
 #ifndef XLLM_HIP_RAW_K
 #define XLLM_HIP_RAW_K 1
 #endif
-constexpr bool raw_k_of(int kt, int tok) { return XLLM_HIP_RAW_K && kv_of(kt) == XLLM_HIP_INT8 && tok == 1; }
+constexpr bool raw_k_of(int kt, int tok) { return XLLM_HIP_RAW_K && kv_of(kt) == XLLM_HIP_INT8 && tok != 2; }
 // LDS placement of raw K rows: 128 bytes each, the eight 16-byte pieces of a row permuted by an XOR
 // whose key takes all eight values over rows r .. r+7 (the MFMA operand read: 8 lanes, same piece,
 // consecutive rows) and differs in bit 2 between rows r and r+1 (the park: 8 lanes write four
@@ -485,7 +485,7 @@ struct RowTile {
                            (int64_t)(it.hk * p.group + gq) * kD;
     float m = 0.0f;
 #pragma unroll
-    for (int c = 0; c < 2; ++c) {
+    for (int c = 0; c < kD / 64; ++c) {
       float f[16];
       q_floats(qrow + 64 * c + 16 * kgl, valid, f);
 #pragma unroll
@@ -509,13 +509,13 @@ struct RowTile {
     float sq = 0.0f;
     q_scale = 1.0f;
     if constexpr (kRawK) {
-      // qf[0], qf[1]: the high parts of elements 64c + 16kg .. + 15 (c = 0, 1), sixteen bytes in the
-      // order the K bytes lie in memory; qf[2], qf[3]: the low parts.
+      // qf[c]: the high parts of elements 64c + 16kg .. + 15 (c = 0 .. kD/64 - 1), sixteen bytes in the
+      // order the K bytes lie in memory; qf[kD/64 + c]: the low parts.
       const float top = fmaxf(absmax, 1e-30f);
       const float inv = 127.0f / top;
       q_scale = top * (1.0f / (127.0f * 256.0f));
 #pragma unroll
-      for (int c = 0; c < 2; ++c) {
+      for (int c = 0; c < kD / 64; ++c) {
         float f[16];
         q_floats(qrow + 64 * c + 16 * kg, valid, f);
         uint32_t hi4[4] = {0, 0, 0, 0}, lo4[4] = {0, 0, 0, 0};
@@ -528,7 +528,7 @@ struct RowTile {
           lo4[e >> 2] |= ((uint32_t)(int)l & 0xffu) << (8 * (e & 3));
         }
         qf[c] = __builtin_bit_cast(Op, u32x4{hi4[0], hi4[1], hi4[2], hi4[3]});
-        qf[2 + c] = __builtin_bit_cast(Op, u32x4{lo4[0], lo4[1], lo4[2], lo4[3]});
+        qf[kD / 64 + c] = __builtin_bit_cast(Op, u32x4{lo4[0], lo4[1], lo4[2], lo4[3]});
       }
     }
 #pragma unroll
@@ -619,7 +619,19 @@ struct RowTile {
     if (TOK == 0) s[0][1] = f32x4{0, 0, 0, 0};  // the halves are added: the offset term enters once
   }
   // Raw K: chunk c (0, 1) of the rows' 128 bytes against the queries' high and low parts.
+  // head_dim 256: the tile's second half holds the same 16 tokens' bytes 128..255, which meet the
+  // queries' chunks 2 and 3; both halves add into one pair of sums.
   __device__ __forceinline__ void scores_step_raw(int c, const i32x4& kf0, const i32x4& kf1, Scores& s) const {
+    if constexpr (TOK == 0) {
+      i32x4 hi = __builtin_bit_cast(i32x4, s[0][0]), lo = __builtin_bit_cast(i32x4, s[1][0]);
+      hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(kf0, __builtin_bit_cast(i32x4, qf[c]), hi, 0, 0, 0);
+      lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(kf0, __builtin_bit_cast(i32x4, qf[4 + c]), lo, 0, 0, 0);
+      hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(kf1, __builtin_bit_cast(i32x4, qf[2 + c]), hi, 0, 0, 0);
+      lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(kf1, __builtin_bit_cast(i32x4, qf[6 + c]), lo, 0, 0, 0);
+      s[0][0] = __builtin_bit_cast(f32x4, hi);
+      s[1][0] = __builtin_bit_cast(f32x4, lo);
+      return;
+    }
     const i32x4 qh = __builtin_bit_cast(i32x4, qf[c]), ql = __builtin_bit_cast(i32x4, qf[2 + c]);
     s[0][0] = __builtin_bit_cast(f32x4, __builtin_amdgcn_mfma_i32_16x16x64_i8(kf0, qh, __builtin_bit_cast(i32x4, s[0][0]), 0, 0, 0));
     s[0][1] = __builtin_bit_cast(f32x4, __builtin_amdgcn_mfma_i32_16x16x64_i8(kf1, qh, __builtin_bit_cast(i32x4, s[0][1]), 0, 0, 0));
@@ -793,10 +805,12 @@ struct RowTile {
     Scores s;
     scores_init(s);
     if constexpr (kRawK) {
+      const uint32_t k0 = kFenced ? opaque(k_off0) : k_off0;
 #pragma unroll
       for (int c = 0; c < 2; ++c) {
-        const uint32_t ko = k_off0 ^ (uint32_t)(c << 6);
+        const uint32_t ko = k0 ^ (uint32_t)(c << 6);
         scores_step_raw(c, *(const i32x4*)(tile + ko), *(const i32x4*)(tile + ko + 2048), s);
+        if (kFenced && c < 1) __builtin_amdgcn_sched_barrier(0);
       }
     } else {
       const uint32_t k0 = kFenced ? opaque(k_off0) : k_off0;
