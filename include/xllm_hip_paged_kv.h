@@ -235,7 +235,12 @@ int xllm_hip_paged_decode_plan(const xllm_hip_kv_cache* cache,
                                size_t workspace_bytes,
                                xllm_hip_stream_t stream);
 
-/* Attention proper; requires a schedule built by xllm_hip_paged_decode_plan in `workspace`.
+/* Attention proper; requires a schedule built by xllm_hip_paged_decode_plan in `workspace` from the same
+ * sizes, block list / length arrays and host-side lengths (max_seq_len, total_kv_len): with host-side
+ * lengths that are nearly equal (max_seq_len * batch <= 1.25 * total_kv_len) a split step stores no
+ * schedule — every work item derives its chunk from its index and its sequence's length — and the plan
+ * call only zeroes the counters of the in-kernel combine, so a run with other host-side lengths than its
+ * plan finds no schedule (its result is then undefined; nothing outside the arguments is read).
  * Split sequences leave normalised partial results in the workspace; up to 16 query rows per kv
  * head the attention kernel combines them itself (the workgroup that finishes a sequence's last
  * chunk; it counts in counters that the plan zeroes and every run leaves at zero), otherwise a merge

@@ -69,6 +69,9 @@ __device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it)
     const SeqChunk s = p.seq_chunks[it.sc < p.max_seq_chunks ? it.sc : 0];
     const PlanHeader hdr = *p.hdr;
     if (rest * p.row_groups >= hdr.total_items || it.sc >= p.max_seq_chunks) return false;
+    // (a record no plan wrote — a run on a workspace that was planned with other host-side lengths —
+    // names no sequence outside the batch)
+    if ((unsigned)s.seq >= (unsigned)p.batch || s.chunk < 0) return false;
     it.b = s.seq;
     it.len = s.len;
     it.chunks = s.chunks;

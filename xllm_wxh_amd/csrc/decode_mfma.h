@@ -792,7 +792,7 @@ struct RowTile {
 #pragma unroll
     for (int dt = 0; dt < kDT; ++dt) {
       accumulate_step<RESCALE>(dt, v_fragment(tile, dt, v0), pf, alpha);
-      if (kFenced && (dt & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+      if (kFenced && (dt & 3) == 3) __builtin_amdgcn_sched_barrier(0);  // (every 2, 8 or 16 tiles: the same time)
     }
     accumulate_weights<RESCALE>(pf, alpha);
   }
