@@ -425,7 +425,10 @@ enum xllm_hip_option {
   XLLM_HIP_OPTION_DECODE_STORED_SCHEDULE = 3, /* != 0: a split step always stores its schedule in the workspace
                                                * (the plan kernel), also when the host-side lengths would let
                                                * every work item derive its chunk by itself */
-  XLLM_HIP_OPTION_COUNT = 4
+  XLLM_HIP_OPTION_DECODE_ITEM_PER_HEAD = 4, /* != 0: a work item is always one kv head, also over a cache whose kv
+                                             * heads lie side by side within a token (NHD), where the 16-row kernel
+                                             * otherwise gives an item four kv heads, one per wave */
+  XLLM_HIP_OPTION_COUNT = 5
 };
 int xllm_hip_set_option(int32_t which, int64_t value);
 int64_t xllm_hip_get_option(int32_t which); /* -1 for an unknown option */

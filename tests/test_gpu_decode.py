@@ -214,23 +214,66 @@ def test_nhd_layout_and_csr_form(gpu, kv):
     a = Case(4, 32, 8, 128, 16, lens, kv=kv, layout="HND", seed=3)
     b = Case(4, 32, 8, 128, 16, lens, kv=kv, layout="NHD", seed=3)
     out_a, lse_a = _check(a)
-    out_b, lse_b = _check(b)
-    assert torch.equal(out_a, out_b) and torch.equal(lse_a, lse_b)  # same values, only the strides differ
-    # CSR form of the same block lists (xllm/core/framework/batch/batch_input_builder.cpp:438-494)
-    lists = [a.table[i, : (L + 15) // 16] for i, L in enumerate(lens)]
-    indptr, indices, last = orc.build_paged_kv_csr(lists, lens, 16)
-    out_c = torch.empty_like(a.q)
-    dev = a.q.device
-    ops.batch_decode_csr(a.q, b.k_cache, b.v_cache, torch.from_numpy(indptr).to(dev), torch.from_numpy(indices).to(dev),
-                         torch.from_numpy(last).to(dev), -1, a.scale, out_c, k_cache_scale=b.k_scale,
-                         v_cache_scale=b.v_scale, kv_layout="NHD")
-    torch.cuda.synchronize()
-    assert torch.equal(out_c, out_a)
+    # Over NHD the 16-row kernel gives a work item four kv heads (one per wave), which changes the order of
+    # the sums; with one kv head per item only the strides differ and the values are the same bits.
+    out_h, lse_h = _check(b)
+    assert torch.allclose(out_h.float(), out_a.float(), rtol=2 ** -7, atol=2e-3)
+    assert torch.allclose(lse_h, lse_a, rtol=0, atol=LSE_TOL_INT8 if kv == "int8" else LSE_TOL)
+    with ops.option("item_per_head"):
+        out_b, lse_b = _check(b)
+        assert torch.equal(out_a, out_b) and torch.equal(lse_a, lse_b)
+        # CSR form of the same block lists (xllm/core/framework/batch/batch_input_builder.cpp:438-494)
+        lists = [a.table[i, : (L + 15) // 16] for i, L in enumerate(lens)]
+        indptr, indices, last = orc.build_paged_kv_csr(lists, lens, 16)
+        out_c = torch.empty_like(a.q)
+        dev = a.q.device
+        ops.batch_decode_csr(a.q, b.k_cache, b.v_cache, torch.from_numpy(indptr).to(dev), torch.from_numpy(indices).to(dev),
+                             torch.from_numpy(last).to(dev), -1, a.scale, out_c, k_cache_scale=b.k_scale,
+                             v_cache_scale=b.v_scale, kv_layout="NHD")
+        torch.cuda.synchronize()
+        assert torch.equal(out_c, out_a)
     table, seq_lens = ops.csr_to_block_table(torch.from_numpy(indptr).to(dev), torch.from_numpy(indices).to(dev),
                                              torch.from_numpy(last).to(dev), 16, a.table.shape[1])
     torch.cuda.synchronize()
     assert seq_lens.cpu().tolist() == lens
     np.testing.assert_array_equal(table.cpu().numpy(), a.table)
+
+
+@pytest.mark.parametrize("kv,qdt", [("bf16", "bf16"), ("fp8", "bf16"), ("int8", "bf16"), ("fp16", "fp16"), ("int8", "fp16")])
+@pytest.mark.parametrize("Hq,Hkv,n", [(32, 8, 1), (32, 8, 4), (16, 4, 2), (64, 8, 2), (12, 12, 1)])
+def test_work_items_of_four_kv_heads_over_nhd(gpu, kv, qdt, Hq, Hkv, n):
+    """Over a 1-byte cache whose kv heads lie side by side within a token (NHD) the 16-row kernel at head_dim
+    128 gives a work item four neighbouring kv heads, one per wave, each wave attending all of the chunk's
+    tokens (16-bit caches, and head counts that are no multiple of four, keep one head per item).  Long and short sequences (split into chunks and merged inside the kernel, or by the merge
+    kernel), an empty one, host-side lengths (no stored schedule) and none, a sliding window — against the
+    oracle, and against the same step with one kv head per item."""
+    print("case four heads per item", kv, qdt, Hq, Hkv, n, flush=True)
+    lens = [9000, 300, 0, 33, 4100, 17]
+    case = Case(len(lens), Hq, Hkv, 128, 16, lens, n=n, kv=kv, qdt=qdt, layout="NHD", seed=93)
+    assert case.variant() == "mfma_d128"
+    tol = {"bf16": REG_TOL, "fp16": 2e-3}.get(kv, REG_TOL_QUANT)
+    lse_tol = LSE_TOL_INT8 if kv == "int8" else LSE_TOL
+    for window in (-1, 300):
+        ref, lse_ref = case.oracle(window)
+        out, lse = case.run(window)
+        assert not torch.isnan(out.float()).any()
+        assert max_abs_err(out, ref) <= tol
+        assert lse_err(lse, lse_ref) <= lse_tol
+        with ops.option("item_per_head"):
+            out_1, lse_1 = case.run(window)
+        assert max_abs_err(out_1, ref) <= tol
+        assert torch.allclose(out.float(), out_1.float(), rtol=2 ** -6, atol=4e-3)
+        with ops.option("separate_merge"):
+            out_s, _ = case.run(window)
+        assert max_abs_err(out_s, ref) <= tol
+    out_h, lse_h = case.run(hints=True)
+    ref, lse_ref = case.oracle()
+    assert max_abs_err(out_h, ref) <= tol and lse_err(lse_h, lse_ref) <= lse_tol
+    # equal lengths with host-side lengths: no stored schedule
+    eq = Case(3, Hq, Hkv, 128, 16, [8192] * 3, n=n, kv=kv, qdt=qdt, layout="NHD", seed=94)
+    ref, lse_ref = eq.oracle()
+    out, lse = eq.run(hints=True)
+    assert max_abs_err(out, ref) <= tol and lse_err(lse, lse_ref) <= lse_tol
 
 
 def test_kv_len_one_returns_value_row_exactly(gpu):

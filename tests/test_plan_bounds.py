@@ -37,6 +37,7 @@ def kernels_for(rows, rng):
     out = [(2048, 2048, 1, 64, 32)]
     if rows <= 16:
         out += [(512, 256, 32, 512, 32), (512, 256, 32, 512, 64), (256, 256, 32, 512, 16)]
+        out += [(512, 256, 32, 512, 32, 4)]  # work items of four kv heads (a cache whose heads lie side by side)
     elif rows <= 32:
         out += [(1024, 1024, 32, 512, 32), (1024, 1024, 32, 512, 64), (512, 512, 32, 512, 16)]
     else:
@@ -54,7 +55,9 @@ def test_chunk_count_never_exceeds_the_workspace(plan, seed):
         g = int(rng.choice([1, 2, 4, 7, 8, 16]))
         n = int(rng.choice([1, 1, 2, 4, 8]))
         choices = kernels_for(g * n, rng)
-        target, small, rows_per_item, min_chunk, tile = choices[int(rng.integers(len(choices)))]
+        choice = choices[int(rng.integers(len(choices)))]
+        target, small, rows_per_item, min_chunk, tile = choice[:5]
+        heads_per_item = choice[5] if len(choice) > 5 and hkv % choice[5] == 0 else 1
         rg = plan.harness_row_groups(n, hkv * g, hkv, rows_per_item)
         if plan.harness_row_groups(n, hkv * g, hkv, 32) > 4:
             continue  # never split
@@ -70,7 +73,7 @@ def test_chunk_count_never_exceeds_the_workspace(plan, seed):
         else:
             lens = np.clip(np.round(rng.lognormal(np.log(2048), 0.8, size=batch)), 16, 32768).astype(np.int64)
         total, max_len = int(lens.sum()), int(lens.max())
-        c = plan.harness_choose_chunk(total, max_len, batch, hkv, rg, target, small, min_chunk, tile)
+        c = plan.harness_choose_chunk(total, max_len, batch, hkv // heads_per_item, rg, target, small, min_chunk, tile)
         assert c >= min_chunk and c % tile == 0
         bound = plan.harness_max_seq_chunks(batch, n, hkv * g, hkv, 128)
         assert _chunks(lens, c) <= bound, (target, small, hkv, rg, batch, total, max_len, c)

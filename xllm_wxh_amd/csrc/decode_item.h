@@ -42,8 +42,9 @@ __device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it)
   }
   it.rg = linear % p.row_groups;
   const int rest = linear / p.row_groups;
-  it.hk = rest % p.num_kv_heads;
-  it.sc = rest / p.num_kv_heads;
+  // (an item that covers several kv heads gets the first of them here; its waves take one each)
+  it.hk = (rest % p.item_heads) * p.heads_per_item;
+  it.sc = rest / p.item_heads;
   int chunk = 0, chunk_tokens = 1 << 30;
   it.chunks = 1;
   bool to_the_end = false;  // the chunk runs to the end of the sequence whatever its length

@@ -1030,7 +1030,13 @@ __device__ inline int first_visible_tile(const DecodeParams& p, const Item& it) 
 // Waves per SIMD the 16-row kernel is compiled for: head_dim 256 needs the registers of one.
 constexpr int decode_waves_per_simd(int tok) { return tok == 0 ? 1 : 2; }
 
-template <int KV_DT, int TOK>
+// HEADS: a work item covers kWaves neighbouring kv heads of a sequence chunk and wave w attends head
+// it.hk + w over all of the chunk's tokens (instead of the four waves sharing one head's tokens).  For a
+// cache whose kv heads lie side by side within a token (the NHD layout) the workgroup then reads runs of
+// four rows — 512 bytes of a 1-byte cache — at about the same time, where a workgroup per head reads
+// 128-byte rows at a 1 KiB stride; a plain streaming kernel measures 6.8 TB/s for the first pattern
+// and 5.5 TB/s for the second on this part.  Every wave finishes its own 16 rows: no exchange between waves.
+template <int KV_DT, int TOK, bool HEADS = false>
 __global__ void __launch_bounds__(64 * kWaves, decode_waves_per_simd(TOK)) decode_mfma_d128_kernel(DecodeParams p) {
   __shared__ __attribute__((aligned(16))) uint8_t lds_all[kWaves * kLdsTile];
   __shared__ float lds_ml[kWaves * 16 * 2];  // (running max, denominator) per wave and query row
@@ -1047,17 +1053,22 @@ __global__ void __launch_bounds__(64 * kWaves, decode_waves_per_simd(TOK)) decod
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: keeps the loop scalar
   const int lane = threadIdx.x & 63;
   uint8_t* tile = lds_all + wave * kLdsTile;  // this wave's private K/V tile
+  if (HEADS) {
+    it.hk += wave;
+    it.head_off = (int64_t)it.hk * p.stride_head;
+    it.sc_head_off = (int64_t)it.hk * p.sc_stride_head;
+  }
 
   RowTile<KV_DT, TOK> rt;
   constexpr bool kRawK = raw_k_of(KV_DT, TOK);
-  rt.init(p, it, 0, lane, kRawK ? rt.q_absmax(p, it, 0, lane) : 0.0f);  // (the four waves hold the same rows)
+  rt.init(p, it, 0, lane, kRawK ? rt.q_absmax(p, it, 0, lane) : 0.0f);  // (the four waves hold the same rows, or each its head's)
   const float park_scale = p.scale_log2 * rt.q_scale;
 
   // This wave's share of the item's tokens.
   const int t0 = first_visible_tile(p, it);
   const int span = it.t_end - t0;
-  const int share = span > 0 ? (((span + kWaves - 1) / kWaves + kT - 1) & ~(kT - 1)) : 0;
-  const int w_begin = t0 + wave * share;
+  const int share = span <= 0 ? 0 : HEADS ? ((span + kT - 1) & ~(kT - 1)) : (((span + kWaves - 1) / kWaves + kT - 1) & ~(kT - 1));
+  const int w_begin = HEADS ? t0 : t0 + wave * share;
   const int w_end = min(it.t_end, w_begin + share);
   const int mask_hi_from = it.len - (it.n - 1);                                    // tiles reaching past this need masks
   const int mask_lo_until = p.window_left >= 0 ? it.len - 1 - p.window_left : 0;  // tiles starting below this too
@@ -1115,9 +1126,16 @@ __global__ void __launch_bounds__(64 * kWaves, decode_waves_per_simd(TOK)) decod
   const __attribute__((address_space(4))) DecodeParams* pm =
       (const __attribute__((address_space(4))) DecodeParams*)__builtin_amdgcn_kernarg_segment_ptr();
   asm volatile("" : "+s"(pm));
-  finish_item<KV_DT, TOK, kWaves>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, 0, wave, lane_id(), 0);
+  if constexpr (HEADS) {
+    finish_item<KV_DT, TOK, 1>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, wave, 0, lane_id(), 0);
+  } else {
+    finish_item<KV_DT, TOK, kWaves>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, 0, wave, lane_id(), 0);
+  }
   // (32 rows in flight make the int8 head_dim-64 instantiation spill)
-  merge_if_last<qf16_of(KV_DT) ? XLLM_HIP_FP16 : XLLM_HIP_BF16, TOK == 0 ? 4 : 2, (TOK == 2 && quant_of(KV_DT)) ? 16 : 32>(*pm, it, &lds_last, wave, lane_id());
+  // (work items of several kv heads leave their split sequences to the merge kernel)
+  if constexpr (!HEADS) {
+    merge_if_last<qf16_of(KV_DT) ? XLLM_HIP_FP16 : XLLM_HIP_BF16, TOK == 0 ? 4 : 2, (TOK == 2 && quant_of(KV_DT)) ? 16 : 32>(*pm, it, &lds_last, wave, lane_id());
+  }
 }
 
 // head_dim 256 over a 16-bit cache: one wave per SIMD (its two tile stages alone are 64 registers).

@@ -43,6 +43,8 @@ struct DecodeParams {
   int32_t n;  // query tokens per sequence (the largest count when q_indptr is set)
   int32_t num_q_heads;
   int32_t num_kv_heads;
+  int32_t heads_per_item;  // kv heads one work item covers: 1, or 4 (one per wave of the 16-row kernel; see fill_params)
+  int32_t item_heads;      // num_kv_heads / heads_per_item: work items per sequence chunk and row group
   int32_t group;  // q heads per kv head
   int32_t rows;   // group * n
   int32_t row_groups;

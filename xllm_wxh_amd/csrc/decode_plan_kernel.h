@@ -61,7 +61,7 @@ __global__ void __launch_bounds__(64) decode_plan_kernel(DecodeParams p) {
   // 2. Chunk size.
   const int chunk = p.fixed_chunk > 0
                         ? p.fixed_chunk
-                        : choose_chunk(total, max_len, p.batch, p.num_kv_heads, p.row_groups, p.target_items,
+                        : choose_chunk(total, max_len, p.batch, p.item_heads, p.row_groups, p.target_items,
                                        p.target_small, p.min_chunk, p.tile_tokens);
 
   // 3. Prefix sums of the full-chunk and tail-chunk counts (lengths are re-derived rather than
@@ -109,7 +109,7 @@ __global__ void __launch_bounds__(64) decode_plan_kernel(DecodeParams p) {
     h.total_full = total_full;
     h.total_tail = total_tail;
     h.chunk_tokens = chunk;
-    h.total_items = (total_full + total_tail) * p.num_kv_heads * p.row_groups;
+    h.total_items = (total_full + total_tail) * p.item_heads * p.row_groups;
     *p.hdr = h;
   }
 

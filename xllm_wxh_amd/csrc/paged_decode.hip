@@ -57,7 +57,7 @@ struct Options {
   Options() {
     static const char* const names[XLLM_HIP_OPTION_COUNT] = {
         "XLLM_HIP_DECODE_FORCE_GENERIC", "XLLM_HIP_DECODE_TARGET_ITEMS", "XLLM_HIP_DECODE_SEPARATE_MERGE",
-        "XLLM_HIP_DECODE_STORED_SCHEDULE"};
+        "XLLM_HIP_DECODE_STORED_SCHEDULE", "XLLM_HIP_DECODE_ITEM_PER_HEAD"};
     for (int i = 0; i < XLLM_HIP_OPTION_COUNT; ++i) {
       const char* e = getenv(names[i]);
       v[i].store(e != nullptr ? atoll(e) : 0, std::memory_order_relaxed);
@@ -208,6 +208,16 @@ static int fill_params(const xllm_hip_kv_cache* c,
   p.tok = variant == kMfmaD64 ? 2 : variant == kMfmaD256 ? 0 : 1;
   p.tile_tokens = variant == kMfmaD256 ? kTileTokens / 2 : kTileTokens * p.tok;
   p.row_groups = row_groups(a->q_per_seq, a->num_q_heads, c->num_kv_heads, p.rows_per_item);
+  // The kv heads of a token lie side by side (the NHD layout: a head's row is followed by the next head's)
+  // and a row is 128 bytes (1-byte cache): the 16-row kernel at head_dim 128 then takes work items of four
+  // kv heads, one per wave, so that a workgroup reads runs of four rows instead of single rows a token's
+  // width apart (fp8, 128 x 8192 tokens: 391 -> 338 us; HND 325).  Over a 16-bit cache, whose rows are 256
+  // bytes, it measured the same as one head per item (166 us), so those keep the simpler form.
+  const bool side_by_side = variant == kMfmaD128 && quant && c->stride_head == c->head_dim &&
+                            c->stride_slot >= (int64_t)c->num_kv_heads * c->head_dim &&
+                            option(XLLM_HIP_OPTION_DECODE_ITEM_PER_HEAD) == 0;
+  p.item_heads = item_heads_of(p.rows, c->num_kv_heads, side_by_side);
+  p.heads_per_item = c->num_kv_heads / p.item_heads;
   p.head_dim = c->head_dim;
   p.block_size = c->block_size;
   p.log2_bs = is_pow2(c->block_size) ? ilog2(c->block_size) : 0;
@@ -224,7 +234,10 @@ static int fill_params(const xllm_hip_kv_cache* c,
   p.target_items = target_items(is_mfma(variant), p.rows, one_wave_per_simd);
   // A small batch on the 16-row kernel: one of the two workgroups a CU holds (the 32-row kernel wants
   // all its slots filled: 4 x 32768 tokens of int8 with 4 draft tokens, 65 us at 1024 items, 84 at 512).
-  p.target_small = is_mfma(variant) && p.rows <= 16 && !one_wave_per_simd ? p.target_items / 2 : p.target_items;
+  // (work items of four kv heads keep every slot as the target: each of their waves streams a head of its own,
+  // so one workgroup per CU would leave half of the loads in flight that two do)
+  p.target_small = is_mfma(variant) && p.rows <= 16 && !one_wave_per_simd && p.heads_per_item == 1 ? p.target_items / 2
+                                                                                                : p.target_items;
   // Only the MFMA kernel finishes single-chunk sequences itself.  When the caller's host-side
   // lengths (the reference keeps both in AttentionMetadata) show that the chunk the plan would
   // pick covers the longest sequence, no sequence is split: the plan is told never to split
@@ -234,10 +247,15 @@ static int fill_params(const xllm_hip_kv_cache* c,
   // With more rows the work of a merge is large enough to want the whole GPU: fused into the 32-row
   // kernel it made the int8 verify workload 7 % slower (401 against 377 us), the tails of all row
   // groups ending together.
-  p.fused_merge = is_mfma(variant) && p.rows <= 16 && option(XLLM_HIP_OPTION_DECODE_SEPARATE_MERGE) == 0 ? 1 : 0;
+  // Nor with work items of four kv heads: the workgroup that finishes last would merge four heads' rows, each
+  // wave its head's one after the other (fp8, 8 rows per kv head: 356 us fused against 338 with the merge kernel).
+  p.fused_merge = is_mfma(variant) && p.rows <= 16 && p.heads_per_item == 1 &&
+                          option(XLLM_HIP_OPTION_DECODE_SEPARATE_MERGE) == 0
+                      ? 1
+                      : 0;
   p.fixed_chunk = 0;
   if (p.direct_single && a->max_seq_len > 0 && a->total_kv_len > 0 &&
-      a->max_seq_len <= choose_chunk(a->total_kv_len, a->max_seq_len, p.batch, p.num_kv_heads, p.row_groups,
+      a->max_seq_len <= choose_chunk(a->total_kv_len, a->max_seq_len, p.batch, p.item_heads, p.row_groups,
                                      p.target_items, p.target_small, p.min_chunk, p.tile_tokens)) {
     p.fixed_chunk = 1 << 30;
   }
@@ -254,7 +272,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
   p.arith_chunks = 0;
   if (p.fixed_chunk == 0 && a->max_seq_len > 0 && a->total_kv_len > 0 &&
       option(XLLM_HIP_OPTION_DECODE_STORED_SCHEDULE) == 0) {
-    const int c = choose_chunk(a->total_kv_len, a->max_seq_len, p.batch, p.num_kv_heads, p.row_groups, p.target_items,
+    const int c = choose_chunk(a->total_kv_len, a->max_seq_len, p.batch, p.item_heads, p.row_groups, p.target_items,
                                p.target_small, p.min_chunk, p.tile_tokens);
     const int64_t per_seq = ((int64_t)a->max_seq_len + c - 1) / c;
     if (per_seq * p.batch <= w.max_seq_chunks && per_seq * p.batch <= INT32_MAX &&
@@ -276,7 +294,10 @@ static int fill_params(const xllm_hip_kv_cache* c,
     if (heads_per_line > c->num_kv_heads) heads_per_line = c->num_kv_heads;
     while (heads_per_line > 1 && c->num_kv_heads % heads_per_line != 0) --heads_per_line;
   }
-  p.cluster = p.row_groups * heads_per_line;
+  // (in work items: an item of four heads covers that many of the line's heads itself)
+  int items_per_line = (heads_per_line + p.heads_per_item - 1) / p.heads_per_item;
+  while (items_per_line > 1 && p.item_heads % items_per_line != 0) --items_per_line;
+  p.cluster = p.row_groups * items_per_line;
   p.q_dtype = a->q_dtype;
   p.scale_log2 = a->sm_scale * 1.4426950408889634f;
   return XLLM_HIP_OK;
@@ -284,7 +305,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
 
 // Upper bound of the work-item count for any lengths (see workspace_layout).
 static int64_t max_items(const DecodeParams& p) {
-  const int64_t per = (int64_t)p.num_kv_heads * p.row_groups;
+  const int64_t per = (int64_t)p.item_heads * p.row_groups;
   int64_t seq_chunks = p.batch;
   if (p.arith_chunks > 0) {
     seq_chunks = (int64_t)p.batch * p.arith_chunks;
@@ -307,6 +328,12 @@ static void launch_mfma_tok(const DecodeParams& p, unsigned grid, hipStream_t st
     if constexpr (!quant_of(KV_DT) && TOK != 0) prefill_mfma_d128_kernel<KV_DT, TOK><<<grid, 256, 0, st>>>(p);
     if constexpr (quant_of(KV_DT) && TOK == 1) prefill_quant_d128_kernel<KV_DT><<<grid, 256, 0, st>>>(p);
   } else if (p.rows <= 16) {
+    if constexpr (TOK == 1) {
+      if (p.heads_per_item > 1) {
+        decode_mfma_d128_kernel<KV_DT, TOK, true><<<grid, 64 * kWaves, 0, st>>>(p);
+        return;
+      }
+    }
     decode_mfma_d128_kernel<KV_DT, TOK><<<grid, 64 * kWaves, 0, st>>>(p);
   } else {
     decode_mfma_d128_rows32_kernel<KV_DT, TOK><<<grid, 128, 0, st>>>(p);

@@ -62,7 +62,8 @@ class option:
     the duration of a block.  Names: "force_generic", "target_items", "separate_merge"."""
 
     _IDS = {"force_generic": _lib.OPTION_DECODE_FORCE_GENERIC, "target_items": _lib.OPTION_DECODE_TARGET_ITEMS,
-            "separate_merge": _lib.OPTION_DECODE_SEPARATE_MERGE, "stored_schedule": _lib.OPTION_DECODE_STORED_SCHEDULE}
+            "separate_merge": _lib.OPTION_DECODE_SEPARATE_MERGE, "stored_schedule": _lib.OPTION_DECODE_STORED_SCHEDULE,
+            "item_per_head": _lib.OPTION_DECODE_ITEM_PER_HEAD}
 
     def __init__(self, name, value=1):
         self.which, self.value = self._IDS[name], int(value)
