@@ -286,10 +286,11 @@ int xllm_hip_paged_decode(const xllm_hip_kv_cache* cache,
  * array of XLLM_HIP_STATIC_WORKSPACE_BYTES bytes that is part of the library's device code: each GPU
  * the library runs on holds its own copy from the first launch until the process ends, and this
  * call neither allocates nor frees anything.  Sizes for which xllm_hip_paged_decode_workspace_bytes
- * exceeds that constant are refused with XLLM_HIP_WORKSPACE_TOO_SMALL and a message (the need is
- * at most 1280 * r * head_dim * 4 bytes, r = min(q_per_seq * num_q_heads / num_kv_heads, 128), plus
+ * exceeds that constant are refused with XLLM_HIP_WORKSPACE_TOO_SMALL and a message (with
+ * r = min(q_per_seq * num_q_heads / num_kv_heads, 128) query rows per kv head the need is at most
+ * 2560 * r * head_dim * 4 bytes for r <= 16 and 1280 * r * head_dim * 4 bytes above, plus
  * r * num_kv_heads * head_dim * 4 bytes per sequence: 20 MiB + 128 KiB per sequence for 32 query rows
- * per kv head at head_dim 128 and 8 kv heads).
+ * per kv head at head_dim 128 and 8 kv heads, 20 MiB + 64 KiB per sequence for 16).
  * Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two streams, two
  * threads) race; calls ordered on a stream, or by events, do not.  Nothing needs clearing between
  * calls: each call rebuilds the schedule and zeroes the counters it uses with a kernel, not a memset.
