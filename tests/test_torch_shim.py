@@ -410,11 +410,16 @@ def test_prefill_chunks_over_a_quantised_cache_take_the_dense_route(gpu, shim, k
 
 
 @pytest.mark.gpu
-def test_forward_qkv_replays_under_hip_graph(gpu, shim):
+@pytest.mark.parametrize("hints", [False, True])
+def test_forward_qkv_replays_under_hip_graph(gpu, shim, hints):
     """AttentionImpl::forward_qkv (norm + rotation + KV write, then decode) captured in a HIP graph and
-    replayed on changing persistent inputs; total_kv_len = 0 in the metadata keeps host-side lengths
-    out of the captured kernel choice.  Every replay is compared with an eager call."""
-    print("case shim graph", flush=True)
+    replayed on changing persistent inputs.  Without hints, total_kv_len = 0 in the metadata keeps host-side
+    lengths out of the captured kernel choice.  With hints the graph is captured for its bucket's bounds
+    (max_seq_len and total_kv_len = batch x max_seq_len, as an engine captures a batch-size bucket): the
+    step then stores no schedule, every work item derives its chunk from the sequence's length on the
+    device, and replays with any shorter lengths stay correct.  Every replay is compared with an eager
+    call, and the hinted form with the unhinted one."""
+    print("case shim graph", hints, flush=True)
     B, Hq, Hkv, D, bs, max_blocks = 4, 32, 8, 128, 16, 260
     nblocks = B * max_blocks + 1
     g = torch.Generator().manual_seed(61)
@@ -432,10 +437,14 @@ def test_forward_qkv_replays_under_hip_graph(gpu, shim):
     kv_cu = torch.zeros(B + 1, dtype=torch.int32, device=gpu)
     q_cu = torch.arange(B + 1, dtype=torch.int32, device=gpu)
     block_table = table_full.to(gpu).contiguous()
-    md = shim.build_decode_metadata(q_cu, kv_cu, slots, block_table, 1, max_blocks * bs, 0)
+    md = shim.build_decode_metadata(q_cu, kv_cu, slots, block_table, 1, max_blocks * bs,
+                                    B * max_blocks * bs if hints else 0)
     md.plan_info.layer_id = 0
     kv_seq_lens = torch.ones(B, dtype=torch.int32, device=gpu)
     md.kv_seq_lens = kv_seq_lens  # persistent, refreshed in place before every replay
+    md_plain = shim.build_decode_metadata(q_cu, kv_cu, slots, block_table, 1, max_blocks * bs, 0)
+    md_plain.plan_info.layer_id = 0
+    md_plain.kv_seq_lens = kv_seq_lens
     attn = shim.AttentionImpl(Hq, D, 1.0 / float(np.sqrt(D)), Hkv, -1)
     cache = shim.KVCache(k_cache, v_cache)
 
@@ -475,6 +484,13 @@ def test_forward_qkv_replays_under_hip_graph(gpu, shim):
         torch.cuda.synchronize()
         assert torch.equal(got, eager), "replay %d differs from eager" % it
         assert torch.equal(k_after, k_cache)
+        if hints:
+            k_cache.copy_(k_before)
+            v_cache.copy_(v_before)
+            qkv.copy_(qkv_src)
+            plain = attn.forward_qkv(md_plain, positions, qkv, cos_sin, False, None, None, 0.0, cache)[0]
+            torch.cuda.synchronize()
+            assert torch.allclose(got.float(), plain.float(), rtol=2 ** -7, atol=2e-3)
         _ = (k_cache[:8].float() @ torch.ones(D, 4, device=gpu)).sum().item()
 
 
