@@ -364,7 +364,8 @@ def main():
     # the FETCH_SIZE / WRITE_SIZE counters, and the kernel's average duration in the kernel trace
     traffic = rocprof_avg = None
     tpath = os.path.join(REPO, "profiles", "hbm_traffic.json")
-    if os.path.exists(tpath):
+    # (they were taken in the default configuration: HND pools with the library's K/V placement)
+    if os.path.exists(tpath) and args.kv_layout == "HND" and args.kv_skew_bytes is None:
         entry = json.load(open(tpath)).get(w.name, {})
         traffic = entry.get("traffic_bytes_per_launch")
         rocprof_avg = entry.get("kernel_avg_us")
