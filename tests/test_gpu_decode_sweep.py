@@ -42,5 +42,10 @@ def test_random_shapes_match_oracle(gpu, seed):
         e = max_abs_err(out, ref)
         print("   variant=%s err=%.3e" % (c.variant(), e), flush=True)
         assert e <= (2.5e-2 if cfg["kv"] in ("fp8", "int8") else 1.2e-2), (cfg, window, e)
-        # (int8 at head_dim 128: the queries are 16-bit fixed point against the work item's largest element)
-        assert lse_err(lse, lse_ref) <= (2.5e-4 if cfg["kv"] == "int8" and cfg["D"] == 128 else 1e-4)
+        # (int8 at head_dim 128 and 256: the queries are 16-bit fixed point against the work item's largest element)
+        lse_tol = 2.5e-4 if cfg["kv"] == "int8" and cfg["D"] != 64 else 1e-4
+        assert lse_err(lse, lse_ref) <= lse_tol
+        # the same step with the host-side lengths an engine has (nearly equal lengths then store no schedule)
+        out_h, lse_h = c.run(window, hints=True)
+        assert max_abs_err(out_h, ref) <= (2.5e-2 if cfg["kv"] in ("fp8", "int8") else 1.2e-2), (cfg, window)
+        assert lse_err(lse_h, lse_ref) <= lse_tol
