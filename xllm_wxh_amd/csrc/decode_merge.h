@@ -38,11 +38,12 @@ __device__ inline float load_partial(const float* ptr) {
 // COLS: columns per lane (2 covers head_dim <= 128, 4 head_dim <= 256).
 // (P: DecodeParams, or DecodeParams qualified with the constant address space when the caller reads
 // its arguments straight from the kernel-argument segment.)
+// `known_chunks`: the sequence's chunk count if the caller has it (a work item carries it), else -1.
 template <int Q_DT, bool COHERENT, int COLS, int MAXB = 32, class P>
-__device__ inline void merge_row_cols(const P& p, int b, int j, int head, int q0, int lane) {
+__device__ inline void merge_row_cols(const P& p, int b, int j, int head, int q0, int lane, int known_chunks = -1) {
   const int nhq = p.n * p.num_q_heads;
   const int rem = j * p.num_q_heads + head;
-  const int cnt = chunks_of_sequence(p, b);
+  const int cnt = known_chunks >= 0 ? known_chunks : chunks_of_sequence(p, b);
   const int D = p.head_dim;
   const float neg_inf = -INFINITY;
   // slot of the sequence's chunk i: its full chunks are consecutive, its tail lies among the tails; or
@@ -220,7 +221,7 @@ __device__ inline void merge_if_last(const P& p, const Item& it, int* lds_flag, 
   const int end = min(first + p.rows_per_item, it.n * p.group);
   for (int r = first + wave; r < end; r += nwaves) {
     const int j = r / p.group;
-    merge_row_cols<Q_DT, true, COLS, MAXB>(p, it.b, j, it.hk * p.group + (r - j * p.group), it.q0, lane);
+    merge_row_cols<Q_DT, true, COLS, MAXB>(p, it.b, j, it.hk * p.group + (r - j * p.group), it.q0, lane, cnt);
   }
 }
 
