@@ -205,7 +205,7 @@ FULL = [n for n in workloads.WORKLOADS if n.startswith("cfg") and n != "cfg1_cpu
 
 
 @pytest.mark.parametrize("name", FULL)
-def test_workload_full_size(gpu, name, monkeypatch):
+def test_workload_full_size(gpu, name):
     print("case workload full", name, flush=True)
     w = workloads.WORKLOADS[name]
     d = build(w, gpu)
@@ -242,13 +242,37 @@ def test_workload_full_size(gpu, name, monkeypatch):
     del k2, v2, ks2, vs2
     # (4) the generic kernel agrees with the MFMA kernel on a slice of the batch
     nb = min(2, w.batch)
-    monkeypatch.setenv("XLLM_HIP_DECODE_FORCE_GENERIC", "1")
     n = w.q_per_seq
     out_g = torch.full_like(d["q"][: nb * n], float("nan"))
-    ops.batch_decode(d["q"][: nb * n], d["k"], out_g, d["block_table"][:nb], d["seq_lens_d"][:nb], d["v"], None, None,
-                     d["ks"], d["vs"], scale=w.sm_scale, q_per_seq=n,
-                     kv_cache_quant_bit_size=8 if d["ks"] is not None else -1)
-    torch.cuda.synchronize()
+    with ops.option("force_generic"):
+        assert ops.decode_variant(d["q"][: nb * n], d["k"], d["v"], d["block_table"][:nb], d["seq_lens_d"][:nb],
+                                  d["ks"], d["vs"], q_per_seq=n) == "generic"
+        ops.batch_decode(d["q"][: nb * n], d["k"], out_g, d["block_table"][:nb], d["seq_lens_d"][:nb], d["v"], None, None,
+                         d["ks"], d["vs"], scale=w.sm_scale, q_per_seq=n,
+                         kv_cache_quant_bit_size=8 if d["ks"] is not None else -1)
+        torch.cuda.synchronize()
     diff = float((out_g.float() - out[: nb * n].float()).abs().max())
     print("   generic vs mfma on %d sequences: %.3e" % (nb, diff), flush=True)
     assert diff <= tol / 2
+
+
+def test_fp8_workload_full_size_over_nhd(gpu):
+    """The fp8 workload at full size over an NHD cache (the reference's CUDA layout), where the 16-row kernel
+    gives a work item four kv heads: oracle on sampled sequences, and agreement with the same step in HND."""
+    print("case workload full nhd fp8", flush=True)
+    w = workloads.WORKLOADS["cfg4_fp8_qwen3_32b"]
+    d = build(w, gpu)
+    out_hnd = decode(d)
+    nhd = lambda t: t.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)  # NHD memory, HND view
+    nhd_s = lambda t: t.permute(0, 2, 1).contiguous().permute(0, 2, 1)
+    k, v, ks, vs = nhd(d["k"]), nhd(d["v"]), nhd_s(d["ks"]), nhd_s(d["vs"])
+    assert k.stride(1) == w.head_dim  # a head's row is followed by the next head's
+    out = decode(d, k=k, v=v, ks=ks, vs=vs)
+    assert not torch.isnan(out.float()).any()
+    err = oracle_on_sample(d, out, [0, w.batch - 1])
+    print("   max-abs err %.3e" % err, flush=True)
+    assert err <= TOL_QUANT_KV
+    assert float((out.float() - out_hnd.float()).abs().max()) <= TOL_QUANT_KV / 4
+    with ops.option("item_per_head"):
+        out_1 = decode(d, k=k, v=v, ks=ks, vs=vs)
+    assert torch.equal(out_1, out_hnd)  # one head per item: only the strides differ
