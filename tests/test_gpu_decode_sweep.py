@@ -49,3 +49,57 @@ def test_random_shapes_match_oracle(gpu, seed):
         out_h, lse_h = c.run(window, hints=True)
         assert max_abs_err(out_h, ref) <= (2.5e-2 if cfg["kv"] in ("fp8", "int8") else 1.2e-2), (cfg, window)
         assert lse_err(lse_h, lse_ref) <= lse_tol
+
+
+def _random_mixed_step(rng):
+    D = int(rng.choice([128, 128, 128, 64, 256]))
+    kv = str(rng.choice(["bf16", "fp8", "int8", "fp16"]))
+    qdt = "fp16" if kv == "fp16" or (kv in ("fp8", "int8") and rng.random() < 0.3) else "bf16"
+    bs = int(rng.choice([16, 32, 128])) if D != 64 else int(rng.choice([32, 64]))
+    Hkv = int(rng.choice([1, 2, 4, 8]))
+    g = int(rng.choice([1, 4, 8]))
+    layout = str(rng.choice(["HND", "NHD"]))
+    lens, counts = [], []
+    for _ in range(int(rng.integers(1, 6))):
+        L = int(rng.integers(1, int(rng.choice([40, 600, 3000]))))
+        lens.append(L)
+        counts.append(min(int(rng.choice([0, 1, 1, 4, 17, 40, 130, 300])), L))
+    if max(counts) == 0:
+        counts[0] = 1
+    window = int(rng.choice([-1, -1, 50, 400]))
+    return dict(Hq=Hkv * g, Hkv=Hkv, D=D, bs=bs, lens=lens, kv=kv, qdt=qdt, layout=layout), counts, window
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_mixed_steps_match_oracle(gpu, seed):
+    """Seeded random mixed steps — sequences with 0 to 300 query tokens each (decode, verify and prefill
+    chunks in one call), every cache type, head size, layout and block size, sliding windows — against
+    the oracle: the 16-row, 32-row and both 128-row kernels under shapes nobody hand-picked."""
+    from oracle import paged_kv_oracle as orc
+    from xllm_wxh_amd import ops
+
+    rng = np.random.default_rng(9000 + seed)
+    for rep in range(4):
+        cfg, counts, window = _random_mixed_step(rng)
+        print("case mixed sweep", seed, rep, cfg, counts, "window", window, flush=True)
+        c = Case(len(cfg["lens"]), cfg["Hq"], cfg["Hkv"], cfg["D"], cfg["bs"], cfg["lens"], kv=cfg["kv"], qdt=cfg["qdt"],
+                 layout=cfg["layout"], seed=seed * 10 + rep)
+        q_indptr = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+        T = int(q_indptr[-1])
+        dt = torch.bfloat16 if cfg["qdt"] == "bf16" else torch.float16
+        q = torch.randn(T, c.Hq, c.D, generator=torch.Generator().manual_seed(seed)).to(dt)
+        qd = q.to(c.q.device)
+        out = torch.full_like(qd, 7.0)
+        lse = torch.full((T, c.Hq), 3.0, dtype=torch.float32, device=qd.device)
+        ops.batch_decode(qd, c.k_cache, out, c.block_table, c.seq_lens, c.v_cache, lse, None, c.k_scale, c.v_scale,
+                         scale=c.scale, return_lse=True, kv_cache_quant_bit_size=8 if c.k_scale is not None else -1,
+                         q_per_seq=max(counts), q_indptr=torch.from_numpy(q_indptr).to(qd.device),
+                         window_size_left=window, kv_layout=cfg["layout"])
+        torch.cuda.synchronize()
+        ref, ref_lse = orc.paged_decode_ragged(q.float().numpy(), c.k_ref, c.v_ref, c.table, c.lens, q_indptr, c.scale,
+                                               window_left=window)
+        got = out.float().cpu().numpy()
+        assert not np.isnan(got).any()
+        assert float(np.abs(got - ref).max()) <= c.tol, (cfg, counts, window)
+        fin = np.isfinite(ref_lse)
+        assert np.allclose(lse.cpu().numpy()[fin], ref_lse[fin], atol=5e-2)
