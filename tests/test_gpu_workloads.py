@@ -17,6 +17,8 @@ from xllm_wxh_amd import ops, workloads
 
 pytestmark = pytest.mark.gpu
 
+REL_TOL = 5e-2  # max-abs error of a sequence's rows over the RMS of its reference rows
+
 TDT = {"bf16": torch.bfloat16, "fp32": torch.float32, "fp8": torch.float8_e4m3fn, "int8": torch.int8}
 
 
@@ -98,7 +100,14 @@ def oracle_on_sample(d, out, sample):
                                   w.sm_scale, q_per_seq=n, acc_dtype=np.float32 if L > 8192 else np.float64)
         got = out[b * n:(b + 1) * n].float().cpu().numpy()
         assert not np.isnan(got).any()
-        worst = max(worst, float(np.abs(got - ref).max()))
+        err = float(np.abs(got - ref).max())
+        worst = max(worst, err)
+        # Long sequences of zero-mean values have outputs of a few hundredths — the size of the absolute
+        # tolerances — so the error is also bounded relative to the sequence's output RMS: a wrong V scale,
+        # a dropped chunk or a wrong merge weight fails this where it would pass the absolute bound.
+        rms = float(np.sqrt(np.mean(ref.astype(np.float64) ** 2)))
+        if rms > 0.0:
+            assert err <= REL_TOL * rms, (b, L, err, rms)
     return worst
 
 
