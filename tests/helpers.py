@@ -120,3 +120,18 @@ def lse_err(lse, ref):
     fin = np.isfinite(ref)
     assert np.array_equal(np.isneginf(got), np.isneginf(ref))
     return float(np.abs(got[fin] - ref[fin]).max()) if fin.any() else 0.0
+
+
+def max_rel_err_ragged(got, ref, q_indptr):
+    """max_rel_err_per_seq for sequences with different numbers of query rows (rows q_indptr[b] ..
+    q_indptr[b+1] belong to sequence b)."""
+    got = np.asarray(got, np.float64)
+    ref = np.asarray(ref, np.float64)
+    worst = 0.0
+    for b in range(len(q_indptr) - 1):
+        lo, hi = int(q_indptr[b]), int(q_indptr[b + 1])
+        if hi > lo:
+            rms = float(np.sqrt(np.mean(ref[lo:hi] ** 2)))
+            if rms > 0.0:
+                worst = max(worst, float(np.abs(got[lo:hi] - ref[lo:hi]).max()) / rms)
+    return worst
