@@ -238,6 +238,15 @@ static int fill_params(const xllm_hip_kv_cache* c,
   // so one workgroup per CU would leave half of the loads in flight that two do)
   p.target_small = is_mfma(variant) && p.rows <= 16 && !one_wave_per_simd && p.heads_per_item == 1 ? p.target_items / 2
                                                                                                 : p.target_items;
+  // ... except over a 1-byte cache, where a wave has half as many bytes in flight per tile and one workgroup
+  // per CU does not saturate HBM (fp8, 16 x 8192 tokens: 65 us at 256 items, 55 at 512; int8, 32 x 32768
+  // tokens with two draft tokens: 423 against 344): every slot, as long as that cuts a sequence into at most
+  // the 32 chunks the in-kernel merge loads in one batch (one 32768-token sequence: 31 us at 256 items, 38 at 512).
+  if (quant && p.target_small < p.target_items) {
+    const int64_t triples = (int64_t)p.batch * p.item_heads * p.row_groups;
+    const int64_t cap = 32 * triples;
+    p.target_small = (int32_t)(cap >= p.target_items ? p.target_items : cap > p.target_small ? cap : p.target_small);
+  }
   // Only the MFMA kernel finishes single-chunk sequences itself.  When the caller's host-side
   // lengths (the reference keeps both in AttentionMetadata) show that the chunk the plan would
   // pick covers the longest sequence, no sequence is split: the plan is told never to split
