@@ -429,7 +429,10 @@ enum xllm_hip_option {
   XLLM_HIP_OPTION_DECODE_ITEM_PER_HEAD = 4, /* != 0: a work item is always one kv head, also over a cache whose kv
                                              * heads lie side by side within a token (NHD), where the 16-row kernel
                                              * otherwise gives an item four kv heads, one per wave */
-  XLLM_HIP_OPTION_COUNT = 5
+  XLLM_HIP_OPTION_DECODE_FOUR_WAVE_ITEMS = 5, /* != 0: the 16-row kernel always runs four waves per work item, also
+                                               * when the launch has at most one item per CU (where it otherwise
+                                               * runs eight) */
+  XLLM_HIP_OPTION_COUNT = 6
 };
 int xllm_hip_set_option(int32_t which, int64_t value);
 int64_t xllm_hip_get_option(int32_t which); /* -1 for an unknown option */

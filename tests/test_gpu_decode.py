@@ -602,8 +602,15 @@ def test_long_context_single_sequence(gpu, kv):
     print("case long context", kv, flush=True)
     case = Case(1, 32, 8, 128, 128, [131072], kv=kv, seed=31, std=0.5)
     out, _ = _check(case)
-    out_h, _ = case.run(hints=True)
-    assert torch.equal(out, out_h)
+    _check(case, hints=True)
+    # with and without the host-side lengths the step is cut the same way; the launch's size differs, and
+    # with it the number of waves per work item over a 1-byte cache unless that is held at four
+    with ops.option("four_wave_items"):
+        out_4, _ = case.run()
+        out_h, _ = case.run(hints=True)
+    assert torch.equal(out_4, out_h)
+    if kv == "bf16":
+        assert torch.equal(out, out_h)
 
 
 def test_large_batch_of_short_sequences(gpu):
@@ -860,10 +867,15 @@ def test_split_step_without_a_stored_schedule(gpu, kv, n, qdt, name, lens):
     tol = {"bf16": REG_TOL, "fp16": 2e-3, "fp32": 1e-4}.get(kv, REG_TOL_QUANT)
     assert max_abs_err(out, ref) <= tol
     assert lse_err(lse, lse_ref) <= (LSE_TOL_INT8 if kv == "int8" else LSE_TOL)
-    with ops.option("stored_schedule"):
-        out_s, lse_s = case.run(workspace=ws, hints=True)
+    # (the stored schedule's launch is sized for any lengths, and a launch of more work items than CUs
+    # runs four waves per item: the comparison holds the other one at four as well)
+    with ops.option("four_wave_items"):
+        out_4, lse_4 = case.run(workspace=ws, hints=True)
+        assert bool((ws[:64] == 0xA5).all())
+        with ops.option("stored_schedule"):
+            out_s, lse_s = case.run(workspace=ws, hints=True)
     assert not bool((ws[:64] == 0xA5).all())
-    assert torch.equal(out, out_s) and torch.equal(lse, lse_s)
+    assert torch.equal(out_4, out_s) and torch.equal(lse_4, lse_s)
     # wrong host-side lengths
     ws.fill_(0xA5)
     longest, total = int(max(lens)), int(sum(lens))

@@ -22,6 +22,7 @@ OK, INVALID_ARGUMENT, UNSUPPORTED, WORKSPACE_TOO_SMALL, RUNTIME_ERROR = 0, 1, 2,
 OPTION_DECODE_FORCE_GENERIC, OPTION_DECODE_TARGET_ITEMS, OPTION_DECODE_SEPARATE_MERGE = 0, 1, 2
 OPTION_DECODE_STORED_SCHEDULE = 3
 OPTION_DECODE_ITEM_PER_HEAD = 4
+OPTION_DECODE_FOUR_WAVE_ITEMS = 5
 
 STATUS_NAMES = {
     OK: "OK",

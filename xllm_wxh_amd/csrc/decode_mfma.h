@@ -1036,10 +1036,17 @@ constexpr int decode_waves_per_simd(int tok) { return tok == 0 ? 1 : 2; }
 // four rows — 512 bytes of a 1-byte cache — at about the same time, where a workgroup per head reads
 // 128-byte rows at a 1 KiB stride; a plain streaming kernel measures 6.8 TB/s for the first pattern
 // and 5.5 TB/s for the second on this part.  Every wave finishes its own 16 rows: no exchange between waves.
-template <int KV_DT, int TOK, bool HEADS = false>
-__global__ void __launch_bounds__(64 * kWaves, decode_waves_per_simd(TOK)) decode_mfma_d128_kernel(DecodeParams p) {
-  __shared__ __attribute__((aligned(16))) uint8_t lds_all[kWaves * kLdsTile];
-  __shared__ float lds_ml[kWaves * 16 * 2];  // (running max, denominator) per wave and query row
+//
+// WAVES: waves that share an item's tokens.  Four, two workgroups to a CU, when the launch has work items
+// for that; eight (one such workgroup fills a CU: its tiles take 134 KiB of LDS) when a launch over a
+// 1-byte cache has at most one item per CU, as a small batch cut into 32 chunks per sequence has: a wave
+// has one tile in flight and converts it before it asks for the next, so four waves leave the CU's memory
+// pipe idle much of the time, and cutting finer instead costs more in the merge than it gains.
+template <int KV_DT, int TOK, bool HEADS = false, int WAVES = kWaves>
+__global__ void __launch_bounds__(64 * WAVES, decode_waves_per_simd(TOK)) decode_mfma_d128_kernel(DecodeParams p) {
+  static_assert(!(HEADS && WAVES != kWaves) && !(TOK == 0 && WAVES != kWaves), "eight waves: head_dim 64 and 128, one kv head per item");
+  __shared__ __attribute__((aligned(16))) uint8_t lds_all[WAVES * kLdsTile];
+  __shared__ float lds_ml[WAVES * 16 * 2];  // (running max, denominator) per wave and query row
   __shared__ int lds_last;
 
   constexpr int kT = tile_tokens_of(TOK);  // tokens per tile
@@ -1067,7 +1074,7 @@ __global__ void __launch_bounds__(64 * kWaves, decode_waves_per_simd(TOK)) decod
   // This wave's share of the item's tokens.
   const int t0 = first_visible_tile(p, it);
   const int span = it.t_end - t0;
-  const int share = span <= 0 ? 0 : HEADS ? ((span + kT - 1) & ~(kT - 1)) : (((span + kWaves - 1) / kWaves + kT - 1) & ~(kT - 1));
+  const int share = span <= 0 ? 0 : HEADS ? ((span + kT - 1) & ~(kT - 1)) : (((span + WAVES - 1) / WAVES + kT - 1) & ~(kT - 1));
   const int w_begin = HEADS ? t0 : t0 + wave * share;
   const int w_end = min(it.t_end, w_begin + share);
   const int mask_hi_from = it.len - (it.n - 1);                                    // tiles reaching past this need masks
@@ -1129,7 +1136,7 @@ __global__ void __launch_bounds__(64 * kWaves, decode_waves_per_simd(TOK)) decod
   if constexpr (HEADS) {
     finish_item<KV_DT, TOK, 1>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, wave, 0, lane_id(), 0);
   } else {
-    finish_item<KV_DT, TOK, kWaves>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, 0, wave, lane_id(), 0);
+    finish_item<KV_DT, TOK, WAVES>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, 0, wave, lane_id(), 0);
   }
   // (32 rows in flight make the int8 head_dim-64 instantiation spill)
   // (work items of several kv heads leave their split sequences to the merge kernel)

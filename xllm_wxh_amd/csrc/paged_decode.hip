@@ -57,7 +57,7 @@ struct Options {
   Options() {
     static const char* const names[XLLM_HIP_OPTION_COUNT] = {
         "XLLM_HIP_DECODE_FORCE_GENERIC", "XLLM_HIP_DECODE_TARGET_ITEMS", "XLLM_HIP_DECODE_SEPARATE_MERGE",
-        "XLLM_HIP_DECODE_STORED_SCHEDULE", "XLLM_HIP_DECODE_ITEM_PER_HEAD"};
+        "XLLM_HIP_DECODE_STORED_SCHEDULE", "XLLM_HIP_DECODE_ITEM_PER_HEAD", "XLLM_HIP_DECODE_FOUR_WAVE_ITEMS"};
     for (int i = 0; i < XLLM_HIP_OPTION_COUNT; ++i) {
       const char* e = getenv(names[i]);
       v[i].store(e != nullptr ? atoll(e) : 0, std::memory_order_relaxed);
@@ -340,6 +340,15 @@ static void launch_mfma_tok(const DecodeParams& p, unsigned grid, hipStream_t st
     if constexpr (TOK == 1) {
       if (p.heads_per_item > 1) {
         decode_mfma_d128_kernel<KV_DT, TOK, true><<<grid, 64 * kWaves, 0, st>>>(p);
+        return;
+      }
+    }
+    if constexpr (TOK != 0 && quant_of(KV_DT)) {
+      // At most one work item per CU over a 1-byte cache: eight waves share it (one 32768-token sequence:
+      // 25 us against 31 for fp8, 26 against 32 for int8; over a 16-bit cache, whose tiles take no
+      // conversion, 31.7 against 31.0).
+      if (grid <= (unsigned)kNumCUs && option(XLLM_HIP_OPTION_DECODE_FOUR_WAVE_ITEMS) == 0) {
+        decode_mfma_d128_kernel<KV_DT, TOK, false, 2 * kWaves><<<grid, 128 * kWaves, 0, st>>>(p);
         return;
       }
     }

@@ -59,11 +59,12 @@ def _require(cond, msg):
 
 class option:
     """Context manager: a process-wide diagnostic switch of the library (xllm_hip_set_option) set for
-    the duration of a block.  Names: "force_generic", "target_items", "separate_merge"."""
+    the duration of a block.  Names: the keys of `_IDS`."""
 
     _IDS = {"force_generic": _lib.OPTION_DECODE_FORCE_GENERIC, "target_items": _lib.OPTION_DECODE_TARGET_ITEMS,
             "separate_merge": _lib.OPTION_DECODE_SEPARATE_MERGE, "stored_schedule": _lib.OPTION_DECODE_STORED_SCHEDULE,
-            "item_per_head": _lib.OPTION_DECODE_ITEM_PER_HEAD}
+            "item_per_head": _lib.OPTION_DECODE_ITEM_PER_HEAD,
+            "four_wave_items": _lib.OPTION_DECODE_FOUR_WAVE_ITEMS}
 
     def __init__(self, name, value=1):
         self.which, self.value = self._IDS[name], int(value)
