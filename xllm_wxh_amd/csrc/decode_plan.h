@@ -51,7 +51,8 @@ constexpr int kPrefillMinRows = 32;
 // items, 53-58 us at 264 to 504.
 //   equal lengths   the item count is exact: k = target_small / triples chunks per sequence (at least
 //                   one: 24 x 8192 tokens x 8 kv heads run unsplit as 192 items in 119 us, cut in three
-//                   for 512 slots — 576 items, a second round — 145 us);
+//                   for 512 slots — 576 items, a second round — 145 us; 20 x 8192 tokens: 104 us as 160
+//                   items, 107 as 480);
 //   else            items <= triples + work / chunk, so chunk = work / (target_small - triples) keeps them
 //                   within target_small; but no coarser than work / (9/16 target_small) — below about 144
 //                   equal items the longest one, streaming alone at some 50 GB/s, would set the time

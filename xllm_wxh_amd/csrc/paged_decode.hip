@@ -238,10 +238,12 @@ static int fill_params(const xllm_hip_kv_cache* c,
   // so one workgroup per CU would leave half of the loads in flight that two do)
   p.target_small = is_mfma(variant) && p.rows <= 16 && !one_wave_per_simd && p.heads_per_item == 1 ? p.target_items / 2
                                                                                                 : p.target_items;
-  // ... except over a 1-byte cache, where a wave has half as many bytes in flight per tile and one workgroup
-  // per CU does not saturate HBM (fp8, 16 x 8192 tokens: 65 us at 256 items, 55 at 512; int8, 32 x 32768
-  // tokens with two draft tokens: 423 against 344): every slot, as long as that cuts a sequence into at most
-  // the 32 chunks the in-kernel merge loads in one batch (one 32768-token sequence: 31 us at 256 items, 38 at 512).
+  // ... except over a 1-byte cache, where four waves have half as many bytes in flight per tile and do not
+  // saturate a CU's share of HBM (fp8, 16 x 8192 tokens: 65 us at 256 items, 55 at 512): every slot, as long
+  // as that cuts a sequence into at most the 32 chunks the in-kernel merge loads in one batch (one
+  // 32768-token sequence: 31 us at 256 items, 38 at 512).  Better still is one workgroup of eight waves per
+  // CU (wide_items below), which needs the launch's size to be known here.
+  const int32_t target_one_per_cu = p.target_small;
   if (quant && p.target_small < p.target_items) {
     const int64_t triples = (int64_t)p.batch * p.item_heads * p.row_groups;
     const int64_t cap = 32 * triples;
@@ -262,34 +264,54 @@ static int fill_params(const xllm_hip_kv_cache* c,
                           option(XLLM_HIP_OPTION_DECODE_SEPARATE_MERGE) == 0
                       ? 1
                       : 0;
-  p.fixed_chunk = 0;
-  if (p.direct_single && a->max_seq_len > 0 && a->total_kv_len > 0 &&
-      a->max_seq_len <= choose_chunk(a->total_kv_len, a->max_seq_len, p.batch, p.item_heads, p.row_groups,
-                                     p.target_items, p.target_small, p.min_chunk, p.tile_tokens)) {
-    p.fixed_chunk = 1 << 30;
-  }
-  // Many query rows per kv head (chunked prefill): the row groups supply the parallelism, and one
-  // partial per chunk and row would be large, so nothing is split.
-  if (never_split(a->q_per_seq, a->num_q_heads, c->num_kv_heads)) p.fixed_chunk = 1 << 30;
-  p.implicit_plan = p.direct_single && p.fixed_chunk == (1 << 30) ? 1 : 0;
-  // A split step whose host-side lengths are (nearly) equal needs no stored schedule: with the chunk
-  // size the device-side plan would choose from the same aggregates, every sequence owns
-  // ceil(max_seq_len / chunk) chunk slots and a work item finds its chunk from its index and the
-  // sequence's length.  No plan kernel runs, and the item's block list, queries and length are
-  // independent loads.  Not for ragged batches: the slots of the shorter sequences would be empty
-  // workgroups (at most a quarter of them may be), and the tails would not be ordered by size.
-  p.arith_chunks = 0;
-  if (p.fixed_chunk == 0 && a->max_seq_len > 0 && a->total_kv_len > 0 &&
-      option(XLLM_HIP_OPTION_DECODE_STORED_SCHEDULE) == 0) {
-    const int c = choose_chunk(a->total_kv_len, a->max_seq_len, p.batch, p.item_heads, p.row_groups, p.target_items,
-                               p.target_small, p.min_chunk, p.tile_tokens);
-    const int64_t per_seq = ((int64_t)a->max_seq_len + c - 1) / c;
-    if (per_seq * p.batch <= w.max_seq_chunks && per_seq * p.batch <= INT32_MAX &&
-        (int64_t)a->max_seq_len * p.batch * 4 <= a->total_kv_len * 5) {
-      p.fixed_chunk = c;
-      p.arith_chunks = (int32_t)per_seq;
+  const bool hints = a->max_seq_len > 0 && a->total_kv_len > 0;
+  const bool stay_whole = never_split(a->q_per_seq, a->num_q_heads, c->num_kv_heads);
+  auto decide = [&]() {
+    p.fixed_chunk = 0;
+    if (p.direct_single && hints &&
+        a->max_seq_len <= choose_chunk(a->total_kv_len, a->max_seq_len, p.batch, p.item_heads, p.row_groups,
+                                       p.target_items, p.target_small, p.min_chunk, p.tile_tokens)) {
+      p.fixed_chunk = 1 << 30;
     }
+    // Many query rows per kv head (chunked prefill): the row groups supply the parallelism, and one
+    // partial per chunk and row would be large, so nothing is split.
+    if (stay_whole) p.fixed_chunk = 1 << 30;
+    p.implicit_plan = p.direct_single && p.fixed_chunk == (1 << 30) ? 1 : 0;
+    // A split step whose host-side lengths are (nearly) equal needs no stored schedule: with the chunk
+    // size the device-side plan would choose from the same aggregates, every sequence owns
+    // ceil(max_seq_len / chunk) chunk slots and a work item finds its chunk from its index and the
+    // sequence's length.  No plan kernel runs, and the item's block list, queries and length are
+    // independent loads.  Not for ragged batches: the slots of the shorter sequences would be empty
+    // workgroups (at most a quarter of them may be), and the tails would not be ordered by size.
+    p.arith_chunks = 0;
+    if (p.fixed_chunk == 0 && hints && option(XLLM_HIP_OPTION_DECODE_STORED_SCHEDULE) == 0) {
+      const int c = choose_chunk(a->total_kv_len, a->max_seq_len, p.batch, p.item_heads, p.row_groups, p.target_items,
+                                 p.target_small, p.min_chunk, p.tile_tokens);
+      const int64_t per_seq = ((int64_t)a->max_seq_len + c - 1) / c;
+      if (per_seq * p.batch <= w.max_seq_chunks && per_seq * p.batch <= INT32_MAX &&
+          (int64_t)a->max_seq_len * p.batch * 4 <= a->total_kv_len * 5) {
+        p.fixed_chunk = c;
+        p.arith_chunks = (int32_t)per_seq;
+      }
+    }
+  };
+  // Over a 1-byte cache the 16-row kernel also comes with eight waves per work item, one such workgroup to a
+  // CU (launch_mfma_tok): with the host-side lengths the launch's size is known here, and a step that can be
+  // cut into at most one item per CU is (fp8, 64 q heads: 32 x 8192 tokens 94 -> 87 us, 2 x 32768 40 -> 33,
+  // 3 x 20000 36 -> 31; int8 with two draft tokens, 32 x 32768: 341 -> 326) — unless that leaves over a
+  // quarter of the CUs without an item (20 x 8192 tokens of fp8: 69 us as 160 items, 65 as 480 in every slot).
+  const bool wide_items = quant && is_mfma(variant) && variant != kMfmaD256 && p.rows <= 16 && p.heads_per_item == 1 &&
+                          hints && option(XLLM_HIP_OPTION_DECODE_FOUR_WAVE_ITEMS) == 0;
+  bool decided = false;
+  if (wide_items && target_one_per_cu < p.target_small) {
+    const int32_t every_slot = p.target_small;
+    p.target_small = target_one_per_cu;
+    decide();
+    const int64_t items = (p.implicit_plan ? (int64_t)p.batch : (int64_t)p.batch * p.arith_chunks) * p.item_heads * p.row_groups;
+    decided = (p.implicit_plan || p.arith_chunks > 0) && items <= kNumCUs && items * 4 >= kNumCUs * 3;
+    if (!decided) p.target_small = every_slot;
   }
+  if (!decided) decide();
   // XCD clusters: the row groups of a (chunk, kv head); and the kv heads whose rows share 128-byte
   // lines — scale rows shorter than a line (HND: block_size * 4 bytes per head; NHD: the heads of a
   // slot are adjacent floats) or cache rows shorter than a line (NHD with 64 one-byte elements).
