@@ -735,6 +735,35 @@ def test_small_batch_chunk_choices(gpu, kv, name, lens):
         assert torch.equal(out, out_h)
 
 
+@pytest.mark.parametrize("kv,qdt", [("fp8", "bf16"), ("int8", "bf16"), ("int8", "fp16")])
+@pytest.mark.parametrize("name,D,bs,n,lens", [
+    ("one long sequence", 128, 16, 1, [32768]),
+    ("split, every CU an item", 128, 128, 2, [6000] * 4),
+    ("not split: a workgroup per (sequence, kv head)", 128, 16, 1, [700 + 16 * i for i in range(30)]),
+    ("nearly equal lengths, one empty", 128, 32, 4, [8192, 7000, 0, 8192, 8100, 7777]),
+    ("head_dim 64", 64, 32, 2, [9000] * 3),
+    ("head_dim 64, not split", 64, 64, 1, [300] * 32),
+])
+def test_eight_wave_items_over_one_byte_caches(gpu, kv, qdt, name, D, bs, n, lens):
+    """With the host's lengths a step over a 1-byte cache that fits one work item per CU runs eight
+    waves per item (the waves share the item's tokens and combine at its end as four do): against the
+    oracle, and against the same step held at four waves."""
+    print("case eight waves", kv, qdt, name, flush=True)
+    case = Case(len(lens), 32, 8, D, bs, lens, n=n, kv=kv, qdt=qdt, seed=63)
+    ref, lse_ref = case.oracle()
+    out, lse = case.run(hints=True)
+    assert not torch.isnan(out.float()).any()
+    assert max_abs_err(out, ref) <= REG_TOL_QUANT
+    assert lse_err(lse, lse_ref) <= lse_tol(kv)
+    with ops.option("four_wave_items"):
+        out_4, lse_4 = case.run(hints=True)
+    # two roundings of 16-bit outputs (2^-8 relative) and fp32 summation order
+    assert max_abs_err(out, out_4.float().cpu().numpy().astype(np.float64)) <= 1.6e-2
+    assert lse_err(lse, lse_4.cpu().numpy().astype(np.float64)) <= 1e-5
+    out2, lse2 = case.run(hints=True)
+    assert torch.equal(out, out2) and torch.equal(lse, lse2)
+
+
 @pytest.mark.parametrize("kv,qdt,tol", [("bf16", "bf16", 2e-2), ("fp16", "fp16", 2e-3), ("int8", "bf16", 2e-2)])
 def test_two_stage_decode_merged_by_lse_equals_one_stage(gpu, kv, qdt, tol):
     """The returned log-sum-exps are base 2 and merge as the reference merges two partial attentions
