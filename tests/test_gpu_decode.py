@@ -735,6 +735,43 @@ def test_small_batch_chunk_choices(gpu, kv, name, lens):
         assert torch.equal(out, out_h)
 
 
+@pytest.mark.parametrize("name,kv,qdt,layout,Hq,Hkv,n,bs,lens", [
+    ("equal lengths, fp8", "fp8", "bf16", "HND", 32, 8, 1, 16, [300] * 256),
+    ("equal lengths, int8, two draft tokens", "int8", "fp16", "HND", 32, 8, 2, 128, [517] * 260),
+    ("equal lengths, four kv heads", "fp8", "bf16", "HND", 16, 4, 1, 32, [130] * 512),
+    ("equal lengths, bf16", "bf16", "bf16", "HND", 32, 8, 1, 16, [100] * 300),
+    ("equal lengths, bf16 over NHD", "bf16", "bf16", "NHD", 32, 8, 1, 16, [64] * 256),
+    ("ragged, int8", "int8", "bf16", "HND", 32, 8, 1, 16, None),
+    ("ragged, bf16", "bf16", "bf16", "HND", 32, 8, 1, 16, None),
+])
+def test_four_head_items_for_many_short_sequences(gpu, name, kv, qdt, layout, Hq, Hkv, n, bs, lens):
+    """A large batch of short sequences, with the host's lengths: a work item is four kv heads of a
+    sequence, one per wave (each wave then has a whole sequence to itself), in any layout — from 512 such
+    items on when the lengths are nearly equal, from 2048 on when they are ragged (long ones are then cut
+    and merged by the merge kernel).  Against the oracle and against the same step with an item per head."""
+    print("case four heads per item, short sequences", name, flush=True)
+    if lens is None:
+        rng = np.random.default_rng(17)
+        top = 700 if kv == "int8" else 190
+        lens = rng.integers(1, top, size=1100).astype(np.int32)
+        lens[::53] = 0
+        lens[7] = 6000 if kv == "int8" else 1500  # one sequence far above the rest: cut into chunks
+    case = Case(len(lens), Hq, Hkv, 128, bs, lens, n=n, kv=kv, qdt=qdt, layout=layout, seed=71)
+    assert case.variant() == "mfma_d128"
+    tol = {"bf16": REG_TOL, "fp16": 2e-3}.get(kv, REG_TOL_QUANT)
+    ref, lse_ref = case.oracle()
+    out, lse = case.run(hints=True)
+    assert not torch.isnan(out.float()).any()
+    assert max_abs_err(out, ref) <= tol
+    assert lse_err(lse, lse_ref) <= lse_tol(kv)
+    with ops.option("item_per_head"):
+        out_1, lse_1 = case.run(hints=True)
+    assert max_abs_err(out_1, ref) <= tol
+    assert torch.allclose(out.float(), out_1.float(), rtol=2 ** -6, atol=4e-3)
+    out2, lse2 = case.run(hints=True)
+    assert torch.equal(out, out2) and torch.equal(lse, lse2)
+
+
 @pytest.mark.parametrize("kv,qdt", [("fp8", "bf16"), ("int8", "bf16"), ("int8", "fp16")])
 @pytest.mark.parametrize("name,D,bs,n,lens", [
     ("one long sequence", 128, 16, 1, [32768]),

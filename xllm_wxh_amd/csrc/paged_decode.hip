@@ -216,7 +216,25 @@ static int fill_params(const xllm_hip_kv_cache* c,
   const bool side_by_side = variant == kMfmaD128 && quant && c->stride_head == c->head_dim &&
                             c->stride_slot >= (int64_t)c->num_kv_heads * c->head_dim &&
                             option(XLLM_HIP_OPTION_DECODE_ITEM_PER_HEAD) == 0;
-  p.item_heads = item_heads_of(p.rows, c->num_kv_heads, side_by_side);
+  // The same work items serve a large batch of short sequences in any layout, when the host-side lengths say
+  // so: a wave that has a kv head's whole sequence to itself runs four times as many tiles between its
+  // prologue and its epilogue as a wave with a quarter of it, and ends without the exchange between the four.
+  // As long as such items fill every workgroup slot: over a 1-byte cache up to 8192 tokens per sequence in
+  // the mean (fp8, 64 q heads: 2048 x 256 tokens 242 -> 203 us, 1024 x 512 211 -> 186, 256 x 2048 177 -> 167,
+  // 256 x 6144 499 -> 492; int8 512 x 1024 198 -> 176; 128 x 8192, which gives 256 such items, 326 -> 333:
+  // not those), over a 16-bit cache up to 192 (4096 x 64 tokens 264 -> 193 us, 2048 x 128 202 -> 182, 256 and more the same).
+  // A ragged batch, whose long sequences are cut, has more of them to cut and to merge when an item is four
+  // heads wide: it takes these items from four times as many on (lognormal lengths, fp8, per layer on an
+  // existing schedule: 1024 sequences around 512 tokens 286 -> 243 us, 2048 around 256 336 -> 268, 1024 around
+  // 1024 508 -> 454; 512 sequences around 1024 the same; 256 around 2048, 243 -> 270: not those).
+  const int64_t four_head_items = (int64_t)p.batch * item_heads_of(p.rows, c->num_kv_heads, true);
+  const int64_t slots = natural_target_items(true, p.rows, false);
+  const bool nearly_equal = (int64_t)a->max_seq_len * p.batch * 4 <= a->total_kv_len * 5;
+  const bool short_sequences = variant == kMfmaD128 && a->max_seq_len > 0 && a->total_kv_len > 0 &&
+                               four_head_items >= (nearly_equal ? slots : 4 * slots) &&
+                               a->total_kv_len <= (int64_t)p.batch * (quant ? 8192 : 192) &&
+                               option(XLLM_HIP_OPTION_DECODE_ITEM_PER_HEAD) == 0;
+  p.item_heads = item_heads_of(p.rows, c->num_kv_heads, side_by_side || short_sequences);
   p.heads_per_item = c->num_kv_heads / p.item_heads;
   p.head_dim = c->head_dim;
   p.block_size = c->block_size;
