@@ -427,8 +427,9 @@ enum xllm_hip_option {
                                                * (the plan kernel), also when the host-side lengths would let
                                                * every work item derive its chunk by itself */
   XLLM_HIP_OPTION_DECODE_ITEM_PER_HEAD = 4, /* != 0: a work item is always one kv head, also over a cache whose kv
-                                             * heads lie side by side within a token (NHD), where the 16-row kernel
-                                             * otherwise gives an item four kv heads, one per wave */
+                                             * heads lie side by side within a token (NHD) and for a large batch of
+                                             * short sequences, where the 16-row kernel otherwise gives an item four
+                                             * kv heads, one per wave */
   XLLM_HIP_OPTION_DECODE_FOUR_WAVE_ITEMS = 5, /* != 0: the 16-row kernel always runs four waves per work item, also
                                                * when the launch has at most one item per CU (where it otherwise
                                                * runs eight) */
