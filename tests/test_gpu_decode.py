@@ -613,18 +613,24 @@ def test_long_context_single_sequence(gpu, kv):
         assert torch.equal(out, out_h)
 
 
-def test_large_batch_of_short_sequences(gpu):
-    """3000 sequences (the plan walks the batch 64 at a time), lengths 1..200, some empty."""
-    print("case large batch", flush=True)
+@pytest.mark.parametrize("B,top", [(3000, 200), (9000, 60)])
+def test_large_batch_of_short_sequences(gpu, B, top):
+    """3000 sequences (the plan walks the batch 64 at a time, their lengths held in LDS), lengths 1..200,
+    some empty; 9000 sequences (more than the plan holds in LDS)."""
+    print("case large batch", B, flush=True)
     rng = np.random.default_rng(3)
-    lens = rng.integers(1, 200, size=3000).astype(np.int32)
+    lens = rng.integers(1, top, size=B).astype(np.int32)
     lens[::97] = 0
-    case = Case(3000, 32, 8, 128, 16, lens, seed=32)
+    lens[5] = 40 * top  # one long sequence: the step is split whatever the mean
+    case = Case(B, 32, 8, 128, 16, lens, seed=32)
     ref, _ = case.oracle()
+    ws = torch.empty(ops.decode_workspace_bytes(B, 1, 32, 8, 128), dtype=torch.uint8, device=gpu)
     for hints in (False, True):
-        out, _ = case.run(hints=hints)
+        out, _ = case.run(hints=hints, workspace=ws)
         assert not torch.isnan(out.float()).any()
-        assert max_abs_err(out, ref) <= REG_TOL
+        # (sequences of a handful of tokens are where the 16-bit weights and outputs cost most: 1.4e-2 at
+        # the worst of 288000 rows)
+        assert max_abs_err(out, ref) <= (REG_TOL if B <= 3000 else 1.6e-2)
         assert float(out[::97].float().abs().max()) == 0.0  # empty sequences give zeros
 
 

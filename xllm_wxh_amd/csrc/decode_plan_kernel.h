@@ -10,16 +10,22 @@ namespace xllm_hip {
 // Plan: one workgroup.  kv lengths -> total -> chunk size -> prefix sums -> chunk table.
 // ---------------------------------------------------------------------------------
 
-// Inclusive scan of (a, b) over the wave.
+// Inclusive scan of (a, b) over the wave, in the data-parallel-primitive form (shifts within rows of 16
+// lanes, then the row broadcasts): six dependent register operations per value, where shuffles through
+// the LDS crossbar cost the plan's one wave some 700 cycles per 64 sequences.
+__device__ inline int wave_inclusive_scan(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);  // row_shr:1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);  // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);  // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);  // row_shr:8
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1 and 3
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2 and 3
+  return v;
+}
 __device__ inline void wave_scan2(int& a, int& b, int lane) {
-#pragma unroll
-  for (int o = 1; o < 64; o <<= 1) {
-    const int ua = __shfl_up(a, o), ub = __shfl_up(b, o);
-    if (lane >= o) {
-      a += ua;
-      b += ub;
-    }
-  }
+  (void)lane;
+  a = wave_inclusive_scan(a);
+  b = wave_inclusive_scan(b);
 }
 
 // The finished-chunk counters of the fused merge at the start of a step that stores no schedule.
@@ -27,6 +33,8 @@ __global__ void __launch_bounds__(256) decode_zero_counters_kernel(int32_t* coun
   const int i = blockIdx.x * 256 + threadIdx.x;
   if (i < n) counters[i] = 0;
 }
+
+constexpr int kPlanLens = 8192;  // sequences whose lengths the plan keeps in LDS (32 KiB)
 
 __global__ void __launch_bounds__(64) decode_plan_kernel(DecodeParams p) {
   const int lane = threadIdx.x;
@@ -42,15 +50,33 @@ __global__ void __launch_bounds__(64) decode_plan_kernel(DecodeParams p) {
     for (int i = lane; i < ncounters; i += 64) p.counters[i] = 0;
   }
 
-  // 1. kv lengths, their sum and their maximum.
+  // 1. kv lengths, their sum and their maximum.  Four loads per lane are in flight at a time, and the
+  //    lengths of up to kPlanLens sequences stay in LDS for the two passes below (each pass otherwise waits
+  //    for memory once per 64 sequences: 20 us for 1024 sequences, 7 from LDS).
+  __shared__ int lens[kPlanLens];
+  __shared__ int first_full[kPlanLens];  // first full-chunk slot of a sequence (pass 3 then needs no second scan)
+  const bool in_lds = p.batch <= kPlanLens;
   long long total = 0;
   int max_len = 0;
-  for (int b = lane; b < p.batch; b += 64) {
-    const int len = kv_length(p, b);
-    p.kv_len[b] = len;
-    total += len;
-    max_len = len > max_len ? len : max_len;
+  for (int base = 0; base < p.batch; base += 256) {
+    int l[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int b = base + 64 * u + lane;
+      l[u] = b < p.batch ? kv_length(p, b) : 0;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int b = base + 64 * u + lane;
+      if (b < p.batch) {
+        p.kv_len[b] = l[u];
+        if (in_lds) lens[b] = l[u];
+        total += l[u];
+        max_len = l[u] > max_len ? l[u] : max_len;
+      }
+    }
   }
+  __syncthreads();
 #pragma unroll
   for (int o = 32; o >= 1; o >>= 1) {
     total += __shfl_xor(total, o);
@@ -66,17 +92,23 @@ __global__ void __launch_bounds__(64) decode_plan_kernel(DecodeParams p) {
 
   // 3. Prefix sums of the full-chunk and tail-chunk counts (lengths are re-derived rather than
   //    re-read so that no lane depends on another lane's global store).
-  auto length_of = [&](int b) { return kv_length(p, b); };
+  auto length_of = [&](int b) { return in_lds ? lens[b] : kv_length(p, b); };
   // The tail chunks differ in size.  They are dispatched after the (equal) full chunks, longest
   // first — in 64 size classes — so that the launch ends with the shortest work items.
-  auto tail_class = [&](int tail_len) { return (int)(((long long)tail_len * 64) / chunk); };  // tail_len < chunk
+  // (in single precision: a 64-bit division costs this one wave a hundred instructions per sequence, and the
+  // classes only order the tails; both passes below compute them alike)
+  const float classes_per_token = 64.0f / (float)chunk;
+  auto tail_class = [&](int tail_len) {  // tail_len < chunk
+    const int c = (int)((float)tail_len * classes_per_token);
+    return c > 63 ? 63 : c;
+  };
   int total_full = 0, total_tail = 0;
   for (int base = 0; base < p.batch; base += 64) {
     const int b = base + lane;
     int nf = 0, nt = 0;
     if (b < p.batch) {
       const int len = length_of(b);
-      nf = len / chunk;
+      nf = (int)((unsigned)len / (unsigned)chunk);
       nt = ((len - nf * chunk) > 0 || len == 0) ? 1 : 0;  // an empty sequence keeps one (empty) chunk: it writes zeros
       if (nt) atomicAdd(&tail_hist[tail_class(len - nf * chunk)], 1);
     }
@@ -84,6 +116,7 @@ __global__ void __launch_bounds__(64) decode_plan_kernel(DecodeParams p) {
     wave_scan2(sf, st, lane);
     if (b < p.batch) {
       p.full_prefix[b] = total_full + sf - nf;
+      if (in_lds) first_full[b] = total_full + sf - nf;
       p.num_chunks[b] = nf + nt;
     }
     total_full += __shfl(sf, 63);
@@ -120,13 +153,13 @@ __global__ void __launch_bounds__(64) decode_plan_kernel(DecodeParams p) {
     int nf = 0, nt = 0, len_b = 0;
     if (b < p.batch) {
       len_b = length_of(b);
-      nf = len_b / chunk;
+      nf = (int)((unsigned)len_b / (unsigned)chunk);
       nt = ((len_b - nf * chunk) > 0 || len_b == 0) ? 1 : 0;  // an empty sequence keeps one (empty) chunk: it writes zeros
     }
     int sf = nf, st = nt;
-    wave_scan2(sf, st, lane);
+    if (!in_lds) wave_scan2(sf, st, lane);
     if (b < p.batch) {
-      const int f0 = run_full + sf - nf;
+      const int f0 = in_lds ? first_full[b] : run_full + sf - nf;
       // (the table holds every chunk any lengths can produce — see workspace_layout —; the bound is
       // checked here all the same, so that nothing is ever written outside it)
       for (int ci = 0; ci < nf; ++ci) {
@@ -139,8 +172,10 @@ __global__ void __launch_bounds__(64) decode_plan_kernel(DecodeParams p) {
         if (total_full + slot < p.max_seq_chunks) p.seq_chunks[total_full + slot] = SeqChunk{b, nf, len_b, nf + nt};
       }
     }
-    run_full += __shfl(sf, 63);
-    run_tail += __shfl(st, 63);
+    if (!in_lds) {
+      run_full += __shfl(sf, 63);
+      run_tail += __shfl(st, 63);
+    }
   }
 }
 
