@@ -1030,7 +1030,8 @@ __device__ inline int first_visible_tile(const DecodeParams& p, const Item& it) 
 // Waves per SIMD the 16-row kernel is compiled for: head_dim 256 needs the registers of one.
 constexpr int decode_waves_per_simd(int tok) { return tok == 0 ? 1 : 2; }
 
-// HEADS: a work item covers kWaves neighbouring kv heads of a sequence chunk and wave w attends head
+// HEADS (with DecodeParams::wave_items: four neighbouring work items, one per wave, for steps that are not
+// split): a work item covers kWaves neighbouring kv heads of a sequence chunk and wave w attends head
 // it.hk + w over all of the chunk's tokens (instead of the four waves sharing one head's tokens).  For a
 // cache whose kv heads lie side by side within a token (the NHD layout) the workgroup then reads runs of
 // four rows — 512 bytes of a 1-byte cache — at about the same time, where a workgroup per head reads
@@ -1054,17 +1055,28 @@ __global__ void __launch_bounds__(64 * WAVES, decode_waves_per_simd(TOK)) decode
   constexpr int kP1 = TOK == 0 ? 1 : 0;    // head_dim 256: the second half is the same tokens' second plane
   static_assert(16 * xch_row_bytes(TOK) <= kLdsTile, "the end-of-item exchange must fit a wave's tile");
 
-  Item it;
-  if (!decode_item(p, blockIdx.x, it)) return;
-
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: keeps the loop scalar
+  Item it;
+  if (HEADS && p.wave_items) {
+    // Every wave a work item of its own: four neighbours in the order of the items (kv head fastest), whatever
+    // the head count.  A wave past the last item keeps step with the others — they meet in a barrier at the
+    // end — as an item without rows or tokens.
+    if (!decode_item(p, (int)blockIdx.x * kWaves + wave, it)) {
+      it = Item{};
+      it.ids = p.block_ids;
+      it.nblk = 1;
+      it.chunks = 1;
+    }
+  } else {
+    if (!decode_item(p, blockIdx.x, it)) return;
+    if (HEADS) {
+      it.hk += wave;
+      it.head_off = (int64_t)it.hk * p.stride_head;
+      it.sc_head_off = (int64_t)it.hk * p.sc_stride_head;
+    }
+  }
   const int lane = threadIdx.x & 63;
   uint8_t* tile = lds_all + wave * kLdsTile;  // this wave's private K/V tile
-  if (HEADS) {
-    it.hk += wave;
-    it.head_off = (int64_t)it.hk * p.stride_head;
-    it.sc_head_off = (int64_t)it.hk * p.sc_stride_head;
-  }
 
   RowTile<KV_DT, TOK> rt;
   constexpr bool kRawK = raw_k_of(KV_DT, TOK);

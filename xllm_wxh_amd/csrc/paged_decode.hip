@@ -330,6 +330,19 @@ static int fill_params(const xllm_hip_kv_cache* c,
     if (!decided) p.target_small = every_slot;
   }
   if (!decided) decide();
+  // Many short sequences when the kv heads are no multiple of four (a tensor-parallel shard's one or two):
+  // four neighbouring work items to a workgroup, one per wave, for the same reason as the four-head items
+  // above.  The step is then not split at all (its items fill every slot four times over), which is why
+  // nearly equal lengths are asked for.
+  p.wave_items = 0;
+  if (variant == kMfmaD128 && p.rows <= 16 && p.heads_per_item == 1 && c->num_kv_heads % kHeadsPerItem != 0 && hints &&
+      nearly_equal && (int64_t)p.batch * c->num_kv_heads >= kHeadsPerItem * slots &&
+      a->total_kv_len <= (int64_t)p.batch * (quant ? 8192 : 192) && option(XLLM_HIP_OPTION_DECODE_ITEM_PER_HEAD) == 0) {
+    p.wave_items = 1;
+    p.fixed_chunk = 1 << 30;
+    p.implicit_plan = 1;
+    p.arith_chunks = 0;
+  }
   // XCD clusters: the row groups of a (chunk, kv head); and the kv heads whose rows share 128-byte
   // lines — scale rows shorter than a line (HND: block_size * 4 bytes per head; NHD: the heads of a
   // slot are adjacent floats) or cache rows shorter than a line (NHD with 64 one-byte elements).
@@ -346,7 +359,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
   // (in work items: an item of four heads covers that many of the line's heads itself)
   int items_per_line = (heads_per_line + p.heads_per_item - 1) / p.heads_per_item;
   while (items_per_line > 1 && p.item_heads % items_per_line != 0) --items_per_line;
-  p.cluster = p.row_groups * items_per_line;
+  p.cluster = p.wave_items ? 1 : p.row_groups * items_per_line;
   p.q_dtype = a->q_dtype;
   p.scale_log2 = a->sm_scale * 1.4426950408889634f;
   return XLLM_HIP_OK;
@@ -368,6 +381,7 @@ static int64_t max_items(const DecodeParams& p) {
     const int64_t clusters = (items + p.cluster - 1) / p.cluster;
     items = (clusters + kXcds - 1) / kXcds * kXcds * p.cluster;
   }
+  if (p.wave_items) items = (items + kWaves - 1) / kWaves;  // four of them to a workgroup
   return items;
 }
 
@@ -378,7 +392,7 @@ static void launch_mfma_tok(const DecodeParams& p, unsigned grid, hipStream_t st
     if constexpr (quant_of(KV_DT) && TOK == 1) prefill_quant_d128_kernel<KV_DT><<<grid, 256, 0, st>>>(p);
   } else if (p.rows <= 16) {
     if constexpr (TOK == 1) {
-      if (p.heads_per_item > 1) {
+      if (p.heads_per_item > 1 || p.wave_items) {
         decode_mfma_d128_kernel<KV_DT, TOK, true><<<grid, 64 * kWaves, 0, st>>>(p);
         return;
       }
