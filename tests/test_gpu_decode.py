@@ -784,6 +784,34 @@ def test_four_head_items_for_many_short_sequences(gpu, name, kv, qdt, layout, Hq
     assert torch.equal(out, out2) and torch.equal(lse, lse2)
 
 
+@pytest.mark.parametrize("name,kv,qdt,layout,Hq,Hkv,n,bs,lens", [
+    ("two kv heads, int8", "int8", "bf16", "HND", 14, 2, 1, 32, [260 - (i % 5) for i in range(1100)]),
+    ("two kv heads, bf16, two draft tokens", "bf16", "bf16", "HND", 14, 2, 2, 32, [1500] * 1024),
+    ("eight kv heads, fp8 over NHD", "fp8", "fp16", "NHD", 32, 8, 1, 64, [411] * 256),
+    ("eight kv heads, fp16, ragged", "fp16", "fp16", "HND", 32, 8, 1, 32, None),
+])
+def test_items_per_wave_at_head_dim_64(gpu, name, kv, qdt, layout, Hq, Hkv, n, bs, lens):
+    """The same work items (four kv heads, or four neighbouring items, one per wave) at head_dim 64."""
+    print("case item per wave, head_dim 64", name, flush=True)
+    if lens is None:
+        rng = np.random.default_rng(19)
+        lens = rng.integers(1, 900, size=1030).astype(np.int32)
+        lens[::41] = 0
+        lens[3] = 9000
+    case = Case(len(lens), Hq, Hkv, 64, bs, lens, n=n, kv=kv, qdt=qdt, layout=layout, seed=73)
+    assert case.variant() == "mfma_d64"
+    tol = {"bf16": REG_TOL, "fp16": 2e-3}.get(kv, REG_TOL_QUANT)
+    ref, lse_ref = case.oracle()
+    out, lse = case.run(hints=True)
+    assert not torch.isnan(out.float()).any()
+    assert max_abs_err(out, ref) <= tol
+    assert lse_err(lse, lse_ref) <= LSE_TOL
+    with ops.option("item_per_head"):
+        out_1, _ = case.run(hints=True)
+    assert max_abs_err(out_1, ref) <= tol
+    assert torch.allclose(out.float(), out_1.float(), rtol=2 ** -6, atol=4e-3)
+
+
 @pytest.mark.parametrize("kv,qdt", [("fp8", "bf16"), ("int8", "bf16"), ("int8", "fp16")])
 @pytest.mark.parametrize("name,D,bs,n,lens", [
     ("one long sequence", 128, 16, 1, [32768]),

@@ -223,6 +223,8 @@ static int fill_params(const xllm_hip_kv_cache* c,
   // the mean (fp8, 64 q heads: 2048 x 256 tokens 242 -> 203 us, 1024 x 512 211 -> 186, 256 x 2048 177 -> 167,
   // 256 x 6144 499 -> 492; int8 512 x 1024 198 -> 176; 128 x 8192, which gives 256 such items, 326 -> 333:
   // not those), over a 16-bit cache up to 192 (4096 x 64 tokens 264 -> 193 us, 2048 x 128 202 -> 182, 256 and more the same).
+  // head_dim 64 likewise, a 16-bit cache up to 2048 tokens (14q/2kv: int8 2048 x 1024 tokens 112 -> 95 us, 4096 x 256
+  // 88 -> 62; bf16 4096 x 128 69 -> 51, 2048 x 768 130 -> 127, 2048 tokens the same).
   // A ragged batch, whose long sequences are cut, has more of them to cut and to merge when an item is four
   // heads wide: it takes these items from four times as many on (lognormal lengths, fp8, per layer on an
   // existing schedule: 1024 sequences around 512 tokens 286 -> 243 us, 2048 around 256 336 -> 268, 1024 around
@@ -230,9 +232,9 @@ static int fill_params(const xllm_hip_kv_cache* c,
   const int64_t four_head_items = (int64_t)p.batch * item_heads_of(p.rows, c->num_kv_heads, true);
   const int64_t slots = natural_target_items(true, p.rows, false);
   const bool nearly_equal = (int64_t)a->max_seq_len * p.batch * 4 <= a->total_kv_len * 5;
-  const bool short_sequences = variant == kMfmaD128 && a->max_seq_len > 0 && a->total_kv_len > 0 &&
+  const bool short_sequences = (variant == kMfmaD128 || variant == kMfmaD64) && a->max_seq_len > 0 && a->total_kv_len > 0 &&
                                four_head_items >= (nearly_equal ? slots : 4 * slots) &&
-                               a->total_kv_len <= (int64_t)p.batch * (quant ? 8192 : 192) &&
+                               a->total_kv_len <= (int64_t)p.batch * (quant ? 8192 : variant == kMfmaD64 ? 2048 : 192) &&
                                option(XLLM_HIP_OPTION_DECODE_ITEM_PER_HEAD) == 0;
   p.item_heads = item_heads_of(p.rows, c->num_kv_heads, side_by_side || short_sequences);
   p.heads_per_item = c->num_kv_heads / p.item_heads;
@@ -335,9 +337,10 @@ static int fill_params(const xllm_hip_kv_cache* c,
   // above.  The step is then not split at all (its items fill every slot four times over), which is why
   // nearly equal lengths are asked for.
   p.wave_items = 0;
-  if (variant == kMfmaD128 && p.rows <= 16 && p.heads_per_item == 1 && c->num_kv_heads % kHeadsPerItem != 0 && hints &&
+  if ((variant == kMfmaD128 || variant == kMfmaD64) && p.rows <= 16 && p.heads_per_item == 1 &&
+      c->num_kv_heads % kHeadsPerItem != 0 && hints &&
       nearly_equal && (int64_t)p.batch * c->num_kv_heads >= kHeadsPerItem * slots &&
-      a->total_kv_len <= (int64_t)p.batch * (quant ? 8192 : 192) && option(XLLM_HIP_OPTION_DECODE_ITEM_PER_HEAD) == 0) {
+      a->total_kv_len <= (int64_t)p.batch * (quant ? 8192 : variant == kMfmaD64 ? 2048 : 192) && option(XLLM_HIP_OPTION_DECODE_ITEM_PER_HEAD) == 0) {
     p.wave_items = 1;
     p.fixed_chunk = 1 << 30;
     p.implicit_plan = 1;
@@ -391,7 +394,7 @@ static void launch_mfma_tok(const DecodeParams& p, unsigned grid, hipStream_t st
     if constexpr (!quant_of(KV_DT) && TOK != 0) prefill_mfma_d128_kernel<KV_DT, TOK><<<grid, 256, 0, st>>>(p);
     if constexpr (quant_of(KV_DT) && TOK == 1) prefill_quant_d128_kernel<KV_DT><<<grid, 256, 0, st>>>(p);
   } else if (p.rows <= 16) {
-    if constexpr (TOK == 1) {
+    if constexpr (TOK != 0) {
       if (p.heads_per_item > 1 || p.wave_items) {
         decode_mfma_d128_kernel<KV_DT, TOK, true><<<grid, 64 * kWaves, 0, st>>>(p);
         return;
