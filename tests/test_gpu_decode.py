@@ -743,24 +743,29 @@ def test_small_batch_chunk_choices(gpu, kv, name, lens):
 
 @pytest.mark.parametrize("name,kv,qdt,layout,Hq,Hkv,n,bs,lens", [
     ("equal lengths, fp8", "fp8", "bf16", "HND", 32, 8, 1, 16, [300] * 256),
-    ("equal lengths, int8, two draft tokens", "int8", "fp16", "HND", 32, 8, 2, 128, [517] * 260),
+    ("equal lengths, int8, two draft tokens", "int8", "fp16", "HND", 32, 8, 2, 128, [517] * 256),
     ("equal lengths, four kv heads", "fp8", "bf16", "HND", 16, 4, 1, 32, [130] * 512),
-    ("equal lengths, bf16", "bf16", "bf16", "HND", 32, 8, 1, 16, [100] * 300),
+    ("equal lengths, bf16", "bf16", "bf16", "HND", 32, 8, 1, 16, [100] * 512),
     ("equal lengths, bf16 over NHD", "bf16", "bf16", "NHD", 32, 8, 1, 16, [64] * 256),
     ("ragged, int8", "int8", "bf16", "HND", 32, 8, 1, 16, None),
     ("ragged, bf16", "bf16", "bf16", "HND", 32, 8, 1, 16, None),
     # kv heads that are no multiple of four: four neighbouring (sequence, kv head) items to a workgroup
-    ("one kv head, fp8, last workgroup with one item", "fp8", "bf16", "HND", 8, 1, 1, 16, [200] * 2101),
-    ("two kv heads, int8, two draft tokens", "int8", "fp16", "HND", 8, 2, 2, 32, [300 - (i % 7) for i in range(1031)]),
-    ("one kv head, bf16", "bf16", "bf16", "HND", 8, 1, 1, 16, [100] * 2050),
-    ("six kv heads over NHD, fp8, some sequences empty", "fp8", "bf16", "NHD", 12, 6, 1, 16, [0 if i % 50 == 3 else 333 for i in range(350)]),
+    ("one kv head, fp8, last workgroup with one item", "fp8", "bf16", "HND", 8, 1, 1, 16, [200] * 2045),
+    ("two kv heads, int8, two draft tokens", "int8", "fp16", "HND", 8, 2, 2, 32, [300 - (i % 7) for i in range(1023)]),
+    ("one kv head, bf16", "bf16", "bf16", "HND", 8, 1, 1, 16, [100] * 2048),
+    # half as many items: two waves to an item, two items to a workgroup (the last one with a single item)
+    ("eight kv heads, fp8, two waves per item", "fp8", "bf16", "HND", 32, 8, 1, 16, [700] * 128),
+    ("one kv head, int8, two waves per item", "int8", "bf16", "HND", 8, 1, 2, 64, [450 - (i % 3) for i in range(1023)]),
+    ("six kv heads over NHD, fp8, some sequences empty", "fp8", "bf16", "NHD", 12, 6, 1, 16, [0 if i % 50 == 3 else 333 for i in range(341)]),
 ])
 def test_four_head_items_for_many_short_sequences(gpu, name, kv, qdt, layout, Hq, Hkv, n, bs, lens):
     """A large batch of short sequences, with the host's lengths: a work item is four kv heads of a
     sequence, one per wave (each wave then has a whole sequence to itself), in any layout — from 512 such
     items on when the lengths are nearly equal, from 2048 on when they are ragged (long ones are then cut
     and merged by the merge kernel); with a head count that is no multiple of four, four neighbouring items
-    of a step that is not split.  Against the oracle and against the same step with an item per head."""
+    of a step that is not split, and with half as many items two waves to an item.  (Batch sizes whose wider
+    workgroups fill whole rounds of the GPU's slots: others keep an item per head.)  Against the oracle
+    and against the same step with an item per head."""
     print("case four heads per item, short sequences", name, flush=True)
     if lens is None:
         rng = np.random.default_rng(17)
@@ -785,7 +790,7 @@ def test_four_head_items_for_many_short_sequences(gpu, name, kv, qdt, layout, Hq
 
 
 @pytest.mark.parametrize("name,kv,qdt,layout,Hq,Hkv,n,bs,lens", [
-    ("two kv heads, int8", "int8", "bf16", "HND", 14, 2, 1, 32, [260 - (i % 5) for i in range(1100)]),
+    ("two kv heads, int8", "int8", "bf16", "HND", 14, 2, 1, 32, [260 - (i % 5) for i in range(1024)]),
     ("two kv heads, bf16, two draft tokens", "bf16", "bf16", "HND", 14, 2, 2, 32, [1500] * 1024),
     ("eight kv heads, fp8 over NHD", "fp8", "fp16", "NHD", 32, 8, 1, 64, [411] * 256),
     ("eight kv heads, fp16, ragged", "fp16", "fp16", "HND", 32, 8, 1, 32, None),

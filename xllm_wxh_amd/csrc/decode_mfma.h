@@ -1057,11 +1057,14 @@ __global__ void __launch_bounds__(64 * WAVES, decode_waves_per_simd(TOK)) decode
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: keeps the loop scalar
   Item it;
-  if (HEADS && p.wave_items) {
-    // Every wave a work item of its own: four neighbours in the order of the items (kv head fastest), whatever
-    // the head count.  A wave past the last item keeps step with the others — they meet in a barrier at the
-    // end — as an item without rows or tokens.
-    if (!decode_item(p, (int)blockIdx.x * kWaves + wave, it)) {
+  // (wave_items: 1 — every wave a work item of its own —, or 2: two waves share an item's tokens, two items to the workgroup)
+  const int item_waves = HEADS ? __builtin_amdgcn_readfirstlane(p.wave_items) : 0;
+  if (HEADS && item_waves) {
+    // Neighbours in the order of the items (kv head fastest), whatever the head count.  A wave past the
+    // last item keeps step with the others — they meet in a barrier at the end — as an item without rows
+    // or tokens.
+    const int vid = item_waves == 2 ? (int)blockIdx.x * 2 + (wave >> 1) : (int)blockIdx.x * kWaves + wave;
+    if (!decode_item(p, vid, it)) {
       it = Item{};
       it.ids = p.block_ids;
       it.nblk = 1;
@@ -1086,8 +1089,9 @@ __global__ void __launch_bounds__(64 * WAVES, decode_waves_per_simd(TOK)) decode
   // This wave's share of the item's tokens.
   const int t0 = first_visible_tile(p, it);
   const int span = it.t_end - t0;
-  const int share = span <= 0 ? 0 : HEADS ? ((span + kT - 1) & ~(kT - 1)) : (((span + WAVES - 1) / WAVES + kT - 1) & ~(kT - 1));
-  const int w_begin = HEADS ? t0 : t0 + wave * share;
+  const int sharers = !HEADS ? WAVES : item_waves == 2 ? 2 : 1;  // waves that split the item's tokens
+  const int share = span <= 0 ? 0 : (((span + sharers - 1) / sharers + kT - 1) & ~(kT - 1));
+  const int w_begin = !HEADS ? t0 + wave * share : item_waves == 2 ? t0 + (wave & 1) * share : t0;
   const int w_end = min(it.t_end, w_begin + share);
   const int mask_hi_from = it.len - (it.n - 1);                                    // tiles reaching past this need masks
   const int mask_lo_until = p.window_left >= 0 ? it.len - 1 - p.window_left : 0;  // tiles starting below this too
@@ -1146,7 +1150,11 @@ __global__ void __launch_bounds__(64 * WAVES, decode_waves_per_simd(TOK)) decode
       (const __attribute__((address_space(4))) DecodeParams*)__builtin_amdgcn_kernarg_segment_ptr();
   asm volatile("" : "+s"(pm));
   if constexpr (HEADS) {
-    finish_item<KV_DT, TOK, 1>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, wave, 0, lane_id(), 0);
+    if (item_waves == 2) {
+      finish_item<KV_DT, TOK, 2>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, wave >> 1, wave & 1, lane_id(), 0);
+    } else {
+      finish_item<KV_DT, TOK, 1>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, wave, 0, lane_id(), 0);
+    }
   } else {
     finish_item<KV_DT, TOK, WAVES>(p, it, rt, lds_all, kLdsTile, lds_ml, wave, 0, wave, lane_id(), 0);
   }

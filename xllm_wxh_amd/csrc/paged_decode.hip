@@ -229,12 +229,34 @@ static int fill_params(const xllm_hip_kv_cache* c,
   // heads wide: it takes these items from four times as many on (lognormal lengths, fp8, per layer on an
   // existing schedule: 1024 sequences around 512 tokens 286 -> 243 us, 2048 around 256 336 -> 268, 1024 around
   // 1024 508 -> 454; 512 sequences around 1024 the same; 256 around 2048, 243 -> 270: not those).
+  // Equal items run in rounds of as many workgroups as there are slots, and a workgroup that does the work of
+  // four makes the last, partly filled round four times as long: 288 sequences of 2048 fp8 tokens x 8 kv heads
+  // are 576 such workgroups, 1.125 rounds, 258 us against 202 as 2304 workgroups of one head each (4.5 rounds);
+  // 320 sequences 261 against 219, 640 (2.5 rounds against 10) 443 against 432.  So for nearly equal lengths
+  // the wider items are taken when (filled share of their rounds) x (their measured gain for the step's mean
+  // length) beats the filled share of the narrow items' rounds.
   const int64_t four_head_items = (int64_t)p.batch * item_heads_of(p.rows, c->num_kv_heads, true);
   const int64_t slots = natural_target_items(true, p.rows, false);
   const bool nearly_equal = (int64_t)a->max_seq_len * p.batch * 4 <= a->total_kv_len * 5;
+  auto wider_items_pay = [&](int64_t narrow_items, int per_workgroup) {
+    auto filled = [&](int64_t workgroups) {
+      const int64_t rounds = (workgroups + slots - 1) / slots;
+      return rounds > 0 ? (double)workgroups / (double)(rounds * slots) : 1.0;
+    };
+    const double mean = (double)a->total_kv_len / (double)(p.batch > 0 ? p.batch : 1);
+    // gain of one wave per item over four, by mean length: 1-byte rows of 128 bytes 100 / L (19 % at 256 tokens,
+    // 5 % at 2048), of 64 bytes 200 / L; 16-bit rows of 256 bytes 16 / L, of 128 bytes 25 / L
+    const double k = variant == kMfmaD64 ? (quant ? 200.0 : 25.0) : (quant ? 100.0 : 16.0);
+    double gain = k / (mean > 1.0 ? mean : 1.0);
+    const double cap = quant ? (variant == kMfmaD64 ? 0.4 : 0.2) : 0.3;
+    gain = gain < cap ? gain : cap;
+    if (per_workgroup == 2) gain *= 0.5;
+    return filled((narrow_items + per_workgroup - 1) / per_workgroup) * (1.0 + gain) > filled(narrow_items) * 1.01;
+  };
   const bool short_sequences = (variant == kMfmaD128 || variant == kMfmaD64) && a->max_seq_len > 0 && a->total_kv_len > 0 &&
                                four_head_items >= (nearly_equal ? slots : 4 * slots) &&
                                a->total_kv_len <= (int64_t)p.batch * (quant ? 8192 : variant == kMfmaD64 ? 2048 : 192) &&
+                               (!nearly_equal || wider_items_pay((int64_t)p.batch * c->num_kv_heads, kHeadsPerItem)) &&
                                option(XLLM_HIP_OPTION_DECODE_ITEM_PER_HEAD) == 0;
   p.item_heads = item_heads_of(p.rows, c->num_kv_heads, side_by_side || short_sequences);
   p.heads_per_item = c->num_kv_heads / p.item_heads;
@@ -335,16 +357,21 @@ static int fill_params(const xllm_hip_kv_cache* c,
   // Many short sequences when the kv heads are no multiple of four (a tensor-parallel shard's one or two):
   // four neighbouring work items to a workgroup, one per wave, for the same reason as the four-head items
   // above.  The step is then not split at all (its items fill every slot four times over), which is why
-  // nearly equal lengths are asked for.
+  // nearly equal lengths are asked for.  With half as many items (from 1024 on, any head count) two waves
+  // share an item and a workgroup takes two (fp8, 128 sequences of 2048 tokens x 8 kv heads: 89.5 -> 86.4 us;
+  // 192 sequences, 1.5 rounds of such workgroups, would take 148 against 134: see wider_items_pay).
   p.wave_items = 0;
-  if ((variant == kMfmaD128 || variant == kMfmaD64) && p.rows <= 16 && p.heads_per_item == 1 &&
-      c->num_kv_heads % kHeadsPerItem != 0 && hints &&
-      nearly_equal && (int64_t)p.batch * c->num_kv_heads >= kHeadsPerItem * slots &&
-      a->total_kv_len <= (int64_t)p.batch * (quant ? 8192 : variant == kMfmaD64 ? 2048 : 192) && option(XLLM_HIP_OPTION_DECODE_ITEM_PER_HEAD) == 0) {
-    p.wave_items = 1;
-    p.fixed_chunk = 1 << 30;
-    p.implicit_plan = 1;
-    p.arith_chunks = 0;
+  if ((variant == kMfmaD128 || variant == kMfmaD64) && p.rows <= 16 && p.heads_per_item == 1 && hints && nearly_equal &&
+      a->total_kv_len <= (int64_t)p.batch * (quant ? 8192 : variant == kMfmaD64 ? 2048 : 192) &&
+      option(XLLM_HIP_OPTION_DECODE_ITEM_PER_HEAD) == 0) {
+    const int64_t items = (int64_t)p.batch * c->num_kv_heads;
+    const int per_group = items >= kHeadsPerItem * slots ? 1 : items >= 2 * slots ? 2 : 0;
+    if (per_group != 0 && wider_items_pay(items, per_group == 1 ? kWaves : 2)) {
+      p.wave_items = per_group;
+      p.fixed_chunk = 1 << 30;
+      p.implicit_plan = 1;
+      p.arith_chunks = 0;
+    }
   }
   // XCD clusters: the row groups of a (chunk, kv head); and the kv heads whose rows share 128-byte
   // lines — scale rows shorter than a line (HND: block_size * 4 bytes per head; NHD: the heads of a
@@ -384,7 +411,8 @@ static int64_t max_items(const DecodeParams& p) {
     const int64_t clusters = (items + p.cluster - 1) / p.cluster;
     items = (clusters + kXcds - 1) / kXcds * kXcds * p.cluster;
   }
-  if (p.wave_items) items = (items + kWaves - 1) / kWaves;  // four of them to a workgroup
+  if (p.wave_items == 1) items = (items + kWaves - 1) / kWaves;  // four of them to a workgroup
+  if (p.wave_items == 2) items = (items + 1) / 2;
   return items;
 }
 
