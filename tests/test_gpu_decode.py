@@ -846,6 +846,46 @@ def test_eight_wave_items_over_one_byte_caches(gpu, kv, qdt, name, D, bs, n, len
     assert torch.equal(out, out2) and torch.equal(lse, lse2)
 
 
+@pytest.mark.parametrize("kv,qdt", [("bf16", "bf16"), ("fp8", "bf16"), ("int8", "fp16")])
+@pytest.mark.parametrize("name,Hq,Hkv,D,n,bs,lens", [
+    ("two sequences past one round", 32, 8, 128, 1, 16, [1500] * 66),
+    ("eight past one round, nearly equal lengths, one empty", 32, 8, 128, 2, 32, [1400 - 3 * (i % 40) for i in range(71)] + [0]),
+    ("a sequence past two rounds", 16, 4, 128, 1, 128, [700] * 257),
+    ("one kv head", 8, 1, 128, 1, 16, [640] * 520),
+    ("head_dim 64", 14, 2, 64, 1, 32, [900] * 260),
+    ("head_dim 256: rounds of 256", 16, 4, 256, 1, 16, [1100] * 66),
+])
+def test_sequences_of_a_partly_filled_round_are_cut(gpu, kv, qdt, name, Hq, Hkv, D, n, bs, lens):
+    """Equal work items a few more than a whole number of rounds of the GPU's workgroup slots: with the host's
+    lengths the sequences of the last round are cut into chunks that fill the slots once more (merged inside
+    the attention kernel) and the others stay whole.  Against the oracle, against the same step left whole
+    (the stored-schedule option keeps it so), on wrong host-side lengths, and twice in a row."""
+    print("case last round cut", kv, name, flush=True)
+    case = Case(len(lens), Hq, Hkv, D, bs, lens, n=n, kv=kv, qdt=qdt, seed=83)
+    tol = {"bf16": REG_TOL, "fp16": 2e-3}.get(kv, REG_TOL_QUANT)
+    ref, lse_ref = case.oracle()
+    nbytes = ops.decode_workspace_bytes(case.B, n, Hq, Hkv, D)
+    ws = torch.full((nbytes,), 0xA5, dtype=torch.uint8, device=gpu)
+    out, lse = case.run(workspace=ws, hints=True)
+    assert not torch.isnan(out.float()).any()
+    assert max_abs_err(out, ref) <= tol
+    assert lse_err(lse, lse_ref) <= lse_tol(kv)
+    with ops.option("stored_schedule"):
+        out_w, lse_w = case.run(workspace=ws, hints=True)
+    assert max_abs_err(out_w, ref) <= tol
+    assert torch.allclose(out.float(), out_w.float(), rtol=2 ** -6, atol=4e-3)
+    # the first sequences are whole either way: the same bits
+    assert torch.equal(out[: 8 * n], out_w[: 8 * n]) and torch.equal(lse[: 8 * n], lse_w[: 8 * n])
+    # some of the last were cut
+    assert not torch.equal(lse[-8 * n:], lse_w[-8 * n:])
+    # host-side lengths that are too small: a sequence's last chunk takes the rest
+    longest, total = int(max(lens)), int(sum(lens))
+    out_s, lse_s = case.run(workspace=ws, max_seq_len=max(1, longest * 3 // 4), total_kv_len=max(1, total * 3 // 4))
+    assert max_abs_err(out_s, ref) <= tol
+    out2, lse2 = case.run(workspace=ws, hints=True, plan=False)
+    assert torch.equal(out2, out) and torch.equal(lse2, lse)
+
+
 @pytest.mark.parametrize("kv,qdt,tol", [("bf16", "bf16", 2e-2), ("fp16", "fp16", 2e-3), ("int8", "bf16", 2e-2)])
 def test_two_stage_decode_merged_by_lse_equals_one_stage(gpu, kv, qdt, tol):
     """The returned log-sum-exps are base 2 and merge as the reference merges two partial attentions

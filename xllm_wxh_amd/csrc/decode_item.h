@@ -55,15 +55,21 @@ __device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it)
     // No stored schedule: slot = sequence * arith_chunks + chunk.  The block list, the queries and the
     // length are then independent loads.  A sequence longer than its slots hold (a host-side
     // max_seq_len that was too small) gives the rest to its last chunk.
-    it.b = it.sc / p.arith_chunks;
-    chunk = it.sc - it.b * p.arith_chunks;
+    // The first arith_whole sequences are not cut: one slot each, ahead of the others' (they are the long
+    // items of the launch, and run first).
+    const bool whole = it.sc < p.arith_whole;
+    const int rest_sc = it.sc - p.arith_whole;
+    it.b = whole ? it.sc : p.arith_whole + rest_sc / p.arith_chunks;
+    chunk = whole ? 0 : rest_sc - (it.b - p.arith_whole) * p.arith_chunks;
     if (it.b >= p.batch) return false;
     it.len = kv_length(p, it.b);
-    const int cnt = chunks_of_length(it.len, p.fixed_chunk);
-    it.chunks = cnt < p.arith_chunks ? cnt : p.arith_chunks;
-    if (chunk >= it.chunks) return false;
-    chunk_tokens = p.fixed_chunk;
-    to_the_end = chunk == p.arith_chunks - 1;
+    if (!whole) {
+      const int cnt = chunks_of_length(it.len, p.fixed_chunk);
+      it.chunks = cnt < p.arith_chunks ? cnt : p.arith_chunks;
+      if (chunk >= it.chunks) return false;
+      chunk_tokens = p.fixed_chunk;
+      to_the_end = chunk == p.arith_chunks - 1;
+    }
   } else {
     // The header and the item's record are independent loads (the record's index is clamped to the
     // table, whose last entries the plan may not have written: such a record is not used).

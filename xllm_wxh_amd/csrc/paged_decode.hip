@@ -362,6 +362,42 @@ static int fill_params(const xllm_hip_kv_cache* c,
     if (!decided) p.target_small = every_slot;
   }
   if (!decided) decide();
+  // Equal items beyond whole rounds of the slots: 66 sequences x 8 kv heads are 528 work items for 512 slots,
+  // and the 16 of the second round take as long as the 512 of the first (fp8, 8192 tokens: 255 us against 167
+  // for 64 sequences).  The sequences of the last, partly filled round are therefore cut into as many chunks
+  // as fill the slots once more — 2 sequences x 8 heads x 32 chunks — while the others stay whole (arith_whole):
+  // the last round then takes a fraction of a whole one.
+  p.arith_whole = 0;
+  if (is_mfma(variant) && p.rows <= 16 && p.heads_per_item == 1 && p.fused_merge && p.implicit_plan && hints &&
+      nearly_equal && option(XLLM_HIP_OPTION_DECODE_STORED_SCHEDULE) == 0) {
+    const int64_t per = (int64_t)p.item_heads * p.row_groups;
+    const int64_t items = (int64_t)p.batch * per;
+    const int64_t round = p.target_items;
+    const int64_t whole_rounds = items / round;
+    // (from four whole rounds on the last one weighs little: 288 x 2048 fp8 tokens, 4.5 rounds, 202 us whole, 206 cut)
+    if (whole_rounds >= 1 && whole_rounds <= 3 && items % round != 0) {
+      const int64_t whole_seqs = whole_rounds * round / per;
+      const int64_t cut_seqs = p.batch - whole_seqs;
+      int64_t k = round / (cut_seqs * per);
+      k = k > 32 ? 32 : k;  // (what the fused merge loads in one batch)
+      // (a 16-bit cache's few items of a last round stream fast enough whole unless they are very few: bf16, 4096
+      // tokens x 8 kv heads, 66 sequences 192 -> 168 us cut, 72 196 -> 191, but 80 204 -> 215 and 96 236 -> 244;
+      // fp8, 8192 tokens: 66 sequences 255 -> 179, 80 260 -> 217, 96 277 -> 258, 136 413 -> 359)
+      if (!quant && k < 8) k = 1;
+      if (k >= 2) {
+        int64_t chunk = ((int64_t)a->max_seq_len + k - 1) / k;
+        chunk = (chunk + p.tile_tokens - 1) / p.tile_tokens * p.tile_tokens;
+        chunk = chunk < p.min_chunk ? p.min_chunk : chunk;
+        k = ((int64_t)a->max_seq_len + chunk - 1) / chunk;
+        if (k >= 2 && whole_seqs + cut_seqs * k <= w.max_seq_chunks) {
+          p.fixed_chunk = (int32_t)chunk;
+          p.arith_chunks = (int32_t)k;
+          p.arith_whole = (int32_t)whole_seqs;
+          p.implicit_plan = 0;
+        }
+      }
+    }
+  }
   // Many short sequences when the kv heads are no multiple of four (a tensor-parallel shard's one or two):
   // four neighbouring work items to a workgroup, one per wave, for the same reason as the four-head items
   // above.  The step is then not split at all (its items fill every slot four times over), which is why
@@ -379,6 +415,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
       p.fixed_chunk = 1 << 30;
       p.implicit_plan = 1;
       p.arith_chunks = 0;
+      p.arith_whole = 0;
     }
   }
   // XCD clusters: the row groups of a (chunk, kv head); and the kv heads whose rows share 128-byte
@@ -408,7 +445,7 @@ static int64_t max_items(const DecodeParams& p) {
   const int64_t per = (int64_t)p.item_heads * p.row_groups;
   int64_t seq_chunks = p.batch;
   if (p.arith_chunks > 0) {
-    seq_chunks = (int64_t)p.batch * p.arith_chunks;
+    seq_chunks = p.arith_whole + (int64_t)(p.batch - p.arith_whole) * p.arith_chunks;
   } else if (p.fixed_chunk != (1 << 30)) {
     int64_t t = 2 * (int64_t)p.target_items;  // choose_chunk may raise the target (by a quarter)
     if (t > kMaxTargetItems) t = kMaxTargetItems;
