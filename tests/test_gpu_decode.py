@@ -846,20 +846,30 @@ def test_eight_wave_items_over_one_byte_caches(gpu, kv, qdt, name, D, bs, n, len
     assert torch.equal(out, out2) and torch.equal(lse, lse2)
 
 
+ALL_KV = ("bf16", "fp8", "int8")
+
+
 @pytest.mark.parametrize("kv,qdt", [("bf16", "bf16"), ("fp8", "bf16"), ("int8", "fp16")])
-@pytest.mark.parametrize("name,Hq,Hkv,D,n,bs,lens", [
-    ("two sequences past one round", 32, 8, 128, 1, 16, [1500] * 66),
-    ("eight past one round, nearly equal lengths, one empty", 32, 8, 128, 2, 32, [1400 - 3 * (i % 40) for i in range(71)] + [0]),
-    ("a sequence past two rounds", 16, 4, 128, 1, 128, [700] * 257),
-    ("one kv head", 8, 1, 128, 1, 16, [640] * 520),
-    ("head_dim 64", 14, 2, 64, 1, 32, [900] * 260),
-    ("head_dim 256: rounds of 256", 16, 4, 256, 1, 16, [1100] * 66),
+@pytest.mark.parametrize("name,Hq,Hkv,D,n,bs,lens,cut_for", [
+    ("two sequences past one round", 32, 8, 128, 1, 16, [1500] * 66, ALL_KV),
+    # (16-bit caches: only when the last round's items are at most an eighth of a round)
+    ("eight past one round, nearly equal lengths, one empty", 32, 8, 128, 2, 32,
+     [1400 - 3 * (i % 40) for i in range(71)] + [0], ("fp8", "int8")),
+    ("a sequence past two rounds", 16, 4, 128, 1, 128, [700] * 257, ALL_KV),
+    ("one kv head", 8, 1, 128, 1, 16, [640] * 520, ALL_KV),
+    ("head_dim 64", 14, 2, 64, 1, 32, [900] * 260, ALL_KV),
+    ("head_dim 256: rounds of 256", 16, 4, 256, 1, 16, [1100] * 66, ALL_KV),
+    # fewer items than slots: 1-byte caches are cut in two throughout, the last sequences finer
+    ("an item per CU and sixteen more", 32, 8, 128, 1, 16, [3200] * 34, ALL_KV),
+    # (... unless the sequences are too short for six chunks)
+    ("an item per CU and eight more, short sequences", 32, 8, 128, 2, 64, [1800] * 33, ("bf16",)),
 ])
-def test_sequences_of_a_partly_filled_round_are_cut(gpu, kv, qdt, name, Hq, Hkv, D, n, bs, lens):
-    """Equal work items a few more than a whole number of rounds of the GPU's workgroup slots: with the host's
-    lengths the sequences of the last round are cut into chunks that fill the slots once more (merged inside
-    the attention kernel) and the others stay whole.  Against the oracle, against the same step left whole
-    (the stored-schedule option keeps it so), on wrong host-side lengths, and twice in a row."""
+def test_sequences_of_a_partly_filled_round_are_cut(gpu, kv, qdt, name, Hq, Hkv, D, n, bs, lens, cut_for):
+    """Equal work items a few more than a whole number of rounds of the GPU (an item per CU over a 16-bit cache,
+    every workgroup slot over a 1-byte one): with the host's lengths the sequences of the last round are cut into
+    chunks that fill a round once more (merged inside the attention kernel) and the others stay as they are.
+    Against the oracle, against the same step left whole (the stored-schedule option keeps it so), on wrong
+    host-side lengths, and twice in a row."""
     print("case last round cut", kv, name, flush=True)
     case = Case(len(lens), Hq, Hkv, D, bs, lens, n=n, kv=kv, qdt=qdt, seed=83)
     tol = {"bf16": REG_TOL, "fp16": 2e-3}.get(kv, REG_TOL_QUANT)
@@ -874,10 +884,13 @@ def test_sequences_of_a_partly_filled_round_are_cut(gpu, kv, qdt, name, Hq, Hkv,
         out_w, lse_w = case.run(workspace=ws, hints=True)
     assert max_abs_err(out_w, ref) <= tol
     assert torch.allclose(out.float(), out_w.float(), rtol=2 ** -6, atol=4e-3)
-    # the first sequences are whole either way: the same bits
-    assert torch.equal(out[: 8 * n], out_w[: 8 * n]) and torch.equal(lse[: 8 * n], lse_w[: 8 * n])
-    # some of the last were cut
-    assert not torch.equal(lse[-8 * n:], lse_w[-8 * n:])
+    rows = 8 * n
+    if kv in cut_for:
+        assert not torch.equal(lse[-rows:], lse_w[-rows:]), "the last sequences were not cut"
+        if len(lens) >= 64 or kv == "bf16":  # (the first sequences stay whole: the same bits)
+            assert torch.equal(out[:rows], out_w[:rows]) and torch.equal(lse[:rows], lse_w[:rows])
+    else:
+        assert torch.equal(out, out_w) and torch.equal(lse, lse_w)
     # host-side lengths that are too small: a sequence's last chunk takes the rest
     longest, total = int(max(lens)), int(sum(lens))
     out_s, lse_s = case.run(workspace=ws, max_seq_len=max(1, longest * 3 // 4), total_kv_len=max(1, total * 3 // 4))

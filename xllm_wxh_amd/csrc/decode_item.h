@@ -55,21 +55,21 @@ __device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it)
     // No stored schedule: slot = sequence * arith_chunks + chunk.  The block list, the queries and the
     // length are then independent loads.  A sequence longer than its slots hold (a host-side
     // max_seq_len that was too small) gives the rest to its last chunk.
-    // The first arith_whole sequences are not cut: one slot each, ahead of the others' (they are the long
-    // items of the launch, and run first).
-    const bool whole = it.sc < p.arith_whole;
-    const int rest_sc = it.sc - p.arith_whole;
-    it.b = whole ? it.sc : p.arith_whole + rest_sc / p.arith_chunks;
-    chunk = whole ? 0 : rest_sc - (it.b - p.arith_whole) * p.arith_chunks;
+    // The first arith_whole sequences own arith_first slots each (one, when they are not cut), ahead of the
+    // others': they are the long items of the launch, and run first.
+    const int first_slots = p.arith_whole * p.arith_first;
+    const bool first = it.sc < first_slots;
+    const int rest_sc = it.sc - first_slots;
+    const int slots = first ? p.arith_first : p.arith_chunks;
+    it.b = first ? it.sc / slots : p.arith_whole + rest_sc / slots;
+    chunk = first ? it.sc - it.b * slots : rest_sc - (it.b - p.arith_whole) * slots;
     if (it.b >= p.batch) return false;
     it.len = kv_length(p, it.b);
-    if (!whole) {
-      const int cnt = chunks_of_length(it.len, p.fixed_chunk);
-      it.chunks = cnt < p.arith_chunks ? cnt : p.arith_chunks;
-      if (chunk >= it.chunks) return false;
-      chunk_tokens = p.fixed_chunk;
-      to_the_end = chunk == p.arith_chunks - 1;
-    }
+    chunk_tokens = first ? p.first_chunk : p.fixed_chunk;
+    const int cnt = chunks_of_length(it.len, chunk_tokens);
+    it.chunks = cnt < slots ? cnt : slots;
+    if (chunk >= it.chunks) return false;
+    to_the_end = chunk == slots - 1;
   } else {
     // The header and the item's record are independent loads (the record's index is clamped to the
     // table, whose last entries the plan may not have written: such a record is not used).

@@ -49,7 +49,9 @@ __device__ inline void merge_row_cols(const P& p, int b, int j, int head, int q0
   // slot of the sequence's chunk i: its full chunks are consecutive, its tail lies among the tails; or
   // (no stored schedule) the sequence owns arith_chunks consecutive slots
   const bool arith = p.arith_chunks > 0;
-  const int f0 = arith ? (b < p.arith_whole ? b : p.arith_whole + (b - p.arith_whole) * p.arith_chunks) : p.full_prefix[b];
+  const int f0 = arith ? (b < p.arith_whole ? b * p.arith_first
+                                              : p.arith_whole * p.arith_first + (b - p.arith_whole) * p.arith_chunks)
+                       : p.full_prefix[b];
   const int nf = arith ? cnt : p.full_prefix[b + 1] - f0;
   const int tail_slot = arith ? 0 : p.hdr->total_full + p.tail_prefix[b];
   auto partial_row = [&](int i) { return (int64_t)(i < nf ? f0 + i : tail_slot) * nhq + rem; };

@@ -68,8 +68,9 @@ struct DecodeParams {
   int32_t arith_chunks;   // > 0: no schedule is stored.  Every sequence owns this many chunk slots of fixed_chunk
                           // tokens (slot = sequence * arith_chunks + chunk); a work item derives its chunk, and a
                           // merge the row's partials, from the sequence's length alone
-  int32_t arith_whole;    // ... except the first arith_whole sequences, which own one slot each and are not cut
-                          // (slot = sequence; then arith_whole + (sequence - arith_whole) * arith_chunks + chunk)
+  int32_t arith_whole;    // ... except the first arith_whole sequences, which own arith_first slots each, for chunks
+  int32_t arith_first;    // of first_chunk tokens (one slot and no cut: first_chunk = 2^30): slot = sequence *
+  int32_t first_chunk;    // arith_first + chunk; then arith_whole * arith_first + (sequence - arith_whole) * arith_chunks + chunk
   int32_t direct_single;  // the attention kernel writes the output rows of single-chunk sequences itself
   int32_t implicit_plan;  // nothing is split and nothing is merged: item = (sequence, kv head, row group),
                           // lengths come straight from the inputs and no plan kernel runs
@@ -109,9 +110,10 @@ __device__ inline int chunks_of_length(int len, int chunk) {
 template <class P>
 __device__ inline int chunks_of_sequence(const P& p, int b) {
   if (p.arith_chunks > 0) {
-    if (b < p.arith_whole) return 1;
-    const int cnt = chunks_of_length(kv_length(p, b), p.fixed_chunk);
-    return cnt < p.arith_chunks ? cnt : p.arith_chunks;
+    const bool first = b < p.arith_whole;
+    const int slots = first ? p.arith_first : p.arith_chunks;
+    const int cnt = chunks_of_length(kv_length(p, b), first ? p.first_chunk : p.fixed_chunk);
+    return cnt < slots ? cnt : slots;
   }
   return p.num_chunks[b];
 }

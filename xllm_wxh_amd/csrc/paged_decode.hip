@@ -368,15 +368,23 @@ static int fill_params(const xllm_hip_kv_cache* c,
   // as fill the slots once more — 2 sequences x 8 heads x 32 chunks — while the others stay whole (arith_whole):
   // the last round then takes a fraction of a whole one.
   p.arith_whole = 0;
+  p.arith_first = 0;
+  p.first_chunk = 1 << 30;
   if (is_mfma(variant) && p.rows <= 16 && p.heads_per_item == 1 && p.fused_merge && p.implicit_plan && hints &&
       nearly_equal && option(XLLM_HIP_OPTION_DECODE_STORED_SCHEDULE) == 0) {
     const int64_t per = (int64_t)p.item_heads * p.row_groups;
     const int64_t items = (int64_t)p.batch * per;
-    const int64_t round = p.target_items;
-    const int64_t whole_rounds = items / round;
-    // (from four whole rounds on the last one weighs little: 288 x 2048 fp8 tokens, 4.5 rounds, 202 us whole, 206 cut)
-    if (whole_rounds >= 1 && whole_rounds <= 3 && items % round != 0) {
-      const int64_t whole_seqs = whole_rounds * round / per;
+    // A round: an item per CU for a 16-bit cache.  What has to balance there is the bytes a CU streams, not
+    // the slots it fills: 33 sequences x 8 kv heads, 264 items of 8192 bf16 tokens, all resident at once, take
+    // 228 us where 256 take 159 — eight CUs stream two items.  Over a 1-byte cache a CU wants two workgroups
+    // to stream at its full rate, so a round is every slot, and a step of fewer items than slots (but more
+    // than the 256 that eight-wave workgroups serve) is first cut in two throughout.
+    const int64_t round = quant || one_wave_per_simd ? p.target_items : kNumCUs;
+    const int64_t first = quant && items < round && 2 * items > round ? 2 : 1;  // chunks of the sequences that stay as they are
+    const int64_t whole_rounds = first * items / round;
+    // (from 2048 items on the last round weighs little: 288 x 2048 fp8 tokens x 8 kv heads 202 us whole, 206 cut)
+    if (whole_rounds >= 1 && items < 4 * p.target_items && (first * items) % round != 0) {
+      const int64_t whole_seqs = whole_rounds * round / (per * first);
       const int64_t cut_seqs = p.batch - whole_seqs;
       int64_t k = round / (cut_seqs * per);
       k = k > 32 ? 32 : k;  // (what the fused merge loads in one batch)
@@ -384,17 +392,27 @@ static int fill_params(const xllm_hip_kv_cache* c,
       // tokens x 8 kv heads, 66 sequences 192 -> 168 us cut, 72 196 -> 191, but 80 204 -> 215 and 96 236 -> 244;
       // fp8, 8192 tokens: 66 sequences 255 -> 179, 80 260 -> 217, 96 277 -> 258, 136 413 -> 359)
       if (!quant && k < 8) k = 1;
-      if (k >= 2) {
-        int64_t chunk = ((int64_t)a->max_seq_len + k - 1) / k;
-        chunk = (chunk + p.tile_tokens - 1) / p.tile_tokens * p.tile_tokens;
-        chunk = chunk < p.min_chunk ? p.min_chunk : chunk;
-        k = ((int64_t)a->max_seq_len + chunk - 1) / chunk;
-        if (k >= 2 && whole_seqs + cut_seqs * k <= w.max_seq_chunks) {
-          p.fixed_chunk = (int32_t)chunk;
-          p.arith_chunks = (int32_t)k;
-          p.arith_whole = (int32_t)whole_seqs;
-          p.implicit_plan = 0;
-        }
+      auto chunk_for = [&](int64_t parts) {
+        int64_t c = ((int64_t)a->max_seq_len + parts - 1) / parts;
+        c = (c + p.tile_tokens - 1) / p.tile_tokens * p.tile_tokens;
+        return c < p.min_chunk ? (int64_t)p.min_chunk : c;
+      };
+      const int64_t chunk1 = first > 1 ? chunk_for(first) : (int64_t)1 << 30;
+      const int64_t k1 = first > 1 ? ((int64_t)a->max_seq_len + chunk1 - 1) / chunk1 : 1;
+      // (no more chunks than the workspace holds partial rows for)
+      const int64_t room = (w.max_seq_chunks - whole_seqs * k1) / cut_seqs;
+      k = k > room ? room : k;
+      const int64_t chunk = chunk_for(k > 1 ? k : 1);
+      k = ((int64_t)a->max_seq_len + chunk - 1) / chunk;
+      // (cut in two throughout, every sequence is merged: that pays while the last round's are few — fp8, 8192 tokens
+      // x 8 kv heads, 33 sequences 129 -> 105 us, 40 132 -> 122, but 48, whose last 16 get four chunks each, 136 -> 144)
+      if (k > k1 && (first == 1 || k >= 6) && whole_seqs * k1 + cut_seqs * k <= w.max_seq_chunks) {
+        p.fixed_chunk = (int32_t)chunk;
+        p.arith_chunks = (int32_t)k;
+        p.arith_whole = (int32_t)whole_seqs;
+        p.arith_first = (int32_t)k1;
+        p.first_chunk = (int32_t)chunk1;
+        p.implicit_plan = 0;
       }
     }
   }
@@ -445,7 +463,7 @@ static int64_t max_items(const DecodeParams& p) {
   const int64_t per = (int64_t)p.item_heads * p.row_groups;
   int64_t seq_chunks = p.batch;
   if (p.arith_chunks > 0) {
-    seq_chunks = p.arith_whole + (int64_t)(p.batch - p.arith_whole) * p.arith_chunks;
+    seq_chunks = (int64_t)p.arith_whole * p.arith_first + (int64_t)(p.batch - p.arith_whole) * p.arith_chunks;
   } else if (p.fixed_chunk != (1 << 30)) {
     int64_t t = 2 * (int64_t)p.target_items;  // choose_chunk may raise the target (by a quarter)
     if (t > kMaxTargetItems) t = kMaxTargetItems;
