@@ -899,6 +899,36 @@ def test_sequences_of_a_partly_filled_round_are_cut(gpu, kv, qdt, name, Hq, Hkv,
     assert torch.equal(out2, out) and torch.equal(lse2, lse)
 
 
+@pytest.mark.parametrize("kv,qdt", [("int8", "bf16"), ("fp8", "fp16")])
+@pytest.mark.parametrize("name,B,L", [
+    ("cut in four, the 33rd sequence finer", 33, 7000),
+    ("cut in two, the last two sequences finer", 66, 3400),
+    ("whole, the last two sequences cut", 130, 1700),
+])
+def test_partly_filled_round_of_the_32_row_kernel(gpu, kv, qdt, name, B, L):
+    """The same over a 1-byte cache with 32 query rows per kv head (four draft tokens): the step's even cut is
+    taken one finer where that overfills a round of the slots by little, and the sequences past the round
+    are cut finer still; the merge kernel combines them."""
+    print("case last round cut, 32 rows", kv, name, flush=True)
+    lens = [L - (i % 3) for i in range(B)]
+    case = Case(B, 64, 8, 128, 128, lens, n=4, kv=kv, qdt=qdt, seed=85)
+    ref, lse_ref = case.oracle()
+    ws = torch.full((ops.decode_workspace_bytes(B, 4, 64, 8, 128),), 0xA5, dtype=torch.uint8, device=gpu)
+    out, lse = case.run(workspace=ws, hints=True)
+    assert not torch.isnan(out.float()).any()
+    assert max_abs_err(out, ref) <= REG_TOL_QUANT
+    assert lse_err(lse, lse_ref) <= lse_tol(kv)
+    with ops.option("stored_schedule"):
+        out_w, lse_w = case.run(workspace=ws, hints=True)
+    assert max_abs_err(out_w, ref) <= REG_TOL_QUANT
+    assert torch.allclose(out.float(), out_w.float(), rtol=2 ** -6, atol=4e-3)
+    assert not torch.equal(lse[-32:], lse_w[-32:]), "the last sequence was not cut finer"
+    out_s, _ = case.run(workspace=ws, max_seq_len=L * 3 // 4, total_kv_len=B * L * 3 // 4)
+    assert max_abs_err(out_s, ref) <= REG_TOL_QUANT
+    out2, lse2 = case.run(workspace=ws, hints=True, plan=False)
+    assert torch.equal(out2, out) and torch.equal(lse2, lse)
+
+
 @pytest.mark.parametrize("kv,qdt,tol", [("bf16", "bf16", 2e-2), ("fp16", "fp16", 2e-3), ("int8", "bf16", 2e-2)])
 def test_two_stage_decode_merged_by_lse_equals_one_stage(gpu, kv, qdt, tol):
     """The returned log-sum-exps are base 2 and merge as the reference merges two partial attentions

@@ -370,8 +370,12 @@ static int fill_params(const xllm_hip_kv_cache* c,
   p.arith_whole = 0;
   p.arith_first = 0;
   p.first_chunk = 1 << 30;
-  if (is_mfma(variant) && p.rows <= 16 && p.heads_per_item == 1 && p.fused_merge && p.implicit_plan && hints &&
-      nearly_equal && option(XLLM_HIP_OPTION_DECODE_STORED_SCHEDULE) == 0) {
+  // (the 32-row kernel over a 1-byte cache as well — int8, four draft tokens, 32768 tokens x 8 kv heads: 66 sequences
+  // 996 us where 64 take 709 —, there also from a step that is already cut evenly, `uniform` chunks a sequence)
+  const bool rows32_quant = quant && p.rows > 16 && p.rows <= kMaxRowsPerItem && p.rows_per_item == kMaxRowsPerItem;
+  const int64_t uniform = p.implicit_plan ? 1 : (rows32_quant && p.arith_chunks > 0 ? p.arith_chunks : 0);
+  if (is_mfma(variant) && ((p.rows <= 16 && p.fused_merge && p.implicit_plan) || (rows32_quant && uniform > 0)) &&
+      p.heads_per_item == 1 && hints && nearly_equal && option(XLLM_HIP_OPTION_DECODE_STORED_SCHEDULE) == 0) {
     const int64_t per = (int64_t)p.item_heads * p.row_groups;
     const int64_t items = (int64_t)p.batch * per;
     // A round: an item per CU for a 16-bit cache.  What has to balance there is the bytes a CU streams, not
@@ -380,7 +384,9 @@ static int fill_params(const xllm_hip_kv_cache* c,
     // to stream at its full rate, so a round is every slot, and a step of fewer items than slots (but more
     // than the 256 that eight-wave workgroups serve) is first cut in two throughout.
     const int64_t round = quant || one_wave_per_simd ? p.target_items : kNumCUs;
-    const int64_t first = quant && items < round && 2 * items > round ? 2 : 1;  // chunks of the sequences that stay as they are
+    // chunks of the sequences that stay as they are: the even cut the step has, or one more when that cut fills
+    // less than nine tenths of a round
+    const int64_t first = quant && uniform * items < round && uniform * items * 10 < round * 9 ? uniform + 1 : uniform;
     const int64_t whole_rounds = first * items / round;
     // (from 2048 items on the last round weighs little: 288 x 2048 fp8 tokens x 8 kv heads 202 us whole, 206 cut)
     if (whole_rounds >= 1 && items < 4 * p.target_items && (first * items) % round != 0) {
@@ -406,7 +412,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
       k = ((int64_t)a->max_seq_len + chunk - 1) / chunk;
       // (cut in two throughout, every sequence is merged: that pays while the last round's are few — fp8, 8192 tokens
       // x 8 kv heads, 33 sequences 129 -> 105 us, 40 132 -> 122, but 48, whose last 16 get four chunks each, 136 -> 144)
-      if (k > k1 && (first == 1 || k >= 6) && whole_seqs * k1 + cut_seqs * k <= w.max_seq_chunks) {
+      if (k > k1 && (first == 1 || k >= 3 * k1) && whole_seqs * k1 + cut_seqs * k <= w.max_seq_chunks) {
         p.fixed_chunk = (int32_t)chunk;
         p.arith_chunks = (int32_t)k;
         p.arith_whole = (int32_t)whole_seqs;
