@@ -852,9 +852,8 @@ ALL_KV = ("bf16", "fp8", "int8")
 @pytest.mark.parametrize("kv,qdt", [("bf16", "bf16"), ("fp8", "bf16"), ("int8", "fp16")])
 @pytest.mark.parametrize("name,Hq,Hkv,D,n,bs,lens,cut_for", [
     ("two sequences past one round", 32, 8, 128, 1, 16, [1500] * 66, ALL_KV),
-    # (16-bit caches: only when the last round's items are at most an eighth of a round)
     ("eight past one round, nearly equal lengths, one empty", 32, 8, 128, 2, 32,
-     [1400 - 3 * (i % 40) for i in range(71)] + [0], ("fp8", "int8")),
+     [1400 - 3 * (i % 40) for i in range(71)] + [0], ALL_KV),
     ("a sequence past two rounds", 16, 4, 128, 1, 128, [700] * 257, ALL_KV),
     ("one kv head", 8, 1, 128, 1, 16, [640] * 520, ALL_KV),
     ("head_dim 64", 14, 2, 64, 1, 32, [900] * 260, ALL_KV),

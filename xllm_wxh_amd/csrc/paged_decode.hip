@@ -394,10 +394,9 @@ static int fill_params(const xllm_hip_kv_cache* c,
       const int64_t cut_seqs = p.batch - whole_seqs;
       int64_t k = round / (cut_seqs * per);
       k = k > 32 ? 32 : k;  // (what the fused merge loads in one batch)
-      // (a 16-bit cache's few items of a last round stream fast enough whole unless they are very few: bf16, 4096
-      // tokens x 8 kv heads, 66 sequences 192 -> 168 us cut, 72 196 -> 191, but 80 204 -> 215 and 96 236 -> 244;
-      // fp8, 8192 tokens: 66 sequences 255 -> 179, 80 260 -> 217, 96 277 -> 258, 136 413 -> 359)
-      if (!quant && k < 8) k = 1;
+      // (bf16, 4096 tokens x 8 kv heads: 66 sequences 192 -> 167 us, 72 196 -> 185, 80, two chunks, 204 -> 206;
+      // 8192 tokens: 33 sequences 228 -> 168, 40 237 -> 203, 44 242 -> 220, 48 247 -> 240.  fp8, 8192 tokens: 66
+      // sequences 255 -> 179, 80 260 -> 217, 96 277 -> 258, 136 413 -> 359)
       auto chunk_for = [&](int64_t parts) {
         int64_t c = ((int64_t)a->max_seq_len + parts - 1) / parts;
         c = (c + p.tile_tokens - 1) / p.tile_tokens * p.tile_tokens;
