@@ -903,9 +903,10 @@ def test_sequences_of_a_partly_filled_round_are_cut(gpu, kv, qdt, name, Hq, Hkv,
     ("cut in two, the last two sequences finer", 66, 3400, "int8", "bf16"),
     ("cut in two, the last two sequences finer", 66, 3400, "fp8", "fp16"),
     ("whole, the last two sequences cut", 130, 1100, "int8", "fp16"),
+    ("16-bit cache: whole, the last two sequences cut", 66, 1300, "bf16", "bf16"),
 ])
 def test_partly_filled_round_of_the_32_row_kernel(gpu, name, B, L, kv, qdt):
-    """The same over a 1-byte cache with 32 query rows per kv head (four draft tokens): the step's even cut is
+    """The same with 32 query rows per kv head (four draft tokens); over a 1-byte cache the step's even cut is
     taken one finer where that overfills a round of the slots by little, and the sequences past the round
     are cut finer still; the merge kernel combines them."""
     print("case last round cut, 32 rows", kv, name, flush=True)
