@@ -373,8 +373,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
   // (the 32-row kernel over a 1-byte cache as well — int8, four draft tokens, 32768 tokens x 8 kv heads: 66 sequences
   // 996 us where 64 take 709 —, there also from a step that is already cut evenly, `uniform` chunks a sequence)
   const bool rows32 = p.rows > 16 && p.rows <= kMaxRowsPerItem && p.rows_per_item == kMaxRowsPerItem;
-  const bool rows32_quant = quant && rows32;
-  const int64_t uniform = p.implicit_plan ? 1 : (rows32_quant && p.arith_chunks > 0 ? p.arith_chunks : 0);
+  const int64_t uniform = p.implicit_plan ? 1 : (rows32 && p.arith_chunks > 0 ? p.arith_chunks : 0);
   if (is_mfma(variant) && ((p.rows <= 16 && p.fused_merge && p.implicit_plan) || (rows32 && uniform > 0)) &&
       p.heads_per_item == 1 && hints && nearly_equal && option(XLLM_HIP_OPTION_DECODE_STORED_SCHEDULE) == 0) {
     const int64_t per = (int64_t)p.item_heads * p.row_groups;
