@@ -238,7 +238,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
   const int64_t four_head_items = (int64_t)p.batch * item_heads_of(p.rows, c->num_kv_heads, true);
   const int64_t slots = natural_target_items(true, p.rows, false);
   const bool nearly_equal = (int64_t)a->max_seq_len * p.batch * 4 <= a->total_kv_len * 5;
-  auto wider_items_pay = [&](int64_t narrow_items, int per_workgroup, double layout_gain = 0.0) {
+  auto wider_items_pay = [&](int64_t narrow_items, int per_workgroup, double layout_gain = 0.0, bool narrow_cut = false) {
     auto filled = [&](int64_t workgroups) {
       if (workgroups <= 0) return 1.0;
       // (fewer than the slots: equal sequences are cut into as many chunks each as still fit)
@@ -255,7 +255,9 @@ static int fill_params(const xllm_hip_kv_cache* c,
     gain = gain < cap ? gain : cap;
     if (per_workgroup == 2) gain *= 0.5;
     gain += layout_gain;
-    return filled((narrow_items + per_workgroup - 1) / per_workgroup) * (1.0 + gain) > filled(narrow_items) * 1.01;
+    // (narrow items whose last round's sequences are cut fill their rounds but for the merges)
+    const double narrow_filled = narrow_cut ? 0.97 : filled(narrow_items);
+    return filled((narrow_items + per_workgroup - 1) / per_workgroup) * (1.0 + gain) > narrow_filled * 1.01;
   };
   const bool short_sequences = (variant == kMfmaD128 || variant == kMfmaD64) && a->max_seq_len > 0 && a->total_kv_len > 0 &&
                                four_head_items >= (nearly_equal ? slots : 4 * slots) &&
@@ -433,7 +435,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
       option(XLLM_HIP_OPTION_DECODE_ITEM_PER_HEAD) == 0) {
     const int64_t items = (int64_t)p.batch * c->num_kv_heads;
     const int per_group = items >= kHeadsPerItem * slots ? 1 : items >= 2 * slots ? 2 : 0;
-    if (per_group != 0 && wider_items_pay(items, per_group == 1 ? kWaves : 2)) {
+    if (per_group != 0 && wider_items_pay(items, per_group == 1 ? kWaves : 2, 0.0, p.arith_whole > 0)) {
       p.wave_items = per_group;
       p.fixed_chunk = 1 << 30;
       p.implicit_plan = 1;
