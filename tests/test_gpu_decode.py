@@ -858,10 +858,11 @@ ALL_KV = ("bf16", "fp8", "int8")
     ("one kv head", 8, 1, 128, 1, 16, [640] * 520, ALL_KV),
     ("head_dim 64", 14, 2, 64, 1, 32, [900] * 260, ALL_KV),
     ("head_dim 256: rounds of 256", 16, 4, 256, 1, 16, [1100] * 66, ALL_KV),
-    # fewer items than slots: 1-byte caches are cut in two throughout, the last sequences finer
+    # up to a quarter more items than CUs: 1-byte caches run eight waves per item, whole items and chunks alike
     ("an item per CU and sixteen more", 32, 8, 128, 1, 16, [3200] * 34, ALL_KV),
-    # (... unless the sequences are too short for six chunks)
-    ("an item per CU and eight more, short sequences", 32, 8, 128, 2, 64, [1800] * 33, ("bf16",)),
+    ("an item per CU and eight more, short sequences", 32, 8, 128, 2, 64, [1800] * 33, ALL_KV),
+    # fewer items than slots: 1-byte caches are cut in two throughout, the last sequences finer
+    ("an item per CU and seventy more", 32, 8, 128, 1, 16, [3300] * 41, ALL_KV),
 ])
 def test_sequences_of_a_partly_filled_round_are_cut(gpu, kv, qdt, name, Hq, Hkv, D, n, bs, lens, cut_for):
     """Equal work items a few more than a whole number of rounds of the GPU (an item per CU over a 16-bit cache,

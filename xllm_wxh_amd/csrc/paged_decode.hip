@@ -372,6 +372,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
   p.arith_whole = 0;
   p.arith_first = 0;
   p.first_chunk = 1 << 30;
+  p.eight_waves = 0;
   // (the 32-row kernel over a 1-byte cache as well — int8, four draft tokens, 32768 tokens x 8 kv heads: 66 sequences
   // 996 us where 64 take 709 —, there also from a step that is already cut evenly, `uniform` chunks a sequence)
   const bool rows32 = p.rows > 16 && p.rows <= kMaxRowsPerItem && p.rows_per_item == kMaxRowsPerItem;
@@ -385,10 +386,15 @@ static int fill_params(const xllm_hip_kv_cache* c,
     // 228 us where 256 take 159 — eight CUs stream two items.  Over a 1-byte cache a CU wants two workgroups
     // to stream at its full rate, so a round is every slot, and a step of fewer items than slots (but more
     // than the 256 that eight-wave workgroups serve) is first cut in two throughout.
-    const int64_t round = quant || one_wave_per_simd ? p.target_items : kNumCUs;
+    // ... or, while the items are at most a quarter more than the CUs, runs eight waves per item like a step of
+    // up to 256 items: a round is then an item per CU, the sequences past it are cut, and their chunks follow the
+    // whole items onto the CUs (fp8, 8192 tokens x 8 kv heads: 33 sequences 105 us cut in two throughout)
+    const bool eight = quant && p.rows <= 16 && p.tok != 0 && uniform == 1 && items > kNumCUs && items * 4 <= kNumCUs * 5 &&
+                       option(XLLM_HIP_OPTION_DECODE_FOUR_WAVE_ITEMS) == 0;
+    const int64_t round = eight ? kNumCUs : quant || one_wave_per_simd ? p.target_items : kNumCUs;
     // chunks of the sequences that stay as they are: the even cut the step has, or one more when that cut fills
     // less than nine tenths of a round
-    const int64_t first = quant && uniform * items < round && uniform * items * 10 < round * 9 ? uniform + 1 : uniform;
+    const int64_t first = !eight && quant && uniform * items < round && uniform * items * 10 < round * 9 ? uniform + 1 : uniform;
     const int64_t whole_rounds = first * items / round;
     // (from 2048 items on the last round weighs little: 288 x 2048 fp8 tokens x 8 kv heads 202 us whole, 206 cut)
     if (whole_rounds >= 1 && items < 4 * p.target_items && (first * items) % round != 0) {
@@ -420,6 +426,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
         p.arith_first = (int32_t)k1;
         p.first_chunk = (int32_t)chunk1;
         p.implicit_plan = 0;
+        p.eight_waves = eight ? 1 : 0;
       }
     }
   }
@@ -502,7 +509,7 @@ static void launch_mfma_tok(const DecodeParams& p, unsigned grid, hipStream_t st
       // At most one work item per CU over a 1-byte cache: eight waves share it (one 32768-token sequence:
       // 25 us against 31 for fp8, 26 against 32 for int8; over a 16-bit cache, whose tiles take no
       // conversion, 31.7 against 31.0).
-      if (grid <= (unsigned)kNumCUs && option(XLLM_HIP_OPTION_DECODE_FOUR_WAVE_ITEMS) == 0) {
+      if ((grid <= (unsigned)kNumCUs || p.eight_waves) && option(XLLM_HIP_OPTION_DECODE_FOUR_WAVE_ITEMS) == 0) {
         decode_mfma_d128_kernel<KV_DT, TOK, false, 2 * kWaves><<<grid, 128 * kWaves, 0, st>>>(p);
         return;
       }
