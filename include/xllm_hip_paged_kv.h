@@ -486,6 +486,25 @@ int xllm_hip_abi_version(void);
 const char* xllm_hip_paged_decode_variant(const xllm_hip_kv_cache* cache,
                                           const xllm_hip_decode_args* args);
 
+/* How xllm_hip_paged_decode_plan / _run would run these arguments on a workspace of `workspace_bytes` (0: of
+ * xllm_hip_paged_decode_workspace_bytes): host-only, launches nothing, reads no device memory (pointers are only
+ * checked for NULL).  No counterpart in the reference; it exists so that the step's schedule can be inspected,
+ * and tested, without a GPU.  Writes up to `count` of
+ *   out[0]  workgroups of the attention launch          out[1]  waves per workgroup (1, 2, 4 or 8)
+ *   out[2]  1: nothing is split (no plan, no merge)     out[3]  1: the schedule is stored by the plan kernel
+ *   out[4]  chunk tokens of the cut sequences (0: chosen on the device)
+ *   out[5]  chunk slots per cut sequence (schedule-free split; else 0)
+ *   out[6]  leading sequences that keep out[7] slots each of out[8] tokens (the others are cut finer)
+ *   out[9]  kv heads per work item                      out[10] work items per workgroup (1, 2 or 4)
+ *   out[11] 1: split sequences are merged inside the attention kernel
+ *   out[12] sequence-chunk slots the workspace holds    out[13] sequence-chunk slots the launch addresses
+ * and returns XLLM_HIP_OK, or the error the same arguments would get. */
+int xllm_hip_paged_decode_describe(const xllm_hip_kv_cache* cache,
+                                   const xllm_hip_decode_args* args,
+                                   size_t workspace_bytes,
+                                   int64_t* out,
+                                   int32_t count);
+
 #ifdef __cplusplus
 }
 #endif

@@ -52,6 +52,7 @@ EXPORTED_SYMBOLS = (
     "xllm_hip_last_error",
     "xllm_hip_abi_version",
     "xllm_hip_paged_decode_variant",
+    "xllm_hip_paged_decode_describe",
 )
 
 
@@ -194,6 +195,9 @@ def load():
     lib.xllm_hip_abi_version.restype = ctypes.c_int
     lib.xllm_hip_paged_decode_variant.argtypes = [P(KvCacheDesc), P(DecodeArgs)]
     lib.xllm_hip_paged_decode_variant.restype = ctypes.c_char_p
+    lib.xllm_hip_paged_decode_describe.argtypes = [P(KvCacheDesc), P(DecodeArgs), ctypes.c_size_t,
+                                                   P(ctypes.c_int64), ctypes.c_int32]
+    lib.xllm_hip_paged_decode_describe.restype = ctypes.c_int
 
     if lib.xllm_hip_abi_version() != ABI_VERSION:
         raise ImportError(

@@ -559,6 +559,62 @@ static int launch_generic(int kv_dtype, const DecodeParams& p, unsigned grid, hi
 
 using namespace xllm_hip;
 
+extern "C" int xllm_hip_paged_decode_describe(const xllm_hip_kv_cache* cache,
+                                              const xllm_hip_decode_args* args,
+                                              size_t workspace_bytes,
+                                              int64_t* out,
+                                              int32_t count) {
+  XLLM_HIP_REQUIRE(out != nullptr && count >= 0, "out is NULL or count negative");
+  XLLM_HIP_REQUIRE(cache != nullptr && args != nullptr, "cache or args is NULL");
+  if (workspace_bytes == 0) {
+    workspace_bytes = workspace_layout(args->batch, args->q_per_seq, args->num_q_heads, cache->num_kv_heads,
+                                       cache->head_dim).total_bytes;
+  }
+  DecodeParams p;
+  // (a workspace address that is never read: every field of it the host forms is an offset from it)
+  if (int s = fill_params(cache, args, (void*)(uintptr_t)4096, workspace_bytes, p)) return s;
+  const Variant v = pick_variant(cache, args);
+  XLLM_HIP_REQUIRE(v != kNone, "no decode kernel for head_dim=%d block_size=%d", cache->head_dim, cache->block_size);
+  const int64_t grid = p.batch == 0 ? 0 : max_items(p);
+  const bool quant = cache->dtype == XLLM_HIP_FP8_E4M3 || cache->dtype == XLLM_HIP_INT8;
+  int64_t waves = 1, per_workgroup = 1;
+  if (is_mfma(v)) {
+    if (p.rows_per_item == kPrefillRowsPerItem) {
+      waves = 4;
+    } else if (p.rows > 16) {
+      waves = 2;
+    } else if (p.heads_per_item > 1 || p.wave_items) {
+      waves = 4;
+      per_workgroup = p.wave_items == 2 ? 2 : (p.wave_items == 1 ? 4 : 1);
+    } else {
+      const bool eight = quant && p.tok != 0 && (grid <= kNumCUs || p.eight_waves) &&
+                         option(XLLM_HIP_OPTION_DECODE_FOUR_WAVE_ITEMS) == 0;
+      waves = eight ? 8 : 4;
+    }
+  }
+  const bool stored = !p.implicit_plan && p.arith_chunks == 0;
+  const int64_t slots_used = p.implicit_plan ? 0
+                             : p.arith_chunks > 0
+                                 ? (int64_t)p.arith_whole * p.arith_first + (int64_t)(p.batch - p.arith_whole) * p.arith_chunks
+                                 : (int64_t)p.max_seq_chunks;
+  const int64_t values[14] = {grid,
+                              waves,
+                              p.implicit_plan,
+                              stored ? 1 : 0,
+                              p.implicit_plan || p.fixed_chunk == (1 << 30) ? 0 : p.fixed_chunk,
+                              p.arith_chunks,
+                              p.arith_whole,
+                              p.arith_whole > 0 ? p.arith_first : 0,
+                              p.arith_whole > 0 ? p.first_chunk : 0,
+                              p.heads_per_item,
+                              per_workgroup,
+                              p.fused_merge && !p.implicit_plan ? 1 : 0,
+                              p.max_seq_chunks,
+                              slots_used};
+  for (int i = 0; i < count && i < 14; ++i) out[i] = values[i];
+  return XLLM_HIP_OK;
+}
+
 extern "C" size_t xllm_hip_paged_decode_workspace_bytes(int32_t batch,
                                                         int32_t q_per_seq,
                                                         int32_t num_q_heads,
