@@ -245,6 +245,9 @@ def main():
 
     variant = ops.decode_variant(q, pools[0][0], pools[0][1], block_table, seq_lens_d, pools[0][2], pools[0][3],
                                  q_per_seq=w.q_per_seq, kv_layout=args.kv_layout)
+    schedule = ops.decode_describe(q, pools[0][0], pools[0][1], block_table, seq_lens_d, pools[0][2], pools[0][3],
+                                   q_per_seq=w.q_per_seq, kv_layout=args.kv_layout, max_seq_len=int(seq_lens.max()),
+                                   total_kv_len=int(seq_lens.sum()))
 
     # HIP events around the attention kernel of every timed step (recorded on the launch stream by
     # the library itself).  torch creates the handles; the first record materialises them.
@@ -420,6 +423,7 @@ def main():
                               % (ops.KV_SKEW_BYTES if args.kv_skew_bytes is None else args.kv_skew_bytes)),
             "kv_pools_rotated": len(pools),
             "kernel_variant": variant,
+            "schedule": schedule,
         },
         "achieved_gbps": round(achieved_gbps, 1),
         "pct_of_hbm_peak": round(100.0 * achieved_gbps / HBM_PEAK_GBPS, 2),

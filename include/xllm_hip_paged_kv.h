@@ -494,7 +494,7 @@ const char* xllm_hip_paged_decode_variant(const xllm_hip_kv_cache* cache,
  *   out[2]  1: nothing is split (no plan, no merge)     out[3]  1: the schedule is stored by the plan kernel
  *   out[4]  chunk tokens of the cut sequences (0: chosen on the device)
  *   out[5]  chunk slots per cut sequence (schedule-free split; else 0)
- *   out[6]  leading sequences that keep out[7] slots each of out[8] tokens (the others are cut finer)
+ *   out[6]  leading sequences that keep out[7] slots each of out[8] tokens (0: whole); the others are cut finer
  *   out[9]  kv heads per work item                      out[10] work items per workgroup (1, 2 or 4)
  *   out[11] 1: split sequences are merged inside the attention kernel
  *   out[12] sequence-chunk slots the workspace holds    out[13] sequence-chunk slots the launch addresses

@@ -605,7 +605,7 @@ extern "C" int xllm_hip_paged_decode_describe(const xllm_hip_kv_cache* cache,
                               p.arith_chunks,
                               p.arith_whole,
                               p.arith_whole > 0 ? p.arith_first : 0,
-                              p.arith_whole > 0 ? p.first_chunk : 0,
+                              p.arith_whole > 0 && p.first_chunk != (1 << 30) ? p.first_chunk : 0,
                               p.heads_per_item,
                               per_workgroup,
                               p.fused_merge && !p.implicit_plan ? 1 : 0,

@@ -389,6 +389,25 @@ def decode_variant(query, k_cache, v_cache, block_table, seq_lens, k_cache_quant
     return _lib.load().xllm_hip_paged_decode_variant(ctypes.byref(desc), ctypes.byref(args)).decode()
 
 
+DESCRIBE_FIELDS = ("workgroups", "waves_per_workgroup", "unsplit", "stored_schedule", "chunk_tokens",
+                   "slots_per_cut_sequence", "kept_sequences", "kept_slots", "kept_chunk_tokens", "kv_heads_per_item",
+                   "items_per_workgroup", "fused_merge", "chunk_slots_held", "chunk_slots_used")
+
+
+def decode_describe(query, k_cache, v_cache, block_table, seq_lens, k_cache_quant_scale=None,
+                    v_cache_quant_scale=None, q_per_seq=None, kv_layout="HND", max_seq_len=0, total_kv_len=0):
+    """How batch_decode would run these tensors (xllm_hip_paged_decode_describe: decided on the host, nothing is
+    launched): a dict of DESCRIBE_FIELDS."""
+    desc = _cache_desc(k_cache, v_cache, k_cache_quant_scale, v_cache_quant_scale, kv_layout)
+    out = torch.empty_like(query)
+    args, _keep = _decode_args(query, out, None, block_table, seq_lens, None, q_per_seq, 1.0, -1, max_seq_len, desc,
+                               total_kv_len=total_kv_len)
+    vals = (ctypes.c_int64 * len(DESCRIBE_FIELDS))()
+    _lib.check(_lib.load().xllm_hip_paged_decode_describe(ctypes.byref(desc), ctypes.byref(args), 0, vals,
+                                                          len(DESCRIBE_FIELDS)))
+    return dict(zip(DESCRIBE_FIELDS, (int(v) for v in vals)))
+
+
 def csr_to_block_table(paged_kv_indptr, paged_kv_indices, paged_kv_last_page_len, block_size, max_blocks_per_seq):
     """Index-only conversion CSR -> (block_table padded with 0, seq_lens)."""
     batch = paged_kv_last_page_len.numel()
