@@ -238,3 +238,34 @@ def test_many_row_kernel_over_one_byte_caches_split_and_garbage(gpu, kv):
     assert float(np.abs(got - ref).max()) <= 1.2e-2
     fin = np.isfinite(lse_ref)
     assert np.allclose(lse.cpu().numpy()[fin], lse_ref[fin], atol=2e-2)
+
+
+@pytest.mark.parametrize("kv,qdt", [("bf16", "bf16"), ("fp32", "fp32")])
+def test_long_chunk_on_the_default_workspace(gpu, kv, qdt):
+    """One sequence's chunk of 4096 query tokens x 32 heads (never split: no partial rows) runs on the
+    shared 128 MiB workspace, on the MFMA and on the generic kernel, which then writes its rows itself.
+    Checked against the oracle on sampled query tokens, each as a decode row of its own kv length
+    (xllm/core/runtime/speculative_worker_impl.cpp:230-243)."""
+    print("case long chunk, default workspace", kv, flush=True)
+    L, n, Hq, Hkv, D = 4096, 4096, 32, 8, 128
+    c = Case(1, Hq, Hkv, D, 16, [L], kv=kv, qdt=qdt, seed=41)
+    assert ops.decode_workspace_bytes(1, n, Hq, Hkv, D) <= 1 << 20
+    dt = torch.bfloat16 if qdt == "bf16" else torch.float32
+    q = torch.randn(n, Hq, D, generator=torch.Generator().manual_seed(79)).to(dt)
+    qd = q.to(c.q.device)
+    out = torch.full_like(qd, 7.0)
+    lse = torch.full((n, Hq), 3.0, dtype=torch.float32, device=qd.device)
+    q_indptr = torch.tensor([0, n], dtype=torch.int32, device=qd.device)
+    ops.batch_decode(qd, c.k_cache, out, c.block_table, c.seq_lens, c.v_cache, lse, scale=c.scale, return_lse=True,
+                     q_per_seq=n, q_indptr=q_indptr)
+    torch.cuda.synchronize()
+    got = out.float().cpu().numpy()
+    assert not np.isnan(got).any()
+    rows = np.array([0, 1, 31, 32, 127, 128, 1000, 2047, 2048, 4094, 4095])
+    table = np.repeat(c.table, len(rows), axis=0)
+    ref, ref_lse = orc.paged_decode(q.float().numpy()[rows], c.k_ref, c.v_ref, table, (L - n + 1 + rows).astype(np.int32),
+                                    c.scale)
+    err = float(np.abs(got[rows] - ref).max())
+    print("   err %.3e" % err, flush=True)
+    assert err <= (1.2e-2 if kv == "bf16" else 1e-4)
+    assert np.allclose(lse.cpu().numpy()[rows], ref_lse, atol=2e-2 if kv == "bf16" else 1e-4)

@@ -20,14 +20,6 @@ pytestmark = pytest.mark.gpu
 REG_TOL = 1.2e-2
 REG_TOL_QUANT = 2.5e-2
 LSE_TOL = 1e-4
-# An int8 cache at head_dim 128 meets the queries in the int8 MFMA: the queries are 16-bit fixed point
-# against the largest query element of the work item (steps of absmax / 32512), where the other
-# paths take them exactly; about 5e-5 in the base-2 log-sum-exp for N(0, 1) inputs.
-LSE_TOL_INT8 = 2.5e-4
-
-
-def lse_tol(kv):
-    return LSE_TOL_INT8 if kv == "int8" else LSE_TOL
 # ... and relative to the size of the outputs: max-abs error of a sequence's rows within this fraction
 # of their RMS (16-bit weights and outputs: a few units of 2^-9 of the largest elements)
 REL_TOL = 3e-2
@@ -44,7 +36,7 @@ def _check(case, window_left=-1, **kw):
     assert e <= case.tol, e
     assert e <= (REG_TOL_QUANT if case.kv in ("fp8", "int8") else REG_TOL), e
     assert re <= REL_TOL, re
-    assert le <= lse_tol(case.kv), le
+    assert le <= LSE_TOL, le
     return out, lse
 
 
@@ -218,7 +210,7 @@ def test_nhd_layout_and_csr_form(gpu, kv):
     # the sums; with one kv head per item only the strides differ and the values are the same bits.
     out_h, lse_h = _check(b)
     assert torch.allclose(out_h.float(), out_a.float(), rtol=2 ** -7, atol=2e-3)
-    assert torch.allclose(lse_h, lse_a, rtol=0, atol=LSE_TOL_INT8 if kv == "int8" else LSE_TOL)
+    assert torch.allclose(lse_h, lse_a, rtol=0, atol=LSE_TOL)
     with ops.option("item_per_head"):
         out_b, lse_b = _check(b)
         assert torch.equal(out_a, out_b) and torch.equal(lse_a, lse_b)
@@ -252,7 +244,7 @@ def test_work_items_of_four_kv_heads_over_nhd(gpu, kv, qdt, Hq, Hkv, n):
     case = Case(len(lens), Hq, Hkv, 128, 16, lens, n=n, kv=kv, qdt=qdt, layout="NHD", seed=93)
     assert case.variant() == "mfma_d128"
     tol = {"bf16": REG_TOL, "fp16": 2e-3}.get(kv, REG_TOL_QUANT)
-    lse_tol = LSE_TOL_INT8 if kv == "int8" else LSE_TOL
+    lse_tol = LSE_TOL
     for window in (-1, 300):
         ref, lse_ref = case.oracle(window)
         out, lse = case.run(window)
@@ -522,7 +514,7 @@ def test_host_length_hints_select_the_unsplit_path(gpu, kv, n):
         e = max_abs_err(out, ref)
         print("   %s err=%.3e" % (kw, e), flush=True)
         assert e <= (REG_TOL_QUANT if kv == "int8" else REG_TOL)
-        assert lse_err(lse, lse_ref) <= lse_tol(kv)
+        assert lse_err(lse, lse_ref) <= LSE_TOL
 
 
 def test_decode_step_replays_under_hip_graph(gpu):
@@ -653,7 +645,7 @@ def test_split_sequences_merge_in_the_attention_kernel_repeatably(gpu, kv, qdt, 
     first, lse_first = case.run()
     assert max_abs_err(first, ref) <= (REG_TOL_QUANT if kv in ("int8", "fp8") else REG_TOL)
     assert max_rel_err_per_seq(first, ref, n) <= REL_TOL
-    assert lse_err(lse_first, lse_ref) <= lse_tol(kv)
+    assert lse_err(lse_first, lse_ref) <= LSE_TOL
     ws = ops.get_workspace(gpu, ops.decode_workspace_bytes(5, n, 64, 8, D))
     for i in range(40):
         out, lse = case.run(workspace=ws, plan=(i == 0))  # one plan, many runs: the counters reset themselves
@@ -780,7 +772,7 @@ def test_four_head_items_for_many_short_sequences(gpu, name, kv, qdt, layout, Hq
     out, lse = case.run(hints=True)
     assert not torch.isnan(out.float()).any()
     assert max_abs_err(out, ref) <= tol
-    assert lse_err(lse, lse_ref) <= lse_tol(kv)
+    assert lse_err(lse, lse_ref) <= LSE_TOL
     with ops.option("item_per_head"):
         out_1, lse_1 = case.run(hints=True)
     assert max_abs_err(out_1, ref) <= tol
@@ -836,7 +828,7 @@ def test_eight_wave_items_over_one_byte_caches(gpu, kv, qdt, name, D, bs, n, len
     out, lse = case.run(hints=True)
     assert not torch.isnan(out.float()).any()
     assert max_abs_err(out, ref) <= REG_TOL_QUANT
-    assert lse_err(lse, lse_ref) <= lse_tol(kv)
+    assert lse_err(lse, lse_ref) <= LSE_TOL
     with ops.option("four_wave_items"):
         out_4, lse_4 = case.run(hints=True)
     # two roundings of 16-bit outputs (2^-8 relative) and fp32 summation order
@@ -879,7 +871,7 @@ def test_sequences_of_a_partly_filled_round_are_cut(gpu, kv, qdt, name, Hq, Hkv,
     out, lse = case.run(workspace=ws, hints=True)
     assert not torch.isnan(out.float()).any()
     assert max_abs_err(out, ref) <= tol
-    assert lse_err(lse, lse_ref) <= lse_tol(kv)
+    assert lse_err(lse, lse_ref) <= LSE_TOL
     with ops.option("stored_schedule"):
         out_w, lse_w = case.run(workspace=ws, hints=True)
     assert max_abs_err(out_w, ref) <= tol
@@ -918,7 +910,7 @@ def test_partly_filled_round_of_the_32_row_kernel(gpu, name, B, L, kv, qdt):
     out, lse = case.run(workspace=ws, hints=True)
     assert not torch.isnan(out.float()).any()
     assert max_abs_err(out, ref) <= REG_TOL_QUANT
-    assert lse_err(lse, lse_ref) <= lse_tol(kv)
+    assert lse_err(lse, lse_ref) <= LSE_TOL
     with ops.option("stored_schedule"):
         out_w, lse_w = case.run(workspace=ws, hints=True)
     assert max_abs_err(out_w, ref) <= REG_TOL_QUANT
@@ -1070,7 +1062,7 @@ def test_split_step_without_a_stored_schedule(gpu, kv, n, qdt, name, lens):
     assert bool((ws[:64] == 0xA5).all()), "a schedule was stored"
     tol = {"bf16": REG_TOL, "fp16": 2e-3, "fp32": 1e-4}.get(kv, REG_TOL_QUANT)
     assert max_abs_err(out, ref) <= tol
-    assert lse_err(lse, lse_ref) <= (LSE_TOL_INT8 if kv == "int8" else LSE_TOL)
+    assert lse_err(lse, lse_ref) <= LSE_TOL
     # (the stored schedule's launch is sized for any lengths, and a launch of more work items than CUs
     # runs four waves per item: the comparison holds the other one at four as well)
     with ops.option("four_wave_items"):
@@ -1085,7 +1077,7 @@ def test_split_step_without_a_stored_schedule(gpu, kv, n, qdt, name, lens):
     longest, total = int(max(lens)), int(sum(lens))
     out_w, lse_w = case.run(workspace=ws, max_seq_len=max(1, longest * 3 // 4), total_kv_len=max(1, total * 3 // 4))
     assert max_abs_err(out_w, ref) <= tol
-    assert lse_err(lse_w, lse_ref) <= (LSE_TOL_INT8 if kv == "int8" else LSE_TOL)
+    assert lse_err(lse_w, lse_ref) <= LSE_TOL
     # ... and a second step on the same workspace without a plan call in between (the counters of the
     # fused merge reset themselves)
     out2, _ = case.run(workspace=ws, hints=True, plan=False)

@@ -92,6 +92,21 @@ def test_workspace_stays_within_the_shared_buffer_of_the_reference():
         assert 0 < need <= 128 << 20, (rows, hkv, d, need)
 
 
+def test_never_split_steps_need_no_partial_rows():
+    """Chunked-prefill and mixed steps (more than 128 query rows per kv head) are never split: their rows are
+    written directly and the workspace holds neither chunk records nor partial rows, so ordinary chunks fit
+    the 128 MiB the libtorch layer reserves (xllm/core/common/global_flags.cpp:564-567) — 1 x 4096 query
+    tokens of 32 heads x 128 would otherwise need 129 MiB of partial rows that nothing touches."""
+    from xllm_wxh_amd import _lib
+
+    lib = _lib.load()
+    for batch, n in ((1, 4096), (1, 8192), (4, 2048), (8, 1024), (16, 512), (64, 512), (256, 128)):
+        need = lib.xllm_hip_paged_decode_workspace_bytes(batch, n, 32, 8, 128)
+        assert 0 < need <= 1 << 20, (batch, n, need)
+    # 128 rows per kv head are still split (and sized for it)
+    assert lib.xllm_hip_paged_decode_workspace_bytes(8, 32, 32, 8, 128) > 1 << 20
+
+
 def test_small_batch_choices(plan):
     def chunk(lens, hkv=8, rg=1, target=512, small=256):
         lens = np.asarray(lens, np.int64)

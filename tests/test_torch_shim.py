@@ -345,6 +345,37 @@ def test_attention_impl_chunked_prefill_step(gpu, shim, kv):
 
 
 @pytest.mark.gpu
+def test_long_prefill_chunk_runs_on_the_default_workspace(gpu, shim):
+    """A chunk of 4096 query tokens x 32 heads through AttentionImpl::forward on the layer's own 128 MiB
+    workspace (a never-split step needs no partial rows); same bits as the C ABI called directly."""
+    from xllm_wxh_amd import ops
+
+    print("case shim long chunk", flush=True)
+    Hq, Hkv, D, bs, L = 32, 8, 128, 16, 4096
+    nblocks = L // bs + 2
+    lst = (np.random.default_rng(3).permutation(nblocks - 1) + 1)[: L // bs].astype(np.int32)
+    slots = np.asarray(orc.kv_cache_slots(lst, bs, 0, L), np.int32)
+    g = torch.Generator().manual_seed(19)
+    qkv = torch.randn(L, (Hq + 2 * Hkv) * D, generator=g).to(torch.bfloat16).to(gpu)
+    cache = shim.KVCache(torch.zeros(nblocks, Hkv, bs, D, dtype=torch.bfloat16, device=gpu),
+                         torch.zeros(nblocks, Hkv, bs, D, dtype=torch.bfloat16, device=gpu))
+    i32 = lambda a: torch.tensor(np.asarray(a), dtype=torch.int32, device=gpu)
+    md = shim.build_decode_metadata(i32([0, L]), i32([0, L]), i32(slots), i32(lst[None, :]), L, L, L)
+    md.plan_info.layer_id = 0
+    md.is_chunked_prefill = True
+    scale = 1.0 / float(np.sqrt(D))
+    attn = shim.AttentionImpl(Hq, D, scale, Hkv, -1)
+    out, _ = attn.forward(md, qkv[:, : Hq * D], qkv[:, Hq * D:(Hq + Hkv) * D], qkv[:, (Hq + Hkv) * D:], cache)
+    torch.cuda.synchronize()
+    want = torch.empty(L, Hq, D, dtype=torch.bfloat16, device=gpu)
+    ops.batch_decode(qkv[:, : Hq * D].reshape(L, Hq, D), cache.get_k_cache(), want, i32(lst[None, :]), i32([L]),
+                     cache.get_v_cache(), scale=scale, q_per_seq=L, q_indptr=i32([0, L]))
+    torch.cuda.synchronize()
+    assert torch.equal(out.reshape(L, Hq, D), want)
+    assert float(out.float().abs().max()) > 0.0
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("kind", ["int8", "fp8"])
 def test_prefill_chunks_over_a_quantised_cache_take_the_dense_route(gpu, shim, kind):
     """Large chunks over a 1-byte cache: AttentionImpl dequantises the cached ranges into a dense copy

@@ -133,9 +133,22 @@ __global__ void __launch_bounds__(64) decode_generic_kernel(DecodeParams p) {
         }
       }
     }
-    const int64_t prow = (int64_t)it.sc * nhq + (int64_t)j * p.num_q_heads + head;
     const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
-    if (lane == 0) p.partial_lse[prow] = l_run > 0.0f ? m_run + __builtin_amdgcn_logf(l_run) : neg_inf;
+    const float lse2 = l_run > 0.0f ? m_run + __builtin_amdgcn_logf(l_run) : neg_inf;
+    if (p.implicit_plan) {
+      // A step that is never split (more query rows per kv head than a split serves): every item is a whole
+      // sequence, so the row is final and no partial is written (the workspace then holds none).
+      const int64_t tok = (int64_t)it.q0 + j;
+      if (lane == 0 && p.lse != nullptr) p.lse[tok * p.num_q_heads + head] = lse2;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int d = lane + 64 * i;
+        if (d < D) Elem<Q_DT>::store(p.out, tok * p.out_token_stride + (int64_t)head * D + d, o[i] * inv);
+      }
+      continue;
+    }
+    const int64_t prow = (int64_t)it.sc * nhq + (int64_t)j * p.num_q_heads + head;
+    if (lane == 0) p.partial_lse[prow] = lse2;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int d = lane + 64 * i;

@@ -132,10 +132,12 @@ struct KvHalf16 {
     int lrow;
     int tok;         // tokens per row
     int second;      // 1 if this lane's piece belongs to the second token of its row
-    __device__ inline void init(const DecodeParams& p, int lane) {
+    // `ptok`: DecodeParams::tok, which the kernels know at compile time (the offsets below that depend on it
+    // alone then become immediates of the instructions that use them)
+    __device__ inline void init(const DecodeParams& p, int lane, int ptok) {
       lrow = lane >> 4;
       const int piece = lane & 15;
-      tok = p.tok == 0 ? 1 : p.tok;  // head_dim 256: rows are tokens here too; `plane` picks the half of the token
+      tok = ptok == 0 ? 1 : ptok;  // head_dim 256: rows are tokens here too; `plane` picks the half of the token
       second = tok == 2 && piece >= 8 ? 1 : 0;
       g_off = (uint32_t)(((lrow * tok + second) * p.stride_slot + (piece & (16 / tok - 1)) * 8) * 2);
       wk = kLdsK + swz_k(lrow, piece);
@@ -277,12 +279,12 @@ struct KvHalfQuant {
     bool sc_on;       // lanes 0 .. 32 * tok - 1 carry a scale: first the K scales, then the V scales
     bool sc_is_v;
     uint32_t wkraw;   // LDS offset of raw K row krow, this lane's 16-byte piece (int8 cache, head_dim 128)
-    __device__ inline void init(const DecodeParams& p, int lane) {
+    __device__ inline void init(const DecodeParams& p, int lane, int ptok) {
       const int chunk = 4 * ((lane >> 3) & 1) + (lane & 3);
       const int pair = (lane >> 2) & 1;
       const int krow = 2 * (lane >> 4) + pair;  // rows r, r+1 alternate between quads (krow < 8)
       vrow = (lane >> 4) + 8 * pair;            // rows r, r+8 alternate between quads (vrow & 7 < 4)
-      tok = p.tok == 0 ? 1 : p.tok;  // head_dim 256: rows are tokens here too; `plane` picks the half of the token
+      tok = ptok == 0 ? 1 : ptok;  // head_dim 256: rows are tokens here too; `plane` picks the half of the token
       second = tok == 2 && chunk >= 4 ? 1 : 0;
       const int in_tok = (chunk & (8 / tok - 1)) * 16;  // byte within the token's row
       gk_off = (uint32_t)((krow * tok + second) * p.stride_slot + in_tok);
@@ -417,8 +419,9 @@ constexpr int xch_row_bytes(int tok) { return head_dim_of(tok) * 4 + 16; }  // a
 // caller that parks them as exact fp16 numbers passes false.
 // FENCED: fragments and per-token factors are read where they are used and the LDS offsets of the
 // fragments are formed every tile anew (scheduling fences; see kFenced), for a kernel with no register to spare.
+// NORM_ROW: see kNormQ.
 template <int KV_DT, int TOK, bool RAWK = raw_k_of(KV_DT, TOK), bool OFFSET = kv_of(KV_DT) == XLLM_HIP_INT8,
-          bool OFFSET_K = OFFSET && !RAWK, bool FENCED = false>
+          bool OFFSET_K = OFFSET && !RAWK, bool FENCED = false, bool NORM_ROW = true>
 struct RowTile {
   static constexpr bool kQuant = quant_of(KV_DT);
   // int8 rows sit in LDS as x + 1152.  With K' = K + 1152 and V' = V + 1152:
@@ -429,11 +432,23 @@ struct RowTile {
   static constexpr bool kOffset = OFFSET;     // V rows (costs an MFMA per tile and its accumulator, wacc)
   static constexpr bool kOffsetK = OFFSET_K;  // K rows (costs nothing per tile: the MFMA's initial C operand)
   // Raw K: the K rows are bytes in LDS and the scores come from the int8 MFMA.  The queries are held as
-  // two int8 parts on one scale for the whole workgroup, q = q_scale * (256 hi + lo) with
-  // q_scale = absmax / (127 * 256), |hi|, |lo| <= 127 — 16 bits against the rows' largest element —
-  // so a score is q_scale * k_scale * (256 S_hi + S_lo) with both sums exact in 32-bit integers
-  // (|S| <= 128 * 127 * 127).  q_scale rides in the per-token factor the park prepares.
+  // two int8 parts on one scale per query row, q = q_scale * (256 hi + lo) with q_scale a power of two,
+  // 2^(e - 15) where 2^e is the first power of two above the row's largest magnitude: 16-bit fixed point
+  // against that element, on a grid on which every bf16 query element within 2^7 of the row's largest is
+  // exact (its own spacing is a multiple of the grid's).  A score is then
+  // q_scale * k_scale * (256 S_hi + S_lo) with both sums exact in 32-bit integers (|S| <= 128 * 128 * 128);
+  // q_scale is a per-lane factor, a query row living in one lane column of the score tile.
   static constexpr bool kRawK = RAWK;
+  // bf16 queries that become fp16 operands are first brought to a largest magnitude in [2^14, 2^15) by a power of
+  // two (exact), so that neither fp16's upper end (65504) nor its lower one (2^-14; nothing below 2^-24) cuts into
+  // queries that bf16 holds well.  Row by row (NORM_ROW: the scores then take the row's factor back, like raw
+  // K's), or, in a kernel with no register to spare for that, by the largest element of the whole work item,
+  // which the caller hands to init and whose factor it folds into the per-token score factors it parks (rows
+  // more than 2^28 below the item's largest element then lose bits).
+  static constexpr bool kNormQ = !RAWK && f16_ops(KV_DT) && !qf16_of(KV_DT);
+  static constexpr bool kNormItem = kNormQ && !NORM_ROW;
+  // The scores carry a factor of their query row (q_scale).
+  static constexpr bool kRowScale = RAWK || (kNormQ && NORM_ROW);
   static constexpr int kD = head_dim_of(TOK);
   static constexpr int kQC = kD / 32;    // 32-element chunks of a query row
   static constexpr int kDT = TOK == 0 ? 16 : 8;  // O^T accumulator tiles
@@ -451,7 +466,7 @@ struct RowTile {
   float m_run;     // reference point of the exponents: follows the running maximum of the log2-scaled scores (of score + log2 v_scale if quantised) lazily, see softmax
   float l_run;     // this lane's share of the softmax denominator
   float s_init;    // initial value of the score accumulators: -1152 * sum_d q[r][d] (int8), else 0
-  float q_scale;   // raw K: see above; else 1
+  float q_scale;   // factor of the lane's query row on its scores (kRowScale); else 1
   int lim;         // tokens >= lim are invisible to the row (causal among draft tokens)
   int lo;          // tokens < lo are outside the sliding window
   uint32_t k_off0; // LDS offset of K row mi, piece kg        (piece 4c + kg: XOR c << 6)
@@ -474,28 +489,42 @@ struct RowTile {
       }
     }
   }
-  // Raw K: largest magnitude among the wave's 16 query rows (every lane gets the wave's value).
-  __device__ inline float q_absmax(const DecodeParams& p, const Item& it, int row_in_item, int lane) const {
-    const int mi = lane & 15, kgl = lane >> 4;
-    const int row = it.rg * p.rows_per_item + row_in_item + mi;
+  // Largest magnitude of the lane's query row (the four lanes that share a row get the same value).
+  __device__ static inline float q_absmax(const uint16_t* qrow, bool valid, int kg) {
+    float m = 0.0f;
+#pragma unroll
+    for (int c = 0; c < kD / 64; ++c) {
+      float f[16];
+      q_floats(qrow + 64 * c + 16 * kg, valid, f);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) m = fmaxf(m, fabsf(f[e]));
+    }
+    return kg_max(m);
+  }
+  // kNormItem: exponent e of the power of two that brings the largest magnitude among the wave's 16 query rows at
+  // `row_in_item` into [2^14, 2^15) (every lane gets the wave's value; waves that share parked per-token factors take the
+  // largest of theirs).
+  __device__ static inline float wave_q_absmax(const DecodeParams& p, const Item& it, int row_in_item, int lane) {
+    const int row = it.rg * p.rows_per_item + row_in_item + (lane & 15);
     const bool valid = row < it.n * p.group;
     const int j = valid ? row / p.group : 0;
     const int gq = valid ? row - j * p.group : 0;
     const uint16_t* qrow = (const uint16_t*)p.q + (int64_t)(it.q0 + j) * p.q_token_stride +
                            (int64_t)(it.hk * p.group + gq) * kD;
-    float m = 0.0f;
-#pragma unroll
-    for (int c = 0; c < kD / 64; ++c) {
-      float f[16];
-      q_floats(qrow + 64 * c + 16 * kgl, valid, f);
-#pragma unroll
-      for (int e = 0; e < 16; ++e) m = fmaxf(m, fabsf(f[e]));
-    }
-    return wave_max(m);
+    return wave_max(q_absmax(qrow, valid, lane >> 4));
+  }
+  __device__ static inline int norm_exponent(float absmax) {
+    return __builtin_amdgcn_readfirstlane(pow2_above(absmax) - 15);
+  }
+  // The power of two 2^e with m < 2^e (m = f * 2^e, f in [0.5, 1)), as its exponent; within +-100 so that
+  // both 2^e and its inverse times 2^15 are ordinary floats (a row of zeros gets the smallest).
+  __device__ static inline int pow2_above(float m) {
+    const int e = (int)((__builtin_bit_cast(uint32_t, m) >> 23) & 0xffu) - 126;
+    return e < -100 ? -100 : (e > 100 ? 100 : e);
   }
 
-  // `absmax`: raw K only, the largest query magnitude of the workgroup's rows (q_absmax of its waves).
-  __device__ inline void init(const DecodeParams& p, const Item& it, int row_in_item, int lane, float absmax = 0.0f) {
+  // `q_exp` (kNormItem): see norm_exponent; the caller folds 2^q_exp into the per-token score factors it parks.
+  __device__ inline void init(const DecodeParams& p, const Item& it, int row_in_item, int lane, int q_exp = 0) {
     const int mi = lane & 15;  // MFMA row of A / column of B and D
     kg = lane >> 4;            // k-group of the operands; row block of D
     const int row = it.rg * p.rows_per_item + row_in_item + mi;
@@ -511,9 +540,12 @@ struct RowTile {
     if constexpr (kRawK) {
       // qf[c]: the high parts of elements 64c + 16kg .. + 15 (c = 0 .. kD/64 - 1), sixteen bytes in the
       // order the K bytes lie in memory; qf[kD/64 + c]: the low parts.
-      const float top = fmaxf(absmax, 1e-30f);
-      const float inv = 127.0f / top;
-      q_scale = top * (1.0f / (127.0f * 256.0f));
+      const float top = q_absmax(qrow, valid, kg);
+      int e2 = pow2_above(top);
+      // (the few values whose grid number would pass 127 * 256 + 127 take the next power of two)
+      if (top * __builtin_amdgcn_ldexpf(1.0f, 15 - e2) > 32639.0f) ++e2;
+      const float inv = __builtin_amdgcn_ldexpf(1.0f, 15 - e2);
+      q_scale = __builtin_amdgcn_ldexpf(1.0f, e2 - 15);
 #pragma unroll
       for (int c = 0; c < kD / 64; ++c) {
         float f[16];
@@ -521,15 +553,22 @@ struct RowTile {
         uint32_t hi4[4] = {0, 0, 0, 0}, lo4[4] = {0, 0, 0, 0};
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-          const float qn = f[e] * inv;
-          const float h = fmaxf(-127.0f, fminf(rintf(qn), 127.0f));
-          const float l = fmaxf(-127.0f, fminf(rintf((qn - h) * 256.0f), 127.0f));
-          hi4[e >> 2] |= ((uint32_t)(int)h & 0xffu) << (8 * (e & 3));
-          lo4[e >> 2] |= ((uint32_t)(int)l & 0xffu) << (8 * (e & 3));
+          int qi = (int)rintf(f[e] * inv);  // |qi| <= 32639
+          qi = qi > 32639 ? 32639 : (qi < -32639 ? -32639 : qi);  // (a NaN or an infinity among the queries)
+          const int h = (qi + 128) >> 8;    // -127 .. 127
+          const int l = qi - (h << 8);      // -128 .. 127
+          hi4[e >> 2] |= ((uint32_t)h & 0xffu) << (8 * (e & 3));
+          lo4[e >> 2] |= ((uint32_t)l & 0xffu) << (8 * (e & 3));
         }
         qf[c] = __builtin_bit_cast(Op, u32x4{hi4[0], hi4[1], hi4[2], hi4[3]});
         qf[kD / 64 + c] = __builtin_bit_cast(Op, u32x4{lo4[0], lo4[1], lo4[2], lo4[3]});
       }
+    }
+    float down = 1.0f;
+    if constexpr (kNormQ) {
+      const int e2 = NORM_ROW ? pow2_above(q_absmax(qrow, valid, kg)) - 15 : q_exp;
+      down = __builtin_amdgcn_ldexpf(1.0f, -e2);
+      if (NORM_ROW) q_scale = __builtin_amdgcn_ldexpf(1.0f, e2);
     }
 #pragma unroll
     for (int c = 0; c < (kRawK ? 0 : kQC); ++c) {
@@ -538,10 +577,9 @@ struct RowTile {
       if constexpr (qf16_of(KV_DT) || !f16_ops(KV_DT)) {
         qf[c] = __builtin_bit_cast(Op, raw);  // the queries already have the operand type
       } else {
-        // bf16 -> fp16 is exact for magnitudes in [2^-14, 65504]; smaller ones lose low bits only
         const bf16x8 qb = __builtin_bit_cast(bf16x8, raw);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) qf[c][e] = (_Float16)(float)qb[e];
+        for (int e = 0; e < 8; ++e) qf[c][e] = (_Float16)((float)qb[e] * down);
       }
       if constexpr (kOffsetK) {
 #pragma unroll
@@ -675,6 +713,7 @@ struct RowTile {
           } else {
             raw = TOK == 0 ? s[0][0][rr] + s[0][1][rr] : s[u][h][rr];
           }
+          if constexpr (kRowScale) raw *= q_scale;
           float v = kFold ? raw : kQuant ? __builtin_fmaf(raw, kscl[i], lv[i]) : raw * scale_log2;
           if (MASKED) {
             const int tok = tb + kU * (16 * h + 4 * kg + rr) + u;
@@ -1081,10 +1120,11 @@ __global__ void __launch_bounds__(64 * WAVES, decode_waves_per_simd(TOK)) decode
   const int lane = threadIdx.x & 63;
   uint8_t* tile = lds_all + wave * kLdsTile;  // this wave's private K/V tile
 
-  RowTile<KV_DT, TOK> rt;
   constexpr bool kRawK = raw_k_of(KV_DT, TOK);
-  rt.init(p, it, 0, lane, kRawK ? rt.q_absmax(p, it, 0, lane) : 0.0f);  // (the four waves hold the same rows, or each its head's)
-  const float park_scale = p.scale_log2 * rt.q_scale;
+  typedef RowTile<KV_DT, TOK> RT;
+  RT rt;
+  rt.init(p, it, 0, lane);  // (the four waves hold the same rows, or each its head's)
+  const float park_scale = p.scale_log2;
 
   // This wave's share of the item's tokens.
   const int t0 = first_visible_tile(p, it);
@@ -1097,7 +1137,7 @@ __global__ void __launch_bounds__(64 * WAVES, decode_waves_per_simd(TOK)) decode
   const int mask_lo_until = p.window_left >= 0 ? it.len - 1 - p.window_left : 0;  // tiles starting below this too
 
   typename KvHalf<KV_DT>::Geom geom;
-  geom.init(p, lane);
+  geom.init(p, lane, TOK);
   // One register stage: the loads of tile i+1 are in flight while tile i is consumed.  (More stages were
   // slower wherever they were tried: two for the 1-byte caches of head_dim 256, which run one wave per
   // SIMD and so have few bytes in flight per CU, 458 against 367 us on 64 x 8192 tokens of fp8 — the
@@ -1192,15 +1232,8 @@ __global__ void __launch_bounds__(128, rows32_waves_per_simd(KV_DT, TOK)) decode
   constexpr bool kRawK = raw_k_of(KV_DT, TOK);
   constexpr bool kInt8 = kv_of(KV_DT) == XLLM_HIP_INT8;
   RowTile<KV_DT, TOK, kRawK, kInt8, kInt8 && !kRawK, rows32_waves_per_simd(KV_DT, TOK) == 2 && TOK == 0> rt;
-  float absmax = 0.0f;
-  if constexpr (kRawK) {  // one scale for the queries of both waves: they share the parked per-token factors
-    lds_ml[wave] = rt.q_absmax(p, it, 16 * rs, lane);
-    __syncthreads();
-    absmax = fmaxf(lds_ml[0], lds_ml[1]);
-    __syncthreads();
-  }
-  rt.init(p, it, 16 * rs, lane, absmax);
-  const float park_scale = p.scale_log2 * rt.q_scale;
+  rt.init(p, it, 16 * rs, lane);
+  const float park_scale = p.scale_log2;
 
   const int w_begin = first_visible_tile(p, it);
   const int w_end = it.t_end;
@@ -1209,7 +1242,7 @@ __global__ void __launch_bounds__(128, rows32_waves_per_simd(KV_DT, TOK)) decode
   const int mask_lo_until = p.window_left >= 0 ? it.len - 1 - p.window_left : 0;
 
   typename KvHalf<KV_DT>::Geom geom;
-  geom.init(p, lane);
+  geom.init(p, lane, TOK);
   // kDepth register stages, used in turn: the loads of tiles i+1 .. i+kDepth are in flight while tile
   // i is consumed (a wave fetches only half a tile, so one stage would leave too few bytes in flight
   // per CU to cover the HBM latency; four stages for head_dim 256, which runs one wave per SIMD,
@@ -1462,8 +1495,11 @@ struct QuantPrefillLoader {
   }
 
   // The wave's rows of the tile at tb: raw -> converted (K, V, per-token factors); see KvHalfQuant::park.
-  template <bool MASKED>
-  __device__ inline void convert(const uint8_t* raw, uint8_t* conv, int tb, int len, float scale_log2) const {
+  // `lds_scale` (LDS_SCALE): where the factor of the K scales is kept in LDS instead of in `scale_log2`, for a
+  // kernel with no scalar register to spare for it through the token loop.
+  template <bool MASKED, bool LDS_SCALE = false>
+  __device__ inline void convert(const uint8_t* raw, uint8_t* conv, int tb, int len, float scale_log2,
+                                 const float* lds_scale = nullptr) const {
     int row8, chunk;
     row_chunk(row8, chunk);
     const int row = 8 * wave + row8;
@@ -1487,6 +1523,7 @@ struct QuantPrefillLoader {
     *(u32x4*)(conv + vo) = vlo;
     *(u32x4*)(conv + (vo ^ 16)) = vhi;
     if (lane < 16) {
+      if (LDS_SCALE) scale_log2 = *lds_scale;
       const float sc = *(const float*)(raw + 8192 + 256 * wave + lane * 4);
       const int t = 8 * wave + (lane & 7);  // token of the tile
       const bool is_v = lane >= 8;
@@ -1519,10 +1556,20 @@ __global__ void __launch_bounds__(256, 2) prefill_quant_d128_kernel(DecodeParams
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
 
-  typedef RowTile<KV_DT, 1, false, false, kv_of(KV_DT) == XLLM_HIP_INT8> RT;
+  typedef RowTile<KV_DT, 1, false, false, kv_of(KV_DT) == XLLM_HIP_INT8, false, false> RT;
   RT rt[2];
-  rt[0].init(p, it, 32 * wave, lane);
-  rt[1].init(p, it, 32 * wave + 16, lane);
+  int q_exp = 0;
+  if constexpr (RT::kNormItem) {  // one factor for the queries of all four waves: they share the converted tile's factors
+    lds_ml[wave] = fmaxf(RT::wave_q_absmax(p, it, 32 * wave, lane), RT::wave_q_absmax(p, it, 32 * wave + 16, lane));
+    __syncthreads();
+    q_exp = RT::norm_exponent(fmaxf(fmaxf(lds_ml[0], lds_ml[1]), fmaxf(lds_ml[2], lds_ml[3])));
+    __syncthreads();
+  }
+  rt[0].init(p, it, 32 * wave, lane, q_exp);
+  rt[1].init(p, it, 32 * wave + 16, lane, q_exp);
+  // (the factor of the K scales waits in LDS, a word per wave: no scalar register is left to hold it through the loop)
+  if constexpr (RT::kNormItem) lds_ml[4 + wave] = __builtin_amdgcn_ldexpf(p.scale_log2, q_exp);
+  const float* lds_scale = lds_ml + 4 + wave;
 
   const int rows = it.n * p.group;
   const int r_first = it.rg * p.rows_per_item + 32 * wave;
@@ -1551,9 +1598,9 @@ __global__ void __launch_bounds__(256, 2) prefill_quant_d128_kernel(DecodeParams
     const int nblk = block_of_const(p, it, tb + 4 * kT + mine);
     __builtin_amdgcn_s_waitcnt(0x0f76);  // vmcnt(6)
     if (tb + kT > it.len) {
-      ld.template convert<true>(raw, conv, tb, it.len, p.scale_log2);
+      ld.template convert<true, RT::kNormItem>(raw, conv, tb, it.len, p.scale_log2, lds_scale);
     } else {
-      ld.template convert<false>(raw, conv, tb, it.len, p.scale_log2);
+      ld.template convert<false, RT::kNormItem>(raw, conv, tb, it.len, p.scale_log2, lds_scale);
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
     __builtin_amdgcn_s_barrier();

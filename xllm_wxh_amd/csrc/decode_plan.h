@@ -167,7 +167,10 @@ inline int64_t max_seq_chunks_for(int batch, int rows, int num_kv_heads) {
 inline WorkspaceLayout workspace_layout(int batch, int q_per_seq, int num_q_heads, int num_kv_heads, int head_dim) {
   WorkspaceLayout w;
   w.max_seq_chunks = max_seq_chunks_for(batch, q_per_seq * (num_q_heads / num_kv_heads), num_kv_heads);
-  if (never_split(q_per_seq, num_q_heads, num_kv_heads)) w.max_seq_chunks = batch + 1;
+  // A step that is never split writes its output rows directly, whichever kernel serves it: no chunk
+  // records and no partial rows (at 4096 query tokens they would be 64 MiB that nothing touches).
+  const bool whole = never_split(q_per_seq, num_q_heads, num_kv_heads);
+  if (whole) w.max_seq_chunks = 0;
   size_t off = 0;
   w.header = off;
   off += sizeof(PlanHeader);

@@ -328,7 +328,8 @@ static int fill_params(const xllm_hip_kv_cache* c,
     // Many query rows per kv head (chunked prefill): the row groups supply the parallelism, and one
     // partial per chunk and row would be large, so nothing is split.
     if (stay_whole) p.fixed_chunk = 1 << 30;
-    p.implicit_plan = p.direct_single && p.fixed_chunk == (1 << 30) ? 1 : 0;
+    // (a step that is never split is whole sequences for the generic kernel too: it then writes the rows itself)
+    p.implicit_plan = (p.direct_single || stay_whole) && p.fixed_chunk == (1 << 30) ? 1 : 0;
     // A split step whose host-side lengths are (nearly) equal needs no stored schedule: with the chunk
     // size the device-side plan would choose from the same aggregates, every sequence owns
     // ceil(max_seq_len / chunk) chunk slots and a work item finds its chunk from its index and the

@@ -354,7 +354,8 @@ void batch_decode(const torch::Tensor& query,
   TORCH_CHECK(seq_lens.scalar_type() == torch::kInt && seq_lens.is_contiguous() && seq_lens.numel() == a.batch,
               "seq_lens must be contiguous int32 [batch]");
   a.block_table = block_table.data_ptr<int32_t>();
-  a.block_table_stride = block_table.stride(0);
+  // (the row stride of a one-row table is arbitrary in torch: such a table is its one row)
+  a.block_table_stride = block_table.size(0) > 1 ? block_table.stride(0) : block_table.size(1);
   a.max_blocks_per_seq = (int32_t)block_table.size(1);
   a.seq_lens = seq_lens.data_ptr<int32_t>();
   a.max_seq_len = (int32_t)max_seq_len;
@@ -401,7 +402,7 @@ void batch_prefill_paged(const torch::Tensor& query, const torch::Tensor& k_cach
   TORCH_CHECK(kv_seq_lens.scalar_type() == torch::kInt && kv_seq_lens.is_contiguous() && kv_seq_lens.numel() == a.batch,
               "kv_seq_lens must be contiguous int32 [batch]");
   a.block_table = block_tables.data_ptr<int32_t>();
-  a.block_table_stride = block_tables.stride(0);
+  a.block_table_stride = block_tables.size(0) > 1 ? block_tables.stride(0) : block_tables.size(1);
   a.max_blocks_per_seq = (int32_t)block_tables.size(1);
   a.seq_lens = kv_seq_lens.data_ptr<int32_t>();
   a.max_seq_len = (int32_t)max_seq_len;

@@ -292,7 +292,8 @@ def _decode_args(query, output, output_lse, block_table, seq_lens, csr, q_per_se
         _require(block_table.size(0) == a.batch and seq_lens.numel() == a.batch,
                  "block_table/seq_lens rows (%d/%d) != batch %d" % (block_table.size(0), seq_lens.numel(), a.batch))
         a.block_table = block_table.data_ptr()
-        a.block_table_stride = block_table.stride(0)
+        # (the row stride of a one-row table is arbitrary in torch: such a table is its one row)
+        a.block_table_stride = block_table.stride(0) if block_table.size(0) > 1 else block_table.size(1)
         a.max_blocks_per_seq = block_table.size(1)
         a.seq_lens = seq_lens.data_ptr()
     else:
