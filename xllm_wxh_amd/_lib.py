@@ -23,6 +23,7 @@ OPTION_DECODE_FORCE_GENERIC, OPTION_DECODE_TARGET_ITEMS, OPTION_DECODE_SEPARATE_
 OPTION_DECODE_STORED_SCHEDULE = 3
 OPTION_DECODE_ITEM_PER_HEAD = 4
 OPTION_DECODE_FOUR_WAVE_ITEMS = 5
+OPTION_PREFILL_KERNEL = 6
 
 STATUS_NAMES = {
     OK: "OK",

@@ -51,7 +51,8 @@ struct DecodeParams {
   int32_t rows;   // group * n
   int32_t row_groups;
   int32_t cluster;        // neighbouring work items kept on one XCD (see decode_item)
-  int32_t rows_per_item;  // query rows one work item handles (32 or 128 MFMA, 1 generic)
+  int32_t rows_per_item;  // query rows one work item handles (32, 128 or 256 MFMA, 1 generic)
+  int32_t prefill_opts;   // XLLM_HIP_OPTION_PREFILL_KERNEL as the 256-row kernel reads it
   int32_t min_chunk;      // smallest chunk the plan may choose
   int32_t head_dim;
   int32_t tok;          // tokens per 256-byte LDS row of the MFMA kernels: 1 (head_dim 128), 2 (head_dim 64),

@@ -28,6 +28,7 @@ constexpr int kMaxTargetItems = 2048; // largest split target of any kernel: eig
 constexpr int kMaxRowsPerItem = 32;   // query rows (g * n) one work item of the MFMA decode kernels handles
 constexpr int kPrefillRowsPerItem = 128;  // ... and of the many-row (prefill) kernel, used above kPrefillMinRows rows
 constexpr int kPrefillMinRows = 32;
+constexpr int kPrefillWideRows = 256;  // ... and of its eight-wave form, used above kPrefillRowsPerItem rows (16-bit caches)
 
 #if defined(__HIPCC__)
 #define XLLM_HIP_HD __host__ __device__

@@ -27,6 +27,7 @@
 #include "decode_item.h"
 #include "decode_merge.h"
 #include "decode_mfma.h"
+#include "prefill_pingpong.h"
 #include "decode_generic.h"
 
 #include <math.h>
@@ -57,7 +58,8 @@ struct Options {
   Options() {
     static const char* const names[XLLM_HIP_OPTION_COUNT] = {
         "XLLM_HIP_DECODE_FORCE_GENERIC", "XLLM_HIP_DECODE_TARGET_ITEMS", "XLLM_HIP_DECODE_SEPARATE_MERGE",
-        "XLLM_HIP_DECODE_STORED_SCHEDULE", "XLLM_HIP_DECODE_ITEM_PER_HEAD", "XLLM_HIP_DECODE_FOUR_WAVE_ITEMS"};
+        "XLLM_HIP_DECODE_STORED_SCHEDULE", "XLLM_HIP_DECODE_ITEM_PER_HEAD", "XLLM_HIP_DECODE_FOUR_WAVE_ITEMS",
+        "XLLM_HIP_PREFILL_KERNEL"};
     for (int i = 0; i < XLLM_HIP_OPTION_COUNT; ++i) {
       const char* e = getenv(names[i]);
       v[i].store(e != nullptr ? atoll(e) : 0, std::memory_order_relaxed);
@@ -204,6 +206,14 @@ static int fill_params(const xllm_hip_kv_cache* c,
                     : (p.rows > kPrefillMinRows && variant != kMfmaD256 && (!quant || variant == kMfmaD128))
                         ? kPrefillRowsPerItem
                         : kMaxRowsPerItem;
+  // More rows than one such item over a 16-bit cache: 256 rows per item, eight waves in two groups that
+  // alternate between their matrix and softmax phases (prefill_pingpong_d128_kernel).
+  p.prefill_opts = (int32_t)option(XLLM_HIP_OPTION_PREFILL_KERNEL);
+  // (head_dim 128: at head_dim 64 a tile is 64 tokens, and its scores and weights do not fit that kernel's registers)
+  if (p.rows_per_item == kPrefillRowsPerItem && p.rows > kPrefillRowsPerItem && !quant && variant == kMfmaD128 &&
+      (p.prefill_opts & 1) == 0) {
+    p.rows_per_item = kPrefillWideRows;
+  }
   p.min_chunk = is_mfma(variant) ? kMinChunkTokens : kMinChunkTokensGeneric;
   p.tok = variant == kMfmaD64 ? 2 : variant == kMfmaD256 ? 0 : 1;
   p.tile_tokens = variant == kMfmaD256 ? kTileTokens / 2 : kTileTokens * p.tok;
@@ -496,7 +506,9 @@ static int64_t max_items(const DecodeParams& p) {
 
 template <int KV_DT, int TOK>
 static void launch_mfma_tok(const DecodeParams& p, unsigned grid, hipStream_t st) {
-  if (p.rows_per_item == kPrefillRowsPerItem) {
+  if (p.rows_per_item == kPrefillWideRows) {
+    if constexpr (!quant_of(KV_DT) && TOK == 1) prefill_pingpong_d128_kernel<KV_DT, TOK><<<grid, 512, 0, st>>>(p);
+  } else if (p.rows_per_item == kPrefillRowsPerItem) {
     if constexpr (!quant_of(KV_DT) && TOK != 0) prefill_mfma_d128_kernel<KV_DT, TOK><<<grid, 256, 0, st>>>(p);
     if constexpr (quant_of(KV_DT) && TOK == 1) prefill_quant_d128_kernel<KV_DT><<<grid, 256, 0, st>>>(p);
   } else if (p.rows <= 16) {
@@ -580,7 +592,9 @@ extern "C" int xllm_hip_paged_decode_describe(const xllm_hip_kv_cache* cache,
   const bool quant = cache->dtype == XLLM_HIP_FP8_E4M3 || cache->dtype == XLLM_HIP_INT8;
   int64_t waves = 1, per_workgroup = 1;
   if (is_mfma(v)) {
-    if (p.rows_per_item == kPrefillRowsPerItem) {
+    if (p.rows_per_item == kPrefillWideRows) {
+      waves = 8;
+    } else if (p.rows_per_item == kPrefillRowsPerItem) {
       waves = 4;
     } else if (p.rows > 16) {
       waves = 2;

@@ -1,0 +1,357 @@
+// Many query rows per kv head over a 16-bit cache, 256 rows per work item: the two-phase ("ping-pong") form of
+// prefill_mfma_d128_kernel.
+#pragma once
+
+#include "decode_mfma.h"
+
+#include <type_traits>
+
+namespace xllm_hip {
+
+// A workgroup is eight waves and 256 query rows of one (sequence, kv head): wave w owns rows 32w .. 32w+31 as
+// two row tiles, as in prefill_mfma_d128_kernel, and all eight walk the item's tokens over the same LDS tiles
+// (global memory -> LDS directly, each wave four rows of K and of V per tile).  The eight waves are two to a
+// SIMD, and what a wave does for a tile is two phases of about the same length that use different parts of the
+// SIMD: the matrix phase (V^T P^T of the previous tile, then K Q^T of this one: 32 MFMAs fed from LDS) and the
+// softmax phase (vector arithmetic only).  Waves 0-3 and waves 4-7 run these phases in opposite order — one
+// group is in its matrix phase while the other is in its softmax phase — and a workgroup barrier at every
+// phase change keeps them there, so that the two waves of a SIMD do not both wait for the same unit.  The
+// second group starts one phase late (an extra barrier at its start, one at the first group's end).
+//
+// Phases and barriers.  Barrier number g of the workgroup: the first group passes 2t before the matrix phase of
+// tile t and 2t+1 before its softmax phase; the second group 2t+1 and 2t+2.  Every wave waits for its own share
+// of tile t+1 before the barrier that precedes its softmax phase of tile t, which for either group comes before
+// any wave reads that tile.  Tile t's buffer is last read in the second group's matrix phase of tile t+1
+// (its V rows), which ends before barrier 2t+4; a wave puts tile t+4 in flight into the buffer of tile t-2
+// after the barrier before its matrix phase of tile t, i.e. after barrier 2t at the earliest.  Six buffers
+// rotate; the loads of tiles t+2 .. t+4 are in flight while tile t+1 is waited for.
+//
+// The tiles every row of the item sees in full take the straight-line form above, six at a time (one per
+// buffer, so that each LDS access names its buffer and the compiler can tell the loads in flight from the
+// tile being read).  The others — the causal edge, the sequence end, a sliding window's lower edge, and up to
+// five tiles that do not fill a group of six — take a form that keeps all three parts of a tile in one step
+// (K Q^T in the matrix phase, softmax and V^T P^T in the other) and lets a wave skip a tile none of its rows
+// sees; both forms pass the same barriers per tile.
+// A wave in its matrix phase runs at a raised priority, so that its MFMAs are issued as soon as their operands
+// are there rather than after the vector instructions of the SIMD's other wave.
+#ifndef XLLM_HIP_PINGPONG_PRIO
+#define XLLM_HIP_PINGPONG_PRIO 1
+#endif
+#if XLLM_HIP_PINGPONG_PRIO
+#define XLLM_HIP_PINGPONG_SETPRIO(n) __builtin_amdgcn_s_setprio(n)
+#else
+#define XLLM_HIP_PINGPONG_SETPRIO(n) ((void)0)
+#endif
+constexpr int kPingPongRows = 256;
+constexpr int kPingPongBuffers = 6;
+
+template <int KV_DT, int TOK>
+struct PingPongLoader {
+  int wave, lane;
+  uint32_t k_off, v_off;  // byte offset of the piece this lane fetches from the first of the wave's tokens
+  int v_tok;              // ... and the token (within the wave's 4 * TOK) its V piece belongs to
+
+  // The piece for position lane % 16 of row 4 * wave + lane / 16 of the tile: token (within the wave's 4 * TOK)
+  // and byte offset.
+  __device__ inline void piece(bool v, int& tok, int& byte) const {
+    const int row4 = lane >> 4;
+    const int row = 4 * wave + row4;
+    const int pos = lane & 15;
+    const int lp = v ? pos ^ (((row & 7) << 1) | ((row >> 3) & 1))  // see swz_v
+                     : pos ^ (row & 15);                             // see swz_k
+    constexpr int kPerTok = 16 / TOK;
+    tok = row4 * TOK + lp / kPerTok;
+    byte = (lp % kPerTok) * 16;
+  }
+  // The two offsets stay in registers of their own for the whole item: a register that addressed a load into LDS
+  // may not be written again before that load has landed, so offsets formed anew for every tile would make
+  // each tile wait for all the tiles in flight.
+  __device__ inline void init(const DecodeParams& p, int wave_, int lane_) {
+    wave = wave_;
+    lane = lane_;
+    int tok, byte;
+    piece(false, tok, byte);
+    k_off = (uint32_t)(tok * p.stride_slot * 2 + byte);
+    piece(true, tok, byte);
+    v_off = (uint32_t)(tok * p.stride_slot * 2 + byte);
+    v_tok = tok;
+  }
+  // Loads of the wave's rows of the tile starting at token tb into `buf` (in flight on return): global memory ->
+  // LDS, 16 bytes per lane, the wave's 64 pieces to consecutive LDS addresses from the one in M0.  Written as
+  // asm so that the waits are this kernel's own (settle): the compiler, which cannot always tell which buffer a
+  // load in flight writes, would otherwise put a wait for all of them in front of LDS reads.  (No "memory"
+  // clobber, which brings those waits back: every read of a tile goes through an address the compiler cannot
+  // see through — RowTile::opaque — and lies between the same two barriers as the wait for that tile, so no
+  // read is merged with one of an earlier tile or moved ahead of its tile's arrival.)
+  __device__ static inline void to_lds(const uint8_t* base, uint32_t offset, uint8_t* lds) {
+    const uint32_t l = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(offset), "s"(base), "s"(l));
+  }
+  __device__ inline void issue(const DecodeParams& p, const Item& it, int tb, int blk, uint8_t* buf) const {
+    const HalfBase b = half_base(p, it, tb + 4 * TOK * wave, blk);
+    to_lds(p.k_cache + b.elem * 2, k_off, buf + kLdsK + 1024 * wave);
+    to_lds(p.v_cache + b.elem * 2, v_off, buf + kLdsV + 1024 * wave);
+  }
+  // Zeros over the V pieces of tokens at or past the sequence end (after the loads have landed).
+  __device__ inline void clear_tail(int tb, int len, uint8_t* buf) const {
+    uint32_t z = 0;
+    asm volatile("" : "+v"(z));  // made here, on the rare path, instead of living in registers through the loop
+    if (tb + 4 * TOK * wave + v_tok >= len) *(u32x4*)(buf + kLdsV + 1024 * wave + lane * 16) = u32x4{z, z, z, z};
+  }
+};
+
+template <int KV_DT, int TOK>
+__global__ void __launch_bounds__(512, 2) prefill_pingpong_d128_kernel(DecodeParams p) {
+  static_assert(!quant_of(KV_DT), "a 1-byte cache needs converting on the way into LDS");
+  static_assert(TOK == 1, "head_dim 128: the scores and weights of a 64-token tile (head_dim 64) do not fit the registers");
+  __shared__ __attribute__((aligned(16))) uint8_t buf0[kPrefillTile];
+  __shared__ __attribute__((aligned(16))) uint8_t buf1[kPrefillTile];
+  __shared__ __attribute__((aligned(16))) uint8_t buf2[kPrefillTile];
+  __shared__ __attribute__((aligned(16))) uint8_t buf3[kPrefillTile];
+  __shared__ __attribute__((aligned(16))) uint8_t buf4[kPrefillTile];
+  __shared__ __attribute__((aligned(16))) uint8_t buf5[kPrefillTile];
+  __shared__ float lds_ml[8 * 16 * 2];
+  constexpr int kT = 32 * TOK;  // tokens per tile
+  constexpr int kNB = kPingPongBuffers;
+  static_assert(2 * 16 * xch_row_bytes(TOK) <= kPrefillTile, "two waves' end-of-item exchanges must fit a tile buffer");
+
+  Item it;
+  if (!decode_item(p, blockIdx.x, it)) return;
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  // The group that runs one phase behind.  Waves w and w + 4 of a workgroup share a SIMD.
+  const bool late = (p.prefill_opts & 2) ? (wave & 1) != 0 : wave >= 4;
+
+  typedef RowTile<KV_DT, TOK> RT;
+  typedef typename RT::Op Op;
+  RT rt[2];
+  rt[0].init(p, it, 32 * wave, lane);
+  rt[1].init(p, it, 32 * wave + 16, lane);
+
+  // What this wave's rows can see (see prefill_mfma_d128_kernel), and what every row of the item sees in full.
+  const int rows = it.n * p.group;
+  const int r_first = it.rg * p.rows_per_item + 32 * wave;
+  const bool has_rows = r_first < rows;
+  const int r_last = min(r_first + 31, rows - 1);
+  const int lim_first = it.len - (it.n - 1 - r_first / p.group);
+  const int lim_last = has_rows ? it.len - (it.n - 1 - r_last / p.group) : 0;
+  const int lo_first = p.window_left >= 0 ? lim_first - 1 - p.window_left : 0;
+  const int lo_last = p.window_left >= 0 ? lim_last - 1 - p.window_left : 0;
+  const int ri_first = it.rg * p.rows_per_item;
+  const int lim_item = it.len - (it.n - 1 - ri_first / p.group);  // the item's first row sees the tokens below this
+
+  const int w_begin = first_visible_tile(p, it);
+  const int w_end = it.t_end;
+  const int iters = w_end > w_begin ? (w_end - w_begin + kT - 1) / kT : 0;
+  // tiles [0, nfast) take the straight-line form, nfast = 1 + 6k (none under a sliding window, whose lower edge
+  // would put masked tiles in front of them)
+  int p1 = lim_item > w_begin ? (lim_item - w_begin) / kT : 0;
+  p1 = p1 < iters ? p1 : iters;
+  const int nfast = p1 >= 1 && p.window_left < 0 ? 1 + (p1 - 1) / kNB * kNB : 0;
+
+  PingPongLoader<KV_DT, TOK> ld;
+  ld.init(p, wave, lane);
+  const int mine = 4 * TOK * wave;  // first of the tokens this wave fetches, within a tile
+
+  auto buffer = [&](auto k) __attribute__((always_inline)) -> uint8_t* {
+    constexpr int K = decltype(k)::value % kNB;
+    if constexpr (K == 0) return buf0;
+    if constexpr (K == 1) return buf1;
+    if constexpr (K == 2) return buf2;
+    if constexpr (K == 3) return buf3;
+    if constexpr (K == 4) return buf4;
+    return buf5;
+  };
+  auto barrier = [&]() __attribute__((always_inline)) {
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  typedef typename RT::Scores Scores;
+  typedef Op Weights[RT::kU];
+  Weights pf0, pf1;  // the weights of the last pipelined tile: they wait for its V^T P^T in the next step
+  int blk = 0;       // block id of this wave's rows of the tile that is put in flight next
+
+  // K Q^T of the tile in `cur` for both row tiles.  `kf`: the fragments of chunk 0, already on their way.
+  // The reads of chunk c + 1 are issued with the MFMAs of chunk c, and nothing moves across the fences: the
+  // compiler would otherwise hoist a phase's 24 fragment reads to its top and hold them all in registers.
+  auto k_fragments = [&](const uint8_t* cur, int c, Op (&kf)[2]) __attribute__((always_inline)) {
+    const uint32_t ko = RT::opaque(rt[0].k_off0) ^ (uint32_t)(c << 6);  // (formed anew for every use: see RowTile::opaque)
+    kf[0] = *(const Op*)(cur + ko);
+    kf[1] = *(const Op*)(cur + ko + 4096);
+  };
+  auto scores_from = [&](const uint8_t* cur, Op (&kf)[2], Scores& s0, Scores& s1) __attribute__((always_inline)) {
+    rt[0].scores_init(s0);
+    rt[1].scores_init(s1);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      Op nf[2];
+      if (c < 3) k_fragments(cur, c + 1, nf);
+      rt[0].scores_step(c, kf[0], kf[1], s0);
+      rt[1].scores_step(c, kf[0], kf[1], s1);
+      if (c < 3) {
+        kf[0] = nf[0];
+        kf[1] = nf[1];
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  auto scores = [&](const uint8_t* cur, Scores& s0, Scores& s1) __attribute__((always_inline)) {
+    Op kf[2];
+    k_fragments(cur, 0, kf);
+    __builtin_amdgcn_sched_barrier(0);
+    scores_from(cur, kf, s0, s1);
+  };
+  // O^T += V^T P^T with the V rows in `buf`: the fragments of head-dim tiles dt + 1 and dt + 2 are on their way
+  // while tile dt's MFMAs are issued.  `then`: what to put in flight with the last two tiles' MFMAs.
+  auto values_then = [&](const uint8_t* buf, const Weights& w0, const Weights& w1, auto then) __attribute__((always_inline)) {
+    Op vf[3];
+    vf[0] = rt[0].v_fragment(buf, 0, RT::opaque(rt[0].v_off0));
+    vf[1] = rt[0].v_fragment(buf, 1, RT::opaque(rt[0].v_off0));
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int dt = 0; dt < 8; ++dt) {
+      if (dt + 2 < 8) vf[(dt + 2) % 3] = rt[0].v_fragment(buf, dt + 2, RT::opaque(rt[0].v_off0));
+      if (dt == 6) then();
+      rt[0].template accumulate_step<false>(dt, vf[dt % 3], w0, 1.0f);
+      rt[1].template accumulate_step<false>(dt, vf[dt % 3], w1, 1.0f);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  auto values = [&](const uint8_t* buf, const Weights& w0, const Weights& w1) __attribute__((always_inline)) {
+    values_then(buf, w0, w1, [] {});
+  };
+  // Softmax of both row tiles; the accumulators follow when a reference point moved (rare after the first tiles).
+  auto weights = [&](auto masked, int tb, const Scores& s0, const Scores& s1, Weights& w0, Weights& w1) __attribute__((always_inline)) {
+    constexpr bool MASKED = decltype(masked)::value;
+    float kscl[RT::kN], lv[RT::kN], rvs[RT::kN];
+    float alpha0, alpha1;
+    const bool moved0 = rt[0].template softmax<MASKED>(s0, kscl, lv, rvs, tb, p.scale_log2, w0, alpha0);
+    __builtin_amdgcn_sched_barrier(0);  // one softmax at a time: interleaving the two costs registers
+    const bool moved1 = rt[1].template softmax<MASKED>(s1, kscl, lv, rvs, tb, p.scale_log2, w1, alpha1);
+    if (moved0 || moved1) {  // (the factor of a tile whose maxima stayed is exactly 1)
+#pragma unroll
+      for (int dt = 0; dt < 8; ++dt) {
+        rt[0].acc[dt] *= alpha0;
+        rt[1].acc[dt] *= alpha1;
+      }
+    }
+  };
+  // Before the barrier that precedes a softmax phase: the block id for the loads issued after the next barrier
+  // (a scalar load, which shares a counter with LDS: it is complete, and out of the way of the matrix phase's
+  // LDS waits, when this returns), this wave's share of the next tile landed, its V rows past the sequence end zeroed.
+  auto settle = [&](int tb, uint8_t* next) __attribute__((always_inline)) {
+    blk = block_of_const(p, it, tb + (kNB - 1) * kT + mine);
+    __builtin_amdgcn_s_waitcnt(0x0f76);  // vmcnt(6): the loads of three tiles may still be in flight
+    if (tb + 2 * kT > it.len) ld.clear_tail(tb + kT, it.len, next);
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+  };
+
+  // One tile, all of it in this step: K Q^T in the matrix phase; softmax and V^T P^T in the other.  (Scores and
+  // weights are the step's own: nothing of a tile outlives its step here.)
+  auto whole = [&](auto ph, int i) __attribute__((always_inline)) {
+    constexpr int PH = decltype(ph)::value;
+    uint8_t* cur = buffer(std::integral_constant<int, PH>{});
+    const int tb = w_begin + i * kT;
+    const bool visible = !(tb >= lim_last || tb + kT <= lo_first);
+    Scores s0, s1;
+    barrier();
+    ld.issue(p, it, tb + (kNB - 2) * kT, blk, buffer(std::integral_constant<int, PH + kNB - 2>{}));
+    if (visible) {
+      XLLM_HIP_PINGPONG_SETPRIO(1);
+      scores(cur, s0, s1);
+      XLLM_HIP_PINGPONG_SETPRIO(0);
+    }
+    settle(tb, buffer(std::integral_constant<int, PH + 1>{}));
+    barrier();
+    if (visible) {
+      Weights w0, w1;
+      if (tb + kT > lim_first || tb < lo_last) {
+        weights(std::true_type{}, tb, s0, s1, w0, w1);
+      } else {
+        weights(std::false_type{}, tb, s0, s1, w0, w1);
+      }
+      values(cur, w0, w1);
+    }
+  };
+  // A tile every row sees in full, after another such tile: V^T P^T of that one, K Q^T of this one, then the softmax.
+  auto pipelined = [&](auto ph, auto first, int i) __attribute__((always_inline)) {
+    constexpr int PH = decltype(ph)::value;
+    uint8_t* cur = buffer(std::integral_constant<int, PH>{});
+    const int tb = w_begin + i * kT;
+    Scores s0, s1;
+    barrier();
+    ld.issue(p, it, tb + (kNB - 2) * kT, blk, buffer(std::integral_constant<int, PH + kNB - 2>{}));
+    XLLM_HIP_PINGPONG_SETPRIO(1);
+    if constexpr (!decltype(first)::value) {
+      Op kf[2];
+      values_then(buffer(std::integral_constant<int, PH + kNB - 1>{}), pf0, pf1,
+                  [&]() __attribute__((always_inline)) { k_fragments(cur, 0, kf); });
+      scores_from(cur, kf, s0, s1);
+    } else {
+      scores(cur, s0, s1);
+    }
+    XLLM_HIP_PINGPONG_SETPRIO(0);
+    settle(tb, buffer(std::integral_constant<int, PH + 1>{}));
+    barrier();
+    weights(std::false_type{}, tb, s0, s1, pf0, pf1);
+  };
+  if (iters > 0) {  // (an item without visible tokens touches no block: its table row may hold anything)
+    // The queries have arrived (they are needed at once; and the compiler, which does not count the tile loads,
+    // would otherwise carry a wait for them into every loop below)
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+    ld.issue(p, it, w_begin, block_of_const(p, it, w_begin + mine), buf0);
+    ld.issue(p, it, w_begin + kT, block_of_const(p, it, w_begin + kT + mine), buf1);
+    ld.issue(p, it, w_begin + 2 * kT, block_of_const(p, it, w_begin + 2 * kT + mine), buf2);
+    ld.issue(p, it, w_begin + 3 * kT, block_of_const(p, it, w_begin + 3 * kT + mine), buf3);
+    settle(w_begin - kT, buf0);  // tile 0 landed; the block id of tile 4
+    if (late) barrier();
+    int i = 0;
+    if (nfast > 0) {
+      pipelined(std::integral_constant<int, 0>{}, std::true_type{}, i);
+      ++i;
+      for (; i + kNB <= nfast; i += kNB) {
+        pipelined(std::integral_constant<int, 1>{}, std::false_type{}, i);
+        pipelined(std::integral_constant<int, 2>{}, std::false_type{}, i + 1);
+        pipelined(std::integral_constant<int, 3>{}, std::false_type{}, i + 2);
+        pipelined(std::integral_constant<int, 4>{}, std::false_type{}, i + 3);
+        pipelined(std::integral_constant<int, 5>{}, std::false_type{}, i + 4);
+        pipelined(std::integral_constant<int, 0>{}, std::false_type{}, i + 5);
+      }
+      values(buf0, pf0, pf1);  // the last pipelined tile's V^T P^T: that tile is in the first buffer
+    }
+    // The other tiles, from the second buffer on (or from the first, when no tile took the straight-line form),
+    // again one step per buffer, so that what is in flight at each step is the same on every path to it.
+    if (nfast == 0) {
+      whole(std::integral_constant<int, 0>{}, 0);
+      i = 1;
+    }
+    while (i < iters) {
+      whole(std::integral_constant<int, 1>{}, i);
+      if (++i >= iters) break;
+      whole(std::integral_constant<int, 2>{}, i);
+      if (++i >= iters) break;
+      whole(std::integral_constant<int, 3>{}, i);
+      if (++i >= iters) break;
+      whole(std::integral_constant<int, 4>{}, i);
+      if (++i >= iters) break;
+      whole(std::integral_constant<int, 5>{}, i);
+      if (++i >= iters) break;
+      whole(std::integral_constant<int, 0>{}, i);
+      ++i;
+    }
+    if (!late) barrier();
+  }
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): nothing lands in LDS any more
+  __syncthreads();  // all tiles consumed: the buffers become the exchange
+  uint8_t* xch = (wave < 2 ? buf0 : wave < 4 ? buf1 : wave < 6 ? buf2 : buf3) + (wave & 1) * (16 * xch_row_bytes(TOK));
+  finish_item<KV_DT, TOK, 1>(p, it, rt[0], xch, 0, lds_ml, wave, wave, 0, lane, 2 * wave);
+  __syncthreads();
+  finish_item<KV_DT, TOK, 1>(p, it, rt[1], xch, 0, lds_ml, wave, wave, 0, lane, 2 * wave + 1);
+}
+
+}  // namespace xllm_hip

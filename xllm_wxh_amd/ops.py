@@ -64,7 +64,7 @@ class option:
     _IDS = {"force_generic": _lib.OPTION_DECODE_FORCE_GENERIC, "target_items": _lib.OPTION_DECODE_TARGET_ITEMS,
             "separate_merge": _lib.OPTION_DECODE_SEPARATE_MERGE, "stored_schedule": _lib.OPTION_DECODE_STORED_SCHEDULE,
             "item_per_head": _lib.OPTION_DECODE_ITEM_PER_HEAD,
-            "four_wave_items": _lib.OPTION_DECODE_FOUR_WAVE_ITEMS}
+            "four_wave_items": _lib.OPTION_DECODE_FOUR_WAVE_ITEMS, "prefill_kernel": _lib.OPTION_PREFILL_KERNEL}
 
     def __init__(self, name, value=1):
         self.which, self.value = self._IDS[name], int(value)
