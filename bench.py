@@ -559,11 +559,30 @@ def aux_kernels(torch, ops, device):
     us = timed(lambda: ops.batch_decode(q, kc, out, table, lens, vc, scale=D ** -0.5, q_per_seq=n, q_indptr=q_indptr,
                                         max_seq_len=L, total_kv_len=B * L), n=10)
     flops = 4.0 * B * Hq * D * sum(L - n + 1 + j for j in range(n))
-    res["entries"].append({"kernel": "chunked prefill (128-row kernel), 4 x 512 tokens on a 3584-token prefix, bf16",
+    res["entries"].append({"kernel": "chunked prefill (256-row kernel), 4 x 512 tokens on a 3584-token prefix, bf16",
                            "us": round(us, 1), "tflops": round(flops / us / 1e6, 1),
                            "frac_of_mfma_peak": round(flops / us / 1e6 / 2500.0, 3),
-                           "note": "flops of the visible (causal) part only; every 128 query rows stream the "
+                           "note": "flops of the visible (causal) part only; every 256 query rows stream the "
                                    "sequence's K/V again, from the L2 of their XCD"})
+    with ops.option("prefill_kernel", 1):
+        us128 = timed(lambda: ops.batch_decode(q, kc, out, table, lens, vc, scale=D ** -0.5, q_per_seq=n, q_indptr=q_indptr,
+                                               max_seq_len=L, total_kv_len=B * L), n=10)
+    res["entries"].append({"kernel": "the same through the 128-row kernel (XLLM_HIP_OPTION_PREFILL_KERNEL = 1)",
+                           "us": round(us128, 1), "tflops": round(flops / us128 / 1e6, 1),
+                           "frac_of_mfma_peak": round(flops / us128 / 1e6 / 2500.0, 3), "note": ""})
+    # a plain prefill: 4 sequences of 4096 tokens from an empty cache (the whole sequence is the chunk)
+    n2 = 4096
+    q2 = torch.randn(B * n2, Hq, D, device=device, dtype=torch.bfloat16, generator=gen)
+    out2 = torch.empty_like(q2)
+    q_indptr2 = (torch.arange(B + 1, device=device) * n2).to(torch.int32)
+    us2 = timed(lambda: ops.batch_decode(q2, kc, out2, table, lens, vc, scale=D ** -0.5, q_per_seq=n2, q_indptr=q_indptr2,
+                                         max_seq_len=L, total_kv_len=B * L), n=5)
+    flops2 = 4.0 * B * Hq * D * sum(j + 1 for j in range(n2))
+    res["entries"].append({"kernel": "prefill (256-row kernel), 4 x 4096 tokens from an empty cache, bf16",
+                           "us": round(us2, 1), "tflops": round(flops2 / us2 / 1e6, 1),
+                           "frac_of_mfma_peak": round(flops2 / us2 / 1e6 / 2500.0, 3),
+                           "note": "causal: flops of the visible part only"})
+    del q2, out2
     us = timed(lambda: ops.batch_decode(q, kq, out, table, lens, vq, None, None, ksc, vsc, scale=D ** -0.5, q_per_seq=n,
                                         q_indptr=q_indptr, max_seq_len=L, total_kv_len=B * L,
                                         kv_cache_quant_bit_size=8), n=10)

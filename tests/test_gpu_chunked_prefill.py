@@ -269,3 +269,54 @@ def test_long_chunk_on_the_default_workspace(gpu, kv, qdt):
     print("   err %.3e" % err, flush=True)
     assert err <= (1.2e-2 if kv == "bf16" else 1e-4)
     assert np.allclose(lse.cpu().numpy()[rows], ref_lse, atol=2e-2 if kv == "bf16" else 1e-4)
+
+
+@pytest.mark.parametrize("qdt", ["bf16", "fp16"])
+@pytest.mark.parametrize("bs,layout", [(16, "HND"), (128, "NHD")])
+def test_256_row_kernel_against_the_128_row_kernel_and_the_oracle(gpu, qdt, bs, layout):
+    """More than 128 query rows per kv head over a 16-bit cache at head_dim 128 take the 256-row kernel (eight
+    waves in two groups that alternate between matrix and softmax phases).  Its straight-line loop takes the
+    tiles every row sees in full, six at a time after the first, and a second form the rest: the prefixes here
+    put 0, 1, 6, 7, 8, 13 and 30 tiles in front of the causal edge, the chunks are one item, one item and a
+    few rows, and several items, one sequence is its own chunk, and one has no query tokens.  The results match
+    the oracle and, to a rounding of a few outputs, the 128-row kernel (XLLM_HIP_OPTION_PREFILL_KERNEL)."""
+    print("case 256-row kernel", qdt, bs, layout, flush=True)
+    q_counts = [64, 40, 33, 70, 64, 200, 64, 0, 129, 300]
+    prefix = [0, 32, 6 * 32, 7 * 32 + 5, 8 * 32, 13 * 32 + 31, 30 * 32 + 1, 100, 0, 1000]
+    lens = [p + n for p, n in zip(prefix, q_counts)]
+    kv = "bf16" if qdt == "bf16" else "fp16"
+    c = Case(len(lens), 32, 8, 128, bs, lens, kv=kv, qdt=qdt, layout=layout, seed=41)
+    q_indptr = np.concatenate([[0], np.cumsum(q_counts)]).astype(np.int32)
+    T = int(q_indptr[-1])
+    dt = torch.bfloat16 if qdt == "bf16" else torch.float16
+    q = torch.randn(T, c.Hq, c.D, generator=torch.Generator().manual_seed(79)).to(dt)
+    qd = q.to(c.q.device)
+    ref, ref_lse = orc.paged_decode_ragged(q.float().numpy(), c.k_ref, c.v_ref, c.table, c.lens, q_indptr, c.scale)
+    ref_w, _ = orc.paged_decode_ragged(q.float().numpy(), c.k_ref, c.v_ref, c.table, c.lens, q_indptr, c.scale, window_left=150)
+    got = {}
+    for name, value in (("rows256", 0), ("rows128", 1)):
+        with ops.option("prefill_kernel", value):
+            for window in (-1, 150):
+                out = torch.full_like(qd, 7.0)
+                lse = torch.full((T, c.Hq), 3.0, dtype=torch.float32, device=qd.device)
+                ops.batch_decode(qd, c.k_cache, out, c.block_table, c.seq_lens, c.v_cache, lse, scale=c.scale, return_lse=True,
+                                 q_per_seq=max(q_counts), q_indptr=torch.from_numpy(q_indptr).to(qd.device), kv_layout=layout,
+                                 window_size_left=window)
+                torch.cuda.synchronize()
+                got[name, window] = (out.float().cpu().numpy(), lse.cpu().numpy())
+    for window, r in ((-1, ref), (150, ref_w)):
+        o256, l256 = got["rows256", window]
+        o128, l128 = got["rows128", window]
+        assert not np.isnan(o256).any()
+        err = float(np.abs(o256 - r).max())
+        print("   window %d err %.3e" % (window, err), flush=True)
+        assert err <= 1.2e-2
+        # (the two kernels do the same arithmetic on the same values; where a reference point moves, the compiler
+        # fuses one of them's rescaled denominator into a multiply-add, so a few outputs may round the other way)
+        assert float(np.abs(o256 - o128).max()) <= 4e-3 and float(np.mean(o256 != o128)) <= 1e-4
+        assert np.allclose(l256, l128, atol=1e-5, equal_nan=True)
+    fin = np.isfinite(ref_lse)
+    assert np.allclose(got["rows256", -1][1][fin], ref_lse[fin], atol=2e-2)
+    d = ops.decode_describe(torch.empty(len(lens) * max(q_counts), c.Hq, c.D, dtype=dt, device=qd.device), c.k_cache, c.v_cache, c.block_table, c.seq_lens,
+                            q_per_seq=max(q_counts), kv_layout=layout)
+    assert d["waves_per_workgroup"] == 8, d

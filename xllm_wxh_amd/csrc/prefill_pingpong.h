@@ -42,6 +42,21 @@ namespace xllm_hip {
 #else
 #define XLLM_HIP_PINGPONG_SETPRIO(n) ((void)0)
 #endif
+// How the matrix phase reads its fragments (see the kernel).  XLLM_HIP_PP_ADDR_REGS: bit 0, the LDS offsets of the
+// eight V fragments stay in registers; bit 1, those of the four K fragments do (otherwise they are formed anew
+// for every read: two vector operations each, in a phase whose vector-issue slots the SIMD's other wave wants —
+// 4 x 512 tokens on a 3584-token prefix: 147-150 us with none, 141 with either V or both).  XLLM_HIP_PP_VDEPTH /
+// XLLM_HIP_PP_KDEPTH: V fragments / K chunks read ahead of the MFMAs that use them (3 or 4 and 2 measured the
+// same as 2 and 1: the phase does not wait for LDS).
+#ifndef XLLM_HIP_PP_ADDR_REGS
+#define XLLM_HIP_PP_ADDR_REGS 3
+#endif
+#ifndef XLLM_HIP_PP_VDEPTH
+#define XLLM_HIP_PP_VDEPTH 2
+#endif
+#ifndef XLLM_HIP_PP_KDEPTH
+#define XLLM_HIP_PP_KDEPTH 1
+#endif
 constexpr int kPingPongRows = 256;
 constexpr int kPingPongBuffers = 6;
 
@@ -174,56 +189,69 @@ __global__ void __launch_bounds__(512, 2) prefill_pingpong_d128_kernel(DecodePar
   typedef typename RT::Scores Scores;
   typedef Op Weights[RT::kU];
   Weights pf0, pf1;  // the weights of the last pipelined tile: they wait for its V^T P^T in the next step
+  Op vpre[XLLM_HIP_PP_VDEPTH];  // ... with the first V fragments of that tile, read ahead of the step's barrier
   int blk = 0;       // block id of this wave's rows of the tile that is put in flight next
 
-  // K Q^T of the tile in `cur` for both row tiles.  `kf`: the fragments of chunk 0, already on their way.
-  // The reads of chunk c + 1 are issued with the MFMAs of chunk c, and nothing moves across the fences: the
-  // compiler would otherwise hoist a phase's 24 fragment reads to its top and hold them all in registers.
+  // Fragment reads run ahead of the MFMAs that use them: kVAhead head-dim tiles of V, kKAhead 32-element chunks
+  // of K.  Nothing moves across the fences: the compiler would otherwise hoist a phase's 24 fragment reads to
+  // its top and hold them all in registers.
+  constexpr int kVAhead = XLLM_HIP_PP_VDEPTH, kKAhead = XLLM_HIP_PP_KDEPTH;
+  auto frag_offset = [&](uint32_t v) __attribute__((always_inline)) { return (XLLM_HIP_PP_ADDR_REGS & 1) ? v : RT::opaque(v); };
+  auto k_frag_offset = [&](uint32_t v) __attribute__((always_inline)) { return (XLLM_HIP_PP_ADDR_REGS & 2) ? v : RT::opaque(v); };
   auto k_fragments = [&](const uint8_t* cur, int c, Op (&kf)[2]) __attribute__((always_inline)) {
-    const uint32_t ko = RT::opaque(rt[0].k_off0) ^ (uint32_t)(c << 6);  // (formed anew for every use: see RowTile::opaque)
+    const uint32_t ko = k_frag_offset(rt[0].k_off0) ^ (uint32_t)(c << 6);
     kf[0] = *(const Op*)(cur + ko);
     kf[1] = *(const Op*)(cur + ko + 4096);
   };
-  auto scores_from = [&](const uint8_t* cur, Op (&kf)[2], Scores& s0, Scores& s1) __attribute__((always_inline)) {
+  // K Q^T of the tile in `cur` for both row tiles.  `kf`: the fragments of the first kKAhead chunks, already on their way.
+  auto scores_from = [&](const uint8_t* cur, Op (&kf)[kKAhead + 1][2], Scores& s0, Scores& s1) __attribute__((always_inline)) {
     rt[0].scores_init(s0);
     rt[1].scores_init(s1);
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
-      Op nf[2];
-      if (c < 3) k_fragments(cur, c + 1, nf);
-      rt[0].scores_step(c, kf[0], kf[1], s0);
-      rt[1].scores_step(c, kf[0], kf[1], s1);
-      if (c < 3) {
-        kf[0] = nf[0];
-        kf[1] = nf[1];
-      }
+      if (c + kKAhead < 4) k_fragments(cur, c + kKAhead, kf[(c + kKAhead) % (kKAhead + 1)]);
+      rt[0].scores_step(c, kf[c % (kKAhead + 1)][0], kf[c % (kKAhead + 1)][1], s0);
+      rt[1].scores_step(c, kf[c % (kKAhead + 1)][0], kf[c % (kKAhead + 1)][1], s1);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
+  auto k_prologue = [&](const uint8_t* cur, Op (&kf)[kKAhead + 1][2]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int c = 0; c < kKAhead; ++c) k_fragments(cur, c, kf[c]);
+  };
   auto scores = [&](const uint8_t* cur, Scores& s0, Scores& s1) __attribute__((always_inline)) {
-    Op kf[2];
-    k_fragments(cur, 0, kf);
+    Op kf[kKAhead + 1][2];
+    k_prologue(cur, kf);
     __builtin_amdgcn_sched_barrier(0);
     scores_from(cur, kf, s0, s1);
   };
-  // O^T += V^T P^T with the V rows in `buf`: the fragments of head-dim tiles dt + 1 and dt + 2 are on their way
-  // while tile dt's MFMAs are issued.  `then`: what to put in flight with the last two tiles' MFMAs.
-  auto values_then = [&](const uint8_t* buf, const Weights& w0, const Weights& w1, auto then) __attribute__((always_inline)) {
-    Op vf[3];
-    vf[0] = rt[0].v_fragment(buf, 0, RT::opaque(rt[0].v_off0));
-    vf[1] = rt[0].v_fragment(buf, 1, RT::opaque(rt[0].v_off0));
+  // O^T += V^T P^T with the V rows in `buf`.  `then`: what to put in flight with the last tiles' MFMAs.
+  // `pre` (PRELOADED): the fragments of the first kVAhead head-dim tiles, read before the step's barrier.
+  auto values_then = [&](const uint8_t* buf, const Weights& w0, const Weights& w1, auto preloaded, const Op (&pre)[kVAhead],
+                         auto then) __attribute__((always_inline)) {
+    Op vf[kVAhead + 1];
+#pragma unroll
+    for (int dt = 0; dt < kVAhead; ++dt) {
+      vf[dt] = decltype(preloaded)::value ? pre[dt] : rt[0].v_fragment(buf, dt, frag_offset(rt[0].v_off0));
+    }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int dt = 0; dt < 8; ++dt) {
-      if (dt + 2 < 8) vf[(dt + 2) % 3] = rt[0].v_fragment(buf, dt + 2, RT::opaque(rt[0].v_off0));
-      if (dt == 6) then();
-      rt[0].template accumulate_step<false>(dt, vf[dt % 3], w0, 1.0f);
-      rt[1].template accumulate_step<false>(dt, vf[dt % 3], w1, 1.0f);
+      if (dt + kVAhead < 8) vf[(dt + kVAhead) % (kVAhead + 1)] = rt[0].v_fragment(buf, dt + kVAhead, frag_offset(rt[0].v_off0));
+      if (dt + kVAhead == 8) then();
+      rt[0].template accumulate_step<false>(dt, vf[dt % (kVAhead + 1)], w0, 1.0f);
+      rt[1].template accumulate_step<false>(dt, vf[dt % (kVAhead + 1)], w1, 1.0f);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
   auto values = [&](const uint8_t* buf, const Weights& w0, const Weights& w1) __attribute__((always_inline)) {
-    values_then(buf, w0, w1, [] {});
+    Op none[kVAhead];
+    values_then(buf, w0, w1, std::false_type{}, none, [] {});
+  };
+  // The first V fragments of the tile in `buf`, put in flight ahead of the barrier behind which they are used.
+  auto v_prologue = [&](const uint8_t* buf, Op (&pre)[kVAhead]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int dt = 0; dt < kVAhead; ++dt) pre[dt] = rt[0].v_fragment(buf, dt, frag_offset(rt[0].v_off0));
   };
   // Softmax of both row tiles; the accumulators follow when a reference point moved (rare after the first tiles).
   auto weights = [&](auto masked, int tb, const Scores& s0, const Scores& s1, Weights& w0, Weights& w1) __attribute__((always_inline)) {
@@ -240,6 +268,48 @@ __global__ void __launch_bounds__(512, 2) prefill_pingpong_d128_kernel(DecodePar
         rt[1].acc[dt] *= alpha1;
       }
     }
+  };
+  // The same for a tile every row sees in full, with the common case — no reference point moves — as the straight
+  // path: whether one moves is asked first (some row's tile maximum more than kLazyRescale above its reference
+  // point: the condition of RowTile::weights), and only then are new reference points, factors and the scaled
+  // accumulators formed.  Same operations on the same values as RowTile::softmax, so the same bits.
+  auto plain_weights_of = [&](RT& r, const Scores& s, Weights& w) __attribute__((always_inline)) {
+    static_assert(RT::kU == 1 && RT::kHalves == 2 && !RT::kQuant && !RT::kRowScale, "16-bit cache, head_dim 128");
+    const float scale = p.scale_log2;
+    float mt = -INFINITY;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) mt = fmaxf(mt, s[0][h][rr]);  // (a chain from -inf: the compiler forms three-input maxima)
+    }
+    mt = kg_max(mt) * scale;
+    if (__builtin_amdgcn_ballot_w64(fmaxf(r.m_run, mt) > r.m_run + kLazyRescale) != 0) {
+      const float m_new = fmaxf(r.m_run, mt);
+      const float m_safe = m_new == -INFINITY ? 0.0f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f(r.m_run - m_safe);
+      r.l_run *= alpha;
+      r.m_run = m_new;
+#pragma unroll
+      for (int dt = 0; dt < 8; ++dt) r.acc[dt] *= alpha;
+    }
+    const float m_safe = r.m_run == -INFINITY ? 0.0f : r.m_run;
+    float e[8];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+        e[4 * h + rr] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[0][h][rr], scale, -m_safe));
+        r.l_run += e[4 * h + rr];
+      }
+    }
+    const u32x4 pw = {Mma<KV_DT>::pack(e[0], e[1]), Mma<KV_DT>::pack(e[2], e[3]), Mma<KV_DT>::pack(e[4], e[5]),
+                      Mma<KV_DT>::pack(e[6], e[7])};
+    w[0] = __builtin_bit_cast(Op, pw);
+  };
+  auto plain_weights = [&](const Scores& s0, const Scores& s1, Weights& w0, Weights& w1) __attribute__((always_inline)) {
+    plain_weights_of(rt[0], s0, w0);
+    __builtin_amdgcn_sched_barrier(0);  // one softmax at a time: interleaving the two costs registers
+    plain_weights_of(rt[1], s1, w1);
   };
   // Before the barrier that precedes a softmax phase: the block id for the loads issued after the next barrier
   // (a scalar load, which shares a counter with LDS: it is complete, and out of the way of the matrix phase's
@@ -273,7 +343,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pingpong_d128_kernel(DecodePar
       if (tb + kT > lim_first || tb < lo_last) {
         weights(std::true_type{}, tb, s0, s1, w0, w1);
       } else {
-        weights(std::false_type{}, tb, s0, s1, w0, w1);
+        plain_weights(s0, s1, w0, w1);
       }
       values(cur, w0, w1);
     }
@@ -288,9 +358,9 @@ __global__ void __launch_bounds__(512, 2) prefill_pingpong_d128_kernel(DecodePar
     ld.issue(p, it, tb + (kNB - 2) * kT, blk, buffer(std::integral_constant<int, PH + kNB - 2>{}));
     XLLM_HIP_PINGPONG_SETPRIO(1);
     if constexpr (!decltype(first)::value) {
-      Op kf[2];
-      values_then(buffer(std::integral_constant<int, PH + kNB - 1>{}), pf0, pf1,
-                  [&]() __attribute__((always_inline)) { k_fragments(cur, 0, kf); });
+      Op kf[kKAhead + 1][2];
+      values_then(buffer(std::integral_constant<int, PH + kNB - 1>{}), pf0, pf1, std::true_type{}, vpre,
+                  [&]() __attribute__((always_inline)) { k_prologue(cur, kf); });
       scores_from(cur, kf, s0, s1);
     } else {
       scores(cur, s0, s1);
@@ -298,7 +368,9 @@ __global__ void __launch_bounds__(512, 2) prefill_pingpong_d128_kernel(DecodePar
     XLLM_HIP_PINGPONG_SETPRIO(0);
     settle(tb, buffer(std::integral_constant<int, PH + 1>{}));
     barrier();
-    weights(std::false_type{}, tb, s0, s1, pf0, pf1);
+    plain_weights(s0, s1, pf0, pf1);
+    __builtin_amdgcn_sched_barrier(0);
+    v_prologue(cur, vpre);  // (this tile's V rows have been in LDS since before its matrix phase)
   };
   if (iters > 0) {  // (an item without visible tokens touches no block: its table row may hold anything)
     // The queries have arrived (they are needed at once; and the compiler, which does not count the tile loads,
@@ -322,7 +394,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pingpong_d128_kernel(DecodePar
         pipelined(std::integral_constant<int, 5>{}, std::false_type{}, i + 4);
         pipelined(std::integral_constant<int, 0>{}, std::false_type{}, i + 5);
       }
-      values(buf0, pf0, pf1);  // the last pipelined tile's V^T P^T: that tile is in the first buffer
+      values_then(buf0, pf0, pf1, std::true_type{}, vpre, [] {});  // the last pipelined tile's V^T P^T: that tile is in the first buffer
     }
     // The other tiles, from the second buffer on (or from the first, when no tile took the straight-line form),
     // again one step per buffer, so that what is in flight at each step is the same on every path to it.
