@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define XLLM_HIP_ABI_VERSION 3
+#define XLLM_HIP_ABI_VERSION 4
 
 /* A hipStream_t, passed as an opaque pointer so that C callers need no HIP headers. */
 typedef void* xllm_hip_stream_t;
@@ -207,6 +207,12 @@ typedef struct xllm_hip_decode_args {
   /* Query token offsets [batch+1] for sequences with different numbers of query tokens; NULL: every
    * sequence has q_per_seq of them. */
   const int32_t* q_indptr;
+  /* != 0: the step's schedule is the one xllm_hip_paged_decode_plan_host (or, from the same arguments,
+   * xllm_hip_paged_decode_plan) stores in the workspace before the step.  Which kernel runs and how its work
+   * items are shaped then follows from the sizes alone and max_seq_len / total_kv_len are ignored, so that a
+   * xllm_hip_paged_decode_run captured in a graph serves every later step of the same sizes: what changes from
+   * step to step lives in the workspace. */
+  int32_t host_plan;
 } xllm_hip_decode_args;
 
 /*
@@ -234,6 +240,35 @@ int xllm_hip_paged_decode_plan(const xllm_hip_kv_cache* cache,
                                void* workspace,
                                size_t workspace_bytes,
                                xllm_hip_stream_t stream);
+
+/*
+ * The same schedule made on the host, from the kv lengths the engine holds there
+ * (xllm/core/framework/model/model_input_params.h:341 kv_seq_lens_vec) — what the reference does before every
+ * step, also before every replay of a captured graph (xllm/core/runtime/cuda_graph_executor_impl.cpp:586-668,
+ * CudaGraphPersistentParam::update -> update_decode_plan_info; xllm/core/layers/cuda/flashinfer_planinfo.cpp:215-324).
+ * With every length known, each sequence is cut into chunks of its own, nearly equal size, how finely is chosen
+ * by the finishing time a list schedule of the step's work items predicts, and the chunks are dispatched longest
+ * first.  args->host_plan must be set (see there); host_kv_lens[b] must be the kv length the device-side arrays
+ * give for sequence b.  The schedule is written into host_staging (xllm_hip_paged_decode_plan_host_bytes bytes,
+ * best pinned) and copied to the head of `workspace` with one hipMemcpyAsync on `stream`; host_staging must stay
+ * untouched until that copy has run.  Nothing is allocated and nothing is read back; the call is made outside a
+ * captured graph, the runs it serves may be inside one.  info, if not NULL, receives {chunk size the cut was made
+ * for (0: nothing is cut), sequence chunks, predicted finishing time in tokens}.
+ */
+size_t xllm_hip_paged_decode_plan_host_bytes(int32_t batch,
+                                             int32_t q_per_seq,
+                                             int32_t num_q_heads,
+                                             int32_t num_kv_heads,
+                                             int32_t head_dim);
+int xllm_hip_paged_decode_plan_host(const xllm_hip_kv_cache* cache,
+                                    const xllm_hip_decode_args* args,
+                                    const int32_t* host_kv_lens,
+                                    void* workspace,
+                                    size_t workspace_bytes,
+                                    void* host_staging,
+                                    size_t host_staging_bytes,
+                                    xllm_hip_stream_t stream,
+                                    int64_t* info);
 
 /* Attention proper; requires a schedule built by xllm_hip_paged_decode_plan in `workspace` from the same
  * sizes, block list / length arrays and host-side lengths (max_seq_len, total_kv_len): with host-side

@@ -10,7 +10,7 @@ import os
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG_DIR, "libxllm_hip_paged_kv.so")
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 STATIC_WORKSPACE_BYTES = 48 << 20
 
 # xllm_hip_dtype
@@ -38,6 +38,8 @@ EXPORTED_SYMBOLS = (
     "xllm_hip_quant_to_paged_cache",
     "xllm_hip_paged_decode_workspace_bytes",
     "xllm_hip_paged_decode_plan",
+    "xllm_hip_paged_decode_plan_host_bytes",
+    "xllm_hip_paged_decode_plan_host",
     "xllm_hip_paged_decode_run",
     "xllm_hip_paged_decode_run_timed",
     "xllm_hip_paged_decode",
@@ -104,6 +106,7 @@ class DecodeArgs(ctypes.Structure):
         ("max_seq_len", ctypes.c_int32),
         ("total_kv_len", ctypes.c_int64),
         ("q_indptr", ctypes.c_void_p),
+        ("host_plan", ctypes.c_int32),
     ]
 
 
@@ -169,6 +172,11 @@ def load():
         fn = getattr(lib, name)
         fn.argtypes = [P(KvCacheDesc), P(DecodeArgs), vp, ctypes.c_size_t, vp]
         fn.restype = ctypes.c_int
+    lib.xllm_hip_paged_decode_plan_host_bytes.argtypes = [i32, i32, i32, i32, i32]
+    lib.xllm_hip_paged_decode_plan_host_bytes.restype = ctypes.c_size_t
+    lib.xllm_hip_paged_decode_plan_host.argtypes = [P(KvCacheDesc), P(DecodeArgs), vp, vp, ctypes.c_size_t, vp, ctypes.c_size_t,
+                                                    vp, P(ctypes.c_int64)]
+    lib.xllm_hip_paged_decode_plan_host.restype = ctypes.c_int
     lib.xllm_hip_paged_decode_run_timed.argtypes = [P(KvCacheDesc), P(DecodeArgs), vp, ctypes.c_size_t, vp, vp, vp]
     lib.xllm_hip_paged_decode_run_timed.restype = ctypes.c_int
     lib.xllm_hip_paged_decode_static.argtypes = [P(KvCacheDesc), P(DecodeArgs), vp]

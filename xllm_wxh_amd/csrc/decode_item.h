@@ -48,6 +48,7 @@ __device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it)
   int chunk = 0, chunk_tokens = 1 << 30;
   it.chunks = 1;
   bool to_the_end = false;  // the chunk runs to the end of the sequence whatever its length
+  int stored_begin = -1, stored_end = 0;  // the chunk's token range as a stored schedule gives it
   if (p.implicit_plan) {
     if (it.sc >= p.batch) return false;
     it.b = it.sc;
@@ -79,11 +80,14 @@ __device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it)
     // (a record no plan wrote — a run on a workspace that was planned with other host-side lengths —
     // names no sequence outside the batch)
     if ((unsigned)s.seq >= (unsigned)p.batch || s.chunk < 0) return false;
+    // (nor a partial slot outside the workspace, nor a token range outside the sequence)
+    if ((unsigned)s.slot >= (unsigned)p.max_seq_chunks || s.t_begin < 0 || s.len < 0) return false;
     it.b = s.seq;
     it.len = s.len;
     it.chunks = s.chunks;
-    chunk = s.chunk;
-    chunk_tokens = hdr.chunk_tokens;
+    it.sc = s.slot;
+    stored_begin = s.t_begin;
+    stored_end = s.t_end < s.len ? s.t_end : s.len;
   }
   if (p.q_indptr != nullptr) {
     it.q0 = p.q_indptr[it.b];
@@ -95,9 +99,14 @@ __device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it)
   }
   if (it.rg * p.rows_per_item >= it.n * p.group) return false;  // this sequence has no rows in the group
   if (p.implicit_plan) it.len = kv_length(p, it.b);
-  it.t_begin = chunk * chunk_tokens;
-  const long long end = (long long)it.t_begin + chunk_tokens;
-  it.t_end = end < it.len && !to_the_end ? (int)end : it.len;
+  if (stored_begin >= 0) {
+    it.t_begin = stored_begin;
+    it.t_end = stored_end;
+  } else {
+    it.t_begin = chunk * chunk_tokens;
+    const long long end = (long long)it.t_begin + chunk_tokens;
+    it.t_end = end < it.len && !to_the_end ? (int)end : it.len;
+  }
   {  // no row of the item sees beyond the causal limit of its last row
     const int rows = it.n * p.group;
     const int last = min((it.rg + 1) * p.rows_per_item, rows) - 1;
@@ -110,6 +119,10 @@ __device__ inline bool decode_item(const DecodeParams& p, int item_id, Item& it)
     it.ids = p.block_ids + (int64_t)it.b * p.bt_stride;
   }
   it.nblk = (it.len + p.block_size - 1) >> p.log2_bs;
+  if (p.kv_indptr != nullptr) {  // (a stored length that the sequence's list cannot hold reads no id outside the list)
+    const int listed = p.kv_indptr[it.b + 1] - p.kv_indptr[it.b];
+    it.nblk = it.nblk < listed ? it.nblk : listed;
+  }
   if (it.nblk < 1) it.nblk = 1;
   it.head_off = (int64_t)it.hk * p.stride_head;
   it.sc_head_off = (int64_t)it.hk * p.sc_stride_head;

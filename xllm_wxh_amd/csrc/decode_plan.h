@@ -91,16 +91,22 @@ XLLM_HIP_HD inline int choose_chunk(long long total, long long max_len, int batc
 struct PlanHeader {
   int32_t total_full;    // number of full sequence-chunks
   int32_t total_tail;    // number of tail sequence-chunks
-  int32_t chunk_tokens;  // C
+  int32_t chunk_tokens;  // C (the device-side plan; a plan made on the host cuts every sequence to its own size)
   int32_t total_items;   // (total_full + total_tail) * num_kv_heads * row_groups
   int32_t pad[12];
 };
 
+// One sequence chunk of the stored schedule, in the order the work items are dispatched.
 struct SeqChunk {
-  int32_t seq;     // sequence index b
-  int32_t chunk;   // chunk index within the sequence (token range [chunk*C, min(L, (chunk+1)*C)))
-  int32_t len;     // kv length of the sequence
-  int32_t chunks;  // chunks of the sequence (full + tail): one record tells a work item all it needs
+  int32_t seq;      // sequence index b
+  int32_t chunk;    // chunk index within the sequence
+  int32_t len;      // kv length of the sequence
+  int32_t chunks;   // chunks of the sequence: one record tells a work item all it needs
+  int32_t t_begin;  // token range of the chunk: [t_begin, t_end), t_begin a multiple of the tile
+  int32_t t_end;
+  int32_t slot;     // where the chunk's partial rows live: full_prefix[seq] + chunk for a full chunk, total_full +
+                    // tail_prefix[seq] for a tail (the device-side plan dispatches in slot order: slot = index)
+  int32_t pad;
 };
 
 struct WorkspaceLayout {

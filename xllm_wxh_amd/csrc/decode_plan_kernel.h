@@ -163,13 +163,17 @@ __global__ void __launch_bounds__(64) decode_plan_kernel(DecodeParams p) {
       // (the table holds every chunk any lengths can produce — see workspace_layout —; the bound is
       // checked here all the same, so that nothing is ever written outside it)
       for (int ci = 0; ci < nf; ++ci) {
-        if (f0 + ci < p.max_seq_chunks) p.seq_chunks[f0 + ci] = SeqChunk{b, ci, len_b, nf + nt};
+        if (f0 + ci < p.max_seq_chunks) {
+          p.seq_chunks[f0 + ci] = SeqChunk{b, ci, len_b, nf + nt, ci * chunk, (ci + 1) * chunk, f0 + ci, 0};
+        }
       }
       if (nt) {
         const int cls = tail_class(len_b - nf * chunk);
         const int slot = tail_hist[cls] + atomicAdd(&tail_fill[cls], 1);
         p.tail_prefix[b] = slot;
-        if (total_full + slot < p.max_seq_chunks) p.seq_chunks[total_full + slot] = SeqChunk{b, nf, len_b, nf + nt};
+        if (total_full + slot < p.max_seq_chunks) {
+          p.seq_chunks[total_full + slot] = SeqChunk{b, nf, len_b, nf + nt, nf * chunk, len_b, total_full + slot, 0};
+        }
       }
     }
     if (!in_lds) {

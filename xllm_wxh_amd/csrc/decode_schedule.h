@@ -1,0 +1,188 @@
+// The split-KV schedule of a decode step, made on the host from the kv lengths the engine holds there
+// (the reference re-plans on the host before every step, also before every replay of a captured graph:
+// xllm/core/runtime/cuda_graph_executor_impl.cpp:586-668, xllm/core/layers/cuda/flashinfer_planinfo.cpp:215-324;
+// the lengths: xllm/core/framework/model/model_input_params.h:341 kv_seq_lens_vec).
+//
+// It fills the same tables as decode_plan_kernel (decode_plan.h), in a host buffer laid out like the head of the
+// workspace, and differs from the device-side plan in what full knowledge of the lengths allows:
+//   * every sequence is cut into chunks of its own, nearly equal size (no short tail behind full chunks);
+//   * how finely to cut is chosen among a few targets by the finishing time a list schedule of the step's work
+//     items predicts (each workgroup slot takes the next item when it falls free, which is what the hardware
+//     dispatcher does with workgroups in index order);
+//   * the chunks are dispatched longest first across all sequences.
+// Host code only: no HIP types.
+#pragma once
+
+#include "decode_plan.h"
+
+#include <stdint.h>
+#include <string.h>
+
+#include <algorithm>
+#include <functional>
+#include <queue>
+#include <vector>
+
+namespace xllm_hip {
+
+struct HostScheduleInput {
+  const int32_t* kv_lens;  // [batch], as the kernels will see them (cut to 0 .. len_cap here)
+  int32_t batch;
+  int32_t len_cap;         // tokens a sequence's block list can hold (INT32_MAX: unknown)
+  int32_t per;             // work items per sequence chunk: kv heads (or head groups) x row groups
+  int32_t slots;           // workgroups the GPU runs at once
+  int32_t tile;            // chunk sizes are multiples of it
+  int32_t min_chunk;       // no chunk of a cut sequence is shorter
+  int64_t max_seq_chunks;  // records and partial rows the workspace holds, and the launch covers
+  int32_t max_per_seq;     // chunks a sequence is cut into at most
+  double item_overhead;    // fixed cost of a work item, in tokens of streaming (prologue, epilogue, partial rows)
+};
+
+struct HostScheduleResult {
+  int32_t chunk_target = 0;    // the chunk size the cut was made for (0: nothing is cut)
+  int64_t total_chunks = 0;
+  double predicted_span = 0;   // finishing time of the list schedule, in tokens
+  size_t bytes = 0;            // bytes of the host buffer that hold the schedule (header .. last record)
+};
+
+inline int32_t schedule_clamped_len(int32_t len, int32_t cap) {
+  len = len < cap ? len : cap;
+  return len > 0 ? len : 0;
+}
+
+// Chunk size and count of a sequence of `len` tokens cut for chunks of about `target` tokens: n nearly equal
+// chunks, tile-aligned, none below min_chunk unless the sequence is whole.
+inline void schedule_cut(int32_t len, int64_t target, const HostScheduleInput& in, int32_t& n, int32_t& chunk) {
+  n = 1;
+  chunk = len;
+  if (target <= 0 || len <= target + target / 4) return;  // (a sequence that would only shed a small piece stays whole)
+  int64_t parts = (len + target - 1) / target;
+  if (parts > in.max_per_seq) parts = in.max_per_seq;
+  int64_t c = (len + parts - 1) / parts;
+  c = (c + in.tile - 1) / in.tile * in.tile;
+  if (c < in.min_chunk) c = in.min_chunk;
+  const int64_t cnt = (len + c - 1) / c;
+  if (cnt <= 1) return;
+  n = (int32_t)cnt;
+  chunk = (int32_t)c;
+}
+
+// Finishing time of the step if its sequence chunks, `per` equal work items each, are handed to `slots` slots
+// longest first.  Items of one sequence chunk start together on `per` slots, so the slots are simulated in
+// groups of `per` (the last group may be narrower; it is treated as a full one: an upper estimate).
+inline double schedule_span(std::vector<int32_t>& sizes, const HostScheduleInput& in) {
+  std::sort(sizes.begin(), sizes.end(), std::greater<int32_t>());
+  int64_t lanes = in.slots / (in.per > 0 ? in.per : 1);
+  if (lanes < 1) lanes = 1;
+  if ((int64_t)sizes.size() <= lanes) return sizes.empty() ? 0.0 : sizes[0] + in.item_overhead;
+  std::priority_queue<double, std::vector<double>, std::greater<double>> free_at;
+  for (int64_t i = 0; i < lanes; ++i) free_at.push(0.0);
+  double span = 0.0;
+  for (int32_t s : sizes) {
+    const double t = free_at.top() + s + in.item_overhead;
+    free_at.pop();
+    free_at.push(t);
+    span = t > span ? t : span;
+  }
+  return span;
+}
+
+// Builds the schedule into `host` (laid out by `w`, the workspace's own layout: header, kv_len, full_prefix,
+// tail_prefix, num_chunks, seq_chunks).  `host_bytes` must cover w.seq_chunks + max_seq_chunks records.
+inline bool host_schedule(const HostScheduleInput& in, const WorkspaceLayout& w, uint8_t* host, size_t host_bytes,
+                          HostScheduleResult& out) {
+  const int64_t room = in.max_seq_chunks < w.max_seq_chunks ? in.max_seq_chunks : w.max_seq_chunks;
+  if (in.batch < 0 || room < in.batch || host_bytes < w.seq_chunks + sizeof(SeqChunk) * (size_t)room) return false;
+  int64_t total = 0;
+  int32_t longest = 0;
+  for (int32_t b = 0; b < in.batch; ++b) {
+    const int32_t l = schedule_clamped_len(in.kv_lens[b], in.len_cap);
+    total += l;
+    longest = l > longest ? l : longest;
+  }
+  // Candidate chunk sizes: nothing cut; then the work spread over 1, 1.5, 2, 3 and 4 times the slots.
+  const int64_t lanes = std::max<int64_t>(1, in.slots / (in.per > 0 ? in.per : 1));
+  int64_t best_target = 0;
+  double best_span = -1.0;
+  int64_t best_count = in.batch;
+  std::vector<int32_t> sizes;
+  sizes.reserve((size_t)room);
+  const int kNum[6] = {0, 2, 3, 4, 6, 8};  // halves of the slots
+  for (int k = 0; k < 6; ++k) {
+    int64_t target = 0;
+    if (kNum[k] > 0) {
+      target = (2 * total + lanes * kNum[k] - 1) / (lanes * kNum[k]);
+      target = (target + in.tile - 1) / in.tile * in.tile;
+      if (target < in.min_chunk) target = in.min_chunk;
+      if (target >= longest) continue;  // cuts nothing
+    }
+    sizes.clear();
+    int64_t count = 0;
+    bool fits = true;
+    double merge_cost = 0.0;
+    for (int32_t b = 0; b < in.batch && fits; ++b) {
+      const int32_t l = schedule_clamped_len(in.kv_lens[b], in.len_cap);
+      int32_t n, c;
+      schedule_cut(l, target, in, n, c);
+      count += n;
+      fits = count <= room;
+      for (int32_t i = 0; i < n && fits; ++i) sizes.push_back(std::min(c, l - i * c));
+      if (n > 1) merge_cost = in.item_overhead;  // the last chunk of a cut sequence also merges it
+    }
+    if (!fits) continue;
+    const double span = schedule_span(sizes, in) + merge_cost;
+    if (best_span < 0.0 || span < best_span * 0.98) {  // (a finer cut must gain at least 2 %: it costs partial rows)
+      best_span = span;
+      best_target = target;
+      best_count = count;
+    }
+  }
+  // Tables.  Partial slots in sequence order (full_prefix), dispatch longest first.
+  PlanHeader hdr;
+  memset(&hdr, 0, sizeof(hdr));
+  int32_t* kv_len = (int32_t*)(host + w.kv_len);
+  int32_t* full_prefix = (int32_t*)(host + w.full_prefix);
+  int32_t* tail_prefix = (int32_t*)(host + w.tail_prefix);
+  int32_t* num_chunks = (int32_t*)(host + w.num_chunks);
+  SeqChunk* table = (SeqChunk*)(host + w.seq_chunks);
+  int32_t slot = 0;
+  for (int32_t b = 0; b < in.batch; ++b) {
+    const int32_t l = schedule_clamped_len(in.kv_lens[b], in.len_cap);
+    int32_t n, c;
+    schedule_cut(l, best_target, in, n, c);
+    kv_len[b] = l;
+    full_prefix[b] = slot;
+    tail_prefix[b] = 0;
+    num_chunks[b] = n;
+    for (int32_t i = 0; i < n; ++i) {
+      SeqChunk r;
+      r.seq = b;
+      r.chunk = i;
+      r.len = l;
+      r.chunks = n;
+      r.t_begin = i * c;
+      r.t_end = std::min<int64_t>((int64_t)(i + 1) * c, l);
+      r.slot = slot + i;
+      r.pad = 0;
+      table[slot + i] = r;
+    }
+    slot += n;
+  }
+  full_prefix[in.batch] = slot;
+  tail_prefix[in.batch] = 0;
+  std::stable_sort(table, table + slot, [](const SeqChunk& a, const SeqChunk& b) {
+    return a.t_end - a.t_begin > b.t_end - b.t_begin;
+  });
+  hdr.total_full = slot;
+  hdr.total_tail = 0;
+  hdr.chunk_tokens = (int32_t)best_target;
+  hdr.total_items = slot * in.per;
+  memcpy(host + w.header, &hdr, sizeof(hdr));
+  out.chunk_target = (int32_t)best_target;
+  out.total_chunks = best_count;
+  out.predicted_span = best_span;
+  out.bytes = w.seq_chunks + sizeof(SeqChunk) * (size_t)slot;
+  return true;
+}
+
+}  // namespace xllm_hip

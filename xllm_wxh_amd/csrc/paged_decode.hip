@@ -19,6 +19,7 @@
 // the CSR contract of xllm/core/kernels/cuda/cuda_ops_api.h:120-136, and the
 // base-2 partial merge of xllm/core/kernels/cuda/xattention/lse_combine.cu:61-73.
 #include "decode_plan.h"
+#include "decode_schedule.h"
 #include "device_utils.h"
 #include "host_utils.h"
 // the device side, in the order a decode step uses it
@@ -121,6 +122,16 @@ static int fill_params(const xllm_hip_kv_cache* c,
                        size_t workspace_bytes,
                        DecodeParams& p) {
   XLLM_HIP_REQUIRE(c != nullptr && a != nullptr, "cache or args is NULL");
+  // A step whose schedule comes from xllm_hip_paged_decode_plan_host: the kernel and the shape of its work items
+  // follow from sizes alone — never from the host-side lengths, which a captured graph would freeze — and the
+  // schedule is always the stored one, which that call (or the device-side plan) rewrites before every step.
+  xllm_hip_decode_args sized;
+  if (a->host_plan != 0) {
+    sized = *a;
+    sized.max_seq_len = 0;
+    sized.total_kv_len = 0;
+    a = &sized;
+  }
   XLLM_HIP_REQUIRE(c->k_cache != nullptr && c->v_cache != nullptr, "k_cache or v_cache is NULL");
   XLLM_HIP_REQUIRE(c->num_blocks > 0 && c->block_size > 0 && c->num_kv_heads > 0 && c->head_dim > 0,
                    "cache sizes must be positive");
@@ -685,6 +696,76 @@ extern "C" int xllm_hip_paged_decode_plan(const xllm_hip_kv_cache* cache,
   }
   decode_plan_kernel<<<1, 64, 0, (hipStream_t)stream>>>(p);
   return check_launch("decode_plan_kernel");
+}
+
+extern "C" size_t xllm_hip_paged_decode_plan_host_bytes(int32_t batch,
+                                                        int32_t q_per_seq,
+                                                        int32_t num_q_heads,
+                                                        int32_t num_kv_heads,
+                                                        int32_t head_dim) {
+  if (batch < 0 || q_per_seq < 1 || num_q_heads < 1 || num_kv_heads < 1 || head_dim < 1) return 0;
+  return workspace_layout(batch, q_per_seq, num_q_heads, num_kv_heads, head_dim).partial_lse;  // header .. last record
+}
+
+extern "C" int xllm_hip_paged_decode_plan_host(const xllm_hip_kv_cache* cache,
+                                               const xllm_hip_decode_args* args,
+                                               const int32_t* host_kv_lens,
+                                               void* workspace,
+                                               size_t workspace_bytes,
+                                               void* host_staging,
+                                               size_t host_staging_bytes,
+                                               xllm_hip_stream_t stream,
+                                               int64_t* info) {
+  XLLM_HIP_REQUIRE(args != nullptr && args->host_plan != 0, "args->host_plan must be set for a plan made on the host");
+  DecodeParams p;
+  if (int s = fill_params(cache, args, workspace, workspace_bytes, p)) return s;
+  if (info != nullptr) info[0] = info[1] = info[2] = 0;
+  if (p.batch == 0 || p.implicit_plan) return XLLM_HIP_OK;  // a step that is never split needs no schedule
+  XLLM_HIP_REQUIRE(host_kv_lens != nullptr && host_staging != nullptr, "host_kv_lens or host_staging is NULL");
+  XLLM_HIP_REQUIRE(p.arith_chunks == 0 && p.fixed_chunk == 0, "a step with a plan made on the host keeps a stored schedule");
+  const WorkspaceLayout w =
+      workspace_layout(args->batch, args->q_per_seq, args->num_q_heads, cache->num_kv_heads, cache->head_dim);
+  if (host_staging_bytes < w.partial_lse) {
+    return fail(XLLM_HIP_WORKSPACE_TOO_SMALL, "host_staging has %zu bytes, need %zu", host_staging_bytes, w.partial_lse);
+  }
+  const bool quant = cache->dtype == XLLM_HIP_FP8_E4M3 || cache->dtype == XLLM_HIP_INT8;
+  const Variant v = pick_variant(cache, args);
+  HostScheduleInput in;
+  in.kv_lens = host_kv_lens;
+  in.batch = p.batch;
+  in.len_cap = p.len_cap;
+  in.per = p.item_heads * p.row_groups;
+  // Slots of the list schedule: the workgroups that stream at once.  Over a 16-bit cache one 16-row workgroup
+  // per CU already streams at the CU's full rate (see choose_chunk), so its second one adds no slot.
+  in.slots = is_mfma(v) && p.rows <= 16 && !quant && p.target_small < p.target_items ? p.target_items / 2 : p.target_items;
+  in.tile = p.tile_tokens;
+  in.min_chunk = p.min_chunk;
+  in.max_seq_chunks = max_items(p) / in.per;  // what the launch covers
+  in.max_per_seq = p.fused_merge ? 32 : 256;  // what a merge loads in one batch
+  {
+    // four microseconds of a slot's streaming, in tokens (6.5 TB/s over the slots; a token of one kv head is K, V and scales)
+    const double bytes_per_token = 2.0 * cache->head_dim * elem_bytes(cache->dtype) * p.heads_per_item + (quant ? 8.0 : 0.0);
+    in.item_overhead = 4.0 * 6.5e6 / ((double)in.slots * bytes_per_token);
+  }
+  HostScheduleResult r;
+  if (!host_schedule(in, w, (uint8_t*)host_staging, host_staging_bytes, r)) {
+    return fail(XLLM_HIP_INVALID_ARGUMENT, "the step's chunks do not fit the workspace (batch %d, %lld records)", p.batch,
+                (long long)in.max_seq_chunks);
+  }
+  if (info != nullptr) {
+    info[0] = r.chunk_target;
+    info[1] = r.total_chunks;
+    info[2] = (int64_t)r.predicted_span;
+  }
+  if (hipMemcpyAsync(workspace, host_staging, r.bytes, hipMemcpyHostToDevice, (hipStream_t)stream) != hipSuccess) {
+    return fail(XLLM_HIP_RUNTIME_ERROR, "hipMemcpyAsync of the schedule failed");
+  }
+  if (p.fused_merge) {
+    const int ncounters = p.batch * p.num_kv_heads * p.row_groups;
+    decode_zero_counters_kernel<<<(unsigned)((ncounters + 255) / 256), 256, 0, (hipStream_t)stream>>>(p.counters, ncounters);
+    return check_launch("decode_zero_counters_kernel");
+  }
+  return XLLM_HIP_OK;
 }
 
 extern "C" int xllm_hip_paged_decode_run(const xllm_hip_kv_cache* cache,

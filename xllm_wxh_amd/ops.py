@@ -307,12 +307,46 @@ def _decode_args(query, output, output_lse, block_table, seq_lens, csr, q_per_se
     return a, (q3, o3)
 
 
-def _run_decode(desc, args, workspace, device, plan=True, run=True, events=None):
+# Pinned host buffers of the schedules made on the host, two per (device, stream) used in turn; each with the
+# event recorded behind its last copy to the device, which is waited for before the buffer is written again.
+_staging = {}
+
+
+def _plan_host(lib, desc, args, host_kv_lens, wptr, wbytes, device):
+    lens = torch.as_tensor(host_kv_lens, dtype=torch.int32, device="cpu").contiguous()
+    _require(lens.numel() == args.batch, "host_kv_lens has %d entries, batch is %d" % (lens.numel(), args.batch))
+    need = lib.xllm_hip_paged_decode_plan_host_bytes(args.batch, args.q_per_seq, args.num_q_heads, desc.num_kv_heads,
+                                                     desc.head_dim)
+    key = (device.index if device.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(device).cuda_stream)
+    slot = _staging.setdefault(key, {"turn": 0, "buffers": [None, None], "events": [None, None]})
+    i = slot["turn"]
+    slot["turn"] = 1 - i
+    if slot["buffers"][i] is None or slot["buffers"][i].numel() < need:
+        slot["buffers"][i] = torch.empty(max(need, 1 << 16), dtype=torch.uint8, pin_memory=True)
+        slot["events"][i] = torch.cuda.Event()
+    else:
+        slot["events"][i].synchronize()
+    buf = slot["buffers"][i]
+    info = (ctypes.c_int64 * 3)()
+    _lib.check(lib.xllm_hip_paged_decode_plan_host(ctypes.byref(desc), ctypes.byref(args), ctypes.c_void_p(lens.data_ptr()),
+                                                   wptr, wbytes, ctypes.c_void_p(buf.data_ptr()), buf.numel(), _stream(),
+                                                   info))
+    slot["events"][i].record(torch.cuda.current_stream(device))
+    return {"chunk_tokens": int(info[0]), "sequence_chunks": int(info[1]), "predicted_span_tokens": int(info[2])}
+
+
+def _run_decode(desc, args, workspace, device, plan=True, run=True, events=None, host_kv_lens=None):
     lib = _lib.load()
     need = lib.xllm_hip_paged_decode_workspace_bytes(args.batch, args.q_per_seq, args.num_q_heads,
                                                      desc.num_kv_heads, desc.head_dim)
     ws = workspace if workspace is not None else get_workspace(device, need)
     wptr, wbytes = ctypes.c_void_p(ws.data_ptr()), ws.numel() * ws.element_size()
+    if host_kv_lens is not None and plan:
+        # the schedule from the host-side lengths; what follows only runs on it
+        info = _plan_host(lib, desc, args, host_kv_lens, wptr, wbytes, device)
+        plan = False
+        if not run:
+            return info
     if events is not None:
         # (ev_begin, ev_end): raw hipEvent_t handles recorded around the attention kernel
         if plan:
@@ -333,7 +367,7 @@ def batch_decode(query, k_cache, output, block_table, seq_lens, v_cache=None, ou
                  alibi_slope=None, mask=None, compute_dtype="float", max_seq_len=0, window_size_left=-1,
                  window_size_right=-1, scale=1.0, return_lse=False, kv_cache_quant_bit_size=-1, *,
                  q_per_seq=None, kv_layout="HND", workspace=None, plan=True, run=True, events=None,
-                 total_kv_len=0, q_indptr=None):
+                 total_kv_len=0, q_indptr=None, host_plan=False, host_kv_lens=None):
     """Paged decode in the block_table form; positional arguments as in
     xllm::kernel::mlu::batch_decode (xllm/core/kernels/mlu/mlu_ops_api.h:126-145).
 
@@ -345,7 +379,11 @@ def batch_decode(query, k_cache, output, block_table, seq_lens, v_cache=None, ou
     host-side sum of the kv lengths, AttentionMetadata.total_kv_len in the reference; together with
     max_seq_len it lets the library drop the merge launch when no sequence needs splitting),
     q_indptr (int32 [batch + 1]: sequences with different numbers of query tokens, the q_cu_seq_lens of
-    a chunked-prefill or mixed step; q_per_seq is then the largest count, max_query_len).
+    a chunked-prefill or mixed step; q_per_seq is then the largest count, max_query_len),
+    host_plan (xllm_hip_decode_args::host_plan: the kernel and its work items follow from sizes alone and the
+    schedule always comes from the workspace, so that a captured run serves every step of these sizes) and
+    host_kv_lens (the kv lengths as a host-side sequence of ints: the plan is then made on the host by
+    xllm_hip_paged_decode_plan_host; implies host_plan).
     """
     _require(v_cache is not None, "v_cache is required (MLA-style single-cache decode is outside this path)")
     for name, t in (("q_quant_scale", q_quant_scale), ("out_quant_scale", out_quant_scale),
@@ -364,13 +402,14 @@ def batch_decode(query, k_cache, output, block_table, seq_lens, v_cache=None, ou
     args, _keep = _decode_args(query, output, output_lse if return_lse or output_lse is not None else None,
                                block_table, seq_lens, None, q_per_seq, scale, window_size_left, max_seq_len, desc,
                                total_kv_len, q_indptr)
-    _run_decode(desc, args, workspace, query.device, plan, run, events)
+    args.host_plan = 1 if (host_plan or host_kv_lens is not None) else 0
+    return _run_decode(desc, args, workspace, query.device, plan, run, events, host_kv_lens)
 
 
 def batch_decode_csr(query, k_cache, v_cache, paged_kv_indptr, paged_kv_indices, paged_kv_last_page_len,
                      window_left, sm_scale, output, output_lse=None, *, k_cache_scale=None, v_cache_scale=None,
                      q_per_seq=None, kv_layout="NHD", workspace=None, plan=True, run=True, max_seq_len=0,
-                     total_kv_len=0):
+                     total_kv_len=0, host_plan=False, host_kv_lens=None):
     """Paged decode in the CSR form of xllm::kernel::cuda::batch_decode
     (xllm/core/kernels/cuda/cuda_ops_api.h:120-136; the FlashInfer plan/workspace/uri
     arguments have no counterpart here).  The CUDA backend's cache layout is NHD."""
@@ -378,7 +417,8 @@ def batch_decode_csr(query, k_cache, v_cache, paged_kv_indptr, paged_kv_indices,
     args, _keep = _decode_args(query, output, output_lse, None, None,
                                (paged_kv_indptr, paged_kv_indices, paged_kv_last_page_len), q_per_seq, sm_scale,
                                window_left, max_seq_len, desc, total_kv_len)
-    _run_decode(desc, args, workspace, query.device, plan, run)
+    args.host_plan = 1 if (host_plan or host_kv_lens is not None) else 0
+    return _run_decode(desc, args, workspace, query.device, plan, run, None, host_kv_lens)
 
 
 def decode_variant(query, k_cache, v_cache, block_table, seq_lens, k_cache_quant_scale=None,
@@ -396,13 +436,15 @@ DESCRIBE_FIELDS = ("workgroups", "waves_per_workgroup", "unsplit", "stored_sched
 
 
 def decode_describe(query, k_cache, v_cache, block_table, seq_lens, k_cache_quant_scale=None,
-                    v_cache_quant_scale=None, q_per_seq=None, kv_layout="HND", max_seq_len=0, total_kv_len=0):
+                    v_cache_quant_scale=None, q_per_seq=None, kv_layout="HND", max_seq_len=0, total_kv_len=0,
+                    host_plan=False):
     """How batch_decode would run these tensors (xllm_hip_paged_decode_describe: decided on the host, nothing is
     launched): a dict of DESCRIBE_FIELDS."""
     desc = _cache_desc(k_cache, v_cache, k_cache_quant_scale, v_cache_quant_scale, kv_layout)
     out = torch.empty_like(query)
     args, _keep = _decode_args(query, out, None, block_table, seq_lens, None, q_per_seq, 1.0, -1, max_seq_len, desc,
                                total_kv_len=total_kv_len)
+    args.host_plan = 1 if host_plan else 0
     vals = (ctypes.c_int64 * len(DESCRIBE_FIELDS))()
     _lib.check(_lib.load().xllm_hip_paged_decode_describe(ctypes.byref(desc), ctypes.byref(args), 0, vals,
                                                           len(DESCRIBE_FIELDS)))
