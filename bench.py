@@ -181,6 +181,61 @@ def engine_step_us(torch, w, pools, table, seq_lens, lists, layout, steps, devic
     return (time.perf_counter() - t0) * 1e6 / (replays * layers)
 
 
+def host_plan_graph_us(torch, ops, w, pools, q, out, block_table, seq_lens_t, seq_lens, layout, steps, layers, bound_lens=None):
+    """Graph mode with a plan made on the host before every replay (the reference's
+    CudaGraphPersistentParam::update, xllm/core/runtime/cuda_graph_executor_impl.cpp:586-668): `layers`
+    xllm_hip_paged_decode_run launches (layer i on KV pool i mod pools) captured once with
+    xllm_hip_decode_args::host_plan — at `bound_lens`, other lengths than the replays' when given, as a graph
+    captured for a batch-size bucket is —, then replayed; before each replay xllm_hip_paged_decode_plan_host makes the
+    schedule from the step's host-side lengths, outside the graph.  Returns (microseconds per layer, microseconds of
+    host time per plan call)."""
+    ws = torch.empty(ops.WORKSPACE_BYTES, dtype=torch.uint8, device=q.device)
+    lens_dev = seq_lens_t.clone()
+    quant = pools[0][2] is not None
+
+    def call(i, plan, run, lens=None):
+        k, v, ks, vs = pools[i % len(pools)]
+        return ops.batch_decode(q, k, out, block_table, lens_dev, v, None, None, ks, vs, scale=w.sm_scale, q_per_seq=w.q_per_seq,
+                                kv_layout=layout, kv_cache_quant_bit_size=8 if quant else -1, workspace=ws, plan=plan, run=run,
+                                host_plan=True, host_kv_lens=lens)
+
+    import numpy as np
+    if bound_lens is not None:
+        lens_dev.copy_(torch.from_numpy(np.asarray(bound_lens, np.int32)))
+    call(0, True, True, bound_lens if bound_lens is not None else seq_lens)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            for i in range(layers):
+                call(i, False, True)
+    torch.cuda.current_stream().wait_stream(side)
+    lens_dev.copy_(seq_lens_t)
+    replays = max(3, (steps + layers - 1) // layers)
+    for _ in range(2):
+        call(0, True, False, seq_lens)
+        graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(replays):
+        call(0, True, False, seq_lens)
+        graph.replay()
+    torch.cuda.synchronize()
+    per_layer = (time.perf_counter() - t0) * 1e6 / (replays * layers)
+    # the plan call by itself, on an idle stream (in the loop above it also waits for the copy of the plan before
+    # last, which stands in the stream behind a whole replay)
+    host = 0.0
+    for _ in range(20):
+        torch.cuda.synchronize()
+        h0 = time.perf_counter()
+        call(0, True, False, seq_lens)
+        host += time.perf_counter() - h0
+    torch.cuda.synchronize()
+    return per_layer, host * 1e6 / 20
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -375,6 +430,13 @@ def main():
         engine_no_hints_us = engine_step_us(torch, w, pools, table, seq_lens, lists, args.kv_layout, args.steps, device,
                                             False, args.engine_layers)
 
+    host_plan_us = host_plan_call_us = None
+    if not args.no_engine_step:
+        # captured at the bucket's bounds (every sequence at the longest length), replayed on the step's own lengths
+        bound = np.full(w.batch, int(seq_lens.max()), np.int32)
+        host_plan_us, host_plan_call_us = host_plan_graph_us(torch, ops, w, pools, q, out, block_table, seq_lens_d, seq_lens,
+                                                             args.kv_layout, args.steps, args.engine_layers, bound)
+
     alg_bytes = workloads.algorithmic_bytes(w, seq_lens)
     achieved_gbps = alg_bytes / us_per_step / 1e3
     kern_gbps = alg_bytes / kern_avg_us / 1e3
@@ -448,6 +510,14 @@ def main():
                                   "layers sharing one AttentionMetadata, captured once in a HIP graph and replayed "
                                   "(layer i on pool i mod pools; the schedule is built at layer 0 only); no_hints: "
                                   "metadata without the host-side total_kv_len",
+        "host_plan_graph_us": None if host_plan_us is None else round(host_plan_us, 2),
+        "host_plan_call_us": None if host_plan_call_us is None else round(host_plan_call_us, 1),
+        "host_plan_graph_note": "per layer: engine_layers xllm_hip_paged_decode_run launches captured once in a HIP graph "
+                                "with xllm_hip_decode_args::host_plan at the bucket's bounds (every sequence at the "
+                                "longest length) and replayed on the step's own lengths; before each replay "
+                                "xllm_hip_paged_decode_plan_host makes the schedule from the host-side lengths, outside "
+                                "the graph (host_plan_call_us: host time of that call through the Python binding). "
+                                "Compare with run_us, the eager run with the step's own hints",
         "roofline": {
             "bound": "hbm",
             "kernel": kernel_name,

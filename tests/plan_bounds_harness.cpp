@@ -26,7 +26,7 @@ int harness_max_target_items() { return xllm_hip::kMaxTargetItems; }
 // kv_len / first_slot / num_chunks; returns the number of records, or -1 when the step does not fit.
 // out[0..2]: chunk size the cut was made for, total items of the header, predicted span.
 long long harness_host_schedule(const int* lens, int batch, int len_cap, int per, int slots, int tile, int min_chunk,
-                                long long max_seq_chunks, int max_per_seq, double item_overhead, int q_per_seq,
+                                long long max_seq_chunks, int max_per_seq, double item_overhead, double solo_speedup, int q_per_seq,
                                 int num_q_heads, int num_kv_heads, int head_dim, int* records, int* kv_len,
                                 int* first_slot, int* num_chunks, long long* out) {
   using namespace xllm_hip;
@@ -43,6 +43,9 @@ long long harness_host_schedule(const int* lens, int batch, int len_cap, int per
   in.max_seq_chunks = max_seq_chunks;
   in.max_per_seq = max_per_seq;
   in.item_overhead = item_overhead;
+  in.solo_speedup = solo_speedup;
+  in.merge_base = item_overhead;
+  in.merge_per_chunk = item_overhead * 0.03;
   HostScheduleResult r;
   if (!host_schedule(in, w, host.data(), host.size(), r)) return -1;
   const PlanHeader* hdr = (const PlanHeader*)(host.data() + w.header);

@@ -21,14 +21,14 @@ def harness(tmp_path_factory):
                     os.path.join(REPO, "tests", "plan_bounds_harness.cpp"), "-o", out], check=True)
     lib = ctypes.CDLL(out)
     ip, llp = ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_longlong)
-    lib.harness_host_schedule.argtypes = [ip] + [ctypes.c_int] * 6 + [ctypes.c_longlong, ctypes.c_int, ctypes.c_double] + \
+    lib.harness_host_schedule.argtypes = [ip] + [ctypes.c_int] * 6 + [ctypes.c_longlong, ctypes.c_int, ctypes.c_double, ctypes.c_double] + \
         [ctypes.c_int] * 4 + [ip, ip, ip, ip, llp]
     lib.harness_host_schedule.restype = ctypes.c_longlong
     return lib
 
 
 def schedule(lib, lens, per=8, slots=512, tile=32, min_chunk=512, cap=None, max_per_seq=32, overhead=200.0, len_cap=2**31 - 1,
-             q_per_seq=1, hq=32, hkv=8, d=128):
+             q_per_seq=1, hq=32, hkv=8, d=128, solo=2.0):
     lens = np.ascontiguousarray(lens, np.int32)
     B = len(lens)
     room = 4096 + B
@@ -37,7 +37,7 @@ def schedule(lib, lens, per=8, slots=512, tile=32, min_chunk=512, cap=None, max_
     out = np.zeros(4, np.int64)
     ptr = lambda a: a.ctypes.data_as(ctypes.POINTER(ctypes.c_int))
     n = lib.harness_host_schedule(ptr(lens), B, len_cap, per, slots, tile, min_chunk, cap if cap is not None else room,
-                                  max_per_seq, overhead, q_per_seq, hq, hkv, d, ptr(rec), ptr(kv_len), ptr(first), ptr(cnt),
+                                  max_per_seq, overhead, solo, q_per_seq, hq, hkv, d, ptr(rec), ptr(kv_len), ptr(first), ptr(cnt),
                                   out.ctypes.data_as(ctypes.POINTER(ctypes.c_longlong)))
     return n, rec[:max(n, 0)], kv_len, first, cnt, out
 
@@ -102,9 +102,12 @@ def test_the_cut_follows_the_lengths(harness):
     # equal sequences that fill the slots exactly stay whole
     n, rec, kv_len, first, cnt, out = schedule(harness, [4096] * 64)
     assert n == 64 and out[0] == 0
-    # a small batch is cut for the slots: 8 sequences x 8 heads over 512 slots -> about 8 chunks each
-    n, rec, kv_len, first, cnt, out = schedule(harness, [8192] * 8)
-    assert 4 <= cnt[0] <= 8 and np.all(cnt == cnt[0])
+    # a small batch is cut for the slots: 8 sequences x 8 heads over 512 slots -> a workgroup per CU (4 chunks each)
+    # where one workgroup streams at its CU's full rate, every slot (8 chunks) where it takes two
+    n, rec, kv_len, first, cnt, out = schedule(harness, [8192] * 8, solo=2.0)
+    assert np.all(cnt == 4)
+    n, rec, kv_len, first, cnt, out = schedule(harness, [8192] * 8, solo=1.3)
+    assert np.all(cnt == 8)
     # ragged: a lognormal batch ends within a fifth of the even share of the work
     rng = np.random.default_rng(3)
     lens = np.clip(np.round(rng.lognormal(np.log(8192), 0.8, 48)), 16, 65536).astype(np.int64)

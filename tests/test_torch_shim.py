@@ -629,3 +629,60 @@ def test_schedule_built_at_layer_zero_serves_every_layer(gpu, shim, kv, n):
     with pytest.raises(RuntimeError, match="layer 0"):
         attend(c0, 1)
     md.block_table = other
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kv,n", [("bf16", 1), ("fp8", 2)])
+def test_plan_info_host_plan_eager_and_under_a_graph(gpu, shim, kv, n):
+    """PlanInfo.kv_lens_host (the engine's kv_seq_lens_vec): layer 0 makes the step's schedule on the host
+    (xllm_hip_paged_decode_plan_host) and the later layers run on it; PlanInfo.host_plan alone fixes the kernel and
+    its work items by the sizes, so that two layers captured in a graph — layer 0's device-side plan with them —
+    serve a replay on other lengths.  Against the oracle."""
+    from oracle import paged_kv_oracle as orc
+    from tests.helpers import Case
+
+    print("case shim host plan", kv, n, flush=True)
+    B, Hq, Hkv, D, bs = 6, 32, 8, 128, 16
+    cap = np.full(B, 9000, np.int32)
+    layers = [Case(B, Hq, Hkv, D, bs, cap, n=n, kv=kv, seed=80, value_seed=80 + i) for i in range(2)]
+    c0 = layers[0]
+    seq_lens = c0.seq_lens.clone()
+    outs = [torch.zeros_like(c.q.view(B, n, Hq, D)) for c in layers]
+    info = shim.PlanInfo()
+
+    def forward():
+        for layer_id, (c, out) in enumerate(zip(layers, outs)):
+            info.layer_id = layer_id
+            shim.batch_decode(c.q.view(B, n, Hq, D), c.k_cache, out, c0.block_table, seq_lens, c.v_cache, None, c.k_scale,
+                              c.v_scale, 0, -1, c.scale, False, 8 if c.k_scale is not None else -1, plan_info=info)
+
+    def check(lens):
+        torch.cuda.synchronize()
+        for c, out in zip(layers, outs):
+            ref, _ = orc.paged_decode(c.q_ref, c.k_ref, c.v_ref, c0.table, lens, c.scale, q_per_seq=n)
+            assert float(np.abs(out.float().cpu().numpy().reshape(ref.shape) - ref).max()) <= c.tol
+
+    lens = np.array([9000, 17, 4100, 800, 1, 2500], np.int32)
+    seq_lens.copy_(torch.from_numpy(lens))
+    info.kv_lens_host = lens.tolist()
+    forward()
+    check(lens)
+    # captured: sizes alone decide the kernels, layer 0's plan kernel is part of the graph
+    info.kv_lens_host = []
+    info.host_plan = True
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        forward()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        forward()
+    for lens in (np.array([300, 9000, 9000, 64, 5000, 33], np.int32), np.array([8000, 1, 2, 3, 4, 9000], np.int32)):
+        seq_lens.copy_(torch.from_numpy(lens))
+        for out in outs:
+            out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        check(lens)

@@ -36,6 +36,10 @@ struct HostScheduleInput {
   int64_t max_seq_chunks;  // records and partial rows the workspace holds, and the launch covers
   int32_t max_per_seq;     // chunks a sequence is cut into at most
   double item_overhead;    // fixed cost of a work item, in tokens of streaming (prologue, epilogue, partial rows)
+  double solo_speedup;     // rate of a workgroup that has its CU to itself, against one that shares it (a CU holds
+                           // two slots: over a 16-bit cache one workgroup already streams at the CU's full rate)
+  double merge_base;       // what a step that cuts sequences ends with: the merge of the last one, in tokens ...
+  double merge_per_chunk;  // ... plus this much per chunk of the sequence with the most
 };
 
 struct HostScheduleResult {
@@ -69,12 +73,18 @@ inline void schedule_cut(int32_t len, int64_t target, const HostScheduleInput& i
 
 // Finishing time of the step if its sequence chunks, `per` equal work items each, are handed to `slots` slots
 // longest first.  Items of one sequence chunk start together on `per` slots, so the slots are simulated in
-// groups of `per` (the last group may be narrower; it is treated as a full one: an upper estimate).
+// groups of `per` (the last group may be narrower; it is treated as a full one: an upper estimate).  A step
+// with no more items than slots runs them all at once, the faster the more CUs hold a single workgroup.
 inline double schedule_span(std::vector<int32_t>& sizes, const HostScheduleInput& in) {
   std::sort(sizes.begin(), sizes.end(), std::greater<int32_t>());
   int64_t lanes = in.slots / (in.per > 0 ? in.per : 1);
   if (lanes < 1) lanes = 1;
-  if ((int64_t)sizes.size() <= lanes) return sizes.empty() ? 0.0 : sizes[0] + in.item_overhead;
+  if (sizes.empty()) return 0.0;
+  if ((int64_t)sizes.size() <= lanes) {
+    const double spare = (double)(lanes - (int64_t)sizes.size()) / (0.5 * (double)lanes);
+    const double rate = 1.0 + (in.solo_speedup - 1.0) * (spare < 1.0 ? spare : 1.0);
+    return sizes[0] / rate + in.item_overhead;
+  }
   std::priority_queue<double, std::vector<double>, std::greater<double>> free_at;
   for (int64_t i = 0; i < lanes; ++i) free_at.push(0.0);
   double span = 0.0;
@@ -100,15 +110,15 @@ inline bool host_schedule(const HostScheduleInput& in, const WorkspaceLayout& w,
     total += l;
     longest = l > longest ? l : longest;
   }
-  // Candidate chunk sizes: nothing cut; then the work spread over 1, 1.5, 2, 3 and 4 times the slots.
+  // Candidate chunk sizes: nothing cut; then the work spread over 0.5, 1, 1.5, 2, 3 and 4 times the slots.
   const int64_t lanes = std::max<int64_t>(1, in.slots / (in.per > 0 ? in.per : 1));
   int64_t best_target = 0;
   double best_span = -1.0;
   int64_t best_count = in.batch;
   std::vector<int32_t> sizes;
   sizes.reserve((size_t)room);
-  const int kNum[6] = {0, 2, 3, 4, 6, 8};  // halves of the slots
-  for (int k = 0; k < 6; ++k) {
+  const int kNum[7] = {0, 1, 2, 3, 4, 6, 8};  // halves of the slots
+  for (int k = 0; k < 7; ++k) {
     int64_t target = 0;
     if (kNum[k] > 0) {
       target = (2 * total + lanes * kNum[k] - 1) / (lanes * kNum[k]);
@@ -116,21 +126,33 @@ inline bool host_schedule(const HostScheduleInput& in, const WorkspaceLayout& w,
       if (target < in.min_chunk) target = in.min_chunk;
       if (target >= longest) continue;  // cuts nothing
     }
-    sizes.clear();
+    // (rounding up sequence by sequence may leave a few chunks more than the slots' multiple that was aimed
+    // for, and those few would take a round of their own: the target grows until they are gone)
+    const int64_t aim = kNum[k] > 0 ? std::max<int64_t>(lanes * kNum[k] / 2, in.batch) : in.batch;
     int64_t count = 0;
-    bool fits = true;
-    double merge_cost = 0.0;
+    for (int attempt = 0; attempt < 12; ++attempt) {
+      count = 0;
+      for (int32_t b = 0; b < in.batch; ++b) {
+        int32_t n, c;
+        schedule_cut(schedule_clamped_len(in.kv_lens[b], in.len_cap), target, in, n, c);
+        count += n;
+      }
+      if (kNum[k] == 0 || count <= aim || target >= longest) break;
+      target += std::max<int64_t>(in.tile, target / 32 / in.tile * in.tile);
+    }
+    const bool fits = count <= room;
+    if (fits && (target == best_target && best_span >= 0.0)) continue;  // (the same cut as the best so far)
+    int32_t most = 1;
+    sizes.clear();
     for (int32_t b = 0; b < in.batch && fits; ++b) {
       const int32_t l = schedule_clamped_len(in.kv_lens[b], in.len_cap);
       int32_t n, c;
       schedule_cut(l, target, in, n, c);
-      count += n;
-      fits = count <= room;
-      for (int32_t i = 0; i < n && fits; ++i) sizes.push_back(std::min(c, l - i * c));
-      if (n > 1) merge_cost = in.item_overhead;  // the last chunk of a cut sequence also merges it
+      for (int32_t i = 0; i < n; ++i) sizes.push_back(std::min(c, l - i * c));
+      most = n > most ? n : most;
     }
     if (!fits) continue;
-    const double span = schedule_span(sizes, in) + merge_cost;
+    const double span = schedule_span(sizes, in) + (most > 1 ? in.merge_base + in.merge_per_chunk * most : 0.0);
     if (best_span < 0.0 || span < best_span * 0.98) {  // (a finer cut must gain at least 2 %: it costs partial rows)
       best_span = span;
       best_target = target;

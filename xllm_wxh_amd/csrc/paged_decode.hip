@@ -735,17 +735,22 @@ extern "C" int xllm_hip_paged_decode_plan_host(const xllm_hip_kv_cache* cache,
   in.batch = p.batch;
   in.len_cap = p.len_cap;
   in.per = p.item_heads * p.row_groups;
-  // Slots of the list schedule: the workgroups that stream at once.  Over a 16-bit cache one 16-row workgroup
-  // per CU already streams at the CU's full rate (see choose_chunk), so its second one adds no slot.
-  in.slots = is_mfma(v) && p.rows <= 16 && !quant && p.target_small < p.target_items ? p.target_items / 2 : p.target_items;
+  in.slots = p.target_items;  // the workgroups the GPU holds at once
   in.tile = p.tile_tokens;
   in.min_chunk = p.min_chunk;
   in.max_seq_chunks = max_items(p) / in.per;  // what the launch covers
   in.max_per_seq = p.fused_merge ? 32 : 256;  // what a merge loads in one batch
   {
-    // four microseconds of a slot's streaming, in tokens (6.5 TB/s over the slots; a token of one kv head is K, V and scales)
+    // Costs in tokens of a slot's streaming (6.5 TB/s over the slots; a token of one kv head is K, V and scales):
+    // four microseconds per work item; a step that cuts sequences ends with a merge of five microseconds and
+    // 0.15 per chunk.  A CU holds two workgroups of the 16-row kernel: over a 16-bit cache one of them alone
+    // already streams at the CU's full rate, over a 1-byte cache at about two thirds of it (see choose_chunk).
     const double bytes_per_token = 2.0 * cache->head_dim * elem_bytes(cache->dtype) * p.heads_per_item + (quant ? 8.0 : 0.0);
-    in.item_overhead = 4.0 * 6.5e6 / ((double)in.slots * bytes_per_token);
+    const double tokens_per_us = 6.5e6 / ((double)in.slots * bytes_per_token);
+    in.item_overhead = 4.0 * tokens_per_us;
+    in.merge_base = 5.0 * tokens_per_us;
+    in.merge_per_chunk = 0.15 * tokens_per_us;
+    in.solo_speedup = !is_mfma(v) || p.rows > 16 ? 1.0 : quant ? 1.3 : 2.0;
   }
   HostScheduleResult r;
   if (!host_schedule(in, w, (uint8_t*)host_staging, host_staging_bytes, r)) {

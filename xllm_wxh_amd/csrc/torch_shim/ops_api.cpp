@@ -1,7 +1,9 @@
 #include "ops_api.h"
 
 #include <c10/hip/HIPStream.h>
+#include <hip/hip_runtime_api.h>
 
+#include <algorithm>
 #include <map>
 #include <mutex>
 #include <utility>
@@ -229,6 +231,20 @@ torch::Tensor decode_workspace(const torch::Device& device, xllm_hip_stream_t st
 
 namespace {
 
+// Pinned host buffers of the schedules made on the host, two per (device, stream) used in turn, each with the
+// event recorded behind its last copy to the device.
+struct HostStaging {
+  torch::Tensor buffer[2];
+  hipEvent_t event[2] = {nullptr, nullptr};
+  int turn = 0;
+};
+HostStaging& host_staging(const torch::Device& device, xllm_hip_stream_t stream) {
+  static std::mutex mu;
+  static std::map<std::pair<int, xllm_hip_stream_t>, HostStaging> all;
+  std::lock_guard<std::mutex> lock(mu);
+  return all[{(int)device.index(), stream}];
+}
+
 // What a schedule depends on (FNV-1a over the fields): a later layer must present the same.
 uint64_t plan_key(const xllm_hip_kv_cache& c, const xllm_hip_decode_args& a) {
   const uint64_t fields[] = {(uint64_t)a.batch,
@@ -245,6 +261,7 @@ uint64_t plan_key(const xllm_hip_kv_cache& c, const xllm_hip_decode_args& a) {
                              (uint64_t)(uintptr_t)a.q_indptr,
                              (uint64_t)a.max_seq_len,
                              (uint64_t)a.total_kv_len,
+                             (uint64_t)a.host_plan,
                              (uint64_t)c.dtype,
                              (uint64_t)c.num_kv_heads,
                              (uint64_t)c.head_dim,
@@ -276,9 +293,33 @@ void run_decode(const xllm_hip_kv_cache& cache, xllm_hip_decode_args& a, const t
     return;
   }
   TORCH_CHECK(plan->layer_id != -1, "Need to set layer_id to PlanInfo.");
+  a.host_plan = plan->host_plan || !plan->kv_lens_host.empty() ? 1 : 0;
   const uint64_t key = plan_key(cache, a);
   if (plan->layer_id == 0) {
-    check_status(xllm_hip_paged_decode_plan(&cache, &a, ws.data_ptr(), (size_t)ws.numel(), stream));
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    (void)hipStreamIsCapturing((hipStream_t)stream, &capturing);
+    if (!plan->kv_lens_host.empty() && capturing == hipStreamCaptureStatusNone) {
+      TORCH_CHECK((int64_t)plan->kv_lens_host.size() == a.batch, "kv_lens_host has ", plan->kv_lens_host.size(),
+                  " entries, the step has ", a.batch, " sequences");
+      HostStaging& st = host_staging(q3.device(), stream);
+      const size_t bytes = xllm_hip_paged_decode_plan_host_bytes(a.batch, a.q_per_seq, a.num_q_heads, cache.num_kv_heads,
+                                                                 cache.head_dim);
+      const int turn = st.turn;
+      st.turn = 1 - turn;
+      if (!st.buffer[turn].defined() || (size_t)st.buffer[turn].numel() < bytes) {
+        st.buffer[turn] = torch::empty({(int64_t)std::max<size_t>(bytes, 1 << 16)},
+                                       torch::TensorOptions().dtype(torch::kUInt8).pinned_memory(true));
+        if (st.event[turn] == nullptr) TORCH_CHECK(hipEventCreateWithFlags(&st.event[turn], hipEventDisableTiming) == hipSuccess);
+      } else {
+        TORCH_CHECK(hipEventSynchronize(st.event[turn]) == hipSuccess);  // its last copy to the device has run
+      }
+      check_status(xllm_hip_paged_decode_plan_host(&cache, &a, plan->kv_lens_host.data(), ws.data_ptr(), (size_t)ws.numel(),
+                                                   st.buffer[turn].data_ptr(), (size_t)st.buffer[turn].numel(), stream,
+                                                   nullptr));
+      TORCH_CHECK(hipEventRecord(st.event[turn], (hipStream_t)stream) == hipSuccess);
+    } else {
+      check_status(xllm_hip_paged_decode_plan(&cache, &a, ws.data_ptr(), (size_t)ws.numel(), stream));
+    }
     plan->workspace = ws.data_ptr();
     plan->key = key;
   } else {

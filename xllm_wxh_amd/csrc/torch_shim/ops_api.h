@@ -10,6 +10,7 @@
 #include <torch/torch.h>
 
 #include <optional>
+#include <vector>
 #include <string>
 
 #include "param.h"
@@ -38,10 +39,18 @@ namespace hip {
 // xllm/core/layers/cuda/flashinfer_planinfo.cpp:252-253).  The schedule depends on the lengths, the
 // block lists' addresses and the sizes, not on q, out or the cache's contents; `key` records what
 // it was built for, and a later layer whose inputs differ is refused.
+// host_plan (no counterpart in the reference, whose plan is always made on the host): the kernel and its work
+// items follow from the step's sizes alone and the schedule always comes from the workspace
+// (xllm_hip_decode_args::host_plan), so that a forward captured in a graph serves later steps of other lengths:
+// captured, layer 0's device-side plan is part of the graph and reads the lengths of each replay.  kv_lens_host,
+// if not empty (the engine's kv_seq_lens_vec, xllm/core/framework/model/model_input_params.h:341), makes layer 0
+// plan on the host instead (xllm_hip_paged_decode_plan_host) when the stream is not being captured.
 struct PlanInfo {
   int32_t layer_id = -1;
   const void* workspace = nullptr;  // where layer 0 left the schedule
   uint64_t key = 0;
+  bool host_plan = false;
+  std::vector<int32_t> kv_lens_host;
 };
 
 // Argument list of xllm::kernel::mlu::batch_decode (xllm/core/kernels/mlu/mlu_ops_api.h:126-145).

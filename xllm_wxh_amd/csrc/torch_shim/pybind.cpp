@@ -1,5 +1,6 @@
 // Python binding of the libtorch host side, so that pytest can drive the C++ operators and the
 // AttentionImpl twin on the GPU box.
+#include <pybind11/stl.h>
 #include <torch/extension.h>
 
 #include "attention.h"
@@ -44,7 +45,9 @@ PYBIND11_MODULE(_xllm_hip_torch, m) {
   m.def("quant_to_paged_cache", &xllm::kernel::quant_to_paged_cache);
   py::class_<xllm::layer::PlanInfo, std::shared_ptr<xllm::layer::PlanInfo>>(m, "PlanInfo")
       .def(py::init<>())
-      .def_readwrite("layer_id", &xllm::layer::PlanInfo::layer_id);
+      .def_readwrite("layer_id", &xllm::layer::PlanInfo::layer_id)
+      .def_readwrite("host_plan", &xllm::layer::PlanInfo::host_plan)
+      .def_readwrite("kv_lens_host", &xllm::layer::PlanInfo::kv_lens_host);
   m.def("batch_decode",
         [](const torch::Tensor& query, const torch::Tensor& k_cache, torch::Tensor output,
            const torch::Tensor& block_table, const torch::Tensor& seq_lens, const std::optional<torch::Tensor>& v_cache,
