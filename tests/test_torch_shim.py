@@ -155,6 +155,21 @@ def test_cpp_ops_match_python_ops(gpu, shim):
                           torch.from_numpy(indices).to(gpu), torch.from_numpy(last).to(gpu), -1, case.scale, out_c)
     torch.cuda.synchronize()
     assert torch.equal(out_c, ref)
+    # ... and over a quantised cache (fp8 KV is what the CUDA-shaped caller anticipates,
+    # xllm/core/kernels/cuda/utils.cpp:275-293): scales in the same NHD shape
+    for kv in ("fp8", "int8"):
+        cq = Case(3, 32, 8, 128, 16, [500, 33, 2000], kv=kv, seed=42)
+        want, _ = cq.oracle()
+        lists = [cq.table[i, : (int(L) + 15) // 16] for i, L in enumerate(cq.lens)]
+        indptr, indices, last = orc.build_paged_kv_csr(lists, cq.lens, 16)
+        out_q = torch.full_like(cq.q, float("nan"))
+        shim.batch_decode_csr(cq.q, cq.k_cache.permute(0, 2, 1, 3).contiguous(), cq.v_cache.permute(0, 2, 1, 3).contiguous(),
+                              torch.from_numpy(indptr).to(gpu), torch.from_numpy(indices).to(gpu),
+                              torch.from_numpy(last).to(gpu), -1, cq.scale, out_q,
+                              k_cache_scale=cq.k_scale.permute(0, 2, 1).contiguous(),
+                              v_cache_scale=cq.v_scale.permute(0, 2, 1).contiguous())
+        torch.cuda.synchronize()
+        assert float(np.abs(out_q.float().cpu().numpy() - want).max()) <= cq.tol
 
 
 @pytest.mark.gpu

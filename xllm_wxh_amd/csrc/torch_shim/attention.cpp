@@ -156,14 +156,18 @@ void AttentionImpl::decoder_forward(const AttentionMetadata& attn_metadata, torc
                                     attn_metadata.total_kv_len, attn_metadata.plan_info.get());
   } else {
     TORCH_CHECK(attn_metadata.paged_kv_indptr.defined(), "neither block_table nor the CSR arrays are set");
-    TORCH_CHECK(!k_cache_scale.has_value(), "the CSR form serves unquantised caches");
     torch::Tensor q3 = query.view({-1, num_heads_, head_size_});
     torch::Tensor o3 = output.view({-1, num_heads_, head_size_});
-    // the CSR entry point takes the CUDA backend's NHD shape: hand it the NHD view of our HND cache
+    // the CSR entry point takes the CUDA backend's NHD shape: hand it the NHD view of our HND cache (and scales)
+    std::optional<torch::Tensor> ks, vs;
+    if (k_cache_scale.has_value()) {
+      ks = k_cache_scale->permute({0, 2, 1});
+      vs = v_cache_scale->permute({0, 2, 1});
+    }
     xllm::kernel::hip::batch_decode_csr(q3, k_cache.permute({0, 2, 1, 3}), v_cache.permute({0, 2, 1, 3}),
                                         attn_metadata.paged_kv_indptr, attn_metadata.paged_kv_indices,
                                         attn_metadata.paged_kv_last_page_len, sliding_window_, scale_, o3, output_lse,
-                                        attn_metadata.plan_info.get());
+                                        attn_metadata.plan_info.get(), ks, vs);
   }
 }
 

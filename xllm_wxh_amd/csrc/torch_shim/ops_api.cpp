@@ -470,10 +470,17 @@ void batch_decode_csr(torch::Tensor query,
                       double sm_scale,
                       torch::Tensor output,
                       std::optional<torch::Tensor>& output_lse,
-                      PlanInfo* plan_info) {
-  // NHD [blocks, block_size, Hkv, D] -> logical [blocks, Hkv, block_size, D] view
-  const xllm_hip_kv_cache cache =
-      make_cache(k_cache.permute({0, 2, 1, 3}), v_cache.permute({0, 2, 1, 3}), std::nullopt, std::nullopt);
+                      PlanInfo* plan_info,
+                      const std::optional<torch::Tensor>& k_cache_scale,
+                      const std::optional<torch::Tensor>& v_cache_scale) {
+  TORCH_CHECK(k_cache_scale.has_value() == v_cache_scale.has_value(), "k_cache_scale and v_cache_scale come together");
+  // NHD [blocks, block_size, Hkv, D] -> logical [blocks, Hkv, block_size, D] view (scales likewise)
+  std::optional<torch::Tensor> ks, vs;
+  if (k_cache_scale.has_value()) {
+    ks = k_cache_scale->permute({0, 2, 1});
+    vs = v_cache_scale->permute({0, 2, 1});
+  }
+  const xllm_hip_kv_cache cache = make_cache(k_cache.permute({0, 2, 1, 3}), v_cache.permute({0, 2, 1, 3}), ks, vs);
   xllm_hip_decode_args a{};
   fill_q_out(a, query, output, 1);
   a.sm_scale = (float)sm_scale;

@@ -115,7 +115,11 @@ void batch_decode_csr(torch::Tensor query,
                       double sm_scale,
                       torch::Tensor output,
                       std::optional<torch::Tensor>& output_lse,
-                      PlanInfo* plan_info = nullptr);
+                      PlanInfo* plan_info = nullptr,
+                      // a quantised cache (fp8 KV is what the CUDA-shaped caller anticipates,
+                      // xllm/core/kernels/cuda/utils.cpp:275-293): fp32 scales [blocks, block_size, Hkv]
+                      const std::optional<torch::Tensor>& k_cache_scale = std::nullopt,
+                      const std::optional<torch::Tensor>& v_cache_scale = std::nullopt);
 
 // xllm::kernel::cuda::fused_qk_norm_rope (xllm/core/kernels/cuda/cuda_ops_api.h:227-241): per-head RMSNorm
 // and rotary embedding of the q and k heads of the fused buffer, in place.

@@ -65,11 +65,15 @@ PYBIND11_MODULE(_xllm_hip_torch, m) {
         py::arg("plan_info") = nullptr);
   m.def("batch_decode_csr",
         [](torch::Tensor query, torch::Tensor k_cache, torch::Tensor v_cache, torch::Tensor indptr, torch::Tensor indices,
-           torch::Tensor last_page_len, int64_t window_left, double sm_scale, torch::Tensor output) {
+           torch::Tensor last_page_len, int64_t window_left, double sm_scale, torch::Tensor output,
+           std::optional<torch::Tensor> k_cache_scale, std::optional<torch::Tensor> v_cache_scale) {
           std::optional<torch::Tensor> lse = std::nullopt;
           xllm::kernel::hip::batch_decode_csr(query, k_cache, v_cache, indptr, indices, last_page_len, window_left,
-                                              sm_scale, output, lse);
-        });
+                                              sm_scale, output, lse, nullptr, k_cache_scale, v_cache_scale);
+        },
+        py::arg("query"), py::arg("k_cache"), py::arg("v_cache"), py::arg("paged_kv_indptr"), py::arg("paged_kv_indices"),
+        py::arg("paged_kv_last_page_len"), py::arg("window_left"), py::arg("sm_scale"), py::arg("output"),
+        py::arg("k_cache_scale") = std::nullopt, py::arg("v_cache_scale") = std::nullopt);
 
   py::class_<KVCache>(m, "KVCache")
       .def(py::init<>())
