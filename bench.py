@@ -653,13 +653,20 @@ def aux_kernels(torch, ops, device):
                            "frac_of_mfma_peak": round(flops2 / us2 / 1e6 / 2500.0, 3),
                            "note": "causal: flops of the visible part only"})
     del q2, out2
-    us = timed(lambda: ops.batch_decode(q, kq, out, table, lens, vq, None, None, ksc, vsc, scale=D ** -0.5, q_per_seq=n,
-                                        q_indptr=q_indptr, max_seq_len=L, total_kv_len=B * L,
-                                        kv_cache_quant_bit_size=8), n=10)
-    res["entries"].append({"kernel": "chunked prefill over an int8 cache in place (128-row kernel for 1-byte caches), 4 x 512 tokens on a 3584-token prefix",
+    def int8_in_place():
+        ops.batch_decode(q, kq, out, table, lens, vq, None, None, ksc, vsc, scale=D ** -0.5, q_per_seq=n,
+                         q_indptr=q_indptr, max_seq_len=L, total_kv_len=B * L, kv_cache_quant_bit_size=8)
+
+    us = timed(int8_in_place, n=10)
+    res["entries"].append({"kernel": "chunked prefill over an int8 cache in place (256-row kernel for 1-byte caches), 4 x 512 tokens on a 3584-token prefix",
                            "us": round(us, 1), "tflops": round(flops / us / 1e6, 1),
                            "frac_of_mfma_peak": round(flops / us / 1e6 / 2500.0, 3),
-                           "note": "every 128 query rows stream the sequence's K/V bytes and convert them to fp16 tiles in LDS again"})
+                           "note": "every 256 query rows stream the sequence's K/V bytes and convert them to fp16 tiles in LDS again"})
+    with ops.option("prefill_kernel", 1):
+        us128 = timed(int8_in_place, n=10)
+    res["entries"].append({"kernel": "the same through the 128-row kernel for 1-byte caches (XLLM_HIP_OPTION_PREFILL_KERNEL = 1)",
+                           "us": round(us128, 1), "tflops": round(flops / us128 / 1e6, 1),
+                           "frac_of_mfma_peak": round(flops / us128 / 1e6 / 2500.0, 3), "note": ""})
     # speculative verify with 64 query rows per kv head (64 q heads, 8 draft tokens)
     B, n, L, Hq2 = 32, 8, 8192, 64
     q = torch.randn(B * n, Hq2, D, device=device, dtype=torch.bfloat16, generator=gen)

@@ -217,11 +217,11 @@ static int fill_params(const xllm_hip_kv_cache* c,
                     : (p.rows > kPrefillMinRows && variant != kMfmaD256 && (!quant || variant == kMfmaD128))
                         ? kPrefillRowsPerItem
                         : kMaxRowsPerItem;
-  // More rows than one such item over a 16-bit cache: 256 rows per item, eight waves in two groups that
-  // alternate between their matrix and softmax phases (prefill_pingpong_d128_kernel).
+  // More rows than one such item: 256 rows per item, eight waves in two groups that alternate between their
+  // matrix and softmax phases (prefill_pingpong_d128_kernel; prefill_pingpong_quant_d128_kernel over a 1-byte cache).
   p.prefill_opts = (int32_t)option(XLLM_HIP_OPTION_PREFILL_KERNEL);
   // (head_dim 128: at head_dim 64 a tile is 64 tokens, and its scores and weights do not fit that kernel's registers)
-  if (p.rows_per_item == kPrefillRowsPerItem && p.rows > kPrefillRowsPerItem && !quant && variant == kMfmaD128 &&
+  if (p.rows_per_item == kPrefillRowsPerItem && p.rows > kPrefillRowsPerItem && variant == kMfmaD128 &&
       (p.prefill_opts & 1) == 0) {
     p.rows_per_item = kPrefillWideRows;
   }
@@ -519,6 +519,7 @@ template <int KV_DT, int TOK>
 static void launch_mfma_tok(const DecodeParams& p, unsigned grid, hipStream_t st) {
   if (p.rows_per_item == kPrefillWideRows) {
     if constexpr (!quant_of(KV_DT) && TOK == 1) prefill_pingpong_d128_kernel<KV_DT, TOK><<<grid, 512, 0, st>>>(p);
+    if constexpr (quant_of(KV_DT) && TOK == 1) prefill_pingpong_quant_d128_kernel<KV_DT><<<grid, 512, 0, st>>>(p);
   } else if (p.rows_per_item == kPrefillRowsPerItem) {
     if constexpr (!quant_of(KV_DT) && TOK != 0) prefill_mfma_d128_kernel<KV_DT, TOK><<<grid, 256, 0, st>>>(p);
     if constexpr (quant_of(KV_DT) && TOK == 1) prefill_quant_d128_kernel<KV_DT><<<grid, 256, 0, st>>>(p);

@@ -426,4 +426,351 @@ __global__ void __launch_bounds__(512, 2) prefill_pingpong_d128_kernel(DecodePar
   finish_item<KV_DT, TOK, 1>(p, it, rt[1], xch, 0, lds_ml, wave, wave, 0, lane, 2 * wave + 1);
 }
 
+// The same over a 1-byte cache (head_dim 128): the two-phase form of prefill_quant_d128_kernel.  A tile's bytes go
+// from global memory straight into a raw LDS buffer (one 16-byte load per lane and tile: lanes 0-31 the wave's four
+// rows of K, lanes 32-63 its four rows of V; one 4-byte load for their fp32 scales), four raw buffers rotate, and
+// the wave that fetched them converts them — it reads back exactly the bytes it fetched — into one of three
+// converted tiles in the layout the MFMA operand reads expect, with the per-token factors of the softmax (see
+// QuantPrefillLoader::convert).  The conversion is vector work and belongs to the softmax phase: in the softmax
+// phase of tile t the first group converts its rows of tile t + 1, the second group, whose matrix phase of that
+// tile comes a phase later but whose softmax phase of tile t comes after the first group has begun to read it,
+// those of tile t + 2.  Tile t + 1 is thus whole before barrier 2t + 2, behind which it is first read, and its
+// buffer's last occupant, tile t - 2, was last read before barrier 2t.  The three converted tiles are one LDS
+// array and the loop is unrolled over them: their offsets are immediates of the LDS instructions.
+constexpr int kPingPongRawTile = 8 * (1024 + 256);  // per wave: 512 bytes of K, 512 of V, a 256-byte scale load
+
+template <int KV_DT>
+struct PingPongQuantLoader {
+  int wave, lane;
+  uint32_t kv_off;  // byte offset of this lane's 16 bytes from the first of the wave's rows (K and V alike)
+  uint32_t sc_off;  // byte offset of this lane's scale from the scale of the wave's first token
+
+  // Row (of the wave's four) and 16-byte chunk of the row that this lane fetches and converts: lanes in quads, as
+  // in QuantPrefillLoader::row_chunk.  (Formed where they are used: two registers fewer through the loop.)
+  __device__ inline void row_chunk(int& row4, int& chunk) const {
+    const int l5 = RowTile<KV_DT, 1>::opaque(lane) & 31;
+    chunk = 4 * ((l5 >> 3) & 1) + (l5 & 3);
+    row4 = 2 * (l5 >> 4) + ((l5 >> 2) & 1);
+  }
+  __device__ inline void init(const DecodeParams& p, int wave_, int lane_) {
+    wave = wave_;
+    lane = lane_;
+    int row4, chunk;
+    row_chunk(row4, chunk);
+    kv_off = (uint32_t)(row4 * p.stride_slot + chunk * 16);
+    sc_off = (uint32_t)((lane & 3) * p.sc_stride_slot * 4);
+  }
+  // Loads of the wave's rows of the tile starting at token tb into `raw` (in flight on return).
+  __device__ inline void issue(const DecodeParams& p, const Item& it, int tb, int blk, uint8_t* raw) const {
+    const HalfBase b = half_base(p, it, tb + 4 * wave, blk);
+    const uint8_t* kv = (lane < 32 ? p.k_cache : p.v_cache) + b.elem + kv_off;
+    const uint8_t* sc = (const uint8_t*)(((lane & 4) ? p.v_scale : p.k_scale) + b.scale) + sc_off;
+    const uint32_t l = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)(raw + 1280 * wave);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(kv), "s"(l));
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" : : "v"(sc), "s"(l + 1024));
+  }
+  // What a lane holds of a raw tile between reading it back and converting it.
+  struct Raw {
+    u32x4 bytes;  // its 16 bytes of a K or V row
+    float sc;     // lanes 0-3: the K scales of the wave's four tokens, lanes 4-7: their V scales
+    float kfac;   // the factor of the K scales (LDS_SCALE: it is kept in LDS, see the kernel)
+  };
+  template <bool LDS_SCALE>
+  __device__ inline Raw fetch(const uint8_t* raw, float scale_log2, const float* lds_scale) const {
+    Raw r;
+    r.bytes = *(const u32x4*)(raw + 1280 * wave + lane * 16);
+    r.sc = *(const float*)(raw + 1280 * wave + 1024 + (lane & 7) * 4);
+    r.kfac = LDS_SCALE ? *lds_scale : scale_log2;
+    return r;
+  }
+  // The wave's rows of the tile at tb: converted (K, V, per-token factors) into `conv`.
+  template <bool MASKED>
+  __device__ inline void store(const Raw& rw, uint8_t* conv, int tb, int len) const {
+    int row4, chunk;
+    row_chunk(row4, chunk);
+    const int row = 4 * wave + row4;
+    u32x4 lo, hi;
+    dequant16<KV_DT>(rw.bytes, lo, hi);
+    uint32_t off = kLdsK + swz_k(row, 2 * chunk);
+    if (lane >= 32) {
+      if constexpr (kv_of(KV_DT) == XLLM_HIP_INT8) {  // 1152 + x -> x, exact in fp16 (see QuantPrefillLoader::convert)
+        lo = __builtin_bit_cast(u32x4, __builtin_bit_cast(f16x8, lo) - (_Float16)kInt8Offset);
+        hi = __builtin_bit_cast(u32x4, __builtin_bit_cast(f16x8, hi) - (_Float16)kInt8Offset);
+      }
+      if (MASKED && tb + row >= len) lo = hi = u32x4{0, 0, 0, 0};
+      off = kLdsV + swz_v(row, 2 * chunk);
+    }
+    *(u32x4*)(conv + off) = lo;
+    *(u32x4*)(conv + (off ^ 16)) = hi;
+    if (lane < 8) {
+      const int t = 4 * wave + (lane & 3);  // token of the tile
+      const bool is_v = lane >= 4;
+      const float vs = fmaxf(rw.sc, 0x1p-100f);
+      float a = is_v ? __builtin_amdgcn_logf(vs) : rw.sc * rw.kfac;
+      float r = __builtin_amdgcn_rcpf(vs);
+      if (MASKED && tb + t >= len) a = r = 0.0f;
+      *(float*)(conv + kLdsSc + (is_v ? 128 : 0) + t * 4) = a;
+      if (is_v) *(float*)(conv + kLdsSc + 256 + t * 4) = r;
+    }
+  }
+};
+
+template <int KV_DT>
+__global__ void __launch_bounds__(512, 2) prefill_pingpong_quant_d128_kernel(DecodeParams p) {
+  static_assert(quant_of(KV_DT), "16-bit caches need no conversion: prefill_pingpong_d128_kernel");
+  constexpr int kT = 32, kConv = 3, kRaw = 4;
+  __shared__ __attribute__((aligned(16))) uint8_t lds[kConv * kLdsTile + kRaw * kPingPongRawTile];
+  __shared__ float lds_ml[8 * 16 * 2];
+  __shared__ float lds_q[16];
+  static_assert(8 * 16 * xch_row_bytes(1) <= kConv * kLdsTile + kRaw * kPingPongRawTile, "the end-of-item exchanges must fit");
+  uint8_t* const raws = lds + kConv * kLdsTile;
+
+  Item it;
+  if (!decode_item(p, blockIdx.x, it)) return;
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  const bool late = wave >= 4;  // the group that runs one phase behind; waves w and w + 4 share a SIMD
+
+  typedef RowTile<KV_DT, 1, false, false, kv_of(KV_DT) == XLLM_HIP_INT8, false, false> RT;
+  typedef typename RT::Op Op;
+  RT rt[2];
+  int q_exp = 0;
+  if constexpr (RT::kNormItem) {  // one factor for the queries of all eight waves: they share the converted tile's factors
+    lds_q[wave] = fmaxf(RT::wave_q_absmax(p, it, 32 * wave, lane), RT::wave_q_absmax(p, it, 32 * wave + 16, lane));
+    __syncthreads();
+    float m = lds_q[0];
+#pragma unroll
+    for (int i = 1; i < 8; ++i) m = fmaxf(m, lds_q[i]);
+    q_exp = RT::norm_exponent(m);
+    __syncthreads();
+  }
+  rt[0].init(p, it, 32 * wave, lane, q_exp);
+  rt[1].init(p, it, 32 * wave + 16, lane, q_exp);
+  // (the factor of the K scales waits in LDS, a word per wave: no scalar register need hold it through the loop)
+  if constexpr (RT::kNormItem) lds_q[8 + wave] = __builtin_amdgcn_ldexpf(p.scale_log2, q_exp);
+  const float* lds_scale = lds_q + 8 + wave;
+
+  const int rows = it.n * p.group;
+  const int r_first = it.rg * p.rows_per_item + 32 * wave;
+  const bool has_rows = r_first < rows;
+  const int r_last = min(r_first + 31, rows - 1);
+  const int lim_first = it.len - (it.n - 1 - r_first / p.group);
+  const int lim_last = has_rows ? it.len - (it.n - 1 - r_last / p.group) : 0;
+  const int lo_first = p.window_left >= 0 ? lim_first - 1 - p.window_left : 0;
+  const int lo_last = p.window_left >= 0 ? lim_last - 1 - p.window_left : 0;
+  const int ri_first = it.rg * p.rows_per_item;
+  const int lim_item = it.len - (it.n - 1 - ri_first / p.group);  // the item's first row sees the tokens below this
+
+  const int w_begin = first_visible_tile(p, it);
+  const int w_end = it.t_end;
+  const int iters = w_end > w_begin ? (w_end - w_begin + kT - 1) / kT : 0;
+  // tiles [0, nfast) take the straight-line form, nfast = 1 + 3k (none under a sliding window)
+  int p1 = lim_item > w_begin ? (lim_item - w_begin) / kT : 0;
+  p1 = p1 < iters ? p1 : iters;
+  const int nfast = p1 >= 1 && p.window_left < 0 ? 1 + (p1 - 1) / kConv * kConv : 0;
+
+  PingPongQuantLoader<KV_DT> ld;
+  ld.init(p, wave, lane);
+  const int mine = 4 * wave;  // first of the tokens this wave fetches, within a tile
+
+  auto barrier = [&]() __attribute__((always_inline)) {
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto conv_tile = [&](auto k) __attribute__((always_inline)) -> uint8_t* { return lds + (decltype(k)::value % kConv) * kLdsTile; };
+
+  typedef typename RT::Scores Scores;
+  typedef Op Weights[RT::kU];
+  Weights pf0, pf1;
+  Op vpre[2];
+  int blk = 0;  // block id of this wave's rows of the tile that is put in flight next
+
+  auto k_fragments = [&](const uint8_t* cur, int c, Op (&kf)[2]) __attribute__((always_inline)) {
+    const uint32_t ko = RT::opaque(rt[0].k_off0) ^ (uint32_t)(c << 6);
+    kf[0] = *(const Op*)(cur + ko);
+    kf[1] = *(const Op*)(cur + ko + 4096);
+  };
+  auto scores_from = [&](const uint8_t* cur, Op (&kf)[2][2], Scores& s0, Scores& s1) __attribute__((always_inline)) {
+    rt[0].scores_init(s0);
+    rt[1].scores_init(s1);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      if (c + 1 < 4) k_fragments(cur, c + 1, kf[(c + 1) & 1]);
+      rt[0].scores_step(c, kf[c & 1][0], kf[c & 1][1], s0);
+      rt[1].scores_step(c, kf[c & 1][0], kf[c & 1][1], s1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  auto scores = [&](const uint8_t* cur, Scores& s0, Scores& s1) __attribute__((always_inline)) {
+    Op kf[2][2];
+    k_fragments(cur, 0, kf[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    scores_from(cur, kf, s0, s1);
+  };
+  auto values_then = [&](const uint8_t* buf, const Weights& w0, const Weights& w1, auto preloaded, const Op (&pre)[2],
+                         auto mid, auto then) __attribute__((always_inline)) {
+    Op vf[3];
+#pragma unroll
+    for (int dt = 0; dt < 2; ++dt) vf[dt] = decltype(preloaded)::value ? pre[dt] : rt[0].v_fragment(buf, dt, RT::opaque(rt[0].v_off0));
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int dt = 0; dt < 8; ++dt) {
+      if (dt + 2 < 8) vf[(dt + 2) % 3] = rt[0].v_fragment(buf, dt + 2, RT::opaque(rt[0].v_off0));
+      if (dt == 2) mid();
+      if (dt == 6) then();
+      rt[0].template accumulate_step<false>(dt, vf[dt % 3], w0, 1.0f);
+      rt[1].template accumulate_step<false>(dt, vf[dt % 3], w1, 1.0f);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  auto values = [&](const uint8_t* buf, const Weights& w0, const Weights& w1) __attribute__((always_inline)) {
+    Op none[2];
+    values_then(buf, w0, w1, std::false_type{}, none, [] {}, [] {});
+  };
+  // Softmax of both row tiles over the converted tile `cur` (its per-token factors live as briefly as they can, as
+  // in attend_pair); the accumulators follow when a reference point moved.
+  auto weights = [&](auto masked, const uint8_t* cur, int tb, const Scores& s0, const Scores& s1, Weights& w0, Weights& w1)
+      __attribute__((always_inline)) {
+    constexpr bool MASKED = decltype(masked)::value;
+    float kscl[RT::kN], lv[RT::kN], rvs[RT::kN];
+    float x0[RT::kN], x1[RT::kN];
+    float alpha0, alpha1;
+    rt[0].load_factor(cur, 0, kscl);
+    rt[0].load_factor(cur, 1, lv);
+    rt[0].template scaled_scores<MASKED>(s0, kscl, lv, tb, p.scale_log2, x0);
+    rt[1].template scaled_scores<MASKED>(s1, kscl, lv, tb, p.scale_log2, x1);
+    __builtin_amdgcn_sched_barrier(0);
+    rt[0].load_factor(cur, 2, rvs);
+    const bool moved0 = rt[0].template weights<MASKED>(x0, rvs, p.scale_log2, w0, alpha0);
+    __builtin_amdgcn_sched_barrier(0);
+    const bool moved1 = rt[1].template weights<MASKED>(x1, rvs, p.scale_log2, w1, alpha1);
+    if (moved0 || moved1) {
+#pragma unroll
+      for (int dt = 0; dt < 8; ++dt) {
+        rt[0].acc[dt] *= alpha0;
+        rt[1].acc[dt] *= alpha1;
+      }
+    }
+  };
+  // In the matrix phase of tile i a wave converts its rows of tile i + 1.  fetch_next, right behind the phase's
+  // barrier: they have landed (the loads of three tiles may still be in flight) and are on their way from the raw
+  // buffer to registers.  store_next, among the phase's MFMAs: converted and written, and the raw buffer takes
+  // the tile four further on.  (`ph`: i modulo the number of converted tiles.)
+  typedef typename PingPongQuantLoader<KV_DT>::Raw Raw;
+  auto fetch_next = [&](int i) __attribute__((always_inline)) -> Raw {
+    __builtin_amdgcn_s_waitcnt(0x0f76);  // vmcnt(6)
+    return ld.template fetch<RT::kNormItem>(raws + ((i + 1) & (kRaw - 1)) * kPingPongRawTile, p.scale_log2, lds_scale);
+  };
+  auto store_next = [&](auto ph, int i, const Raw& rw) __attribute__((always_inline)) {
+    constexpr int PH = decltype(ph)::value;
+    const int tb = w_begin + (i + 1) * kT;
+    uint8_t* conv = lds + ((PH + 1) % kConv) * kLdsTile;
+    if (tb + kT > it.len) {
+      ld.template store<true>(rw, conv, tb, it.len);
+    } else {
+      ld.template store<false>(rw, conv, tb, it.len);
+    }
+    blk = block_of_const(p, it, tb + kRaw * kT + mine);
+    __builtin_amdgcn_sched_barrier(0);  // (the raw bytes are in registers: their buffer may be written)
+    ld.issue(p, it, tb + kRaw * kT, blk, raws + ((i + 1) & (kRaw - 1)) * kPingPongRawTile);
+  };
+
+  auto whole = [&](auto ph, int i) __attribute__((always_inline)) {
+    uint8_t* cur = conv_tile(ph);
+    const int tb = w_begin + i * kT;
+    const bool visible = !(tb >= lim_last || tb + kT <= lo_first);
+    Scores s0, s1;
+    barrier();
+    const Raw rw = fetch_next(i);
+    if (visible) {
+      XLLM_HIP_PINGPONG_SETPRIO(1);
+      scores(cur, s0, s1);
+      XLLM_HIP_PINGPONG_SETPRIO(0);
+    }
+    store_next(ph, i, rw);
+    barrier();
+    if (visible) {
+      Weights w0, w1;
+      if (tb + kT > lim_first || tb < lo_last) {
+        weights(std::true_type{}, cur, tb, s0, s1, w0, w1);
+      } else {
+        weights(std::false_type{}, cur, tb, s0, s1, w0, w1);
+      }
+      values(cur, w0, w1);
+    }
+  };
+  auto pipelined = [&](auto ph, auto first, int i) __attribute__((always_inline)) {
+    constexpr int PH = decltype(ph)::value;
+    uint8_t* cur = conv_tile(ph);
+    const int tb = w_begin + i * kT;
+    Scores s0, s1;
+    barrier();
+    const Raw rw = fetch_next(i);
+    XLLM_HIP_PINGPONG_SETPRIO(1);
+    if constexpr (!decltype(first)::value) {
+      Op kf[2][2];
+      values_then(conv_tile(std::integral_constant<int, PH + kConv - 1>{}), pf0, pf1, std::true_type{}, vpre,
+                  [&]() __attribute__((always_inline)) { store_next(ph, i, rw); },
+                  [&]() __attribute__((always_inline)) { k_fragments(cur, 0, kf[0]); });
+      scores_from(cur, kf, s0, s1);
+    } else {
+      store_next(ph, i, rw);
+      scores(cur, s0, s1);
+    }
+    XLLM_HIP_PINGPONG_SETPRIO(0);
+    barrier();
+    weights(std::false_type{}, cur, tb, s0, s1, pf0, pf1);
+    __builtin_amdgcn_sched_barrier(0);
+    vpre[0] = rt[0].v_fragment(cur, 0, RT::opaque(rt[0].v_off0));
+    vpre[1] = rt[0].v_fragment(cur, 1, RT::opaque(rt[0].v_off0));
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  if (iters > 0) {  // (an item without visible tokens touches no block: its table row may hold anything)
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the queries have arrived (see prefill_pingpong_d128_kernel)
+    ld.issue(p, it, w_begin, block_of_const(p, it, w_begin + mine), raws);
+    ld.issue(p, it, w_begin + kT, block_of_const(p, it, w_begin + kT + mine), raws + kPingPongRawTile);
+    ld.issue(p, it, w_begin + 2 * kT, block_of_const(p, it, w_begin + 2 * kT + mine), raws + 2 * kPingPongRawTile);
+    ld.issue(p, it, w_begin + 3 * kT, block_of_const(p, it, w_begin + 3 * kT + mine), raws + 3 * kPingPongRawTile);
+    // tile 0 is converted before the first barrier (fetch_next(i) and store_next(.., i, ..) handle tile i + 1)
+    {
+      const Raw rw = fetch_next(-1);
+      store_next(std::integral_constant<int, kConv - 1>{}, -1, rw);
+    }
+    if (late) barrier();
+    int i = 0;
+    if (nfast > 0) {
+      pipelined(std::integral_constant<int, 0>{}, std::true_type{}, i);
+      ++i;
+      for (; i + kConv <= nfast; i += kConv) {
+        pipelined(std::integral_constant<int, 1>{}, std::false_type{}, i);
+        pipelined(std::integral_constant<int, 2>{}, std::false_type{}, i + 1);
+        pipelined(std::integral_constant<int, 0>{}, std::false_type{}, i + 2);
+      }
+      values_then(lds, pf0, pf1, std::true_type{}, vpre, [] {}, [] {});  // the last pipelined tile's V^T P^T: that tile is in the first buffer
+    }
+    if (nfast == 0) {
+      whole(std::integral_constant<int, 0>{}, 0);
+      i = 1;
+    }
+    while (i < iters) {
+      whole(std::integral_constant<int, 1>{}, i);
+      if (++i >= iters) break;
+      whole(std::integral_constant<int, 2>{}, i);
+      if (++i >= iters) break;
+      whole(std::integral_constant<int, 0>{}, i);
+      ++i;
+    }
+    if (!late) barrier();
+  }
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): nothing lands in LDS any more
+  __syncthreads();  // all tiles consumed: the buffers become the exchange
+  uint8_t* xch = lds + wave * (16 * xch_row_bytes(1));
+  finish_item<KV_DT, 1, 1>(p, it, rt[0], xch, 0, lds_ml, wave, wave, 0, lane, 2 * wave);
+  __syncthreads();
+  finish_item<KV_DT, 1, 1>(p, it, rt[1], xch, 0, lds_ml, wave, wave, 0, lane, 2 * wave + 1);
+}
+
 }  // namespace xllm_hip
