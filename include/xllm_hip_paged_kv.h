@@ -468,12 +468,12 @@ enum xllm_hip_option {
   XLLM_HIP_OPTION_DECODE_FOUR_WAVE_ITEMS = 5, /* != 0: the 16-row kernel always runs four waves per work item, also
                                                * when the launch has at most one item per CU (where it otherwise
                                                * runs eight) */
-  XLLM_HIP_OPTION_PREFILL_KERNEL = 6, /* bit 0: steps of more than 128 query rows per kv head over a 16-bit cache
-                                       * take the 128-row kernel (four waves per work item) instead of the
-                                       * 256-row one (eight waves in two groups that alternate between their
+  XLLM_HIP_OPTION_PREFILL_KERNEL = 6, /* bit 0: steps of more than 128 query rows per kv head at head_dim 128
+                                       * take the 128-row kernels (four waves per work item) instead of the
+                                       * 256-row ones (eight waves in two groups that alternate between their
                                        * matrix and softmax phases); bit 1: the late group of the 256-row kernel
-                                       * is the odd waves instead of waves 4-7; bit 2: no raised wave priority
-                                       * in its matrix phase */
+                                       * for 16-bit caches is the odd waves instead of waves 4-7 (two waves of
+                                       * different SIMDs: for measurements) */
   XLLM_HIP_OPTION_COUNT = 7
 };
 int xllm_hip_set_option(int32_t which, int64_t value);

@@ -50,7 +50,8 @@ def test_struct_sizes_match_the_header_layout():
     assert _lib.DecodeArgs.block_table.offset == 64
     assert _lib.DecodeArgs.max_seq_len.offset == 120
     assert _lib.DecodeArgs.q_indptr.offset == 136
-    assert ctypes.sizeof(_lib.DecodeArgs) == 144
+    assert _lib.DecodeArgs.host_plan.offset == 144
+    assert ctypes.sizeof(_lib.DecodeArgs) == 152  # (+ 4 bytes of padding)
     # xllm_hip_rope_args: ptr, 2 i64, 6 i32, 2 ptr, f32 + i32, ptr, i64, ptr, 3 i32 (+ 4 bytes of padding)
     assert _lib.RopeArgs.q_weight.offset == 48 and _lib.RopeArgs.cos_sin_cache.offset == 72
     assert _lib.RopeArgs.positions_int32.offset == 104

@@ -320,3 +320,66 @@ def test_256_row_kernel_against_the_128_row_kernel_and_the_oracle(gpu, qdt, bs, 
     d = ops.decode_describe(torch.empty(len(lens) * max(q_counts), c.Hq, c.D, dtype=dt, device=qd.device), c.k_cache, c.v_cache, c.block_table, c.seq_lens,
                             q_per_seq=max(q_counts), kv_layout=layout)
     assert d["waves_per_workgroup"] == 8, d
+
+
+@pytest.mark.parametrize("kv", ["fp8", "int8"])
+@pytest.mark.parametrize("qdt", ["bf16", "fp16"])
+@pytest.mark.parametrize("bs,layout", [(16, "HND"), (128, "NHD")])
+def test_256_row_kernel_over_one_byte_caches(gpu, kv, qdt, bs, layout):
+    """The same over a 1-byte cache: raw bytes and scales reach LDS by DMA and each wave converts its rows of the
+    next tile during its matrix phase, three converted tiles rotating.  Its straight-line loop takes the tiles
+    every row sees in full three at a time after the first: the prefixes put 0, 1, 3, 4, 5, 7 and 30 tiles in
+    front of the causal edge.  Every slot no sequence owns holds bytes that decode to NaN or 127 and a NaN scale.
+    The results match the oracle and the 128-row kernel for 1-byte caches, which converts the same values the
+    same way."""
+    print("case 256-row kernel, 1-byte cache", kv, qdt, bs, layout, flush=True)
+    q_counts = [64, 40, 33, 70, 64, 200, 64, 0, 129, 300]
+    prefix = [0, 32, 3 * 32, 4 * 32 + 5, 5 * 32, 7 * 32 + 31, 30 * 32 + 1, 100, 0, 1000]
+    lens = [p + n for p, n in zip(prefix, q_counts)]
+    c = Case(len(lens), 32, 8, 128, bs, lens, kv=kv, qdt=qdt, layout=layout, seed=43)
+    used = torch.zeros(c.k_cache.size(0), bs, dtype=torch.bool)
+    for b, L in enumerate(lens):
+        for t in range(L):
+            used[c.table[b, t // bs], t % bs] = True
+    mask = (~used).to(c.k_cache.device)
+    for cache in (c.k_cache, c.v_cache):
+        view = cache.view(torch.uint8)
+        (view if layout == "NHD" else view.permute(0, 2, 1, 3))[mask] = 0x7F  # NaN in e4m3fn, 127 in int8
+    for sc in (c.k_scale, c.v_scale):
+        (sc if layout == "NHD" else sc.permute(0, 2, 1))[mask] = float("nan")
+    q_indptr = np.concatenate([[0], np.cumsum(q_counts)]).astype(np.int32)
+    T = int(q_indptr[-1])
+    dt = torch.bfloat16 if qdt == "bf16" else torch.float16
+    q = torch.randn(T, c.Hq, c.D, generator=torch.Generator().manual_seed(79)).to(dt)
+    qd = q.to(c.q.device)
+    refs = {w: orc.paged_decode_ragged(q.float().numpy(), c.k_ref, c.v_ref, c.table, c.lens, q_indptr, c.scale, window_left=w)
+            for w in (-1, 150)}
+    got = {}
+    for name, value in (("rows256", 0), ("rows128", 1)):
+        with ops.option("prefill_kernel", value):
+            for window in (-1, 150):
+                out = torch.full_like(qd, 7.0)
+                lse = torch.full((T, c.Hq), 3.0, dtype=torch.float32, device=qd.device)
+                ops.batch_decode(qd, c.k_cache, out, c.block_table, c.seq_lens, c.v_cache, lse, None, c.k_scale, c.v_scale,
+                                 scale=c.scale, return_lse=True, q_per_seq=max(q_counts), kv_cache_quant_bit_size=8,
+                                 q_indptr=torch.from_numpy(q_indptr).to(qd.device), kv_layout=layout, window_size_left=window)
+                torch.cuda.synchronize()
+                got[name, window] = (out.float().cpu().numpy(), lse.cpu().numpy())
+    for window in (-1, 150):
+        ref, ref_lse = refs[window]
+        o256, l256 = got["rows256", window]
+        o128, l128 = got["rows128", window]
+        assert not np.isnan(o256).any()
+        err = float(np.abs(o256 - ref).max())
+        print("   window %d err %.3e" % (window, err), flush=True)
+        assert err <= 1.2e-2
+        # (bf16 queries become fp16 operands on one power-of-two factor per work item, which the two kernels take
+        # over 256 and over 128 rows: exact either way unless a row lies 2^28 below its item's largest element)
+        assert float(np.abs(o256 - o128).max()) <= 4e-3 and float(np.mean(o256 != o128)) <= 1e-4
+        assert np.allclose(l256, l128, atol=1e-5, equal_nan=True)
+        fin = np.isfinite(ref_lse)
+        assert np.allclose(l256[fin], ref_lse[fin], atol=2e-2)
+    d = ops.decode_describe(torch.empty(len(lens) * max(q_counts), c.Hq, c.D, dtype=dt, device=qd.device), c.k_cache, c.v_cache,
+                            c.block_table, c.seq_lens, q_per_seq=max(q_counts), kv_layout=layout, k_cache_quant_scale=c.k_scale,
+                            v_cache_quant_scale=c.v_scale)
+    assert d["waves_per_workgroup"] == 8, d

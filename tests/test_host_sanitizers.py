@@ -27,10 +27,11 @@ def test_host_code_runs_clean_under_asan_and_ubsan(tmp_path):
     for inc in ce.include_paths() + [os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "include")]:
         cmd += ["-isystem", inc]
     cmd += [os.path.join(REPO, "tests", "host_sanitizer_harness.cpp"), os.path.join(CSRC, "torch_shim", "ops_api.cpp")]
-    lib_dirs = ce.library_paths() + [xbuild.PKG_DIR]
+    # (ops_api.cpp calls the HIP runtime itself: events and pinned memory of the host-side plan's staging buffers)
+    lib_dirs = ce.library_paths() + [xbuild.PKG_DIR, os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "lib")]
     for d in lib_dirs:
         cmd += ["-L" + d, "-Wl,-rpath," + d]
-    cmd += ["-l:" + xbuild.LIB_NAME, "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch", "-o", exe]
+    cmd += ["-l:" + xbuild.LIB_NAME, "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch", "-lamdhip64", "-o", exe]
     build = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     assert build.returncode == 0, build.stdout[-4000:]
     # libtorch keeps a few allocations for the life of the process; leak checking is not the point here

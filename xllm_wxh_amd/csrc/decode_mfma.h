@@ -101,9 +101,6 @@ constexpr bool qf16_of(int kt) { return (kt & kQF16) != 0 || kv_of(kt) == XLLM_H
 constexpr bool quant_of(int kt) { return kv_of(kt) == XLLM_HIP_FP8_E4M3 || kv_of(kt) == XLLM_HIP_INT8; }
 // An int8 cache at head_dim 128 or 256: the K rows stay bytes in LDS and meet the queries in the int8 MFMA
 // (v_mfma_i32_16x16x64_i8); see RowTile.  V is still converted to fp16 for the second MFMA.
-#ifndef XLLM_HIP_ASM_MAX
-#define XLLM_HIP_ASM_MAX 1
-#endif
 #ifndef XLLM_HIP_RAW_K
 #define XLLM_HIP_RAW_K 1
 #endif
@@ -383,22 +380,26 @@ __device__ inline void lane_swap16(float& a, float& b) {
 __device__ inline void lane_swap32(float& a, float& b) {
   asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
 }
-// (the maximum as the instruction alone: fmaxf first brings each operand to canonical form, an operation of its own)
-__device__ inline float max_plain(float a, float b) {
-#if XLLM_HIP_ASM_MAX
-  float r;
-  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
-  return r;
-#else
-  return fmaxf(a, b);
-#endif
+// The maximum over the four lanes that hold a query row's scores.  PLAIN: the maximum as the instruction alone
+// (fmaxf first brings each operand to canonical form, an operation of its own; the same value for operands that
+// are no signalling NaNs).  Only where it pays: it changes the register allocation of the kernels around it.
+template <bool PLAIN>
+__device__ inline float max_of(float a, float b) {
+  if constexpr (PLAIN) {
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+  } else {
+    return fmaxf(a, b);
+  }
 }
+template <bool PLAIN = false>
 __device__ inline float kg_max(float v) {
   float a = v, b = v;
   lane_swap16(a, b);
-  a = b = max_plain(a, b);
+  a = b = max_of<PLAIN>(a, b);
   lane_swap32(a, b);
-  return max_plain(a, b);
+  return max_of<PLAIN>(a, b);
 }
 __device__ inline float kg_sum(float v) {
   float a = v, b = v;

@@ -282,7 +282,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pingpong_d128_kernel(DecodePar
 #pragma unroll
       for (int rr = 0; rr < 4; ++rr) mt = fmaxf(mt, s[0][h][rr]);  // (a chain from -inf: the compiler forms three-input maxima)
     }
-    mt = kg_max(mt) * scale;
+    mt = kg_max<true>(mt) * scale;
     if (__builtin_amdgcn_ballot_w64(fmaxf(r.m_run, mt) > r.m_run + kLazyRescale) != 0) {
       const float m_new = fmaxf(r.m_run, mt);
       const float m_safe = m_new == -INFINITY ? 0.0f : m_new;
@@ -629,20 +629,19 @@ __global__ void __launch_bounds__(512, 2) prefill_pingpong_quant_d128_kernel(Dec
     Op none[2];
     values_then(buf, w0, w1, std::false_type{}, none, [] {}, [] {});
   };
-  // Softmax of both row tiles over the converted tile `cur` (its per-token factors live as briefly as they can, as
-  // in attend_pair); the accumulators follow when a reference point moved.
-  auto weights = [&](auto masked, const uint8_t* cur, int tb, const Scores& s0, const Scores& s1, Weights& w0, Weights& w1)
-      __attribute__((always_inline)) {
+  // Softmax of both row tiles over the converted tile `cur`, whose factors of the K scales and logarithms of the V
+  // scales the caller has read (`kscl`, `lv`; the reciprocals of the V scales are read here, ahead of the
+  // arithmetic that hides their latency); the accumulators follow when a reference point moved.
+  auto weights_with = [&](auto masked, const uint8_t* cur, int tb, const Scores& s0, const Scores& s1, const float (&kscl)[RT::kN],
+                          const float (&lv)[RT::kN], Weights& w0, Weights& w1) __attribute__((always_inline)) {
     constexpr bool MASKED = decltype(masked)::value;
-    float kscl[RT::kN], lv[RT::kN], rvs[RT::kN];
+    float rvs[RT::kN];
     float x0[RT::kN], x1[RT::kN];
     float alpha0, alpha1;
-    rt[0].load_factor(cur, 0, kscl);
-    rt[0].load_factor(cur, 1, lv);
+    rt[0].load_factor(cur, 2, rvs);
     rt[0].template scaled_scores<MASKED>(s0, kscl, lv, tb, p.scale_log2, x0);
     rt[1].template scaled_scores<MASKED>(s1, kscl, lv, tb, p.scale_log2, x1);
     __builtin_amdgcn_sched_barrier(0);
-    rt[0].load_factor(cur, 2, rvs);
     const bool moved0 = rt[0].template weights<MASKED>(x0, rvs, p.scale_log2, w0, alpha0);
     __builtin_amdgcn_sched_barrier(0);
     const bool moved1 = rt[1].template weights<MASKED>(x1, rvs, p.scale_log2, w1, alpha1);
@@ -653,6 +652,13 @@ __global__ void __launch_bounds__(512, 2) prefill_pingpong_quant_d128_kernel(Dec
         rt[1].acc[dt] *= alpha1;
       }
     }
+  };
+  auto weights = [&](auto masked, const uint8_t* cur, int tb, const Scores& s0, const Scores& s1, Weights& w0, Weights& w1)
+      __attribute__((always_inline)) {
+    float kscl[RT::kN], lv[RT::kN];
+    rt[0].load_factor(cur, 0, kscl);
+    rt[0].load_factor(cur, 1, lv);
+    weights_with(masked, cur, tb, s0, s1, kscl, lv, w0, w1);
   };
   // In the matrix phase of tile i a wave converts its rows of tile i + 1.  fetch_next, right behind the phase's
   // barrier: they have landed (the loads of three tiles may still be in flight) and are on their way from the raw
@@ -672,9 +678,13 @@ __global__ void __launch_bounds__(512, 2) prefill_pingpong_quant_d128_kernel(Dec
     } else {
       ld.template store<false>(rw, conv, tb, it.len);
     }
-    blk = block_of_const(p, it, tb + kRaw * kT + mine);
     __builtin_amdgcn_sched_barrier(0);  // (the raw bytes are in registers: their buffer may be written)
     ld.issue(p, it, tb + kRaw * kT, blk, raws + ((i + 1) & (kRaw - 1)) * kPingPongRawTile);
+  };
+  // The block id for the loads that the matrix phase of tile i issues (tile i + 5): a scalar load, which shares a
+  // counter with LDS, so it is made where a wait for it delays nothing: ahead of the barrier before that phase.
+  auto next_block = [&](int i) __attribute__((always_inline)) {
+    blk = block_of_const(p, it, w_begin + (i + 1 + kRaw) * kT + mine);
   };
 
   auto whole = [&](auto ph, int i) __attribute__((always_inline)) {
@@ -700,6 +710,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pingpong_quant_d128_kernel(Dec
       }
       values(cur, w0, w1);
     }
+    next_block(i + 1);
   };
   auto pipelined = [&](auto ph, auto first, int i) __attribute__((always_inline)) {
     constexpr int PH = decltype(ph)::value;
@@ -719,12 +730,18 @@ __global__ void __launch_bounds__(512, 2) prefill_pingpong_quant_d128_kernel(Dec
       store_next(ph, i, rw);
       scores(cur, s0, s1);
     }
+    float kscl[RT::kN], lv[RT::kN];  // on their way across the barrier
+    rt[0].load_factor(cur, 0, kscl);
+    rt[0].load_factor(cur, 1, lv);
     XLLM_HIP_PINGPONG_SETPRIO(0);
     barrier();
-    weights(std::false_type{}, cur, tb, s0, s1, pf0, pf1);
+    weights_with(std::false_type{}, cur, tb, s0, s1, kscl, lv, pf0, pf1);
     __builtin_amdgcn_sched_barrier(0);
     vpre[0] = rt[0].v_fragment(cur, 0, RT::opaque(rt[0].v_off0));
     vpre[1] = rt[0].v_fragment(cur, 1, RT::opaque(rt[0].v_off0));
+    next_block(i + 1);
+    // (waited for here: behind the barrier it would make the first MFMA wait for the raw bytes' way to registers as well)
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
     __builtin_amdgcn_sched_barrier(0);
   };
 
@@ -736,8 +753,10 @@ __global__ void __launch_bounds__(512, 2) prefill_pingpong_quant_d128_kernel(Dec
     ld.issue(p, it, w_begin + 3 * kT, block_of_const(p, it, w_begin + 3 * kT + mine), raws + 3 * kPingPongRawTile);
     // tile 0 is converted before the first barrier (fetch_next(i) and store_next(.., i, ..) handle tile i + 1)
     {
+      next_block(-1);
       const Raw rw = fetch_next(-1);
       store_next(std::integral_constant<int, kConv - 1>{}, -1, rw);
+      next_block(0);
     }
     if (late) barrier();
     int i = 0;
