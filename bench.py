@@ -59,6 +59,10 @@ def parse_args():
                          "kernel against which the rocprofv3 FETCH_SIZE / WRITE_SIZE counters are scaled")
     ap.add_argument("--settle-ms", type=float, default=150.0,
                     help="untimed steps run for this long before the warm-up steps (clock and TLB settling)")
+    ap.add_argument("--schedule-audit", action="store_true",
+                    help="time the scheduling rules' choice against each forced alternative over a grid of shapes "
+                         "(cache type x batch x length, equal and lognormal lengths); one JSON line per cell")
+    ap.add_argument("--audit-cells", default="", help="comma-separated substrings: only cells whose name holds one")
     ap.add_argument("--aux", action="store_true",
                     help="time the kernels around the decode path instead (KV writes, norm + rotary embedding + "
                          "write, block copy, a chunked-prefill step) and print one JSON line of their own")
@@ -265,6 +269,9 @@ def main():
         return
     if args.aux:
         print(json.dumps(aux_kernels(torch, ops, device)), flush=True)
+        return
+    if args.schedule_audit:
+        schedule_audit(torch, ops, device, args.audit_cells)
         return
     w = workloads.WORKLOADS[args.workload]
     if args.set:
@@ -678,6 +685,126 @@ def aux_kernels(torch, ops, device):
     add("verify, 64 rows per kv head (128-row kernel, half of its waves idle), 32 x 8192 tokens bf16", us,
         B * L * Hkv * D * 2 * 2, "K/V bytes")
     return res
+
+
+def schedule_audit(torch, ops, device, only=""):
+    """For every cell of a fixed grid, the decode step as the library's rules shape it (hints = the true lengths)
+    against the same step with each rule forced the other way (xllm_hip_set_option), without hints, and with the
+    schedule made on the host.  Timed per layer on an existing schedule (plan once, then runs), the figure
+    `run_us` is; a cell's `loss_pct` is how far the rules' choice is behind the fastest alternative."""
+    import numpy as np
+
+    Hq, Hkv, D, bs = 32, 8, 128, 16
+    max_tokens = 4 << 20
+    nb = max_tokens // bs + 4096
+    gen = torch.Generator(device=device)
+    gen.manual_seed(11)
+    rng = np.random.default_rng(11)
+    caches = {}
+
+    def cache(kind):
+        if kind not in caches:
+            caches.clear()  # one pool at a time
+            torch.cuda.empty_cache()
+            if kind == "bf16":
+                k = torch.randn(nb, Hkv, bs, D, device=device, dtype=torch.bfloat16, generator=gen)
+                v = torch.randn(nb, Hkv, bs, D, device=device, dtype=torch.bfloat16, generator=gen)
+                caches[kind] = (k, v, None, None)
+            else:
+                raw = torch.randint(-100, 100, (2, nb, Hkv, bs, D), device=device, dtype=torch.int8, generator=gen)
+                if kind == "fp8":
+                    raw = (raw.to(torch.float32) / 16).to(torch.float8_e4m3fn)
+                sc = torch.rand(2, nb, Hkv, bs, device=device, generator=gen) * 0.01 + 0.005
+                caches[kind] = (raw[0], raw[1], sc[0], sc[1])
+        return caches[kind]
+
+    def timed(fn, n):
+        for _ in range(3):
+            fn()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(n):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) * 1e3 / n
+
+    alternatives = [("no_hints", {}, "nohints"), ("host_plan", {}, "host"), ("stored_schedule", {"stored_schedule": 1}, None),
+                    ("item_per_head", {"item_per_head": 1}, None), ("four_wave_items", {"four_wave_items": 1}, None),
+                    ("separate_merge", {"separate_merge": 1}, None), ("target_256", {"target_items": 256}, None)]
+    wanted = [t for t in only.split(",") if t]
+    worst, host_wins = [], []
+    for kind in ("bf16", "fp8", "int8"):
+        for B in (16, 64, 256, 1024):
+            for mean in (256, 2048, 8192, 32768):
+                for dist in ("equal", "lognormal"):
+                    name = "%s_b%d_l%d_%s" % (kind, B, mean, dist)
+                    if B * mean > max_tokens // 2 or (wanted and not any(t in name for t in wanted)):
+                        continue
+                    if dist == "equal":
+                        lens = np.full(B, mean, dtype=np.int64)
+                    else:
+                        lens = np.clip(rng.lognormal(np.log(mean), 0.8, B), 16, 4 * mean).astype(np.int64)
+                        lens = np.minimum(lens, max(16, (max_tokens - 16 * B) // B * 4))
+                        while lens.sum() > max_tokens - 16 * B:
+                            lens = np.maximum(lens * 9 // 10, 16)
+                    k, v, ks, vs = cache(kind)
+                    blocks = (lens + bs - 1) // bs
+                    table = torch.zeros(B, int(blocks.max()), dtype=torch.int32, device=device)
+                    perm = torch.randperm(nb, device=device, generator=gen).to(torch.int32)
+                    o = 0
+                    for b in range(B):
+                        table[b, : blocks[b]] = perm[o: o + blocks[b]]
+                        o += int(blocks[b])
+                    seq_lens = torch.from_numpy(lens.astype(np.int32)).to(device)
+                    q = torch.randn(B, Hq, D, device=device, dtype=torch.bfloat16, generator=gen)
+                    out = torch.empty_like(q)
+                    ws = torch.empty(ops.WORKSPACE_BYTES, dtype=torch.uint8, device=device)
+                    host_lens = [int(x) for x in lens]
+
+                    base = dict(scale=D ** -0.5, q_per_seq=1, workspace=ws, kv_cache_quant_bit_size=8 if ks is not None else -1)
+                    by_mode = {"host": dict(base, host_plan=True), "nohints": base,
+                               None: dict(base, max_seq_len=int(lens.max()), total_kv_len=int(lens.sum()))}
+
+                    def step(mode, plan, run):
+                        # (the same host-side work in every mode: a step of under 20 us is timed by its launch)
+                        kw = by_mode[mode]
+                        if mode == "host" and plan:
+                            kw = dict(kw, host_kv_lens=host_lens)
+                        ops.batch_decode(q, k, out, table, seq_lens, v, None, None, ks, vs, plan=plan, run=run, **kw)
+
+                    def measure(mode, opts):
+                        import contextlib
+                        with contextlib.ExitStack() as st:
+                            for key, val in opts.items():
+                                st.enter_context(ops.option(key, val))
+                            step(mode, True, False)
+                            n = max(5, min(50, int(20000 / max(20.0, B * mean / 4000.0))))
+                            return timed(lambda: step(mode, False, True), n)
+
+                    measure(None, {})  # (the cell's first measurement runs on cold caches and a ramping clock)
+                    rule = measure(None, {})
+                    res = {alt: round(measure(mode, opts), 1) for alt, opts, mode in alternatives}
+                    rule = min(rule, measure(None, {}))  # (and once more behind the alternatives: the smaller counts)
+                    # the forced alternatives (and the call without hints) against the rules' choice; the schedule made
+                    # on the host is another entry point, which needs every length on the host: reported beside them
+                    host_us = res.pop("host_plan")
+                    best_name = min(res, key=res.get)
+                    best = min(res[best_name], rule)
+                    loss = (rule - best) / best * 100.0
+                    kv_bytes = float(lens.sum()) * Hkv * D * 2 * (2 if kind == "bf16" else 1)
+                    line = {"cell": name, "rule_us": round(rule, 1), "frac_of_8TBs": round(kv_bytes / rule / 8e6, 3),
+                            "alternatives_us": res, "best": best_name if res[best_name] < rule else "rule",
+                            "loss_pct": round(loss, 1), "host_plan_us": host_us,
+                            "host_plan_gain_pct": round((rule - host_us) / host_us * 100.0, 1)}
+                    print(json.dumps(line), flush=True)
+                    if loss > 3.0:
+                        worst.append((name, round(loss, 1), best_name))
+                    if rule > host_us * 1.03:
+                        host_wins.append((name, line["host_plan_gain_pct"]))
+                    del table, seq_lens, q, out, ws
+    print(json.dumps({"schedule_audit_summary": True, "cells_where_a_forced_alternative_wins_by_over_3_pct": worst,
+                      "cells_where_the_host_plan_wins_by_over_3_pct": host_wins}), flush=True)
 
 
 def cpu_baseline(w, torch, pool, q, block_table, seq_lens, out, step, args):
