@@ -59,6 +59,8 @@ def parse_args():
                          "kernel against which the rocprofv3 FETCH_SIZE / WRITE_SIZE counters are scaled")
     ap.add_argument("--settle-ms", type=float, default=150.0,
                     help="untimed steps run for this long before the warm-up steps (clock and TLB settling)")
+    ap.add_argument("--no-sustained", action="store_true",
+                    help="skip the interleaved and sustained timing legs (profiling runs: fewer dispatches to trace)")
     ap.add_argument("--schedule-audit", action="store_true",
                     help="time the scheduling rules' choice against each forced alternative over a grid of shapes "
                          "(cache type x batch x length, equal and lognormal lengths); one JSON line per cell")
@@ -430,6 +432,44 @@ def main():
     plan_us = plan_graph_us()
     plan_or_run(0, True)
 
+    def interleaved_us(rounds=4, per=50):
+        # `value` (plan + run per call) and `run_us` (runs on an existing schedule) in alternating legs, so that a
+        # drift of the clocks over the benchmark's run shows in both series instead of between them
+        full, runs = [], []
+        for _ in range(rounds):
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            for i in range(per):
+                step(i)
+            torch.cuda.synchronize()
+            full.append(round((time.perf_counter() - t) * 1e6 / per, 2))
+            plan_or_run(0, True)
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            for i in range(per):
+                plan_or_run(i, False)
+            torch.cuda.synchronize()
+            runs.append(round((time.perf_counter() - t) * 1e6 / per, 2))
+        return full, runs
+
+    def sustained_us(seconds=1.0):
+        # back-to-back steps for at least a second (the queue is drained every 256 steps, so that the clock below
+        # follows the GPU and not the enqueueing)
+        n = 0
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        while time.perf_counter() - t < seconds:
+            for i in range(256):
+                step(n + i)
+            n += 256
+            torch.cuda.synchronize()
+        return (time.perf_counter() - t) * 1e6 / n, n
+
+    interleaved_full = interleaved_runs = sustained = sustained_steps = None
+    if not args.no_sustained:
+        interleaved_full, interleaved_runs = interleaved_us()
+        sustained, sustained_steps = sustained_us()
+
     engine_us = engine_no_hints_us = None
     if io_dtype == torch.bfloat16 and not args.no_engine_step:
         engine_us = engine_step_us(torch, w, pools, table, seq_lens, lists, args.kv_layout, args.steps, device, True,
@@ -453,13 +493,14 @@ def main():
                    "decode_mfma_d128_kernel" if rows_per_kv_head <= 16 else "decode_mfma_d128_rows32_kernel")
     # figures of the committed rocprofv3 runs of this same command (profiles/): HBM bytes per launch from
     # the FETCH_SIZE / WRITE_SIZE counters, and the kernel's average duration in the kernel trace
-    traffic = rocprof_avg = None
+    traffic = rocprof_avg = rocprof_commit = None
     tpath = os.path.join(REPO, "profiles", "hbm_traffic.json")
     # (they were taken in the default configuration: HND pools with the library's K/V placement)
     if os.path.exists(tpath) and args.kv_layout == "HND" and args.kv_skew_bytes is None:
         entry = json.load(open(tpath)).get(w.name, {})
         traffic = entry.get("traffic_bytes_per_launch")
         rocprof_avg = entry.get("kernel_avg_us")
+        rocprof_commit = entry.get("commit", json.load(open(tpath)).get("_commit"))
 
     result = {
         "metric": "decode-attn us/step + achieved HBM GB/s (% of 8 TB/s), Llama-3-8B shape b64 ctx4k",
@@ -509,6 +550,13 @@ def main():
                          "(xllm_hip_paged_decode_plan; no launch at all when the host-side lengths show that nothing "
                          "is split), run_us: attention (+ merge) on an existing schedule (xllm_hip_paged_decode_run), "
                          "what every layer after layer 0 costs an engine that plans once per step",
+        "interleaved_value_us": interleaved_full,
+        "interleaved_run_us": interleaved_runs,
+        "sustained_us": None if sustained is None else round(sustained, 2),
+        "sustained_steps": sustained_steps,
+        "timing_note": "interleaved_*: four alternating legs of 50 steps each of plan + run (what `value` times) and "
+                       "of runs on an existing schedule (run_us), in the order they ran; sustained_us: plan + run per "
+                       "step over at least a second of back-to-back steps",
         "engine_layers": args.engine_layers,
         "write_plus_attend_us": None if engine_us is None else round(engine_us, 2),
         "write_plus_attend_no_hints_us": None if engine_no_hints_us is None else round(engine_no_hints_us, 2),
@@ -541,6 +589,9 @@ def main():
                         "events); an event pair adds about 2 us of command-processor time to the kernel's own "
                         "duration, which is rocprof_kernel_avg_us" % (args.steps, us_per_step_with_events),
             "rocprof_kernel_avg_us": rocprof_avg,
+            "rocprof_commit": rocprof_commit,
+            "rocprof_note": "traffic and rocprof_kernel_avg_us are stored figures, read from profiles/hbm_traffic.json: "
+                            "they were measured by rocprofv3 on the tree of rocprof_commit, not in this run",
         },
     }
 

@@ -453,6 +453,18 @@ def test_prefill_chunks_over_a_quantised_cache_take_the_dense_route(gpu, shim, k
         assert err <= 5e-2
     # the dense copy is the dequantised cache rounded to bf16: the two routes differ by that rounding only
     assert float(np.abs(outs[0] - outs[1]).max()) <= 2e-2
+    # The dense route layer by layer, as the model's loop drives it: layer 0 makes the copy's block table and the
+    # step's schedule, later layers reuse both, and every layer's copy goes through the same persistent buffers.
+    attn = shim.AttentionImpl(Hq, D, scale, Hkv, -1)
+    attn.set_prefill_dequant_rows(128)
+    cache = fresh_cache()
+    qkv_d = qkv.to(gpu)
+    for layer in (0, 1, 2):
+        md.plan_info.layer_id = layer
+        out, _ = attn.forward(md, qkv_d[:, : Hq * D], qkv_d[:, Hq * D:(Hq + Hkv) * D], qkv_d[:, (Hq + Hkv) * D:], cache)
+        torch.cuda.synchronize()
+        assert np.array_equal(out.float().cpu().numpy().reshape(T, Hq, D), outs[0]), layer
+    md.plan_info.layer_id = 0
 
 
 @pytest.mark.gpu

@@ -141,15 +141,17 @@ inline bool never_split(int q_per_seq, int num_q_heads, int num_kv_heads) {
 // 16-row and the 128-row MFMA kernels is four waves, one per SIMD of a CU, and two fit on a CU (256
 // VGPRs, < 80 KiB of LDS); four two-wave workgroups of the 32-row kernel do; the generic kernel runs
 // one wave per item, eight per CU.  head_dim 256 runs one wave per SIMD: half as many workgroups.
-constexpr int kNumCUs = 256;
+// CUs of the device the sizes are for: the callers pass what the device reports (hipDeviceAttributeMultiprocessorCount,
+// read once per device); this is the MI355X's count, for code that sizes things with no device at hand.
+constexpr int kDefaultCUs = 256;
 // Up to 16 query rows per kv head, over a cache whose kv heads lie side by side within a token, a work item
 // covers four kv heads (one per wave of the 16-row kernel) when the head count allows it.
 constexpr int kHeadsPerItem = 4;
 inline int item_heads_of(int rows, int num_kv_heads, bool heads_side_by_side) {
   return heads_side_by_side && rows <= 16 && num_kv_heads % kHeadsPerItem == 0 ? num_kv_heads / kHeadsPerItem : num_kv_heads;
 }
-inline int natural_target_items(bool mfma, int rows, bool one_wave_per_simd) {
-  int v = !mfma ? 8 * kNumCUs : (rows > 16 && rows <= kPrefillMinRows) ? 4 * kNumCUs : 2 * kNumCUs;
+inline int natural_target_items(bool mfma, int rows, bool one_wave_per_simd, int cus = kDefaultCUs) {
+  int v = !mfma ? 8 * cus : (rows > 16 && rows <= kPrefillMinRows) ? 4 * cus : 2 * cus;
   if (one_wave_per_simd) v /= 2;
   return v;
 }
@@ -162,18 +164,19 @@ inline int natural_target_items(bool mfma, int rows, bool one_wave_per_simd) {
 //   MFMA kernels     up to 16 rows T = 512, 17..32 rows T = 1024 (RG = 1); more rows T = 512 with 128
 //                    (16-bit cache) or 32 (1-byte cache) rows per item: RG >= ceil(rows / 128)
 //   16-row MFMA kernel over a cache whose heads lie side by side (work items of kHeadsPerItem kv heads): Hkv / 4 in place of Hkv
-inline int64_t max_seq_chunks_for(int batch, int rows, int num_kv_heads) {
+inline int64_t max_seq_chunks_for(int batch, int rows, int num_kv_heads, int cus = kDefaultCUs) {
   auto bound = [&](int64_t target, int64_t rg, int64_t heads) { return (target + target / 4 + heads * rg - 1) / (heads * rg); };
-  const int64_t generic = bound(natural_target_items(false, rows, false), rows, num_kv_heads);
-  const int64_t mfma = bound(natural_target_items(true, rows, false),
+  const int64_t generic = bound(natural_target_items(false, rows, false, cus), rows, num_kv_heads);
+  const int64_t mfma = bound(natural_target_items(true, rows, false, cus),
                              rows <= kPrefillMinRows ? 1 : (rows + kPrefillRowsPerItem - 1) / kPrefillRowsPerItem,
                              item_heads_of(rows, num_kv_heads, true));
   return (generic > mfma ? generic : mfma) + batch + 1;
 }
 
-inline WorkspaceLayout workspace_layout(int batch, int q_per_seq, int num_q_heads, int num_kv_heads, int head_dim) {
+inline WorkspaceLayout workspace_layout(int batch, int q_per_seq, int num_q_heads, int num_kv_heads, int head_dim,
+                                        int cus = kDefaultCUs) {
   WorkspaceLayout w;
-  w.max_seq_chunks = max_seq_chunks_for(batch, q_per_seq * (num_q_heads / num_kv_heads), num_kv_heads);
+  w.max_seq_chunks = max_seq_chunks_for(batch, q_per_seq * (num_q_heads / num_kv_heads), num_kv_heads, cus);
   // A step that is never split writes its output rows directly, whichever kernel serves it: no chunk
   // records and no partial rows (at 4096 query tokens they would be 64 MiB that nothing touches).
   const bool whole = never_split(q_per_seq, num_q_heads, num_kv_heads);

@@ -25,6 +25,48 @@
 
 namespace xllm_hip {
 
+// The thresholds by which the host shapes a decode step (fill_params in paged_decode.hip reads them here; the
+// reasoning stands beside each use), each with the measurement it came from — per layer on an existing schedule,
+// one MI355X, 8 kv heads of 128 elements unless noted.  `bench.py --schedule-audit` times every choice they lead
+// to against the forced alternatives.
+struct ShapeRules {
+  // Lengths count as nearly equal when max_len * batch <= total * 5 / 4: every sequence then owns the same number
+  // of chunk slots and at most a fifth of the launch's workgroups find nothing to do (fixed-length buckets; the
+  // ragged workload, lognormal sigma 0.8, has max * batch = 4 x total and keeps the stored schedule).
+  int nearly_equal_num = 5, nearly_equal_den = 4;
+  // One wave per kv head (work items of four heads, or four items to a workgroup) up to this mean length:
+  // 1-byte cache 2048 x 256 tokens 242 -> 203 us, 256 x 6144 499 -> 492, 128 x 8192 326 -> 333 (not those);
+  // 16-bit cache 4096 x 64 tokens 264 -> 193, 2048 x 128 202 -> 182, 256 tokens and more the same;
+  // head_dim 64 over a 16-bit cache 4096 x 128 69 -> 51, 2048 x 768 130 -> 127, 2048 tokens the same.
+  int wave_per_head_max_mean_quant = 8192, wave_per_head_max_mean_d64 = 2048, wave_per_head_max_mean_16bit = 192;
+  // Its gain over four waves per head, as k / mean length up to a cap (fitted to the rows above): 1-byte rows of
+  // 128 bytes 100 / L (19 % at 256 tokens, 5 % at 2048), of 64 bytes 200 / L; 16-bit rows of 256 bytes 16 / L, of
+  // 128 bytes 25 / L.
+  double wave_per_head_k_quant = 100.0, wave_per_head_k_quant_d64 = 200.0, wave_per_head_k_16bit = 16.0, wave_per_head_k_16bit_d64 = 25.0;
+  double wave_per_head_cap_quant = 0.2, wave_per_head_cap_quant_d64 = 0.4, wave_per_head_cap_16bit = 0.3;
+  // Four-head items over a 1-byte cache whose heads lie side by side gain this much from the layout alone
+  // (fp8, 128 x 8192 tokens, NHD: 391 -> 338 us).
+  double side_by_side_gain = 0.16;
+  // Narrow items whose last round's sequences are cut fill their rounds but for the merges; the wider form must
+  // beat the narrow one by this factor to be taken (192 sequences of 2048 fp8 tokens, 1.5 rounds of four-head
+  // workgroups: 148 us against 134).
+  double cut_rounds_filled = 0.97, wider_items_hurdle = 1.01;
+  // Eight waves per item (1-byte caches) when the launch has at most one item per CU and at least three quarters
+  // of the CUs get one (20 x 8192 fp8 tokens: 69 us as 160 eight-wave items, 65 as 480 four-wave items), and
+  // while the items are at most a quarter more than the CUs, the sequences past a round being cut (33 sequences x
+  // 8192 fp8 tokens: 105 -> 100 us, 40: 122 -> 116).
+  int eight_waves_min_num = 3, eight_waves_min_den = 4, eight_waves_over_num = 5, eight_waves_over_den = 4;
+  // The fused merge loads 32 partials in one batch: no sequence is cut finer by the rules that rely on it (one
+  // 32768-token fp8 sequence: 31 us at 256 items, 38 at 512).
+  int fused_merge_max_chunks = 32;
+  // The sequences of a partly filled last round are cut while the step is under four rounds (288 x 2048 fp8
+  // tokens, 4.5 rounds: 202 us whole, 206 cut); an even cut that fills under nine tenths of a round is taken one
+  // finer first (1-byte caches); cut in two throughout, the last round's sequences must get at least three times
+  // the others' chunks (fp8, 8192 tokens: 40 sequences 132 -> 122 us, 48, four chunks each, 136 -> 144).
+  int cut_last_round_below_rounds = 4, round_fill_num = 9, round_fill_den = 10, last_round_min_ratio = 3;
+};
+constexpr ShapeRules kShapeRules{};
+
 struct HostScheduleInput {
   const int32_t* kv_lens;  // [batch], as the kernels will see them (cut to 0 .. len_cap here)
   int32_t batch;

@@ -73,10 +73,31 @@ static Options& options() {
 }
 static int64_t option(int which) { return options().v[which].load(std::memory_order_relaxed); }
 
+// CUs of the current device, as the runtime reports them (asked once per device; kDefaultCUs where there is no
+// device to ask: the size functions are also called on hosts without a GPU).
+static int device_cus() {
+  constexpr int kMaxDevices = 64;
+  static std::atomic<int> cached[kMaxDevices];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    (void)hipGetLastError();
+    return kDefaultCUs;
+  }
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+      (void)hipGetLastError();
+      n = kDefaultCUs;
+    }
+    cached[dev].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
+
 // Work items to aim for (natural_target_items), or fewer when the diagnostic option says so: the
 // workspace is sized for the natural targets, so the option can only lower them.
 static int target_items(int variant_is_mfma, int rows, bool one_wave_per_simd) {
-  const int v = natural_target_items(variant_is_mfma != 0, rows, one_wave_per_simd);
+  const int v = natural_target_items(variant_is_mfma != 0, rows, one_wave_per_simd, device_cus());
   const int64_t t = option(XLLM_HIP_OPTION_DECODE_TARGET_ITEMS);
   return t > 0 && t < v ? (int)t : v;
 }
@@ -159,7 +180,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
                      "q/out token stride smaller than num_q_heads*head_dim");
   }
   const WorkspaceLayout w =
-      workspace_layout(a->batch, a->q_per_seq, a->num_q_heads, c->num_kv_heads, c->head_dim);
+      workspace_layout(a->batch, a->q_per_seq, a->num_q_heads, c->num_kv_heads, c->head_dim, device_cus());
   if (workspace == nullptr || workspace_bytes < w.total_bytes) {
     return fail(XLLM_HIP_WORKSPACE_TOO_SMALL, "workspace has %zu bytes, need %zu", workspace_bytes, w.total_bytes);
   }
@@ -257,8 +278,10 @@ static int fill_params(const xllm_hip_kv_cache* c,
   // the wider items are taken when (filled share of their rounds) x (their measured gain for the step's mean
   // length) beats the filled share of the narrow items' rounds.
   const int64_t four_head_items = (int64_t)p.batch * item_heads_of(p.rows, c->num_kv_heads, true);
-  const int64_t slots = natural_target_items(true, p.rows, false);
-  const bool nearly_equal = (int64_t)a->max_seq_len * p.batch * 4 <= a->total_kv_len * 5;
+  const int cus = device_cus();
+  const int64_t slots = natural_target_items(true, p.rows, false, cus);
+  const ShapeRules& R = kShapeRules;
+  const bool nearly_equal = (int64_t)a->max_seq_len * p.batch * R.nearly_equal_den <= a->total_kv_len * R.nearly_equal_num;
   auto wider_items_pay = [&](int64_t narrow_items, int per_workgroup, double layout_gain = 0.0, bool narrow_cut = false) {
     auto filled = [&](int64_t workgroups) {
       if (workgroups <= 0) return 1.0;
@@ -270,25 +293,26 @@ static int fill_params(const xllm_hip_kv_cache* c,
     const double mean = (double)a->total_kv_len / (double)(p.batch > 0 ? p.batch : 1);
     // gain of one wave per item over four, by mean length: 1-byte rows of 128 bytes 100 / L (19 % at 256 tokens,
     // 5 % at 2048), of 64 bytes 200 / L; 16-bit rows of 256 bytes 16 / L, of 128 bytes 25 / L
-    const double k = variant == kMfmaD64 ? (quant ? 200.0 : 25.0) : (quant ? 100.0 : 16.0);
+    const double k = variant == kMfmaD64 ? (quant ? R.wave_per_head_k_quant_d64 : R.wave_per_head_k_16bit_d64)
+                                         : (quant ? R.wave_per_head_k_quant : R.wave_per_head_k_16bit);
     double gain = k / (mean > 1.0 ? mean : 1.0);
-    const double cap = quant ? (variant == kMfmaD64 ? 0.4 : 0.2) : 0.3;
+    const double cap = quant ? (variant == kMfmaD64 ? R.wave_per_head_cap_quant_d64 : R.wave_per_head_cap_quant) : R.wave_per_head_cap_16bit;
     gain = gain < cap ? gain : cap;
     if (per_workgroup == 2) gain *= 0.5;
     gain += layout_gain;
     // (narrow items whose last round's sequences are cut fill their rounds but for the merges)
-    const double narrow_filled = narrow_cut ? 0.97 : filled(narrow_items);
-    return filled((narrow_items + per_workgroup - 1) / per_workgroup) * (1.0 + gain) > narrow_filled * 1.01;
+    const double narrow_filled = narrow_cut ? R.cut_rounds_filled : filled(narrow_items);
+    return filled((narrow_items + per_workgroup - 1) / per_workgroup) * (1.0 + gain) > narrow_filled * R.wider_items_hurdle;
   };
   const bool short_sequences = (variant == kMfmaD128 || variant == kMfmaD64) && a->max_seq_len > 0 && a->total_kv_len > 0 &&
                                four_head_items >= (nearly_equal ? slots : 4 * slots) &&
-                               a->total_kv_len <= (int64_t)p.batch * (quant ? 8192 : variant == kMfmaD64 ? 2048 : 192) &&
+                               a->total_kv_len <= (int64_t)p.batch * (quant ? R.wave_per_head_max_mean_quant : variant == kMfmaD64 ? R.wave_per_head_max_mean_d64 : R.wave_per_head_max_mean_16bit) &&
                                (!nearly_equal || wider_items_pay((int64_t)p.batch * c->num_kv_heads, kHeadsPerItem)) &&
                                option(XLLM_HIP_OPTION_DECODE_ITEM_PER_HEAD) == 0;
   // (the four-head items of a 1-byte cache with its heads side by side gain 16 % from the layout alone, 391 -> 338
   // us: they too give way where their rounds would be poorly filled and the host-side lengths show it)
   const bool side_by_side_pays = !(a->max_seq_len > 0 && a->total_kv_len > 0 && nearly_equal) ||
-                                 wider_items_pay((int64_t)p.batch * c->num_kv_heads, kHeadsPerItem, 0.16);
+                                 wider_items_pay((int64_t)p.batch * c->num_kv_heads, kHeadsPerItem, R.side_by_side_gain);
   p.item_heads = item_heads_of(p.rows, c->num_kv_heads, (side_by_side && side_by_side_pays) || short_sequences);
   p.heads_per_item = c->num_kv_heads / p.item_heads;
   p.head_dim = c->head_dim;
@@ -319,7 +343,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
   const int32_t target_one_per_cu = p.target_small;
   if (quant && p.target_small < p.target_items) {
     const int64_t triples = (int64_t)p.batch * p.item_heads * p.row_groups;
-    const int64_t cap = 32 * triples;
+    const int64_t cap = R.fused_merge_max_chunks * triples;
     p.target_small = (int32_t)(cap >= p.target_items ? p.target_items : cap > p.target_small ? cap : p.target_small);
   }
   // Only the MFMA kernel finishes single-chunk sequences itself.  When the caller's host-side
@@ -387,7 +411,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
     p.target_small = target_one_per_cu;
     decide();
     const int64_t items = (p.implicit_plan ? (int64_t)p.batch : (int64_t)p.batch * p.arith_chunks) * p.item_heads * p.row_groups;
-    decided = (p.implicit_plan || p.arith_chunks > 0) && items <= kNumCUs && items * 4 >= kNumCUs * 3;
+    decided = (p.implicit_plan || p.arith_chunks > 0) && items <= cus && items * R.eight_waves_min_den >= (int64_t)cus * R.eight_waves_min_num;
     if (!decided) p.target_small = every_slot;
   }
   if (!decided) decide();
@@ -416,19 +440,19 @@ static int fill_params(const xllm_hip_kv_cache* c,
     // ... or, while the items are at most a quarter more than the CUs, runs eight waves per item like a step of
     // up to 256 items: a round is then an item per CU, the sequences past it are cut, and their chunks follow the
     // whole items onto the CUs (fp8, 8192 tokens x 8 kv heads: 33 sequences 105 us cut in two throughout)
-    const bool eight = quant && p.rows <= 16 && p.tok != 0 && uniform == 1 && items > kNumCUs && items * 4 <= kNumCUs * 5 &&
+    const bool eight = quant && p.rows <= 16 && p.tok != 0 && uniform == 1 && items > cus && items * R.eight_waves_over_den <= (int64_t)cus * R.eight_waves_over_num &&
                        option(XLLM_HIP_OPTION_DECODE_FOUR_WAVE_ITEMS) == 0;
-    const int64_t round = eight ? kNumCUs : quant || one_wave_per_simd ? p.target_items : kNumCUs;
+    const int64_t round = eight ? cus : quant || one_wave_per_simd ? p.target_items : cus;
     // chunks of the sequences that stay as they are: the even cut the step has, or one more when that cut fills
     // less than nine tenths of a round
-    const int64_t first = !eight && quant && uniform * items < round && uniform * items * 10 < round * 9 ? uniform + 1 : uniform;
+    const int64_t first = !eight && quant && uniform * items < round && uniform * items * R.round_fill_den < round * R.round_fill_num ? uniform + 1 : uniform;
     const int64_t whole_rounds = first * items / round;
     // (from 2048 items on the last round weighs little: 288 x 2048 fp8 tokens x 8 kv heads 202 us whole, 206 cut)
-    if (whole_rounds >= 1 && items < 4 * p.target_items && (first * items) % round != 0) {
+    if (whole_rounds >= 1 && items < (int64_t)R.cut_last_round_below_rounds * p.target_items && (first * items) % round != 0) {
       const int64_t whole_seqs = whole_rounds * round / (per * first);
       const int64_t cut_seqs = p.batch - whole_seqs;
       int64_t k = round / (cut_seqs * per);
-      k = k > 32 ? 32 : k;  // (what the fused merge loads in one batch)
+      k = k > R.fused_merge_max_chunks ? R.fused_merge_max_chunks : k;  // (what the fused merge loads in one batch)
       // (bf16, 4096 tokens x 8 kv heads: 66 sequences 192 -> 167 us, 72 196 -> 185, 80, two chunks, 204 -> 206;
       // 8192 tokens: 33 sequences 228 -> 168, 40 237 -> 203, 44 242 -> 220, 48 247 -> 240.  fp8, 8192 tokens: 66
       // sequences 255 -> 179, 80 260 -> 217, 96 277 -> 258, 136 413 -> 359)
@@ -446,7 +470,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
       k = ((int64_t)a->max_seq_len + chunk - 1) / chunk;
       // (cut in two throughout, every sequence is merged: that pays while the last round's are few — fp8, 8192 tokens
       // x 8 kv heads, 33 sequences 129 -> 105 us, 40 132 -> 122, but 48, whose last 16 get four chunks each, 136 -> 144)
-      if (k > k1 && (first == 1 || k >= 3 * k1) && whole_seqs * k1 + cut_seqs * k <= w.max_seq_chunks) {
+      if (k > k1 && (first == 1 || k >= R.last_round_min_ratio * k1) && whole_seqs * k1 + cut_seqs * k <= w.max_seq_chunks) {
         p.fixed_chunk = (int32_t)chunk;
         p.arith_chunks = (int32_t)k;
         p.arith_whole = (int32_t)whole_seqs;
@@ -465,7 +489,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
   // 192 sequences, 1.5 rounds of such workgroups, would take 148 against 134: see wider_items_pay).
   p.wave_items = 0;
   if ((variant == kMfmaD128 || variant == kMfmaD64) && p.rows <= 16 && p.heads_per_item == 1 && hints && nearly_equal &&
-      a->total_kv_len <= (int64_t)p.batch * (quant ? 8192 : variant == kMfmaD64 ? 2048 : 192) &&
+      a->total_kv_len <= (int64_t)p.batch * (quant ? R.wave_per_head_max_mean_quant : variant == kMfmaD64 ? R.wave_per_head_max_mean_d64 : R.wave_per_head_max_mean_16bit) &&
       option(XLLM_HIP_OPTION_DECODE_ITEM_PER_HEAD) == 0) {
     const int64_t items = (int64_t)p.batch * c->num_kv_heads;
     const int per_group = items >= kHeadsPerItem * slots ? 1 : items >= 2 * slots ? 2 : 0;
@@ -539,7 +563,7 @@ static void launch_mfma_tok(const DecodeParams& p, unsigned grid, hipStream_t st
       // At most one work item per CU over a 1-byte cache: eight waves share it (one 32768-token sequence:
       // 25 us against 31 for fp8, 26 against 32 for int8; over a 16-bit cache, whose tiles take no
       // conversion, 31.7 against 31.0).
-      if ((grid <= (unsigned)kNumCUs || p.eight_waves) && option(XLLM_HIP_OPTION_DECODE_FOUR_WAVE_ITEMS) == 0) {
+      if ((grid <= (unsigned)device_cus() || p.eight_waves) && option(XLLM_HIP_OPTION_DECODE_FOUR_WAVE_ITEMS) == 0) {
         decode_mfma_d128_kernel<KV_DT, TOK, false, 2 * kWaves><<<grid, 128 * kWaves, 0, st>>>(p);
         return;
       }
@@ -598,7 +622,7 @@ extern "C" int xllm_hip_paged_decode_describe(const xllm_hip_kv_cache* cache,
   XLLM_HIP_REQUIRE(cache != nullptr && args != nullptr, "cache or args is NULL");
   if (workspace_bytes == 0) {
     workspace_bytes = workspace_layout(args->batch, args->q_per_seq, args->num_q_heads, cache->num_kv_heads,
-                                       cache->head_dim).total_bytes;
+                                       cache->head_dim, device_cus()).total_bytes;
   }
   DecodeParams p;
   // (a workspace address that is never read: every field of it the host forms is an offset from it)
@@ -619,7 +643,7 @@ extern "C" int xllm_hip_paged_decode_describe(const xllm_hip_kv_cache* cache,
       waves = 4;
       per_workgroup = p.wave_items == 2 ? 2 : (p.wave_items == 1 ? 4 : 1);
     } else {
-      const bool eight = quant && p.tok != 0 && (grid <= kNumCUs || p.eight_waves) &&
+      const bool eight = quant && p.tok != 0 && (grid <= device_cus() || p.eight_waves) &&
                          option(XLLM_HIP_OPTION_DECODE_FOUR_WAVE_ITEMS) == 0;
       waves = eight ? 8 : 4;
     }
@@ -653,7 +677,7 @@ extern "C" size_t xllm_hip_paged_decode_workspace_bytes(int32_t batch,
                                                         int32_t num_kv_heads,
                                                         int32_t head_dim) {
   if (batch < 0 || q_per_seq < 1 || num_q_heads < 1 || num_kv_heads < 1 || head_dim < 1) return 0;
-  return workspace_layout(batch, q_per_seq, num_q_heads, num_kv_heads, head_dim).total_bytes;
+  return workspace_layout(batch, q_per_seq, num_q_heads, num_kv_heads, head_dim, device_cus()).total_bytes;
 }
 
 extern "C" int xllm_hip_set_option(int32_t which, int64_t value) {
@@ -710,7 +734,7 @@ extern "C" size_t xllm_hip_paged_decode_plan_host_bytes(int32_t batch,
                                                         int32_t num_kv_heads,
                                                         int32_t head_dim) {
   if (batch < 0 || q_per_seq < 1 || num_q_heads < 1 || num_kv_heads < 1 || head_dim < 1) return 0;
-  return workspace_layout(batch, q_per_seq, num_q_heads, num_kv_heads, head_dim).partial_lse;  // header .. last record
+  return workspace_layout(batch, q_per_seq, num_q_heads, num_kv_heads, head_dim, device_cus()).partial_lse;  // header .. last record
 }
 
 extern "C" int xllm_hip_paged_decode_plan_host(const xllm_hip_kv_cache* cache,
@@ -730,7 +754,7 @@ extern "C" int xllm_hip_paged_decode_plan_host(const xllm_hip_kv_cache* cache,
   XLLM_HIP_REQUIRE(host_kv_lens != nullptr && host_staging != nullptr, "host_kv_lens or host_staging is NULL");
   XLLM_HIP_REQUIRE(p.arith_chunks == 0 && p.fixed_chunk == 0, "a step with a plan made on the host keeps a stored schedule");
   const WorkspaceLayout w =
-      workspace_layout(args->batch, args->q_per_seq, args->num_q_heads, cache->num_kv_heads, cache->head_dim);
+      workspace_layout(args->batch, args->q_per_seq, args->num_q_heads, cache->num_kv_heads, cache->head_dim, device_cus());
   if (host_staging_bytes < w.partial_lse) {
     return fail(XLLM_HIP_WORKSPACE_TOO_SMALL, "host_staging has %zu bytes, need %zu", host_staging_bytes, w.partial_lse);
   }
@@ -909,7 +933,7 @@ extern "C" int xllm_hip_paged_decode_static(const xllm_hip_kv_cache* cache,
                        cache->head_dim >= 1,
                    "bad batch/q_per_seq/num_q_heads/num_kv_heads/head_dim");
   const size_t need =
-      workspace_layout(args->batch, args->q_per_seq, args->num_q_heads, cache->num_kv_heads, cache->head_dim)
+      workspace_layout(args->batch, args->q_per_seq, args->num_q_heads, cache->num_kv_heads, cache->head_dim, device_cus())
           .total_bytes;
   if (need > (size_t)XLLM_HIP_STATIC_WORKSPACE_BYTES) {
     return fail(XLLM_HIP_WORKSPACE_TOO_SMALL,

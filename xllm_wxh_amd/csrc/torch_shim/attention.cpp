@@ -2,7 +2,49 @@
 
 #include "ops_api.h"
 
+#include <c10/hip/HIPStream.h>
+#include <hip/hip_runtime_api.h>
+
+#include <map>
+#include <mutex>
+#include <tuple>
+
 namespace xllm::layer {
+
+namespace {
+
+// The dense 16-bit copy of a step's cached K/V ranges (decoder_forward's route for very many query rows over a
+// 1-byte cache) and the block table over it.  One per (device, stream, element type), kept for the life of the
+// process and only ever grown — outside stream capture: a captured graph holds the addresses.
+struct DenseCopy {
+  torch::Tensor k, v;        // flat, in the queries' type
+  torch::Tensor table;       // [batch, blocks of the longest sequence]: consecutive blocks of the copy
+  torch::Tensor row_offset;  // [batch]: first row of each sequence in the copy
+};
+
+DenseCopy& dense_copy(const torch::Device& device, const torch::TensorOptions& options, int64_t elements) {
+  static std::mutex mu;
+  static std::map<std::tuple<int, int64_t, int>, DenseCopy> copies;
+  const auto stream = c10::hip::getCurrentHIPStream(device.index());
+  std::lock_guard<std::mutex> lock(mu);
+  DenseCopy& dc = copies[std::make_tuple((int)device.index(), (int64_t)stream.id(), (int)c10::typeMetaToScalarType(options.dtype()))];
+  if (!dc.k.defined() || dc.k.numel() < elements) {
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    (void)hipStreamIsCapturing(stream.stream(), &capturing);
+    TORCH_CHECK(capturing == hipStreamCaptureStatusNone,
+                "the dense copy of the cached K/V must grow to ", elements, " elements: run the largest step of the "
+                "bucket once on this stream before capturing it");
+    // (a quarter more than asked for: steps of a serving loop grow token by token)
+    const int64_t n = elements + elements / 4;
+    dc.k = torch::Tensor();
+    dc.v = torch::Tensor();
+    dc.k = torch::empty({n}, options);
+    dc.v = torch::empty({n}, options);
+  }
+  return dc;
+}
+
+}  // namespace
 
 AttentionImpl::AttentionImpl(int64_t num_heads, int64_t head_size, float scale, int64_t num_kv_heads,
                              int64_t sliding_window)
@@ -101,16 +143,25 @@ void AttentionImpl::decoder_forward(const AttentionMetadata& attn_metadata, torc
       // of consecutive blocks.
       const int64_t bs = k_cache.size(2);
       const int64_t total_blocks = (attn_metadata.total_kv_len + batch * (bs - 1)) / bs + 1;
-      const auto i32 = torch::TensorOptions().dtype(torch::kInt32).device(query.device());
-      torch::Tensor blocks_per_seq = torch::div(attn_metadata.kv_seq_lens + (bs - 1), bs, "floor").to(torch::kInt32);
-      torch::Tensor first_block = (torch::cumsum(blocks_per_seq, 0) - blocks_per_seq).to(torch::kInt32);
-      const int64_t max_blocks = (attn_metadata.max_seq_len + bs - 1) / bs;
-      torch::Tensor dense_table =
-          torch::clamp_max(first_block.unsqueeze(1) + torch::arange(max_blocks, i32).unsqueeze(0), total_blocks - 1)
-              .to(torch::kInt32)
-              .contiguous();
-      torch::Tensor dk = torch::empty({total_blocks, bs, num_kv_heads_, head_size_}, query.options());
-      torch::Tensor dv = torch::empty_like(dk);
+      // The copy and its block table live in buffers that every layer of the process shares, one set per
+      // (device, stream), grown to the largest step seen and then reused: layer after layer on a stream consumes
+      // its copy before the next one overwrites it.  The table and the rows' offsets depend on the lengths alone:
+      // layer 0 of a step makes them (plan_info.layer_id; every call if the metadata carries no plan_info).
+      PlanInfo* plan_info = attn_metadata.plan_info.get();
+      DenseCopy& dc = dense_copy(query.device(), query.options(), total_blocks * bs * num_kv_heads_ * head_size_);
+      if (plan_info == nullptr || plan_info->layer_id == 0 || !dc.table.defined()) {
+        const auto i32 = torch::TensorOptions().dtype(torch::kInt32).device(query.device());
+        torch::Tensor blocks_per_seq = torch::div(attn_metadata.kv_seq_lens + (bs - 1), bs, "floor").to(torch::kInt32);
+        torch::Tensor first_block = (torch::cumsum(blocks_per_seq, 0) - blocks_per_seq).to(torch::kInt32);
+        const int64_t max_blocks = (attn_metadata.max_seq_len + bs - 1) / bs;
+        dc.table = torch::clamp_max(first_block.unsqueeze(1) + torch::arange(max_blocks, i32).unsqueeze(0), total_blocks - 1)
+                       .to(torch::kInt32)
+                       .contiguous();
+        dc.row_offset = (first_block * bs).to(torch::kInt32);
+      }
+      TORCH_CHECK(dc.table.size(0) == batch, "the dense copy's block table was made for another batch: layer 0 of the step must come first");
+      torch::Tensor dk = dc.k.narrow(0, 0, total_blocks * bs * num_kv_heads_ * head_size_).view({total_blocks, bs, num_kv_heads_, head_size_});
+      torch::Tensor dv = dc.v.narrow(0, 0, total_blocks * bs * num_kv_heads_ * head_size_).view({total_blocks, bs, num_kv_heads_, head_size_});
       xllm::kernel::ReshapeFromCacheParams g;
       g.key = dk.view({-1, num_kv_heads_, head_size_});
       g.value = dv.view({-1, num_kv_heads_, head_size_});
@@ -118,7 +169,7 @@ void AttentionImpl::decoder_forward(const AttentionMetadata& attn_metadata, torc
       g.value_cache = v_cache;
       g.context_lengths = attn_metadata.kv_seq_lens;
       g.max_context_len = attn_metadata.max_seq_len;
-      g.context_seq_offset = (first_block * bs).to(torch::kInt32);
+      g.context_seq_offset = dc.row_offset;
       g.block_tables = attn_metadata.block_table;
       g.key_cache_quant_scale = k_cache_scale;
       g.value_cache_quant_scale = v_cache_scale;
@@ -126,9 +177,9 @@ void AttentionImpl::decoder_forward(const AttentionMetadata& attn_metadata, torc
       // the dense copy is token-major ([blocks, slots, heads, dim]); the kernels take its HND view
       xllm::kernel::hip::batch_prefill_paged(q3, dk.permute({0, 2, 1, 3}), dv.permute({0, 2, 1, 3}), o3, output_lse,
                                              attn_metadata.q_cu_seq_lens, attn_metadata.kv_seq_lens, std::nullopt,
-                                             std::nullopt, dense_table, attn_metadata.max_query_len,
+                                             std::nullopt, dc.table, attn_metadata.max_query_len,
                                              attn_metadata.max_seq_len, scale_, sliding_window_, false,
-                                             attn_metadata.total_kv_len);
+                                             attn_metadata.total_kv_len, plan_info);
       return;
     }
     xllm::kernel::hip::batch_prefill_paged(q3, k_cache, v_cache, o3, output_lse, attn_metadata.q_cu_seq_lens,

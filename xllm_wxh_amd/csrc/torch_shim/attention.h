@@ -48,6 +48,9 @@ class AttentionImpl {
   // the order of operations of the reference's MLU layer (xllm/core/layers/mlu/attention.cpp:179-228);
   // with that many row groups per sequence one conversion is cheaper than one per row group
   // (2 x 2048 tokens on 6144: 710 us against 840 us in place; 4 x 512 on 3584: 261 against 256).
+  // The copy lives in buffers shared by all layers, one set per (device, stream), grown outside stream capture to
+  // the largest step seen and then reused; with AttentionMetadata::plan_info, layer 0 makes the copy's block table
+  // and the step's schedule and later layers reuse both.
   // 0 disables the dense route.
   void set_prefill_dequant_rows(int64_t rows) { prefill_dequant_rows_ = rows; }
 
