@@ -656,6 +656,15 @@ def test_schedule_built_at_layer_zero_serves_every_layer(gpu, shim, kv, n):
     with pytest.raises(RuntimeError, match="layer 0"):
         attend(c0, 1)
     md.block_table = other
+    # ... or that comes after one of the library's switches was toggled (they shape the work items), or with a cache
+    # in another layout
+    from xllm_wxh_amd import ops
+
+    attend(c0, 0)
+    with ops.option("separate_merge", 1):
+        with pytest.raises(RuntimeError, match="layer 0"):
+            attend(c0, 1)
+    attend(c0, 1)
 
 
 @pytest.mark.gpu

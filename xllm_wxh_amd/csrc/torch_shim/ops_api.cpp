@@ -267,15 +267,25 @@ uint64_t plan_key(const xllm_hip_kv_cache& c, const xllm_hip_decode_args& a) {
                              (uint64_t)c.head_dim,
                              (uint64_t)c.block_size,
                              (uint64_t)c.num_blocks,
-                             // the kernel family chosen (it also depends on strides and alignments)
+                             // the layout decides the shape of the work items (kv heads side by side: four to an item)
+                             (uint64_t)c.stride_block,
+                             (uint64_t)c.stride_head,
+                             (uint64_t)c.stride_slot,
+                             (uint64_t)c.scale_stride_block,
+                             (uint64_t)c.scale_stride_head,
+                             (uint64_t)c.scale_stride_slot,
+                             // the kernel family chosen (it also depends on alignments)
                              (uint64_t)(uintptr_t)xllm_hip_paged_decode_variant(&c, &a)};
   uint64_t h = 1469598103934665603ull;
-  for (uint64_t f : fields) {
+  auto mix = [&](uint64_t f) {
     for (int i = 0; i < 8; ++i) {
       h ^= (f >> (8 * i)) & 0xff;
       h *= 1099511628211ull;
     }
-  }
+  };
+  // ... and so do the library's diagnostic switches: one toggled between two layers changes it under the schedule
+  for (int32_t o = 0; o < XLLM_HIP_OPTION_COUNT; ++o) mix((uint64_t)xllm_hip_get_option(o));
+  for (uint64_t f : fields) mix(f);
   return h;
 }
 
