@@ -399,6 +399,15 @@ def main():
                          plan=plan, run=not plan)
 
     def run_loop_us():
+        # (the legs before this one end in host-side pauses — graph captures, synchronisations — after which the
+        # first few hundred launches run up to 15 % slower: settle as before the main leg)
+        t_settle = time.perf_counter()
+        i = 0
+        while (time.perf_counter() - t_settle) * 1e3 < args.settle_ms:
+            plan_or_run(i, False)
+            i += 1
+            if i % 16 == 0:
+                torch.cuda.synchronize()
         for i in range(max(3, args.warmup // 2)):
             plan_or_run(i, False)
         torch.cuda.synchronize()
@@ -436,6 +445,8 @@ def main():
         # `value` (plan + run per call) and `run_us` (runs on an existing schedule) in alternating legs, so that a
         # drift of the clocks over the benchmark's run shows in both series instead of between them
         full, runs = [], []
+        for i in range(per):  # (settled: see run_loop_us)
+            step(i)
         for _ in range(rounds):
             torch.cuda.synchronize()
             t = time.perf_counter()
