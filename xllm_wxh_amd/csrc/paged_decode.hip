@@ -29,7 +29,6 @@
 #include "decode_merge.h"
 #include "decode_mfma.h"
 #include "prefill_pingpong.h"
-#include "prefill_pingpong32.h"
 #include "decode_generic.h"
 
 #include <math.h>
@@ -548,14 +547,7 @@ static int64_t max_items(const DecodeParams& p) {
 template <int KV_DT, int TOK>
 static void launch_mfma_tok(const DecodeParams& p, unsigned grid, hipStream_t st) {
   if (p.rows_per_item == kPrefillWideRows) {
-    if constexpr (!quant_of(KV_DT) && TOK == 1) {
-      // (the 32x32x16 MFMA: half as many MFMA issues per tile; option bit 2: the 16x16x32 form, for comparisons)
-      if (p.prefill_opts & 4) {
-        prefill_pingpong_d128_kernel<KV_DT, TOK><<<grid, 512, 0, st>>>(p);
-      } else {
-        prefill_pingpong_wide_d128_kernel<KV_DT><<<grid, 512, 0, st>>>(p);
-      }
-    }
+    if constexpr (!quant_of(KV_DT) && TOK == 1) prefill_pingpong_d128_kernel<KV_DT, TOK><<<grid, 512, 0, st>>>(p);
     if constexpr (quant_of(KV_DT) && TOK == 1) prefill_pingpong_quant_d128_kernel<KV_DT><<<grid, 512, 0, st>>>(p);
   } else if (p.rows_per_item == kPrefillRowsPerItem) {
     if constexpr (!quant_of(KV_DT) && TOK != 0) prefill_mfma_d128_kernel<KV_DT, TOK><<<grid, 256, 0, st>>>(p);
