@@ -483,25 +483,31 @@ struct PingPongQuantLoader {
     r.kfac = LDS_SCALE ? *lds_scale : scale_log2;
     return r;
   }
-  // The wave's rows of the tile at tb: converted (K, V, per-token factors) into `conv`.
-  template <bool MASKED>
-  __device__ inline void store(const Raw& rw, uint8_t* conv, int tb, int len) const {
+  // The wave's rows of the tile at tb: converted (K, V, per-token factors) into `conv`.  `dst`: where in a
+  // converted tile this lane's two 16-byte pieces go (conv_offset; it depends on the lane alone and is kept in a
+  // register: formed anew for every tile it was a third of the conversion's instructions).
+  __device__ inline uint32_t conv_offset() const {
     int row4, chunk;
     row_chunk(row4, chunk);
     const int row = 4 * wave + row4;
+    return lane >= 32 ? kLdsV + swz_v(row, 2 * chunk) : kLdsK + swz_k(row, 2 * chunk);
+  }
+  template <bool MASKED>
+  __device__ inline void store(const Raw& rw, uint8_t* conv, uint32_t dst, int tb, int len) const {
     u32x4 lo, hi;
     dequant16<KV_DT>(rw.bytes, lo, hi);
-    uint32_t off = kLdsK + swz_k(row, 2 * chunk);
-    if (lane >= 32) {
-      if constexpr (kv_of(KV_DT) == XLLM_HIP_INT8) {  // 1152 + x -> x, exact in fp16 (see QuantPrefillLoader::convert)
-        lo = __builtin_bit_cast(u32x4, __builtin_bit_cast(f16x8, lo) - (_Float16)kInt8Offset);
-        hi = __builtin_bit_cast(u32x4, __builtin_bit_cast(f16x8, hi) - (_Float16)kInt8Offset);
-      }
-      if (MASKED && tb + row >= len) lo = hi = u32x4{0, 0, 0, 0};
-      off = kLdsV + swz_v(row, 2 * chunk);
+    if constexpr (kv_of(KV_DT) == XLLM_HIP_INT8) {  // V rows: 1152 + x -> x, exact in fp16 (see QuantPrefillLoader::convert)
+      const _Float16 sub = lane >= 32 ? (_Float16)kInt8Offset : (_Float16)0.0f;
+      lo = __builtin_bit_cast(u32x4, __builtin_bit_cast(f16x8, lo) - sub);
+      hi = __builtin_bit_cast(u32x4, __builtin_bit_cast(f16x8, hi) - sub);
     }
-    *(u32x4*)(conv + off) = lo;
-    *(u32x4*)(conv + (off ^ 16)) = hi;
+    if (MASKED && lane >= 32) {
+      int row4, chunk;
+      row_chunk(row4, chunk);
+      if (tb + 4 * wave + row4 >= len) lo = hi = u32x4{0, 0, 0, 0};
+    }
+    *(u32x4*)(conv + dst) = lo;
+    *(u32x4*)(conv + (dst ^ 16)) = hi;
     if (lane < 8) {
       const int t = 4 * wave + (lane & 3);  // token of the tile
       const bool is_v = lane >= 4;
@@ -572,6 +578,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pingpong_quant_d128_kernel(Dec
 
   PingPongQuantLoader<KV_DT> ld;
   ld.init(p, wave, lane);
+  const uint32_t conv_dst = ld.conv_offset();
   const int mine = 4 * wave;  // first of the tokens this wave fetches, within a tile
 
   auto barrier = [&]() __attribute__((always_inline)) {
@@ -674,9 +681,9 @@ __global__ void __launch_bounds__(512, 2) prefill_pingpong_quant_d128_kernel(Dec
     const int tb = w_begin + (i + 1) * kT;
     uint8_t* conv = lds + ((PH + 1) % kConv) * kLdsTile;
     if (tb + kT > it.len) {
-      ld.template store<true>(rw, conv, tb, it.len);
+      ld.template store<true>(rw, conv, conv_dst, tb, it.len);
     } else {
-      ld.template store<false>(rw, conv, tb, it.len);
+      ld.template store<false>(rw, conv, conv_dst, tb, it.len);
     }
     __builtin_amdgcn_sched_barrier(0);  // (the raw bytes are in registers: their buffer may be written)
     ld.issue(p, it, tb + kRaw * kT, blk, raws + ((i + 1) & (kRaw - 1)) * kPingPongRawTile);
