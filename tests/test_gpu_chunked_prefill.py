@@ -322,9 +322,8 @@ def test_256_row_kernel_against_the_128_row_kernel_and_the_oracle(gpu, qdt, bs, 
     assert d["waves_per_workgroup"] == 8, d
 
 
-@pytest.mark.parametrize("kv", ["fp8", "int8"])
-@pytest.mark.parametrize("qdt", ["bf16", "fp16"])
-@pytest.mark.parametrize("bs,layout", [(16, "HND"), (128, "NHD")])
+@pytest.mark.parametrize("kv,qdt,bs,layout", [("fp8", "bf16", 16, "HND"), ("int8", "fp16", 16, "HND"),
+                                               ("fp8", "fp16", 128, "NHD"), ("int8", "bf16", 128, "NHD")])
 def test_256_row_kernel_over_one_byte_caches(gpu, kv, qdt, bs, layout):
     """The same over a 1-byte cache: raw bytes and scales reach LDS by DMA and each wave converts its rows of the
     next tile during its matrix phase, three converted tiles rotating.  Its straight-line loop takes the tiles
