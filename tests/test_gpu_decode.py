@@ -232,17 +232,23 @@ def test_nhd_layout_and_csr_form(gpu, kv):
 
 
 @pytest.mark.parametrize("kv,qdt", [("bf16", "bf16"), ("fp8", "bf16"), ("int8", "bf16"), ("fp16", "fp16"), ("int8", "fp16")])
-@pytest.mark.parametrize("Hq,Hkv,n", [(32, 8, 1), (32, 8, 4), (16, 4, 2), (64, 8, 2), (12, 12, 1)])
+@pytest.mark.parametrize("Hq,Hkv,n", [(32, 8, 1), (32, 8, 4), (16, 4, 2), (64, 8, 2), (12, 12, 1), (64, 8, 4), (32, 8, 5)])
 def test_work_items_of_four_kv_heads_over_nhd(gpu, kv, qdt, Hq, Hkv, n):
     """Over a 1-byte cache whose kv heads lie side by side within a token (NHD) the 16-row kernel at head_dim
     128 gives a work item four neighbouring kv heads, one per wave, each wave attending all of the chunk's
-    tokens (16-bit caches, and head counts that are no multiple of four, keep one head per item).  Long and short sequences (split into chunks and merged inside the kernel, or by the merge
+    tokens, and the 32-row kernel (17 to 32 query rows per kv head: the last two shapes) a pair of waves per head,
+    eight waves to the workgroup (16-bit caches, and head counts that are no multiple of four, keep one head per item).  Long and short sequences (split into chunks and merged inside the kernel, or by the merge
     kernel), an empty one, host-side lengths (no stored schedule) and none, a sliding window — against the
     oracle, and against the same step with one kv head per item."""
     print("case four heads per item", kv, qdt, Hq, Hkv, n, flush=True)
     lens = [9000, 300, 0, 33, 4100, 17]
     case = Case(len(lens), Hq, Hkv, 128, 16, lens, n=n, kv=kv, qdt=qdt, layout="NHD", seed=93)
     assert case.variant() == "mfma_d128"
+    shape = ops.decode_describe(case.q, case.k_cache, case.v_cache, case.block_table, case.seq_lens, case.k_scale, case.v_scale,
+                                q_per_seq=n, kv_layout="NHD")
+    assert shape["kv_heads_per_item"] == (4 if kv in ("fp8", "int8") and Hkv % 4 == 0 else 1), shape
+    if n * (Hq // Hkv) > 16:
+        assert shape["waves_per_workgroup"] == (8 if shape["kv_heads_per_item"] == 4 else 2), shape
     tol = {"bf16": REG_TOL, "fp16": 2e-3}.get(kv, REG_TOL_QUANT)
     lse_tol = LSE_TOL
     for window in (-1, 300):

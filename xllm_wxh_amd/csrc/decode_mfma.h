@@ -1222,13 +1222,17 @@ __global__ void __launch_bounds__(64 * WAVES, decode_waves_per_simd(TOK)) decode
 // head_dim 256 over a 16-bit cache: one wave per SIMD (its two tile stages alone are 64 registers).
 constexpr int rows32_waves_per_simd(int kv_dt, int tok) { return tok == 0 && !quant_of(kv_dt) ? 1 : 2; }
 
-template <int KV_DT, int TOK>
-__global__ void __launch_bounds__(128, rows32_waves_per_simd(KV_DT, TOK)) decode_mfma_d128_rows32_kernel(DecodeParams p) {
-  // A workgroup is one pair of waves: wave w owns query rows 16w .. 16w+15 and fetches rows 16w ..
+// PAIRS = 4: a work item of four kv heads whose rows lie side by side within a token (a 1-byte cache in the NHD
+// layout), one pair of waves per head, eight waves to the workgroup and one such workgroup to a CU: the four pairs
+// walk the same tokens in step (they meet at every tile's barrier), so that what the workgroup asks of memory at
+// a time is a run of four rows, 512 bytes, instead of single rows a token's width apart.
+template <int KV_DT, int TOK, int PAIRS = 1>
+__global__ void __launch_bounds__(128 * PAIRS, rows32_waves_per_simd(KV_DT, TOK)) decode_mfma_d128_rows32_kernel(DecodeParams p) {
+  // A pair of waves: wave w of it owns query rows 16w .. 16w+15 and fetches rows 16w ..
   // of every tile.  A tile is parked while both waves still read the previous one from the other
-  // buffer, so one barrier (of two waves) per tile suffices.  Four such workgroups share a CU.
-  __shared__ __attribute__((aligned(16))) uint8_t lds_all[2 * kLdsTile];
-  __shared__ float lds_ml[2 * 16 * 2];
+  // buffer, so one barrier per tile suffices.  Four such pairs share a CU.
+  __shared__ __attribute__((aligned(16))) uint8_t lds_pairs[PAIRS * 2 * kLdsTile];
+  __shared__ float lds_ml_pairs[PAIRS * 2 * 16 * 2];
 
   constexpr int kT = tile_tokens_of(TOK);  // tokens per tile
   constexpr int kH = half_tokens_of(TOK);  // tokens from the tile's first half to its second
@@ -1238,10 +1242,19 @@ __global__ void __launch_bounds__(128, rows32_waves_per_simd(KV_DT, TOK)) decode
   Item it;
   if (!decode_item(p, blockIdx.x, it)) return;
 
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wave_of_group = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int pair = PAIRS > 1 ? wave_of_group >> 1 : 0;
+  const int wave = wave_of_group & 1;  // within the pair
   const int rs = wave;  // row set; also the tile half this wave fetches
   const int lane = threadIdx.x & 63;
+  uint8_t* lds_all = lds_pairs + pair * (2 * kLdsTile);
+  float* lds_ml = lds_ml_pairs + pair * (2 * 16 * 2);
   uint8_t* tiles = lds_all;
+  if (PAIRS > 1) {  // (the item names the first of its kv heads)
+    it.hk += pair;
+    it.head_off = (int64_t)it.hk * p.stride_head;
+    it.sc_head_off = (int64_t)it.hk * p.sc_stride_head;
+  }
 
   constexpr bool kRawK = raw_k_of(KV_DT, TOK);
   constexpr bool kInt8 = kv_of(KV_DT) == XLLM_HIP_INT8;

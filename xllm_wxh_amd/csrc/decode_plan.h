@@ -147,8 +147,11 @@ constexpr int kDefaultCUs = 256;
 // Up to 16 query rows per kv head, over a cache whose kv heads lie side by side within a token, a work item
 // covers four kv heads (one per wave of the 16-row kernel) when the head count allows it.
 constexpr int kHeadsPerItem = 4;
-inline int item_heads_of(int rows, int num_kv_heads, bool heads_side_by_side) {
-  return heads_side_by_side && rows <= 16 && num_kv_heads % kHeadsPerItem == 0 ? num_kv_heads / kHeadsPerItem : num_kv_heads;
+// (17 to 32 rows: the 32-row kernel's form of the same, a pair of waves per head; `rows32` says that the caller means it)
+inline int item_heads_of(int rows, int num_kv_heads, bool heads_side_by_side, bool rows32 = false) {
+  return heads_side_by_side && (rows <= 16 || (rows32 && rows <= 32)) && num_kv_heads % kHeadsPerItem == 0
+             ? num_kv_heads / kHeadsPerItem
+             : num_kv_heads;
 }
 inline int natural_target_items(bool mfma, int rows, bool one_wave_per_simd, int cus = kDefaultCUs) {
   int v = !mfma ? 8 * cus : (rows > 16 && rows <= kPrefillMinRows) ? 4 * cus : 2 * cus;

@@ -314,6 +314,10 @@ static int fill_params(const xllm_hip_kv_cache* c,
   const bool side_by_side_pays = !(a->max_seq_len > 0 && a->total_kv_len > 0 && nearly_equal) ||
                                  wider_items_pay((int64_t)p.batch * c->num_kv_heads, kHeadsPerItem, R.side_by_side_gain);
   p.item_heads = item_heads_of(p.rows, c->num_kv_heads, (side_by_side && side_by_side_pays) || short_sequences);
+  // 17 to 32 rows per kv head over such a cache (the heads side by side, rows of 128 bytes): the 32-row kernel's
+  // form of the four-head item, eight waves to the workgroup and one workgroup to a CU.
+  const bool side_by_side32 = side_by_side && p.rows > 16 && p.rows <= kMaxRowsPerItem && p.rows_per_item == kMaxRowsPerItem;
+  if (side_by_side32) p.item_heads = item_heads_of(p.rows, c->num_kv_heads, true, true);
   p.heads_per_item = c->num_kv_heads / p.item_heads;
   p.head_dim = c->head_dim;
   p.block_size = c->block_size;
@@ -329,6 +333,8 @@ static int fill_params(const xllm_hip_kv_cache* c,
   // 32-row kernel over a 1-byte cache, which fits two
   const bool one_wave_per_simd = variant == kMfmaD256 && !(p.rows > 16 && quant);
   p.target_items = target_items(is_mfma(variant), p.rows, one_wave_per_simd);
+  // (the 32-row kernel's four-head items: one workgroup of eight waves per CU where four of two waves are)
+  if (side_by_side32 && p.heads_per_item > 1) p.target_items = p.target_items / kHeadsPerItem > 0 ? p.target_items / kHeadsPerItem : 1;
   // A small batch on the 16-row kernel: one of the two workgroups a CU holds (the 32-row kernel wants
   // all its slots filled: 4 x 32768 tokens of int8 with 4 draft tokens, 65 us at 1024 items, 84 at 512).
   // (work items of four kv heads keep every slot as the target: each of their waves streams a head of its own,
@@ -570,6 +576,12 @@ static void launch_mfma_tok(const DecodeParams& p, unsigned grid, hipStream_t st
     }
     decode_mfma_d128_kernel<KV_DT, TOK><<<grid, 64 * kWaves, 0, st>>>(p);
   } else {
+    if constexpr (TOK == 1 && quant_of(KV_DT)) {
+      if (p.heads_per_item > 1) {
+        decode_mfma_d128_rows32_kernel<KV_DT, TOK, kHeadsPerItem><<<grid, 128 * kHeadsPerItem, 0, st>>>(p);
+        return;
+      }
+    }
     decode_mfma_d128_rows32_kernel<KV_DT, TOK><<<grid, 128, 0, st>>>(p);
   }
 }
@@ -638,7 +650,7 @@ extern "C" int xllm_hip_paged_decode_describe(const xllm_hip_kv_cache* cache,
     } else if (p.rows_per_item == kPrefillRowsPerItem) {
       waves = 4;
     } else if (p.rows > 16) {
-      waves = 2;
+      waves = p.heads_per_item > 1 ? 2 * kHeadsPerItem : 2;
     } else if (p.heads_per_item > 1 || p.wave_items) {
       waves = 4;
       per_workgroup = p.wave_items == 2 ? 2 : (p.wave_items == 1 ? 4 : 1);
