@@ -179,12 +179,11 @@ def test_thirty_three_to_sixty_four_rows(gpu, g, n, D, bs, qdt):
         assert float(np.abs(out_r - ref_r).max()) <= 1.2e-2
 
 
-@pytest.mark.parametrize("kv", ["fp8", "int8"])
-@pytest.mark.parametrize("bs", [16, 128])
-@pytest.mark.parametrize("qdt", ["bf16", "fp16"])
+@pytest.mark.parametrize("kv,bs,qdt", [("fp8", 16, "bf16"), ("int8", 16, "fp16"), ("fp8", 128, "fp16"), ("int8", 128, "bf16")])
 def test_many_row_kernel_over_one_byte_caches(gpu, kv, bs, qdt):
-    """1-byte caches at head_dim 128 with more than 32 query rows per kv head take the 128-row kernel
-    that brings raw bytes and scales to LDS and converts each tile once per row group: lengths around
+    """1-byte caches at head_dim 128 with more than 32 query rows per kv head take the many-row kernels
+    that bring raw bytes and scales to LDS and convert each tile once per row group (here, with up to 1200 rows
+    per kv head, the 256-row one; the 128-row one in the next test and beside the 256-row one further down): lengths around
     its tile (32 tokens) and its four raw buffers, chunks that are the whole sequence, chunks shorter
     than one row group, sequences without query tokens; then a sliding window."""
     print("case many rows, 1-byte cache", kv, bs, qdt, flush=True)
