@@ -161,6 +161,9 @@ inline bool host_schedule(const HostScheduleInput& in, const WorkspaceLayout& w,
   sizes.reserve((size_t)room);
   const int kNum[7] = {0, 1, 2, 3, 4, 6, 8};  // halves of the slots
   for (int k = 0; k < 7; ++k) {
+    // (a cut aimed at a quarter as many chunks as there are sequences changes nothing that matters — a batch of
+    // that many rounds is balanced by its number — so a large batch ends here, after one pass over its lengths)
+    if (kNum[k] > 0 && 2 * lanes * kNum[k] <= in.batch) continue;
     int64_t target = 0;
     if (kNum[k] > 0) {
       target = (2 * total + lanes * kNum[k] - 1) / (lanes * kNum[k]);
@@ -183,6 +186,10 @@ inline bool host_schedule(const HostScheduleInput& in, const WorkspaceLayout& w,
       target += std::max<int64_t>(in.tile, target / 32 / in.tile * in.tile);
     }
     const bool fits = count <= room;
+    if (kNum[k] == 0 && fits && 2 * lanes * kNum[6] <= in.batch) {  // (the only candidate: its finishing time is not asked for)
+      best_span = 0.0;
+      continue;
+    }
     if (fits && (target == best_target && best_span >= 0.0)) continue;  // (the same cut as the best so far)
     int32_t most = 1;
     sizes.clear();
