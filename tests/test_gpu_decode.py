@@ -792,6 +792,10 @@ def test_four_head_items_for_many_short_sequences(gpu, name, kv, qdt, layout, Hq
     ("two kv heads, bf16, two draft tokens", "bf16", "bf16", "HND", 14, 2, 2, 32, [1500] * 1024),
     ("eight kv heads, fp8 over NHD", "fp8", "fp16", "NHD", 32, 8, 1, 64, [411] * 256),
     ("eight kv heads, fp16, ragged", "fp16", "fp16", "HND", 32, 8, 1, 32, None),
+    # rows of 64 bytes, two kv heads to a 128-byte line: the waves of a workgroup walk their tokens in step, each
+    # as many tiles as the longest of the four (lengths either side of a tile's end)
+    ("two kv heads, int8 over NHD, a wave per item", "int8", "bf16", "NHD", 14, 2, 1, 32, [250 + 5 * (i % 7) for i in range(1024)]),
+    ("two kv heads, fp8 over NHD, two waves per item", "fp8", "bf16", "NHD", 14, 2, 1, 32, [1000 + 9 * (i % 5) for i in range(1000)]),
 ])
 def test_items_per_wave_at_head_dim_64(gpu, name, kv, qdt, layout, Hq, Hkv, n, bs, lens):
     """The same work items (four kv heads, or four neighbouring items, one per wave) at head_dim 64."""
@@ -803,6 +807,11 @@ def test_items_per_wave_at_head_dim_64(gpu, name, kv, qdt, layout, Hq, Hkv, n, b
         lens[3] = 9000
     case = Case(len(lens), Hq, Hkv, 64, bs, lens, n=n, kv=kv, qdt=qdt, layout=layout, seed=73)
     assert case.variant() == "mfma_d64"
+    if "per item" in name:
+        lens_np = np.asarray(lens)
+        shape = ops.decode_describe(case.q, case.k_cache, case.v_cache, case.block_table, case.seq_lens, case.k_scale, case.v_scale,
+                                    q_per_seq=n, kv_layout=layout, max_seq_len=int(lens_np.max()), total_kv_len=int(lens_np.sum()))
+        assert shape["items_per_workgroup"] == (4 if "a wave per item" in name else 2), shape
     tol = {"bf16": REG_TOL, "fp16": 2e-3}.get(kv, REG_TOL_QUANT)
     ref, lse_ref = case.oracle()
     out, lse = case.run(hints=True)

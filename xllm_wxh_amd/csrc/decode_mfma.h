@@ -155,6 +155,7 @@ struct KvHalf16 {
   u32x4 v[4];
 
   // `plane` (head_dim 256 only): 0 = elements 0..127 of the 16 tokens, 1 = elements 128..255.
+  template <bool KEEP = false>
   __device__ inline void issue(const DecodeParams& p, const Item& it, int tok, int blk, const Geom& g, int plane = 0) {
     const HalfBase b = half_base(p, it, tok, blk);
     const uint8_t* kb = p.k_cache + b.elem * 2 + plane * 256;
@@ -316,14 +317,22 @@ struct KvHalfQuant {
   // `plane` (head_dim 256 only): 0 = elements 0..127 of the 16 tokens, 1 = elements 128..255.  Both
   // planes carry the tokens' scales (the second copy comes from the cache and lands in the unused
   // half of the factor arrays).
+  // KEEP: ordinary loads, whose lines may stay in the CU's cache, for a workgroup whose other waves ask for the
+  // rest of the same lines.
+  template <bool KEEP = false>
   __device__ inline void issue(const DecodeParams& p, const Item& it, int tok, int blk, const Geom& g, int plane = 0) {
     const HalfBase b = half_base(p, it, tok, blk);
     const uint8_t* kb = p.k_cache + b.elem + plane * 128;
     const uint8_t* vb = p.v_cache + b.elem + plane * 128;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      k[j] = ldg_stream(kb + j * 8 * p.stride_slot * g.tok + g.gk_off);
-      v[j] = ldg_stream(vb + j * 4 * p.stride_slot * g.tok + g.gv_off);
+      if constexpr (KEEP) {
+        k[j] = *(const u32x4*)(kb + j * 8 * p.stride_slot * g.tok + g.gk_off);
+        v[j] = *(const u32x4*)(vb + j * 4 * p.stride_slot * g.tok + g.gv_off);
+      } else {
+        k[j] = ldg_stream(kb + j * 8 * p.stride_slot * g.tok + g.gk_off);
+        v[j] = ldg_stream(vb + j * 4 * p.stride_slot * g.tok + g.gv_off);
+      }
     }
     const float* sb = (g.sc_is_v ? p.v_scale : p.k_scale) + b.scale;
     if (g.sc_on) sc = *(const float*)((const uint8_t*)sb + g.sc_g);
@@ -1096,9 +1105,15 @@ constexpr int decode_waves_per_simd(int tok) { return tok == 0 ? 1 : 2; }
 // 1-byte cache has at most one item per CU, as a small batch cut into 32 chunks per sequence has: a wave
 // has one tile in flight and converts it before it asks for the next, so four waves leave the CU's memory
 // pipe idle much of the time, and cutting finer instead costs more in the merge than it gains.
-template <int KV_DT, int TOK, bool HEADS = false, int WAVES = kWaves>
+//
+// LOCK (with HEADS, for cache rows shorter than a 128-byte line whose neighbour in the line is the next kv head's
+// row, which another wave of the workgroup attends): the four waves meet before every tile and load with ordinary
+// loads, so that the two halves of a line are asked for at about the same time, the second finds it in the CU's
+// cache, and the line crosses HBM once.
+template <int KV_DT, int TOK, bool HEADS = false, int WAVES = kWaves, bool LOCK = false>
 __global__ void __launch_bounds__(64 * WAVES, decode_waves_per_simd(TOK)) decode_mfma_d128_kernel(DecodeParams p) {
   static_assert(!(HEADS && WAVES != kWaves) && !(TOK == 0 && WAVES != kWaves), "eight waves: head_dim 64 and 128, one kv head per item");
+  static_assert(!LOCK || HEADS, "in step: waves that attend neighbouring kv heads");
   __shared__ __attribute__((aligned(16))) uint8_t lds_all[WAVES * kLdsTile];
   __shared__ float lds_ml[WAVES * 16 * 2];  // (running max, denominator) per wave and query row
   __shared__ int lds_last;
@@ -1175,8 +1190,8 @@ __global__ void __launch_bounds__(64 * WAVES, decode_waves_per_simd(TOK)) decode
       st[1].template park<false, kRawK>(tile, 1, tb + kH, it.len, park_scale, geom);
     }
     if (tb + kT < w_end) {
-      st[0].issue(p, it, tb + kT, blk[0], geom);
-      st[1].issue(p, it, tb + kT + kH, blk[1], geom, kP1);
+      st[0].template issue<LOCK>(p, it, tb + kT, blk[0], geom);
+      st[1].template issue<LOCK>(p, it, tb + kT + kH, blk[1], geom, kP1);
     }
     blk[0] = nblk0;
     blk[1] = nblk1;
@@ -1186,9 +1201,27 @@ __global__ void __launch_bounds__(64 * WAVES, decode_waves_per_simd(TOK)) decode
       rt.template attend<false>(tile, tb, p.scale_log2);
     }
   };
-  if (w_begin < w_end) {
-    st[0].issue(p, it, w_begin, block_of(p, it, w_begin), geom);
-    st[1].issue(p, it, w_begin + kH, block_of(p, it, w_begin + kH), geom, kP1);
+  if constexpr (LOCK) {
+    // In step: every wave walks as many tiles as the workgroup's longest share has, and the four meet before
+    // each — every wave reaches every barrier, with or without a tile of its own.
+    __shared__ int lds_tiles[kWaves];
+    if (lane == 0) lds_tiles[wave] = w_begin < w_end ? (w_end - w_begin + kT - 1) / kT : 0;
+    __syncthreads();
+    const int tiles = __builtin_amdgcn_readfirstlane(max(max(lds_tiles[0], lds_tiles[1]), max(lds_tiles[2], lds_tiles[3])));
+    if (w_begin < w_end) {
+      st[0].template issue<LOCK>(p, it, w_begin, block_of(p, it, w_begin), geom);
+      st[1].template issue<LOCK>(p, it, w_begin + kH, block_of(p, it, w_begin + kH), geom, kP1);
+      blk[0] = block_of(p, it, w_begin + kT);
+      blk[1] = block_of(p, it, w_begin + kT + kH);
+    }
+    int tb = w_begin;
+    for (int i = 0; i < tiles; ++i, tb += kT) {
+      __builtin_amdgcn_s_barrier();
+      if (tb < w_end) step(tb);
+    }
+  } else if (w_begin < w_end) {
+    st[0].template issue<LOCK>(p, it, w_begin, block_of(p, it, w_begin), geom);
+    st[1].template issue<LOCK>(p, it, w_begin + kH, block_of(p, it, w_begin + kH), geom, kP1);
     blk[0] = block_of(p, it, w_begin + kT);
     blk[1] = block_of(p, it, w_begin + kT + kH);
     for (int tb = w_begin; tb < w_end; tb += kT) step(tb);

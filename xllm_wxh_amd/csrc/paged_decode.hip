@@ -517,6 +517,18 @@ static int fill_params(const xllm_hip_kv_cache* c,
     };
     heads_per_line = shared_by(c->stride_head * elem_bytes(c->dtype));
     if (quant) heads_per_line = max(heads_per_line, shared_by(c->scale_stride_head * 4));
+    // Cache rows shorter than a line, and waves of a workgroup that attend neighbouring kv heads (1-byte caches at
+    // head_dim 64 over NHD): the waves walk their tokens in step, a barrier per tile, and load with ordinary loads
+    // instead of streaming ones, so that the halves of a line are asked for together — the second from the CU's
+    // cache — and cross HBM once.  int8, 2 kv heads, 512 x 8192 tokens: 1.60x the algorithmic bytes fetched and
+    // 265 us as independent waves, 225 us in step (1.13x), 209 us with ordinary loads as well (HND 173); fp8
+    // 266 -> 206; 8 kv heads, 128 x 8192 tokens 314 -> 253 us, 1024 x 1024 tokens 268 -> 237.  Rows of a whole
+    // line gain nothing from it and lose the waves' independence (fp8, head_dim 128, 128 x 8192 tokens over
+    // NHD: 350 -> 365 us): not those.
+    p.lockstep = (p.wave_items || p.heads_per_item > 1) && c->num_kv_heads > 1 && quant && variant == kMfmaD64 &&
+                         shared_by(c->stride_head * elem_bytes(c->dtype)) > 1
+                     ? 1
+                     : 0;
     if (heads_per_line > c->num_kv_heads) heads_per_line = c->num_kv_heads;
     while (heads_per_line > 1 && c->num_kv_heads % heads_per_line != 0) --heads_per_line;
   }
@@ -561,6 +573,12 @@ static void launch_mfma_tok(const DecodeParams& p, unsigned grid, hipStream_t st
   } else if (p.rows <= 16) {
     if constexpr (TOK != 0) {
       if (p.heads_per_item > 1 || p.wave_items) {
+        if constexpr (TOK == 2 && quant_of(KV_DT)) {  // (the one shape whose rows are shorter than a line)
+          if (p.lockstep) {
+            decode_mfma_d128_kernel<KV_DT, TOK, true, kWaves, true><<<grid, 64 * kWaves, 0, st>>>(p);
+            return;
+          }
+        }
         decode_mfma_d128_kernel<KV_DT, TOK, true><<<grid, 64 * kWaves, 0, st>>>(p);
         return;
       }
