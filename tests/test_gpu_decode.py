@@ -787,6 +787,40 @@ def test_four_head_items_for_many_short_sequences(gpu, name, kv, qdt, layout, Hq
     assert torch.equal(out, out2) and torch.equal(lse, lse2)
 
 
+@pytest.mark.parametrize("kv,qdt", [("fp8", "bf16"), ("int8", "bf16"), ("int8", "fp16"), ("bf16", "bf16")])
+@pytest.mark.parametrize("Hq,Hkv,n", [(32, 8, 1), (16, 4, 2), (14, 2, 1)])
+def test_work_items_of_four_kv_heads_over_nhd_at_head_dim_64(gpu, kv, qdt, Hq, Hkv, n):
+    """head_dim 64 over a 1-byte NHD cache (rows of 64 bytes, two kv heads to a 128-byte line): work items of four kv
+    heads for any step, split sequences included, their waves walking the tokens in step; 16-bit caches and two kv
+    heads keep one head per item here (their steps are split)."""
+    print("case four heads per item, head_dim 64", kv, qdt, Hq, Hkv, n, flush=True)
+    lens = [9000, 300, 0, 33, 4100, 17, 64, 65]
+    case = Case(len(lens), Hq, Hkv, 64, 32, lens, n=n, kv=kv, qdt=qdt, layout="NHD", seed=97)
+    assert case.variant() == "mfma_d64"
+    shape = ops.decode_describe(case.q, case.k_cache, case.v_cache, case.block_table, case.seq_lens, case.k_scale, case.v_scale,
+                                q_per_seq=n, kv_layout="NHD")
+    assert shape["kv_heads_per_item"] == (4 if kv in ("fp8", "int8") and Hkv % 4 == 0 else 1), shape
+    tol = {"bf16": REG_TOL, "fp16": 2e-3}.get(kv, REG_TOL_QUANT)
+    for window in (-1, 300):
+        ref, lse_ref = case.oracle(window)
+        out, lse = case.run(window)
+        assert not torch.isnan(out.float()).any()
+        assert max_abs_err(out, ref) <= tol
+        assert lse_err(lse, lse_ref) <= LSE_TOL
+        with ops.option("item_per_head"):
+            out_1, _ = case.run(window)
+        assert max_abs_err(out_1, ref) <= tol
+        assert torch.allclose(out.float(), out_1.float(), rtol=2 ** -6, atol=4e-3)
+    out_h, lse_h = case.run(hints=True)
+    ref, lse_ref = case.oracle()
+    assert max_abs_err(out_h, ref) <= tol and lse_err(lse_h, lse_ref) <= LSE_TOL
+    # long equal sequences with host-side lengths: not split, a wave (or two) per (sequence, kv head)
+    eq = Case(300, Hq, Hkv, 64, 32, [1100 + (i % 3) for i in range(300)], n=n, kv=kv, qdt=qdt, layout="NHD", seed=98)
+    ref, lse_ref = eq.oracle()
+    out, lse = eq.run(hints=True)
+    assert max_abs_err(out, ref) <= tol and lse_err(lse, lse_ref) <= LSE_TOL
+
+
 @pytest.mark.parametrize("name,kv,qdt,layout,Hq,Hkv,n,bs,lens", [
     ("two kv heads, int8", "int8", "bf16", "HND", 14, 2, 1, 32, [260 - (i % 5) for i in range(1024)]),
     ("two kv heads, bf16, two draft tokens", "bf16", "bf16", "HND", 14, 2, 2, 32, [1500] * 1024),

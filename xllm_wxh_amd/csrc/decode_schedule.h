@@ -47,6 +47,10 @@ struct ShapeRules {
   // Four-head items over a 1-byte cache whose heads lie side by side gain this much from the layout alone
   // (fp8, 128 x 8192 tokens, NHD: 391 -> 338 us).
   double side_by_side_gain = 0.16;
+  // The same where the rows are 64 bytes and two kv heads share a 128-byte line (head_dim 64, 1-byte cache, NHD):
+  // waves that attend neighbouring heads in step, against four waves to a head (int8, 14q/2kv, 512 x 8192 tokens
+  // 259 -> 209 us; 32q/8kv, 64 x 16384 tokens 314 -> 232).
+  double short_rows_gain = 0.24;
   // Narrow items whose last round's sequences are cut fill their rounds but for the merges; the wider form must
   // beat the narrow one by this factor to be taken (192 sequences of 2048 fp8 tokens, 1.5 rounds of four-head
   // workgroups: 148 us against 134).

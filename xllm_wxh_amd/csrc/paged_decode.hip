@@ -255,8 +255,15 @@ static int fill_params(const xllm_hip_kv_cache* c,
   // kv heads, one per wave, so that a workgroup reads runs of four rows instead of single rows a token's
   // width apart (fp8, 128 x 8192 tokens: 391 -> 338 us; HND 325).  Over a 16-bit cache, whose rows are 256
   // bytes, it measured the same as one head per item (166 us), so those keep the simpler form.
-  const bool side_by_side = variant == kMfmaD128 && quant && c->stride_head == c->head_dim &&
-                            c->stride_slot >= (int64_t)c->num_kv_heads * c->head_dim &&
+  // At head_dim 64 such rows are 64 bytes, two kv heads to a 128-byte line: there the waves of a workgroup should
+  // attend neighbouring heads wherever they can, and walk their tokens in step (see DecodeParams::lockstep
+  // below), whatever the sequences' lengths (int8, 14q/2kv, 512 x 16384 tokens: 542 us with four waves to a
+  // head, against 349 in HND).
+  const bool short_rows = variant == kMfmaD64 && quant && c->stride_head == c->head_dim && c->num_kv_heads > 1 &&
+                          c->stride_slot >= (int64_t)c->num_kv_heads * c->head_dim;
+  const bool side_by_side = ((variant == kMfmaD128 && quant && c->stride_head == c->head_dim &&
+                              c->stride_slot >= (int64_t)c->num_kv_heads * c->head_dim) ||
+                             short_rows) &&
                             option(XLLM_HIP_OPTION_DECODE_ITEM_PER_HEAD) == 0;
   // The same work items serve a large batch of short sequences in any layout, when the host-side lengths say
   // so: a wave that has a kv head's whole sequence to itself runs four times as many tiles between its
@@ -306,17 +313,17 @@ static int fill_params(const xllm_hip_kv_cache* c,
   };
   const bool short_sequences = (variant == kMfmaD128 || variant == kMfmaD64) && a->max_seq_len > 0 && a->total_kv_len > 0 &&
                                four_head_items >= (nearly_equal ? slots : 4 * slots) &&
-                               a->total_kv_len <= (int64_t)p.batch * (quant ? R.wave_per_head_max_mean_quant : variant == kMfmaD64 ? R.wave_per_head_max_mean_d64 : R.wave_per_head_max_mean_16bit) &&
+                               (short_rows || a->total_kv_len <= (int64_t)p.batch * (quant ? R.wave_per_head_max_mean_quant : variant == kMfmaD64 ? R.wave_per_head_max_mean_d64 : R.wave_per_head_max_mean_16bit)) &&
                                (!nearly_equal || wider_items_pay((int64_t)p.batch * c->num_kv_heads, kHeadsPerItem)) &&
                                option(XLLM_HIP_OPTION_DECODE_ITEM_PER_HEAD) == 0;
   // (the four-head items of a 1-byte cache with its heads side by side gain 16 % from the layout alone, 391 -> 338
   // us: they too give way where their rounds would be poorly filled and the host-side lengths show it)
   const bool side_by_side_pays = !(a->max_seq_len > 0 && a->total_kv_len > 0 && nearly_equal) ||
-                                 wider_items_pay((int64_t)p.batch * c->num_kv_heads, kHeadsPerItem, R.side_by_side_gain);
+                                 wider_items_pay((int64_t)p.batch * c->num_kv_heads, kHeadsPerItem, short_rows ? R.short_rows_gain : R.side_by_side_gain);
   p.item_heads = item_heads_of(p.rows, c->num_kv_heads, (side_by_side && side_by_side_pays) || short_sequences);
   // 17 to 32 rows per kv head over such a cache (the heads side by side, rows of 128 bytes): the 32-row kernel's
   // form of the four-head item, eight waves to the workgroup and one workgroup to a CU.
-  const bool side_by_side32 = side_by_side && p.rows > 16 && p.rows <= kMaxRowsPerItem && p.rows_per_item == kMaxRowsPerItem;
+  const bool side_by_side32 = side_by_side && variant == kMfmaD128 && p.rows > 16 && p.rows <= kMaxRowsPerItem && p.rows_per_item == kMaxRowsPerItem;
   if (side_by_side32) p.item_heads = item_heads_of(p.rows, c->num_kv_heads, true, true);
   p.heads_per_item = c->num_kv_heads / p.item_heads;
   p.head_dim = c->head_dim;
@@ -495,11 +502,11 @@ static int fill_params(const xllm_hip_kv_cache* c,
   // 192 sequences, 1.5 rounds of such workgroups, would take 148 against 134: see wider_items_pay).
   p.wave_items = 0;
   if ((variant == kMfmaD128 || variant == kMfmaD64) && p.rows <= 16 && p.heads_per_item == 1 && hints && nearly_equal &&
-      a->total_kv_len <= (int64_t)p.batch * (quant ? R.wave_per_head_max_mean_quant : variant == kMfmaD64 ? R.wave_per_head_max_mean_d64 : R.wave_per_head_max_mean_16bit) &&
+      (short_rows || a->total_kv_len <= (int64_t)p.batch * (quant ? R.wave_per_head_max_mean_quant : variant == kMfmaD64 ? R.wave_per_head_max_mean_d64 : R.wave_per_head_max_mean_16bit)) &&
       option(XLLM_HIP_OPTION_DECODE_ITEM_PER_HEAD) == 0) {
     const int64_t items = (int64_t)p.batch * c->num_kv_heads;
     const int per_group = items >= kHeadsPerItem * slots ? 1 : items >= 2 * slots ? 2 : 0;
-    if (per_group != 0 && wider_items_pay(items, per_group == 1 ? kWaves : 2, 0.0, p.arith_whole > 0)) {
+    if (per_group != 0 && wider_items_pay(items, per_group == 1 ? kWaves : 2, short_rows ? R.short_rows_gain : 0.0, p.arith_whole > 0)) {
       p.wave_items = per_group;
       p.fixed_chunk = 1 << 30;
       p.implicit_plan = 1;
@@ -525,10 +532,7 @@ static int fill_params(const xllm_hip_kv_cache* c,
     // 266 -> 206; 8 kv heads, 128 x 8192 tokens 314 -> 253 us, 1024 x 1024 tokens 268 -> 237.  Rows of a whole
     // line gain nothing from it and lose the waves' independence (fp8, head_dim 128, 128 x 8192 tokens over
     // NHD: 350 -> 365 us): not those.
-    p.lockstep = (p.wave_items || p.heads_per_item > 1) && c->num_kv_heads > 1 && quant && variant == kMfmaD64 &&
-                         shared_by(c->stride_head * elem_bytes(c->dtype)) > 1
-                     ? 1
-                     : 0;
+    p.lockstep = (p.wave_items || p.heads_per_item > 1) && short_rows ? 1 : 0;
     if (heads_per_line > c->num_kv_heads) heads_per_line = c->num_kv_heads;
     while (heads_per_line > 1 && c->num_kv_heads % heads_per_line != 0) --heads_per_line;
   }
