@@ -787,8 +787,8 @@ def test_four_head_items_for_many_short_sequences(gpu, name, kv, qdt, layout, Hq
     assert torch.equal(out, out2) and torch.equal(lse, lse2)
 
 
-@pytest.mark.parametrize("kv,qdt", [("fp8", "bf16"), ("int8", "bf16"), ("int8", "fp16"), ("bf16", "bf16")])
-@pytest.mark.parametrize("Hq,Hkv,n", [(32, 8, 1), (16, 4, 2), (14, 2, 1)])
+@pytest.mark.parametrize("kv,qdt,Hq,Hkv,n", [("fp8", "bf16", 32, 8, 1), ("int8", "bf16", 16, 4, 2), ("int8", "fp16", 32, 8, 1),
+                                            ("bf16", "bf16", 32, 8, 1), ("int8", "bf16", 14, 2, 1), ("fp8", "bf16", 14, 2, 1)])
 def test_work_items_of_four_kv_heads_over_nhd_at_head_dim_64(gpu, kv, qdt, Hq, Hkv, n):
     """head_dim 64 over a 1-byte NHD cache (rows of 64 bytes, two kv heads to a 128-byte line): work items of four kv
     heads for any step, split sequences included, their waves walking the tokens in step; 16-bit caches and two kv
