@@ -38,6 +38,7 @@ def kernels_for(rows, rng):
     if rows <= 16:
         out += [(512, 256, 32, 512, 32), (512, 256, 32, 512, 64), (256, 256, 32, 512, 16)]
         out += [(512, 256, 32, 512, 32, 4)]  # work items of four kv heads (a cache whose heads lie side by side)
+        out += [(512, 256, 32, 512, 64, 4), (512, 512, 32, 512, 64, 4)]  # ... at head_dim 64 (1-byte rows of 64 bytes)
         out += [(512, 512, 32, 512, 32), (512, 384, 32, 512, 32)]  # 1-byte caches: small batches are cut for more slots
     elif rows <= 32:
         out += [(1024, 1024, 32, 512, 32), (1024, 1024, 32, 512, 64), (512, 512, 32, 512, 16)]
