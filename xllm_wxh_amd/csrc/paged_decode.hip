@@ -505,7 +505,11 @@ static int fill_params(const xllm_hip_kv_cache* c,
       (short_rows || a->total_kv_len <= (int64_t)p.batch * (quant ? R.wave_per_head_max_mean_quant : variant == kMfmaD64 ? R.wave_per_head_max_mean_d64 : R.wave_per_head_max_mean_16bit)) &&
       option(XLLM_HIP_OPTION_DECODE_ITEM_PER_HEAD) == 0) {
     const int64_t items = (int64_t)p.batch * c->num_kv_heads;
-    const int per_group = items >= kHeadsPerItem * slots ? 1 : items >= 2 * slots ? 2 : 0;
+    // (64-byte rows, see short_rows: two waves to an item from one round of items on, if that leaves more workgroups than
+    // CUs — int8, 14q/2kv over NHD, 400 x 4096 tokens 111 -> 102 us, 500 x 2048 65 -> 59; 256 x 8192, a workgroup per CU, 130 -> 133)
+    const int per_group = items >= kHeadsPerItem * slots ? 1
+                          : items >= 2 * slots || (short_rows && items >= slots && items / 2 > cus) ? 2
+                                                                                                     : 0;
     if (per_group != 0 && wider_items_pay(items, per_group == 1 ? kWaves : 2, short_rows ? R.short_rows_gain : 0.0, p.arith_whole > 0)) {
       p.wave_items = per_group;
       p.fixed_chunk = 1 << 30;
