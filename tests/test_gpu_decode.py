@@ -815,7 +815,7 @@ def test_work_items_of_four_kv_heads_over_nhd_at_head_dim_64(gpu, kv, qdt, Hq, H
     ref, lse_ref = case.oracle()
     assert max_abs_err(out_h, ref) <= tol and lse_err(lse_h, lse_ref) <= LSE_TOL
     # long equal sequences with host-side lengths: not split, a wave (or two) per (sequence, kv head)
-    eq = Case(300, Hq, Hkv, 64, 32, [1100 + (i % 3) for i in range(300)], n=n, kv=kv, qdt=qdt, layout="NHD", seed=98)
+    eq = Case(280, Hq, Hkv, 64, 32, [700 + (i % 3) for i in range(280)], n=n, kv=kv, qdt=qdt, layout="NHD", seed=98)
     ref, lse_ref = eq.oracle()
     out, lse = eq.run(hints=True)
     assert max_abs_err(out, ref) <= tol and lse_err(lse, lse_ref) <= LSE_TOL
@@ -943,7 +943,6 @@ def test_sequences_of_a_partly_filled_round_are_cut(gpu, kv, qdt, name, Hq, Hkv,
 @pytest.mark.parametrize("name,B,L,kv,qdt", [
     ("cut in four, the 33rd sequence finer", 33, 6200, "int8", "bf16"),
     ("cut in two, the last two sequences finer", 66, 3400, "int8", "bf16"),
-    ("cut in two, the last two sequences finer", 66, 3400, "fp8", "fp16"),
     ("whole, the last two sequences cut", 130, 1100, "int8", "fp16"),
     ("16-bit cache: whole, the last two sequences cut", 66, 1300, "bf16", "bf16"),
 ])
