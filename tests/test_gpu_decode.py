@@ -830,6 +830,9 @@ def test_work_items_of_four_kv_heads_over_nhd_at_head_dim_64(gpu, kv, qdt, Hq, H
     # as many tiles as the longest of the four (lengths either side of a tile's end)
     ("two kv heads, int8 over NHD, a wave per item", "int8", "bf16", "NHD", 14, 2, 1, 32, [250 + 5 * (i % 7) for i in range(1024)]),
     ("two kv heads, fp8 over NHD, two waves per item", "fp8", "bf16", "NHD", 14, 2, 1, 32, [1000 + 9 * (i % 5) for i in range(1000)]),
+    # ... and over a schedule that is kept (ragged lengths, one sequence split, some empty): two items to a workgroup too
+    ("two kv heads, int8 over NHD, ragged", "int8", "bf16", "NHD", 14, 2, 1, 32, None),
+    ("two kv heads, fp8 over NHD, ragged, two draft tokens", "fp8", "fp16", "NHD", 14, 2, 2, 64, None),
 ])
 def test_items_per_wave_at_head_dim_64(gpu, name, kv, qdt, layout, Hq, Hkv, n, bs, lens):
     """The same work items (four kv heads, or four neighbouring items, one per wave) at head_dim 64."""

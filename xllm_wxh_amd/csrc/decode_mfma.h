@@ -1092,8 +1092,8 @@ __device__ inline int first_visible_tile(const DecodeParams& p, const Item& it) 
 // Waves per SIMD the 16-row kernel is compiled for: head_dim 256 needs the registers of one.
 constexpr int decode_waves_per_simd(int tok) { return tok == 0 ? 1 : 2; }
 
-// HEADS (with DecodeParams::wave_items: four neighbouring work items, one per wave, for steps that are not
-// split): a work item covers kWaves neighbouring kv heads of a sequence chunk and wave w attends head
+// HEADS (with DecodeParams::wave_items: four neighbouring work items, one per wave, or two of two waves each; for steps
+// that are not split, and the latter over any schedule, the merge kernel combining what is split): a work item covers kWaves neighbouring kv heads of a sequence chunk and wave w attends head
 // it.hk + w over all of the chunk's tokens (instead of the four waves sharing one head's tokens).  For a
 // cache whose kv heads lie side by side within a token (the NHD layout) the workgroup then reads runs of
 // four rows — 512 bytes of a 1-byte cache — at about the same time, where a workgroup per head reads

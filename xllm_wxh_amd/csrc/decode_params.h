@@ -46,7 +46,7 @@ struct DecodeParams {
   int32_t heads_per_item;  // kv heads one work item covers: 1, or 4 (one per wave of the 16-row kernel; see fill_params)
   int32_t item_heads;      // num_kv_heads / heads_per_item: work items per sequence chunk and row group
   int32_t eight_waves;     // != 0: the 16-row kernel runs eight waves per work item whatever the launch's size (1-byte caches)
-  int32_t wave_items;      // 1: every wave of a 16-row workgroup is a work item of its own (item 4 * workgroup + wave); 2: two waves to an item, two items to a workgroup; steps that are not split only
+  int32_t wave_items;      // 1: every wave of a 16-row workgroup is a work item of its own (item 4 * workgroup + wave); 2: two waves to an item, two items to a workgroup; steps that are not split, and (2 only) a 1-byte cache of 64-byte rows with an even number of kv heads, whose split sequences the merge kernel combines
   int32_t lockstep;        // != 0: the 16-row kernel's waves, each attending a kv head of its own, walk their tokens in step (its LOCK form; 1-byte caches at head_dim 64 whose kv heads lie side by side)
   int32_t group;  // q heads per kv head
   int32_t rows;   // group * n

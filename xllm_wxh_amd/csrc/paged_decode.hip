@@ -518,6 +518,20 @@ static int fill_params(const xllm_hip_kv_cache* c,
       p.arith_whole = 0;
     }
   }
+  // 64-byte rows whose kv heads come in pairs but not in fours (short_rows; a tensor-parallel shard's two), in a
+  // step that keeps its schedule, split or ragged: the same workgroups of two items, two waves each, over the
+  // schedule's items as they are — neighbours 2j and 2j + 1 in their order are a chunk's kv heads 2j and 2j + 1, the
+  // two halves of the same lines — and split sequences go to the merge kernel, as those of four-head items do.
+  // From a round of items on, more workgroups than CUs (a small batch keeps eight waves to an item).  int8, 14q/2kv
+  // over NHD: 300 x 12000 tokens 235 -> 216 us (HND 163), 272 x 8192 150 -> 144, 260 x 16384 277 -> 268; lognormal
+  // lengths, 512 sequences around 4096 tokens 194 -> 192, 1024 around 512 75 -> 73.
+  if (p.wave_items == 0 && short_rows && p.rows <= 16 && p.heads_per_item == 1 && c->num_kv_heads % 2 == 0 &&
+      (int64_t)p.batch * c->num_kv_heads >= slots && (int64_t)p.batch * c->num_kv_heads / 2 > cus &&
+      option(XLLM_HIP_OPTION_DECODE_ITEM_PER_HEAD) == 0) {
+    p.wave_items = 2;
+    p.fused_merge = 0;
+    p.eight_waves = 0;
+  }
   // XCD clusters: the row groups of a (chunk, kv head); and the kv heads whose rows share 128-byte
   // lines — scale rows shorter than a line (HND: block_size * 4 bytes per head; NHD: the heads of a
   // slot are adjacent floats) or cache rows shorter than a line (NHD with 64 one-byte elements).
